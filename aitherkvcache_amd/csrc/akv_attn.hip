@@ -1,0 +1,351 @@
+// Paged decode attention over a uniform TurboQuant cache (2/3/4-bit):
+//   prologue  : q' = Pi q for every (sequence, query head) + per-sequence block prefix
+//   main      : stream-K walk over (sequence, block) pairs, all kv heads per workgroup
+//   reduce    : log-sum-exp merge of the partials, /l, out = Pi^T a, cast
+// This file holds the prologue, the reduce and the general main kernel (any of the three
+// bit widths, head_dim 64/128/256).  The MFMA main kernel for 4-bit / head_dim 128 is in
+// akv_attn_mfma.hip and plugs into the same prologue / reduce.
+#include "akv_attn_common.h"
+
+
+// ----------------------------------------------------------------------------------
+// prologue
+// ----------------------------------------------------------------------------------
+template <int QDT>
+__global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
+    const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
+    int S, int QH, int D, const void* context_lens, int cl_itype, int block_size,
+    int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qrot) {
+  __shared__ float q_lds[256];
+  __shared__ int32_t scratch[257];
+  const int b = blockIdx.x;
+  if (b == S * QH) {
+    akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
+    return;
+  }
+  const int s = b / QH, h = b % QH;
+  const int tid = threadIdx.x;
+  if (tid < D) q_lds[tid] = akv_elem<QDT>::load(query, s * qs_seq + h * qs_head + tid);
+  __syncthreads();
+  if (tid < D) {
+    float acc = 0.f;
+    for (int j = 0; j < D; ++j) acc = fmaf(PiT[(size_t)j * D + tid], q_lds[j], acc);
+    qrot[((size_t)s * QH + h) * D + tid] = acc;
+  }
+}
+
+// ----------------------------------------------------------------------------------
+// reduce: one wavefront per (sequence, query head)
+// ----------------------------------------------------------------------------------
+template <int D, int ODT>
+__global__ __launch_bounds__(64) void akv_attn_reduce_kernel(
+    const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
+    const float* __restrict__ part_ml, const float* __restrict__ Pi, int S, int QH, int G,
+    void* __restrict__ out, int64_t os_seq, int64_t os_head) {
+  constexpr int DPL = D / 64;
+  __shared__ float a_lds[D];
+  const int s = blockIdx.x / QH, h = blockIdx.x % QH;
+  const int lane = threadIdx.x;
+  const int b0 = prefix[s], b1 = prefix[s + 1];
+  const int64_t obase = s * os_seq + h * os_head;
+  if (b1 <= b0) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, obase + lane * DPL + i, 0.f);
+    return;
+  }
+  const int total = prefix[S];
+  const int per = (total + G - 1) / G;
+  const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
+  float m = -INFINITY, l = 0.f, acc[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+  for (int w = w_lo; w <= w_hi; ++w) {
+    const size_t slot = (size_t)(w + s) * QH + h;
+    const float ms = part_ml[slot * 2], ls = part_ml[slot * 2 + 1];
+    float alpha, beta;
+    akv_lse_merge(m, l, ms, ls, alpha, beta);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i)
+      acc[i] = alpha * acc[i] + beta * part_acc[slot * D + lane * DPL + i];
+  }
+  const float inv = l > 0.f ? 1.f / l : 1.f;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) a_lds[lane * DPL + i] = acc[i] * inv;
+  __syncthreads();
+  float o[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) o[i] = 0.f;
+  for (int k = 0; k < D; ++k) {
+    const float a = a_lds[k];
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) o[i] = fmaf(a, Pi[(size_t)k * D + lane * DPL + i], o[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, obase + lane * DPL + i, o[i]);
+}
+
+// ----------------------------------------------------------------------------------
+// general main kernel: 8 wavefronts, wavefront <-> kv head.  Per 64-token chunk a wavefront
+// first scores with lanes <-> tokens (packed K row in registers, q' broadcast from LDS),
+// updates the running softmax, then accumulates V with lanes <-> coordinates (V rows and
+// weights staged in the wavefront's own LDS slice).  The query heads of a kv head are taken
+// GQ at a time (GQ = 4 when the GQA ratio is a multiple of 4, else 1).
+// ----------------------------------------------------------------------------------
+#define AKV_ATTN_WAVES 8
+
+template <int D, int BITS, int GQ>
+struct akv_attn_gen_cfg {
+  static constexpr int ROWDW = D * BITS / 32;
+  static constexpr int VROW = ROWDW + 1;  // padded row stride in dwords
+  static constexpr size_t wave_floats = 64 * GQ + 64 * VROW;
+  static size_t lds_bytes(int QH) { return ((size_t)QH * D + AKV_ATTN_WAVES * wave_floats + 16) * 4; }
+};
+
+template <int D, int BITS, int GQ>
+__global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) {
+  typedef akv_attn_gen_cfg<D, BITS, GQ> cfg;
+  constexpr int DPL = D / 64;
+  constexpr int ROWDW = cfg::ROWDW;
+  constexpr int VROW = cfg::VROW;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  float* q_lds = (float*)lds_raw;                          // [QH][D]
+  float* wave_base = q_lds + (size_t)a.QH * D;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* p_lds = wave_base + wave * cfg::wave_floats;      // [64][GQ]
+  uint32_t* v_lds = (uint32_t*)(p_lds + 64 * GQ);          // [64][VROW]
+  float* cen = wave_base + AKV_ATTN_WAVES * cfg::wave_floats;
+
+  if (threadIdx.x < (1 << BITS)) cen[threadIdx.x] = a.centroids[threadIdx.x];
+
+  const int G = gridDim.x;
+  const int total = a.prefix[a.S];
+  const int per = (total + G - 1) / G;
+  const int g0 = blockIdx.x * per;
+  const int g1 = min(total, g0 + per);
+  const int gqa = a.QH / a.KVH;
+  const int bs = a.block_size;
+
+  int g = g0;
+  while (g < g1) {
+    const int s = akv_find_seq(a.prefix, a.S, g);
+    const int sb0 = a.prefix[s], sb1 = a.prefix[s + 1];
+    const int blk_lo = g - sb0;
+    const int blk_hi = min(g1, sb1) - sb0;
+    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
+    const int t0 = blk_lo * bs;
+    const int t1 = (int)min((int64_t)blk_hi * bs, ctx);
+    g = sb0 + blk_hi;
+
+    __syncthreads();  // previous segment done with q_lds
+    for (int i = threadIdx.x; i < a.QH * D; i += blockDim.x)
+      q_lds[i] = a.qrot[(size_t)s * a.QH * D + i];
+    __syncthreads();
+
+    for (int h = wave; h < a.KVH; h += AKV_ATTN_WAVES) {
+      for (int qg = 0; qg < gqa; qg += GQ) {
+        float m[GQ], l[GQ], acc[GQ][DPL];
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) {
+          m[q] = -INFINITY; l[q] = 0.f;
+#pragma unroll
+          for (int i = 0; i < DPL; ++i) acc[q][i] = 0.f;
+        }
+        const float* qh = q_lds + (size_t)(h * gqa + qg) * D;
+
+        for (int c0 = t0; c0 < t1; c0 += 64) {
+          const int t = c0 + lane;
+          const bool valid = t < t1;
+          const int tc = valid ? t : t1 - 1;
+          const int64_t phys = akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs);
+          const int pos = tc % bs;
+          // ---- scores: lanes <-> tokens; 32 coordinates (= BITS dwords of codes) per step
+          const uint32_t* kr = (const uint32_t*)(a.kp + phys * a.kps_blk + pos * a.kps_pos + h * a.kps_head);
+          float sc[GQ];
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+#pragma unroll 1
+          for (int u = 0; u < D / 32; ++u) {
+            uint32_t kw[BITS];
+#pragma unroll
+            for (int i = 0; i < BITS; ++i) kw[i] = kr[u * BITS + i];
+            const float* qu = qh + u * 32;
+#pragma unroll
+            for (int d = 0; d < 32; ++d) {
+              const uint32_t code = akv_stream_code<BITS>(d, [&](int o) { return (kw[o >> 2] >> (8 * (o & 3))) & 0xffu; });
+              const float kv = cen[code];
+#pragma unroll
+              for (int q = 0; q < GQ; ++q) sc[q] = fmaf(qu[q * D + d], kv, sc[q]);
+            }
+          }
+          const float knorm = a.kn[phys * a.kns_blk + pos * a.kns_pos + h * a.kns_head];
+          const float vnorm = valid ? a.vn[phys * a.vns_blk + pos * a.vns_pos + h * a.vns_head] : 0.f;
+          // ---- running softmax
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) {
+            const float sv = valid ? sc[q] * knorm * a.scale : -INFINITY;
+            const float mt = akv_wave_max(sv);
+            const float mn = fmaxf(m[q], mt);
+            const float alpha = __expf(m[q] - mn);
+            const float p = valid ? __expf(sv - mn) : 0.f;
+            l[q] = l[q] * alpha + p;
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) acc[q][i] *= alpha;
+            m[q] = mn;
+            p_lds[lane * GQ + q] = p * vnorm;
+          }
+          // ---- stage the V rows
+          {
+            const uint32_t* vr = (const uint32_t*)(a.vp + phys * a.vps_blk + pos * a.vps_pos + h * a.vps_head);
+#pragma unroll
+            for (int i = 0; i < ROWDW; ++i) v_lds[lane * VROW + i] = vr[i];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          // ---- values: lanes <-> coordinates
+          const int nt = min(64, t1 - c0);
+          for (int tt = 0; tt < nt; ++tt) {
+            const uint8_t* vb = (const uint8_t*)(v_lds + tt * VROW);
+            float vv[DPL];
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+              const uint32_t code = akv_stream_code<BITS>(lane * DPL + i, [&](int o) { return (uint32_t)vb[o]; });
+              vv[i] = cen[code];
+            }
+#pragma unroll
+            for (int q = 0; q < GQ; ++q) {
+              const float pw = p_lds[tt * GQ + q];
+#pragma unroll
+              for (int i = 0; i < DPL; ++i) acc[q][i] = fmaf(pw, vv[i], acc[q][i]);
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        // ---- partial for this (workgroup, sequence, query heads)
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) {
+          const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + qg + q);
+          const float lsum = akv_wave_sum(l[q]);
+#pragma unroll
+          for (int i = 0; i < DPL; ++i) a.part_acc[slot * D + lane * DPL + i] = acc[q][i];
+          if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------
+// host entry
+// ----------------------------------------------------------------------------------
+// MFMA main kernel (akv_attn_mfma.hip); AKV_ERR_UNSUPPORTED when it does not apply.
+int akv_attn_mfma_try(const akv_attn_args& a, int d, int bits, int grid, hipStream_t stream);
+
+extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
+  if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
+  return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, d, akv_attn_grid()).bytes;
+}
+
+template <int D, int BITS, int GQ>
+static int akv_launch_attn_general_gq(const akv_attn_args& a, int grid, hipStream_t stream) {
+  const size_t lds = akv_attn_gen_cfg<D, BITS, GQ>::lds_bytes(a.QH);
+  if (lds > 160 * 1024)
+    return akv_fail(AKV_ERR_UNSUPPORTED, "paged_attn: num_q_heads*head_dim too large for LDS (%zu bytes)", lds);
+  AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_general_kernel<D, BITS, GQ>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  akv_attn_general_kernel<D, BITS, GQ><<<grid, 512, lds, stream>>>(a);
+  AKV_LAUNCH_CHECK("akv_attn_general_kernel");
+  return AKV_OK;
+}
+
+template <int D, int BITS>
+static int akv_launch_attn_general(const akv_attn_args& a, int grid, hipStream_t stream) {
+  const int gqa = a.QH / a.KVH;
+  if (gqa % 4 == 0) return akv_launch_attn_general_gq<D, BITS, 4>(a, grid, stream);
+  return akv_launch_attn_general_gq<D, BITS, 1>(a, grid, stream);
+}
+
+template <int D>
+static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, int G, void* out,
+                             int64_t os_seq, int64_t os_head, hipStream_t stream) {
+  const int grid = a.S * a.QH;
+  switch (odt) {
+    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+  }
+  AKV_LAUNCH_CHECK("akv_attn_reduce_kernel");
+  return AKV_OK;
+}
+
+extern "C" int akv_paged_attn(
+    const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+    const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+    const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
+    const uint8_t* v_packed, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+    const float* v_norms, int64_t vns_blk, int64_t vns_pos, int64_t vns_head,
+    const void* block_tables, int bt_itype, int64_t bt_stride,
+    const void* context_lens, int cl_itype,
+    const void* rot_prep, const float* centroids, int bits,
+    void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+    int num_seqs, int num_q_heads, int num_kv_heads, int d,
+    int block_size, int64_t max_blocks_per_seq, float scale,
+    void* workspace, size_t workspace_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  AKV_REQUIRE(num_seqs >= 0 && num_q_heads > 0 && num_kv_heads > 0, "akv_paged_attn: bad head/seq counts");
+  AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_paged_attn: num_q_heads %% num_kv_heads != 0");
+  AKV_REQUIRE(akv_valid_dtype(q_dtype) && akv_valid_dtype(out_dtype), "akv_paged_attn: bad dtype");
+  AKV_REQUIRE(akv_valid_itype(bt_itype) && akv_valid_itype(cl_itype), "akv_paged_attn: bad index type");
+  AKV_REQUIRE(block_size > 0 && max_blocks_per_seq >= 0, "akv_paged_attn: bad block_size / table width");
+  AKV_REQUIRE(bits >= 2 && bits <= 4, "akv_paged_attn: bits=%d not in {2,3,4}", bits);
+  if (!(d == 64 || d == 128 || d == 256))
+    return akv_fail(AKV_ERR_UNSUPPORTED, "akv_paged_attn: head_dim=%d not in {64,128,256}", d);
+  if (num_seqs == 0) return AKV_OK;
+  AKV_REQUIRE(query && out && rot_prep && centroids && context_lens, "akv_paged_attn: null pointer");
+  AKV_REQUIRE(max_blocks_per_seq == 0 || (k_packed && k_norms && v_packed && v_norms && block_tables),
+              "akv_paged_attn: null cache pointer");
+  AKV_REQUIRE((((uintptr_t)k_packed | (uintptr_t)v_packed | (uintptr_t)kps_blk | (uintptr_t)kps_pos |
+                (uintptr_t)kps_head | (uintptr_t)vps_blk | (uintptr_t)vps_pos | (uintptr_t)vps_head) & 3) == 0,
+              "akv_paged_attn: packed rows must be 4-byte aligned");
+  const int G = akv_attn_grid();
+  AKV_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0, "akv_paged_attn: workspace null or not 256-byte aligned");
+  akv_attn_ws ws = akv_attn_ws_layout(workspace, num_seqs, num_q_heads, d, G);
+  if (workspace_bytes < ws.bytes)
+    return akv_fail(AKV_ERR_WORKSPACE, "akv_paged_attn: workspace %zu < %zu bytes", workspace_bytes, ws.bytes);
+
+  const float* Pi = (const float*)rot_prep;
+  const float* PiT = Pi + (size_t)d * d;
+  const int pgrid = num_seqs * num_q_heads + 1;
+#define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot)
+  if (q_dtype == AKV_F16) AKV_PRO(AKV_F16); else if (q_dtype == AKV_BF16) AKV_PRO(AKV_BF16); else AKV_PRO(AKV_F32);
+#undef AKV_PRO
+  AKV_LAUNCH_CHECK("akv_attn_prologue_kernel");
+
+  akv_attn_args a;
+  a.kp = k_packed; a.kps_blk = kps_blk; a.kps_pos = kps_pos; a.kps_head = kps_head;
+  a.kn = k_norms; a.kns_blk = kns_blk; a.kns_pos = kns_pos; a.kns_head = kns_head;
+  a.vp = v_packed; a.vps_blk = vps_blk; a.vps_pos = vps_pos; a.vps_head = vps_head;
+  a.vn = v_norms; a.vns_blk = vns_blk; a.vns_pos = vns_pos; a.vns_head = vns_head;
+  a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
+  a.context_lens = context_lens; a.cl_itype = cl_itype;
+  a.centroids = centroids;
+  a.S = num_seqs; a.QH = num_q_heads; a.KVH = num_kv_heads; a.block_size = block_size;
+  a.max_blocks_per_seq = max_blocks_per_seq; a.scale = scale;
+  a.prefix = ws.prefix; a.qrot = ws.qrot; a.part_acc = ws.part_acc; a.part_ml = ws.part_ml;
+
+  int rc = akv_attn_mfma_try(a, d, bits, G, stream);
+  if (rc == AKV_ERR_UNSUPPORTED) {
+    rc = AKV_ERR_UNSUPPORTED;
+#define AKV_CASE(DD, BB) if (d == DD && bits == BB) rc = akv_launch_attn_general<DD, BB>(a, G, stream);
+    AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
+    AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
+    AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+#undef AKV_CASE
+  }
+  if (rc) return rc;
+  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
+  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
+  return akv_launch_reduce<256>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
+}

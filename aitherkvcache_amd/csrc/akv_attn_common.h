@@ -1,0 +1,134 @@
+// Work partition shared by the paged decode-attention kernels.
+//
+// The (sequence, KV block) pairs of a batch are laid end to end into one global block axis
+// of length total = sum_i ceil(ctx_i / block_size).  The main kernel runs a fixed grid of G
+// workgroups; workgroup w owns global blocks [w*per, (w+1)*per) with per = ceil(total / G),
+// for ALL kv heads, and walks the sequences that range intersects.  Every (workgroup,
+// sequence) intersection produces one partial (running max, running sum, unnormalised
+// accumulator) per query head, stored in slot w + seq -- unique because both w and seq are
+// non-decreasing along the walk and at least one of them grows at every step.  A reduce
+// kernel merges the slots of a sequence with the log-sum-exp rule
+// (aither_kvcache/fused_attention.py:513-522) and applies the inverse rotation.
+// Everything is derived on the device from context_lens, so the launch needs no host
+// synchronisation and the sequence can be recorded into a HIP graph.
+#pragma once
+#include "akv_common.h"
+
+#define AKV_ATTN_WG_PER_CU 2
+
+struct akv_attn_args {
+  const uint8_t* kp; int64_t kps_blk, kps_pos, kps_head;
+  const float* kn;   int64_t kns_blk, kns_pos, kns_head;
+  const uint8_t* vp; int64_t vps_blk, vps_pos, vps_head;
+  const float* vn;   int64_t vns_blk, vns_pos, vns_head;
+  const void* block_tables; int bt_itype; int64_t bt_stride;
+  const void* context_lens; int cl_itype;
+  const float* centroids;
+  int S, QH, KVH, block_size;
+  int64_t max_blocks_per_seq;
+  float scale;
+  const int32_t* prefix;
+  const float* qrot;
+  float* part_acc;
+  float* part_ml;
+};
+
+static inline int akv_attn_grid() {
+  int cus = akv_cached_cu_count();
+  return (cus > 0 ? cus : 256) * AKV_ATTN_WG_PER_CU;
+}
+
+static inline size_t akv_align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Workspace carve-up.  acc_floats = floats of accumulator per query head
+// (head_dim for the uniform codec, 256 for tq35).
+struct akv_attn_ws {
+  int32_t* prefix;   // [S + 1] exclusive prefix of blocks per sequence; prefix[S] = total
+  float* qrot;       // [S][QH][acc_floats] transformed queries
+  float* part_acc;   // [G + S][QH][acc_floats]
+  float* part_ml;    // [G + S][QH][2]  (max, sum)
+  size_t bytes;
+};
+
+static inline akv_attn_ws akv_attn_ws_layout(void* base, int S, int QH, int acc_floats, int G) {
+  akv_attn_ws w;
+  size_t off = 0;
+  w.prefix = (int32_t*)((char*)base + off);
+  off += akv_align256((size_t)(S + 1) * 4);
+  w.qrot = (float*)((char*)base + off);
+  off += akv_align256((size_t)S * QH * acc_floats * 4);
+  w.part_acc = (float*)((char*)base + off);
+  off += akv_align256((size_t)(G + S) * QH * acc_floats * 4);
+  w.part_ml = (float*)((char*)base + off);
+  off += akv_align256((size_t)(G + S) * QH * 2 * 4);
+  w.bytes = off;
+  return w;
+}
+
+// blocks a sequence occupies, clamped to the table width
+__device__ __forceinline__ int akv_seq_blocks(const void* context_lens, int cl_itype, int s,
+                                              int block_size, int64_t max_blocks_per_seq) {
+  int64_t ctx = akv_load_index(context_lens, cl_itype, s);
+  if (ctx < 0) ctx = 0;
+  int64_t nb = (ctx + block_size - 1) / block_size;
+  if (nb > max_blocks_per_seq) nb = max_blocks_per_seq;
+  return (int)nb;
+}
+
+__device__ __forceinline__ int64_t akv_seq_tokens(const void* context_lens, int cl_itype, int s,
+                                                  int block_size, int64_t max_blocks_per_seq) {
+  int64_t ctx = akv_load_index(context_lens, cl_itype, s);
+  if (ctx < 0) ctx = 0;
+  const int64_t cap = max_blocks_per_seq * block_size;
+  return ctx < cap ? ctx : cap;
+}
+
+// One workgroup (256 threads) writes prefix[0..S].
+__device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, int cl_itype, int S,
+                                                      int block_size, int64_t max_blocks_per_seq,
+                                                      int32_t* prefix, int32_t* scratch /*[257] LDS*/) {
+  const int tid = threadIdx.x;
+  const int chunk = (S + 255) / 256;
+  const int lo = min(S, tid * chunk), hi = min(S, lo + chunk);
+  int sum = 0;
+  for (int s = lo; s < hi; ++s) sum += akv_seq_blocks(context_lens, cl_itype, s, block_size, max_blocks_per_seq);
+  scratch[tid] = sum;
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int t = 0; t < 256; ++t) {
+      const int v = scratch[t];
+      scratch[t] = run;
+      run += v;
+    }
+    scratch[256] = run;
+  }
+  __syncthreads();
+  int run = scratch[tid];
+  for (int s = lo; s < hi; ++s) {
+    prefix[s] = run;
+    run += akv_seq_blocks(context_lens, cl_itype, s, block_size, max_blocks_per_seq);
+  }
+  if (tid == 0) prefix[S] = scratch[256];
+}
+
+// largest s with prefix[s] <= g  (prefix non-decreasing, prefix[0] = 0, g < prefix[S])
+__device__ __forceinline__ int akv_find_seq(const int32_t* __restrict__ prefix, int S, int g) {
+  int lo = 0, hi = S;  // invariant: prefix[lo] <= g < prefix[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (prefix[mid] <= g) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// merge (m, l, acc) <- (m, l, acc) (+) (ms, ls, accs)
+__device__ __forceinline__ void akv_lse_merge(float& m, float& l, float ms, float ls,
+                                              float& alpha, float& beta) {
+  const float mn = fmaxf(m, ms);
+  if (mn == -INFINITY) { alpha = 1.f; beta = 0.f; return; }
+  alpha = __expf(m - mn);
+  beta = __expf(ms - mn);
+  l = alpha * l + beta * ls;
+  m = mn;
+}

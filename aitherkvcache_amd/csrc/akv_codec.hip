@@ -1,0 +1,503 @@
+// TurboQuant codec kernels: rotation preparation, quantize+pack, unpack+lookup, encode
+// (flat and paged scatter), decode.  General kernels (any float dtype, head_dim 64/128/256,
+// 2/3/4-bit); the MFMA fast path for fp16 / head_dim 128 lives in akv_encode_mfma.hip.
+#include "akv_common.h"
+
+// ----------------------------------------------------------------------------------
+// host state
+// ----------------------------------------------------------------------------------
+char* akv_error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+int akv_cached_cu_count() {
+  static int cached = -1;
+  if (cached < 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cached = prop.multiProcessorCount;
+    else
+      return 0;
+  }
+  return cached;
+}
+
+extern "C" const char* akv_version(void) { return "aitherkv-hip 0.1 (gfx950)"; }
+extern "C" const char* akv_last_error(void) { return akv_error_buffer(); }
+extern "C" int akv_device_cu_count(int* cu_count) {
+  AKV_REQUIRE(cu_count != nullptr, "akv_device_cu_count: null output");
+  *cu_count = akv_cached_cu_count();
+  if (*cu_count <= 0) return akv_fail(AKV_ERR_HIP, "no HIP device available");
+  return AKV_OK;
+}
+
+// ----------------------------------------------------------------------------------
+// rotation preparation
+// ----------------------------------------------------------------------------------
+__global__ void akv_prepare_rotation_kernel(const float* __restrict__ R, float* __restrict__ prep,
+                                            int d) {
+  // 32x32 tiled transpose through LDS; also copies Pi itself.
+  __shared__ float tile[32][33];
+  const int bx = blockIdx.x * 32, by = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 256 threads: ty 0..7
+  for (int r = ty; r < 32; r += 8) {
+    const float v = R[(size_t)(by + r) * d + bx + tx];
+    prep[(size_t)(by + r) * d + bx + tx] = v;
+    tile[r][tx] = v;
+  }
+  __syncthreads();
+  float* RT = prep + (size_t)d * d;
+  for (int r = ty; r < 32; r += 8) RT[(size_t)(bx + r) * d + by + tx] = tile[tx][r];
+}
+
+int akv_prepare_rotation_mfma(const float* rotation, int d, void* prep, hipStream_t stream);
+
+extern "C" size_t akv_rotation_prepared_bytes(int d) { return akv_prep_floats(d) * sizeof(float); }
+
+extern "C" int akv_rotation_prepare(const float* rotation, int d, void* prep, size_t prep_bytes,
+                                    void* stream) {
+  AKV_REQUIRE(rotation && prep, "akv_rotation_prepare: null pointer");
+  AKV_REQUIRE(d == 64 || d == 128 || d == 256, "akv_rotation_prepare: head_dim %d not in {64,128,256}", d);
+  AKV_REQUIRE(prep_bytes >= akv_rotation_prepared_bytes(d), "akv_rotation_prepare: prep buffer too small");
+  AKV_REQUIRE(((uintptr_t)prep & 255) == 0, "akv_rotation_prepare: prep must be 256-byte aligned");
+  dim3 grid(d / 32, d / 32);
+  akv_prepare_rotation_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rotation, (float*)prep, d);
+  AKV_LAUNCH_CHECK("akv_prepare_rotation_kernel");
+  if (d == 128) return akv_prepare_rotation_mfma(rotation, d, prep, (hipStream_t)stream);
+  return AKV_OK;
+}
+
+// ----------------------------------------------------------------------------------
+// quantize + pack / unpack + lookup   (triton_ops.py:220-259)
+// ----------------------------------------------------------------------------------
+template <int BITS>
+__global__ __launch_bounds__(256) void akv_quantize_pack_kernel(
+    const float* __restrict__ y, int64_t n, int d, int64_t y_stride,
+    const float* __restrict__ bnd_g, uint8_t* __restrict__ out, int64_t out_stride) {
+  __shared__ float bnd[16];
+  if (threadIdx.x < (1 << BITS) - 1) bnd[threadIdx.x] = bnd_g[threadIdx.x];
+  __syncthreads();
+  const int P = d * BITS / 8;
+  const int64_t total = n * P;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / P;
+    const int k = (int)(i - row * P);
+    const float* yr = y + row * y_stride;
+    out[row * out_stride + k] =
+        (uint8_t)akv_stream_byte<BITS>(k, [&](int dim) { return akv_search<BITS>(yr[dim], bnd); });
+  }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void akv_unpack_lookup_kernel(
+    const uint8_t* __restrict__ packed, int64_t n, int d, int64_t packed_stride,
+    const float* __restrict__ cen_g, float* __restrict__ out, int64_t out_stride) {
+  __shared__ float cen[16];
+  if (threadIdx.x < (1 << BITS)) cen[threadIdx.x] = cen_g[threadIdx.x];
+  __syncthreads();
+  const int64_t total = n * d;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / d;
+    const int dim = (int)(i - row * d);
+    const uint8_t* pr = packed + row * packed_stride;
+    const uint32_t c = akv_stream_code<BITS>(dim, [&](int o) { return (uint32_t)pr[o]; });
+    out[row * out_stride + dim] = cen[c];
+  }
+}
+
+static inline int akv_grid_for(int64_t work_items, int block) {
+  int64_t g = (work_items + block - 1) / block;
+  int cus = akv_cached_cu_count();
+  int64_t cap = (int64_t)(cus > 0 ? cus : 256) * 8;
+  if (g > cap) g = cap;
+  if (g < 1) g = 1;
+  return (int)g;
+}
+
+extern "C" int akv_quantize_pack(const float* y, int64_t n, int d, int64_t y_stride,
+                                 const float* boundaries, int bits, uint8_t* out,
+                                 int64_t out_stride, void* stream) {
+  AKV_REQUIRE(n >= 0 && d > 0 && d % 8 == 0, "akv_quantize_pack: bad n=%lld d=%d", (long long)n, d);
+  AKV_REQUIRE(bits >= 2 && bits <= 4, "akv_quantize_pack: bits=%d not in {2,3,4}", bits);
+  if (n == 0) return AKV_OK;
+  AKV_REQUIRE(y && boundaries && out, "akv_quantize_pack: null pointer");
+  const int grid = akv_grid_for(n * akv_packed_size(d, bits), 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (bits == 4) akv_quantize_pack_kernel<4><<<grid, 256, 0, s>>>(y, n, d, y_stride, boundaries, out, out_stride);
+  else if (bits == 3) akv_quantize_pack_kernel<3><<<grid, 256, 0, s>>>(y, n, d, y_stride, boundaries, out, out_stride);
+  else akv_quantize_pack_kernel<2><<<grid, 256, 0, s>>>(y, n, d, y_stride, boundaries, out, out_stride);
+  AKV_LAUNCH_CHECK("akv_quantize_pack_kernel");
+  return AKV_OK;
+}
+
+extern "C" int akv_unpack_lookup(const uint8_t* packed, int64_t n, int d, int64_t packed_stride,
+                                 const float* centroids, int bits, float* out, int64_t out_stride,
+                                 void* stream) {
+  AKV_REQUIRE(n >= 0 && d > 0 && d % 8 == 0, "akv_unpack_lookup: bad n=%lld d=%d", (long long)n, d);
+  AKV_REQUIRE(bits >= 2 && bits <= 4, "akv_unpack_lookup: bits=%d not in {2,3,4}", bits);
+  if (n == 0) return AKV_OK;
+  AKV_REQUIRE(packed && centroids && out, "akv_unpack_lookup: null pointer");
+  const int grid = akv_grid_for(n * d, 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (bits == 4) akv_unpack_lookup_kernel<4><<<grid, 256, 0, s>>>(packed, n, d, packed_stride, centroids, out, out_stride);
+  else if (bits == 3) akv_unpack_lookup_kernel<3><<<grid, 256, 0, s>>>(packed, n, d, packed_stride, centroids, out, out_stride);
+  else akv_unpack_lookup_kernel<2><<<grid, 256, 0, s>>>(packed, n, d, packed_stride, centroids, out, out_stride);
+  AKV_LAUNCH_CHECK("akv_unpack_lookup_kernel");
+  return AKV_OK;
+}
+
+// ----------------------------------------------------------------------------------
+// general encode / decode: one workgroup of 4 wavefronts, each wavefront rotates VPW vectors
+// at a time with lanes owning D/64 output coordinates; the matrix (Pi^T for encode, Pi for
+// decode) is staged in LDS as [k][out].
+// ----------------------------------------------------------------------------------
+#define AKV_GEN_WAVES 4
+#define AKV_GEN_VPW 8
+
+
+// acc[v][i] += sum_k in[v][k] * M[k][lane*DPL + i], k in [k0, k0 + KT)
+template <int D, int KT>
+__device__ __forceinline__ void akv_rotate_tile(const float* __restrict__ m_lds,  // [KT][D]
+                                                const float* __restrict__ in_lds, // [VPW][D]
+                                                int k0, int lane,
+                                                float (&acc)[AKV_GEN_VPW][D / 64]) {
+  constexpr int DPL = D / 64;
+#pragma unroll 2
+  for (int k = 0; k < KT; k += 4) {
+    float m[4][DPL];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) m[kk][i] = m_lds[(k + kk) * D + lane * DPL + i];
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v) {
+      const float4 u = *(const float4*)(in_lds + v * D + k0 + k);
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        acc[v][i] = fmaf(m[0][i], u.x, acc[v][i]);
+        acc[v][i] = fmaf(m[1][i], u.y, acc[v][i]);
+        acc[v][i] = fmaf(m[2][i], u.z, acc[v][i]);
+        acc[v][i] = fmaf(m[3][i], u.w, acc[v][i]);
+      }
+    }
+  }
+}
+
+template <int D> struct akv_gen_cfg {
+  static constexpr int KT = (D <= 128) ? D : 64;  // matrix rows staged at a time (<= 64 KiB)
+  static constexpr size_t mat_floats = (size_t)KT * D;
+  static constexpr size_t in_floats = (size_t)AKV_GEN_WAVES * AKV_GEN_VPW * D;
+  static constexpr size_t code_bytes = (size_t)AKV_GEN_WAVES * AKV_GEN_VPW * D;
+  static constexpr size_t lds_bytes = (mat_floats + in_floats) * 4 + code_bytes + 64;
+};
+
+template <int D, int BITS, int XDT, bool PAGED>
+__global__ __launch_bounds__(256) void akv_encode_general_kernel(akv_gen_args a) {
+  constexpr int DPL = D / 64;
+  constexpr int KT = akv_gen_cfg<D>::KT;
+  constexpr int P = D * BITS / 8;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  float* m_lds = (float*)lds_raw;
+  float* in_lds = m_lds + akv_gen_cfg<D>::mat_floats;
+  uint8_t* c_lds = (uint8_t*)(in_lds + akv_gen_cfg<D>::in_floats);
+  float* bnd = (float*)(c_lds + akv_gen_cfg<D>::code_bytes);  // 16 floats
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x < (1 << BITS) - 1) bnd[threadIdx.x] = a.table[threadIdx.x];
+  if (KT == D) {
+    for (int i = threadIdx.x * 4; i < D * D; i += 256 * 4)
+      *(float4*)(m_lds + i) = *(const float4*)(a.mat + i);
+  }
+  __syncthreads();
+
+  float* my_in = in_lds + wave * AKV_GEN_VPW * D;
+  uint8_t* my_c = c_lds + wave * AKV_GEN_VPW * D;
+  const int64_t tile_vecs = AKV_GEN_WAVES * AKV_GEN_VPW;
+  const int64_t num_tiles = (a.n + tile_vecs - 1) / tile_vecs;
+
+  for (int64_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+    const int64_t base = tile * tile_vecs + wave * AKV_GEN_VPW;
+    float nrm[AKV_GEN_VPW];
+    // 1) load, norm, normalise
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v) {
+      const int64_t n = base + v;
+      float xv[DPL];
+      float ss = 0.f;
+      if (n < a.n) {
+        const int64_t off = PAGED ? (n / a.heads) * a.xs0 + (n % a.heads) * a.xs1 : n * a.xs0;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) {
+          xv[i] = akv_elem<XDT>::load(a.x, off + lane * DPL + i);
+          ss = fmaf(xv[i], xv[i], ss);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) xv[i] = 0.f;
+      }
+      ss = akv_wave_sum(ss);
+      nrm[v] = sqrtf(ss);
+      const float den = nrm[v] + 1e-10f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) my_in[v * D + lane * DPL + i] = xv[i] / den;
+    }
+    // 2) rotate
+    float acc[AKV_GEN_VPW][DPL];
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v)
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) acc[v][i] = 0.f;
+    if (KT == D) {
+      __syncthreads();
+      akv_rotate_tile<D, KT>(m_lds, my_in, 0, lane, acc);
+    } else {
+      for (int k0 = 0; k0 < D; k0 += KT) {
+        __syncthreads();
+        for (int i = threadIdx.x * 4; i < KT * D; i += 256 * 4)
+          *(float4*)(m_lds + i) = *(const float4*)(a.mat + (size_t)k0 * D + i);
+        __syncthreads();
+        akv_rotate_tile<D, KT>(m_lds, my_in, k0, lane, acc);
+      }
+    }
+    // 3) codebook search -> code bytes in LDS
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v)
+#pragma unroll
+      for (int i = 0; i < DPL; ++i)
+        my_c[v * D + lane * DPL + i] = (uint8_t)akv_search<BITS>(acc[v][i], bnd);
+    __syncthreads();
+    // 4) pack + store
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v) {
+      const int64_t n = base + v;
+      if (n >= a.n) continue;
+      uint8_t* prow;
+      float* nptr;
+      if (PAGED) {
+        const int64_t tok = n / a.heads, head = n % a.heads;
+        const int64_t slot = akv_load_index(a.slots, a.slot_itype, tok);
+        if (slot < 0) continue;
+        const int64_t blk = slot / a.block_size, pos = slot % a.block_size;
+        if (blk >= a.max_blocks) continue;
+        prow = a.packed + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+        nptr = a.norms + blk * a.ns0 + pos * a.ns1 + head * a.ns2;
+      } else {
+        prow = a.packed + n * a.ps0;
+        nptr = a.norms + n;
+      }
+      const uint8_t* cv = my_c + v * D;
+      for (int k = lane; k < P; k += 64)
+        prow[k] = (uint8_t)akv_stream_byte<BITS>(k, [&](int dim) { return (uint32_t)cv[dim]; });
+      if (lane == 0) *nptr = nrm[v];
+    }
+    __syncthreads();
+  }
+}
+
+template <int D, int BITS, int ODT>
+__global__ __launch_bounds__(256) void akv_decode_general_kernel(akv_gen_args a) {
+  constexpr int DPL = D / 64;
+  constexpr int KT = akv_gen_cfg<D>::KT;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  float* m_lds = (float*)lds_raw;
+  float* in_lds = m_lds + akv_gen_cfg<D>::mat_floats;
+  uint8_t* c_lds = (uint8_t*)(in_lds + akv_gen_cfg<D>::in_floats);
+  float* cen = (float*)(c_lds + akv_gen_cfg<D>::code_bytes);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x < (1 << BITS)) cen[threadIdx.x] = a.table[threadIdx.x];
+  if (KT == D) {
+    for (int i = threadIdx.x * 4; i < D * D; i += 256 * 4)
+      *(float4*)(m_lds + i) = *(const float4*)(a.mat + i);
+  }
+  __syncthreads();
+
+  float* my_in = in_lds + wave * AKV_GEN_VPW * D;
+  const int64_t tile_vecs = AKV_GEN_WAVES * AKV_GEN_VPW;
+  const int64_t num_tiles = (a.n + tile_vecs - 1) / tile_vecs;
+
+  for (int64_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+    const int64_t base = tile * tile_vecs + wave * AKV_GEN_VPW;
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v) {
+      const int64_t n = base + v;
+      const uint8_t* prow = a.packed + (n < a.n ? n : 0) * a.ps0;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        float val = 0.f;
+        if (n < a.n) {
+          const uint32_t c = akv_stream_code<BITS>(lane * DPL + i, [&](int o) { return (uint32_t)prow[o]; });
+          val = cen[c];
+        }
+        my_in[v * D + lane * DPL + i] = val;
+      }
+    }
+    float acc[AKV_GEN_VPW][DPL];
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v)
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) acc[v][i] = 0.f;
+    if (KT == D) {
+      __syncthreads();
+      akv_rotate_tile<D, KT>(m_lds, my_in, 0, lane, acc);
+    } else {
+      for (int k0 = 0; k0 < D; k0 += KT) {
+        __syncthreads();
+        for (int i = threadIdx.x * 4; i < KT * D; i += 256 * 4)
+          *(float4*)(m_lds + i) = *(const float4*)(a.mat + (size_t)k0 * D + i);
+        __syncthreads();
+        akv_rotate_tile<D, KT>(m_lds, my_in, k0, lane, acc);
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < AKV_GEN_VPW; ++v) {
+      const int64_t n = base + v;
+      if (n >= a.n) continue;
+      const float nv = a.norms[n];
+#pragma unroll
+      for (int i = 0; i < DPL; ++i)
+        akv_elem<ODT>::store(a.out, n * a.os0 + lane * DPL + i, acc[v][i] * nv);
+    }
+    __syncthreads();
+  }
+}
+
+template <typename K>
+static int akv_launch_gen(K kernel, const char* name, size_t lds, const akv_gen_args& a, void* stream) {
+  static thread_local const void* configured[64];
+  static thread_local int nconf = 0;
+  bool seen = false;
+  for (int i = 0; i < nconf; ++i) seen |= (configured[i] == (const void*)kernel);
+  if (!seen) {
+    AKV_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (nconf < 64) configured[nconf++] = (const void*)kernel;
+  }
+  const int64_t tile_vecs = AKV_GEN_WAVES * AKV_GEN_VPW;
+  int64_t tiles = (a.n + tile_vecs - 1) / tile_vecs;
+  int cus = akv_cached_cu_count();
+  int64_t cap = (int64_t)(cus > 0 ? cus : 256) * 2;
+  int grid = (int)(tiles < cap ? tiles : cap);
+  kernel<<<grid, 256, lds, (hipStream_t)stream>>>(a);
+  AKV_LAUNCH_CHECK(name);
+  return AKV_OK;
+}
+
+template <int D, int BITS, bool PAGED>
+static int akv_encode_dispatch_dtype(int dt, const akv_gen_args& a, void* stream) {
+  const size_t lds = akv_gen_cfg<D>::lds_bytes;
+  switch (dt) {
+    case AKV_F16: return akv_launch_gen(akv_encode_general_kernel<D, BITS, AKV_F16, PAGED>, "akv_encode_general_kernel", lds, a, stream);
+    case AKV_BF16: return akv_launch_gen(akv_encode_general_kernel<D, BITS, AKV_BF16, PAGED>, "akv_encode_general_kernel", lds, a, stream);
+    default: return akv_launch_gen(akv_encode_general_kernel<D, BITS, AKV_F32, PAGED>, "akv_encode_general_kernel", lds, a, stream);
+  }
+}
+
+template <bool PAGED>
+static int akv_encode_dispatch(int d, int bits, int dt, const akv_gen_args& a, void* stream) {
+#define AKV_CASE(DD, BB) \
+  if (d == DD && bits == BB) return akv_encode_dispatch_dtype<DD, BB, PAGED>(dt, a, stream);
+  AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
+  AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
+  AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+#undef AKV_CASE
+  return akv_fail(AKV_ERR_UNSUPPORTED, "encode: no kernel for head_dim=%d bits=%d", d, bits);
+}
+
+// MFMA fast path (akv_encode_mfma.hip); returns AKV_ERR_UNSUPPORTED when it does not apply.
+int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, int bits,
+                        const void* rot_prep, hipStream_t stream);
+
+static int akv_check_codec_args(const char* fn, int d, int bits) {
+  if (!(d == 64 || d == 128 || d == 256))
+    return akv_fail(AKV_ERR_UNSUPPORTED, "%s: head_dim=%d not in {64,128,256}", fn, d);
+  if (bits < 2 || bits > 4) return akv_fail(AKV_ERR_INVALID, "%s: bits=%d not in {2,3,4}", fn, bits);
+  return AKV_OK;
+}
+
+extern "C" int akv_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride,
+                          const void* rot_prep, const float* boundaries, int bits,
+                          uint8_t* out_packed, int64_t packed_stride, float* out_norms,
+                          void* stream) {
+  AKV_REQUIRE(n >= 0, "akv_encode: n=%lld", (long long)n);
+  AKV_REQUIRE(akv_valid_dtype(x_dtype), "akv_encode: bad dtype %d", x_dtype);
+  int rc = akv_check_codec_args("akv_encode", d, bits);
+  if (rc) return rc;
+  if (n == 0) return AKV_OK;
+  AKV_REQUIRE(x && rot_prep && boundaries && out_packed && out_norms, "akv_encode: null pointer");
+  AKV_REQUIRE(x_stride >= d && packed_stride >= akv_packed_size(d, bits), "akv_encode: stride smaller than row");
+  akv_gen_args a = {};
+  a.x = x; a.n = n; a.xs0 = x_stride; a.heads = 1;
+  a.mat = (const float*)rot_prep + (size_t)d * d;  // Pi^T: [k = input coord][out coord]
+  a.table = boundaries;
+  a.packed = out_packed; a.ps0 = packed_stride;
+  a.norms = out_norms;
+  rc = akv_encode_mfma_try(a, false, x_dtype, d, bits, rot_prep, (hipStream_t)stream);
+  if (rc != AKV_ERR_UNSUPPORTED) return rc;
+  return akv_encode_dispatch<false>(d, bits, x_dtype, a, stream);
+}
+
+extern "C" int akv_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads,
+                                int d, int64_t xs_token, int64_t xs_head, const void* slot_mapping,
+                                int slot_itype, const void* rot_prep, const float* boundaries,
+                                int bits, uint8_t* out_packed, int64_t ps_blk, int64_t ps_pos,
+                                int64_t ps_head, float* out_norms, int64_t ns_blk, int64_t ns_pos,
+                                int64_t ns_head, int block_size, int64_t max_blocks, void* stream) {
+  AKV_REQUIRE(num_tokens >= 0 && num_kv_heads > 0, "akv_encode_paged: bad sizes");
+  AKV_REQUIRE(akv_valid_dtype(x_dtype) && akv_valid_itype(slot_itype), "akv_encode_paged: bad dtype");
+  AKV_REQUIRE(block_size > 0 && max_blocks >= 0, "akv_encode_paged: bad block_size/max_blocks");
+  int rc = akv_check_codec_args("akv_encode_paged", d, bits);
+  if (rc) return rc;
+  if (num_tokens == 0 || max_blocks == 0) return AKV_OK;
+  AKV_REQUIRE(x && slot_mapping && rot_prep && boundaries && out_packed && out_norms,
+              "akv_encode_paged: null pointer");
+  akv_gen_args a = {};
+  a.x = x; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
+  a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
+  a.mat = (const float*)rot_prep + (size_t)d * d;
+  a.table = boundaries;
+  a.packed = out_packed; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
+  a.norms = out_norms; a.ns0 = ns_blk; a.ns1 = ns_pos; a.ns2 = ns_head;
+  rc = akv_encode_mfma_try(a, true, x_dtype, d, bits, rot_prep, (hipStream_t)stream);
+  if (rc != AKV_ERR_UNSUPPORTED) return rc;
+  return akv_encode_dispatch<true>(d, bits, x_dtype, a, stream);
+}
+
+template <int D, int BITS>
+static int akv_decode_dispatch_dtype(int dt, const akv_gen_args& a, void* stream) {
+  const size_t lds = akv_gen_cfg<D>::lds_bytes;
+  switch (dt) {
+    case AKV_F16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F16>, "akv_decode_general_kernel", lds, a, stream);
+    case AKV_BF16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_BF16>, "akv_decode_general_kernel", lds, a, stream);
+    default: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F32>, "akv_decode_general_kernel", lds, a, stream);
+  }
+}
+
+extern "C" int akv_decode(const uint8_t* packed, int64_t packed_stride, const float* norms,
+                          int64_t n, int d, const void* rot_prep, const float* centroids, int bits,
+                          void* out, int out_dtype, int64_t out_stride, void* stream) {
+  AKV_REQUIRE(n >= 0, "akv_decode: n=%lld", (long long)n);
+  AKV_REQUIRE(akv_valid_dtype(out_dtype), "akv_decode: bad dtype %d", out_dtype);
+  int rc = akv_check_codec_args("akv_decode", d, bits);
+  if (rc) return rc;
+  if (n == 0) return AKV_OK;
+  AKV_REQUIRE(packed && norms && rot_prep && centroids && out, "akv_decode: null pointer");
+  AKV_REQUIRE(out_stride >= d && packed_stride >= akv_packed_size(d, bits), "akv_decode: stride smaller than row");
+  akv_gen_args a = {};
+  a.n = n;
+  a.mat = (const float*)rot_prep;  // Pi: [k = rotated coord][out coord]
+  a.table = centroids;
+  a.packed = const_cast<uint8_t*>(packed); a.ps0 = packed_stride;
+  a.norms = const_cast<float*>(norms);
+  a.out = out; a.os0 = out_stride;
+#define AKV_CASE(DD, BB) \
+  if (d == DD && bits == BB) return akv_decode_dispatch_dtype<DD, BB>(out_dtype, a, stream);
+  AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
+  AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
+  AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+#undef AKV_CASE
+  return akv_fail(AKV_ERR_UNSUPPORTED, "decode: no kernel for head_dim=%d bits=%d", d, bits);
+}

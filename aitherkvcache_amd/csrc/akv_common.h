@@ -1,0 +1,185 @@
+// Shared device/host helpers for the gfx950 TurboQuant kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/aitherkv.h"
+
+#define AKV_WAVE 64
+
+// ----------------------------------------------------------------------------------
+// host: status + message
+// ----------------------------------------------------------------------------------
+char* akv_error_buffer();  // thread-local, 512 bytes (defined in akv_codec.hip)
+
+static inline int akv_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(akv_error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define AKV_REQUIRE(cond, ...)                                  \
+  do {                                                          \
+    if (!(cond)) return akv_fail(AKV_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+#define AKV_HIP(call)                                                                         \
+  do {                                                                                        \
+    hipError_t e_ = (call);                                                                   \
+    if (e_ != hipSuccess)                                                                     \
+      return akv_fail(AKV_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),     \
+                      __FILE__, __LINE__);                                                    \
+  } while (0)
+
+#define AKV_LAUNCH_CHECK(name)                                                                \
+  do {                                                                                        \
+    hipError_t e_ = hipGetLastError();                                                        \
+    if (e_ != hipSuccess)                                                                     \
+      return akv_fail(AKV_ERR_HIP, "launch of %s failed: %s", name, hipGetErrorString(e_));   \
+  } while (0)
+
+static inline bool akv_valid_dtype(int t) { return t == AKV_F16 || t == AKV_BF16 || t == AKV_F32; }
+static inline bool akv_valid_itype(int t) { return t == AKV_I32 || t == AKV_I64; }
+static inline int akv_packed_size(int d, int bits) { return d * bits / 8; }
+
+int akv_cached_cu_count();  // 0 when no device (defined in akv_codec.hip)
+
+// Offsets (in floats) into the prepared-rotation buffer.
+//   [0, d*d)        Pi     row-major  (y_i = sum_j Pi[i][j] x_j)
+//   [d*d, 2*d*d)    Pi^T   row-major
+//   [2*d*d, 4*d*d)  fp16 hi / scaled-lo operand tiles for the MFMA encode kernel
+static inline size_t akv_prep_floats(int d) { return (size_t)4 * d * d; }
+
+// Arguments of the encode / decode kernels (flat and paged forms share one struct).
+struct akv_gen_args {
+  // encode input
+  const void* x;
+  int64_t n;        // vectors (paged: num_tokens * num_kv_heads)
+  int64_t xs0, xs1; // flat: xs0 = row stride; paged: xs0 = token stride, xs1 = head stride
+  int heads;        // paged: num_kv_heads
+  const void* slots;
+  int slot_itype;
+  int block_size;
+  int64_t max_blocks;
+  const float* mat;   // [D][D] staged matrix, [k][out]
+  const float* table; // boundaries (encode) or centroids (decode)
+  // packed side
+  uint8_t* packed;
+  int64_t ps0, ps1, ps2; // flat: ps0 = row stride (bytes); paged: blk, pos, head strides (bytes)
+  float* norms;
+  int64_t ns0, ns1, ns2;
+  // decode output
+  void* out;
+  int64_t os0;
+};
+
+// ----------------------------------------------------------------------------------
+// device: element loads / stores
+// ----------------------------------------------------------------------------------
+struct akv_f16 { uint16_t v; };
+struct akv_bf16 { uint16_t v; };
+
+__device__ __forceinline__ float akv_to_float(__half h) { return __half2float(h); }
+__device__ __forceinline__ float akv_bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ uint16_t akv_float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                            // RNE
+  return (uint16_t)(u >> 16);
+}
+
+template <int DT> struct akv_elem;
+template <> struct akv_elem<AKV_F16> {
+  typedef __half type;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) {
+    return __half2float(((const __half*)p)[i]);
+  }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) {
+    ((__half*)p)[i] = __float2half_rn(v);
+  }
+};
+template <> struct akv_elem<AKV_BF16> {
+  typedef uint16_t type;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) {
+    return akv_bf16_bits_to_float(((const uint16_t*)p)[i]);
+  }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) {
+    ((uint16_t*)p)[i] = akv_float_to_bf16_bits(v);
+  }
+};
+template <> struct akv_elem<AKV_F32> {
+  typedef float type;
+  static __device__ __forceinline__ float load(const void* p, int64_t i) {
+    return ((const float*)p)[i];
+  }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) {
+    ((float*)p)[i] = v;
+  }
+};
+
+__device__ __forceinline__ int64_t akv_load_index(const void* p, int itype, int64_t i) {
+  return itype == AKV_I64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
+}
+
+// ----------------------------------------------------------------------------------
+// device: wavefront (64-lane) reductions; every lane receives the result
+// ----------------------------------------------------------------------------------
+__device__ __forceinline__ float akv_wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, AKV_WAVE);
+  return v;
+}
+__device__ __forceinline__ float akv_wave_max(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, AKV_WAVE));
+  return v;
+}
+
+// ----------------------------------------------------------------------------------
+// device: MSB-first code streams (covers pack_4bit / pack_2bit / pack_3bit of
+// aither_kvcache/packing.py and pack_multibit of hybrid_quantizer.py:310-352 -- all four
+// are the same big-endian bit stream with BITS bits per index)
+// ----------------------------------------------------------------------------------
+// Byte k of the stream, given a callable code_of(dim).
+template <int BITS, class F>
+__device__ __forceinline__ uint32_t akv_stream_byte(int k, F code_of) {
+  const int p0 = 8 * k;
+  const int dim0 = p0 / BITS;
+  const int dim1 = (p0 + 7) / BITS;
+  uint32_t byte = 0;
+  for (int dim = dim0; dim <= dim1; ++dim) {
+    const uint32_t c = code_of(dim);
+    const int shift = (p0 + 8) - (dim * BITS + BITS);
+    byte |= shift >= 0 ? (c << shift) : (c >> (-shift));
+  }
+  return byte & 0xffu;
+}
+
+// Index `dim` of the stream, given a callable byte_of(offset).
+template <int BITS, class F>
+__device__ __forceinline__ uint32_t akv_stream_code(int dim, F byte_of) {
+  const int p = dim * BITS;
+  const int o = p >> 3;
+  const int r = p & 7;
+  uint32_t w = byte_of(o) << 8;
+  if (r + BITS > 8) w |= byte_of(o + 1);
+  return (w >> (16 - BITS - r)) & ((1u << BITS) - 1u);
+}
+
+// code = #{b in boundaries : b < y}  (torch.searchsorted(right=False), quantizer.py:203-207)
+template <int BITS>
+__device__ __forceinline__ uint32_t akv_search(float y, const float* bnd) {
+  uint32_t c = 0;
+#pragma unroll
+  for (int k = 0; k < (1 << BITS) - 1; ++k) c += (bnd[k] < y) ? 1u : 0u;
+  if (y != y) c = (1u << BITS) - 1u;  // searchsorted places NaN after every boundary
+  return c;
+}

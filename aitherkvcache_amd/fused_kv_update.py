@@ -1,0 +1,81 @@
+"""Encode-on-write into the paged TurboQuant cache: one HIP kernel does norm, normalise,
+rotation, codebook search, bit packing and the scatter through slot_mapping.
+
+Same call surface as the reference's aither_kvcache/fused_kv_update.py
+(fused_tq4_kv_update :300-405, fused_encode_and_store :412-468) with the semantics of its
+torch fallback (:220-293): the stored norm is the plain L2 norm, the divisor is norm + 1e-10,
+ties go to the lower bin, tokens with a negative slot or a block index >= max_blocks are
+skipped.  Besides 4-bit (the only width the reference fuses) 3- and 2-bit are supported via
+`bits=` / fused_kv_update().
+"""
+import logging
+
+import torch
+
+from . import _lib
+from .packing import packed_size
+from .quantizer import prepared_rotation_for
+
+logger = logging.getLogger("aither.turboquant.fused_kv_update")
+
+HAS_HIP = _lib.available()
+HAS_TRITON = HAS_HIP
+
+__all__ = ["fused_tq4_kv_update", "fused_kv_update", "fused_encode_and_store", "HAS_TRITON", "HAS_HIP"]
+
+
+def fused_kv_update(x, slot_mapping, out_packed, out_norms, rotation, boundaries, bits,
+                    block_size=16, max_blocks=0, prepared=None) -> None:
+    """Quantize-and-store for one cache tensor (K or V) at `bits` in {2, 3, 4}.
+
+    x            [num_tokens, num_kv_heads, head_dim] float16 / bfloat16 / float32
+    slot_mapping [num_tokens] int64 or int32; negative = padding
+    out_packed   [max_blocks, block_size, num_kv_heads, >= packed_dim] uint8 (strides honoured)
+    out_norms    [max_blocks, block_size, num_kv_heads] float32 (strides honoured)
+    rotation     [head_dim, head_dim] float32;  boundaries [2**bits - 1] float32
+    """
+    if max_blocks == 0:
+        max_blocks = out_packed.shape[0]
+    num_tokens, num_kv_heads, head_dim = x.shape
+    if num_tokens == 0:
+        return
+    if head_dim <= 0 or (head_dim & (head_dim - 1)) != 0:
+        raise ValueError(f"head_dim must be a power of 2, got {head_dim}")
+    dev = _lib.require_gpu(x, slot_mapping, out_packed, out_norms, rotation, boundaries)
+    if out_packed.dtype != torch.uint8 or out_norms.dtype != torch.float32:
+        raise ValueError("out_packed must be uint8 and out_norms float32")
+    if out_packed.shape[-1] < packed_size(head_dim, bits) or out_packed.stride(-1) != 1:
+        raise ValueError("out_packed rows are too short or not contiguous in the last dim")
+    if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        x = x.float()
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    slots = slot_mapping if slot_mapping.is_contiguous() else slot_mapping.contiguous()
+    prep = prepared if prepared is not None else prepared_rotation_for(rotation)
+    bnd = boundaries if (boundaries.dtype == torch.float32 and boundaries.is_contiguous()) \
+        else boundaries.float().contiguous()
+    _lib.check(_lib.lib().akv_encode_paged(
+        x.data_ptr(), _lib.dtype_code(x), num_tokens, num_kv_heads, head_dim, x.stride(0), x.stride(1),
+        slots.data_ptr(), _lib.itype_code(slots), prep.ptr, bnd.data_ptr(), bits,
+        out_packed.data_ptr(), out_packed.stride(0), out_packed.stride(1), out_packed.stride(2),
+        out_norms.data_ptr(), out_norms.stride(0), out_norms.stride(1), out_norms.stride(2),
+        block_size, max_blocks, _lib.stream_ptr(dev)))
+
+
+def fused_tq4_kv_update(x, slot_mapping, out_packed, out_norms, rotation, boundaries,
+                        block_size: int = 16, max_blocks: int = 0) -> None:
+    """4-bit quantize-and-store, signature of the reference (fused_kv_update.py:300-309)."""
+    fused_kv_update(x, slot_mapping, out_packed, out_norms, rotation, boundaries, 4,
+                    block_size=block_size, max_blocks=max_blocks)
+
+
+def fused_encode_and_store(tq_cache, layer_idx: int, key, value, slot_mapping) -> None:
+    """K then V for one layer into a cache object with attributes tq, k_packed, k_norms,
+    v_packed, v_norms, block_size, max_blocks (reference: fused_kv_update.py:412-468)."""
+    tq = tq_cache.tq
+    prep = tq.prepared_rotation() if hasattr(tq, "prepared_rotation") else None
+    for x, packed, norms in ((key, tq_cache.k_packed, tq_cache.k_norms),
+                             (value, tq_cache.v_packed, tq_cache.v_norms)):
+        fused_kv_update(x, slot_mapping, packed[layer_idx], norms[layer_idx], tq.rotation,
+                        tq.boundaries_inner, tq.bits, block_size=tq_cache.block_size,
+                        max_blocks=tq_cache.max_blocks, prepared=prep)

@@ -1,0 +1,94 @@
+"""Encode-on-write and paged decode attention for the tq35 hybrid cache.
+
+The reference has no fused path for hybrid data: its tq::hybrid_decode_step
+(aither_kvcache/vllm/hooks.py:240-345) encodes the new token, decompresses every block the
+batch addresses with HybridTurboQuant.decode and runs dense SDPA.  Here the same attention
+(softmax(q K^T * scale) V over the decoded rows) is computed directly on the packed 64-byte
+rows by one kernel sequence, and the new token is written by one scatter kernel.
+Cache tensors are uint8 [num_blocks, block_size, num_kv_heads, >= 64] (norms are inside the
+rows); strided views with 4-byte aligned rows are accepted.
+"""
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+def hybrid_encode_and_store(htq, x: torch.Tensor, slot_mapping: torch.Tensor, cache: torch.Tensor,
+                            block_size: int = 16, max_blocks: int = 0) -> None:
+    """Write x [num_tokens, num_kv_heads, 128] into cache[blk, pos, head, :64] for
+    slot = blk * block_size + pos; negative slots and blocks >= max_blocks are skipped."""
+    if max_blocks == 0:
+        max_blocks = cache.shape[0]
+    num_tokens, num_kv_heads, head_dim = x.shape
+    if num_tokens == 0:
+        return
+    table = htq.kernel_table
+    dev = _lib.require_gpu(x, slot_mapping, cache, table)
+    if cache.dtype != torch.uint8 or cache.stride(-1) != 1 or cache.shape[-1] < htq.packed_dim:
+        raise ValueError(f"cache must be uint8 with contiguous rows of >= {htq.packed_dim} bytes")
+    if head_dim != htq.head_dim:
+        raise ValueError(f"head_dim {head_dim} != {htq.head_dim}")
+    if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        x = x.float()
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    slots = slot_mapping if slot_mapping.is_contiguous() else slot_mapping.contiguous()
+    _lib.check(_lib.lib().akv_hybrid_encode_paged(
+        x.data_ptr(), _lib.dtype_code(x), num_tokens, num_kv_heads, x.stride(0), x.stride(1),
+        slots.data_ptr(), _lib.itype_code(slots), table.data_ptr(),
+        cache.data_ptr(), cache.stride(0), cache.stride(1), cache.stride(2),
+        block_size, max_blocks, _lib.stream_ptr(dev)))
+
+
+class HybridPagedAttention:
+    """attn = HybridPagedAttention(htq, num_query_heads=32)
+    out = attn.forward(query, k_cache, v_cache, block_tables, context_lens, scale=...)"""
+
+    def __init__(self, htq, num_query_heads: int):
+        self._htq = htq
+        self.num_query_heads = num_query_heads
+        self.head_dim = htq.head_dim
+        self._workspace: Optional[torch.Tensor] = None
+
+    def forward(self, query, k_cache, v_cache, block_tables, context_lens, block_size: int = 16,
+                num_kv_heads: Optional[int] = None, scale: Optional[float] = None) -> torch.Tensor:
+        if num_kv_heads is None:
+            num_kv_heads = k_cache.shape[2]
+        if scale is None:
+            scale = 1.0 / (self.head_dim ** 0.5)
+        table = self._htq.kernel_table
+        dev = _lib.require_gpu(query, k_cache, v_cache, block_tables, context_lens, table)
+        num_seqs, num_q_heads, head_dim = query.shape
+        if head_dim != self.head_dim or num_q_heads != self.num_query_heads:
+            raise ValueError(f"query shape {tuple(query.shape)} does not match heads="
+                             f"{self.num_query_heads}, head_dim={self.head_dim}")
+        q = query
+        if q.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            q = q.float()
+        if q.stride(-1) != 1:
+            q = q.contiguous()
+        out = torch.empty((num_seqs, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+        if num_seqs == 0:
+            return out
+        for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if t.dtype != torch.uint8 or t.stride(-1) != 1 or t.shape[-1] < 64:
+                raise ValueError(f"{name} must be uint8 with contiguous rows of >= 64 bytes")
+        bt = block_tables if block_tables.stride(-1) == 1 else block_tables.contiguous()
+        cl = context_lens if context_lens.is_contiguous() else context_lens.contiguous()
+        L = _lib.lib()
+        need = L.akv_hybrid_paged_attn_workspace_bytes(num_seqs, num_q_heads)
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != dev:
+            self._workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+        ws = self._workspace
+        _lib.check(L.akv_hybrid_paged_attn(
+            q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
+            k_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+            v_cache.data_ptr(), v_cache.stride(0), v_cache.stride(1), v_cache.stride(2),
+            bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
+            table.data_ptr(),
+            out.data_ptr(), _lib.dtype_code(out), out.stride(0), out.stride(1),
+            num_seqs, num_q_heads, num_kv_heads, block_size, bt.shape[1], float(scale),
+            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev)))
+        return out if out.dtype == query.dtype else out.to(query.dtype)

@@ -1,0 +1,8 @@
+"""TriAttention: spectral KV compression with trigonometric-series scoring (decode path)."""
+from .config import TriAttentionConfig
+from .encoder import SpectralEncoding, SpectralKVEncoder
+from .attention import TriAttention
+from .spectral import rope_frequencies
+
+__all__ = ["TriAttentionConfig", "SpectralEncoding", "SpectralKVEncoder", "TriAttention",
+           "rope_frequencies"]

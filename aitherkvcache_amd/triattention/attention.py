@@ -1,0 +1,93 @@
+"""TriAttention decode step on MI355X (reference: aither_kvcache/triattention/attention.py:186-280
+with TrigSeriesScorer.score, scorer.py:115-208).
+
+score(q, k_t) = (1/sqrt d) sum_f [ c_f cos(delta theta_f) + s_f sin(delta theta_f) ] over the
+token's retained RoPE pairs, softmax over the cached tokens, and a weighted scatter-add of the
+value coefficients -- one HIP kernel over the spectral cache plus a merge kernel, instead of the
+reference's chain of [B, QH, S, F] float32 temporaries.
+"""
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+from .config import TriAttentionConfig
+from .encoder import SpectralEncoding, SpectralKVEncoder
+from .spectral import rope_frequencies
+
+
+class TriAttention:
+    def __init__(self, config: TriAttentionConfig, device: str = "cpu"):
+        self.config = config
+        self.device = device
+        self.head_dim = config.head_dim
+        self.num_query_heads = config.num_query_heads
+        self.num_kv_heads = config.num_kv_heads
+        self.gqa_ratio = config.gqa_ratio
+        self.scale = 1.0 / math.sqrt(config.head_dim)
+        self.encoder = SpectralKVEncoder(config)
+        # float32 table evaluated on the host exactly as the reference does, then moved
+        self._theta = rope_frequencies(config.head_dim, config.rope_base, device="cpu").to(device)
+        self._workspace: Optional[torch.Tensor] = None
+
+    def to(self, device: str) -> "TriAttention":
+        self.device = device
+        self._theta = self._theta.to(device)
+        return self
+
+    def encode_kv(self, keys: torch.Tensor, values: torch.Tensor) -> Tuple[SpectralEncoding, SpectralEncoding]:
+        """keys / values [B, S, num_kv_heads, head_dim] (keys before RoPE)."""
+        return self.encoder.encode(keys), self.encoder.encode(values)
+
+    def decode_step(self, query: torch.Tensor, k_enc: SpectralEncoding, v_enc: SpectralEncoding,
+                    query_pos: Optional[torch.Tensor] = None,
+                    key_positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """query [B, QH, D]; encodings with indices/packed [B, S, KVH, F], scales [B, S, KVH];
+        query_pos [B] (default S), key_positions [B, S] (default 0..S-1) -> float32 [B, QH, D]."""
+        if not self.config.pre_rope:
+            raise NotImplementedError("post-RoPE scoring is not built")
+        dev = _lib.require_gpu(query, k_enc.indices, k_enc.packed, k_enc.scales,
+                               v_enc.indices, v_enc.packed, v_enc.scales, query_pos, key_positions)
+        if self._theta.device != dev:
+            self._theta = self._theta.to(dev)
+        B, QH, D = query.shape
+        _, S, KVH, F = k_enc.indices.shape
+        if v_enc.indices.shape != k_enc.indices.shape:
+            raise ValueError("k_enc and v_enc must have the same [B, S, KVH, F] shape")
+        if D != self.head_dim or QH % KVH != 0:
+            raise ValueError(f"bad shapes: query {tuple(query.shape)}, encodings {tuple(k_enc.indices.shape)}")
+        q = query if query.dtype in (torch.float16, torch.bfloat16, torch.float32) else query.float()
+        q = q.contiguous()
+
+        def u8(t):
+            if t.dtype != torch.uint8:
+                raise ValueError("indices / packed must be uint8 (int4 coefficients)")
+            return t.contiguous()
+
+        ki, kc, vi, vc = u8(k_enc.indices), u8(k_enc.packed), u8(v_enc.indices), u8(v_enc.packed)
+        ks = k_enc.scales.to(torch.float16).contiguous()
+        vs = v_enc.scales.to(torch.float16).contiguous()
+
+        def pos(t, shape):
+            if t is None:
+                return None
+            if t.dtype not in (torch.int32, torch.int64):
+                t = t.long()
+            return t.expand(shape).contiguous()
+
+        qp = pos(query_pos, (B,))
+        kp = pos(key_positions, (B, S))
+        out = torch.empty(B, QH, D, dtype=torch.float32, device=dev)
+        L = _lib.lib()
+        need = L.akv_tri_decode_workspace_bytes(B, QH, D)
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != dev:
+            self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        _lib.check(L.akv_tri_decode_step(
+            q.data_ptr(), _lib.dtype_code(q), ki.data_ptr(), kc.data_ptr(), ks.data_ptr(),
+            vi.data_ptr(), vc.data_ptr(), vs.data_ptr(), self._theta.data_ptr(),
+            _lib.ptr(qp), _lib.itype_code(qp) if qp is not None else 0,
+            _lib.ptr(kp), _lib.itype_code(kp) if kp is not None else 0,
+            out.data_ptr(), B, S, QH, KVH, D, F,
+            self._workspace.data_ptr(), self._workspace.numel(), _lib.stream_ptr(dev)))
+        return out

@@ -1,0 +1,200 @@
+/*
+ * aitherkv.h -- C ABI of the MI355X (gfx950) TurboQuant KV-cache hot path.
+ *
+ * The reference (aither-kvcache) has no FFI of its own: its hot path is Python
+ * calling torch ops and Triton kernels.  This header is the boundary a binding
+ * for that path would use: plain device pointers, element strides, sizes, enums
+ * and a hipStream_t; every function returns an akv_status and never aborts
+ * (the reference's callers wrap the path in try/except and fall back,
+ * aither_kvcache/vllm/backend.py:527-530,552-555).  Each entry point cites the
+ * reference function it stands in for.
+ *
+ * Conventions
+ *   - all pointers are DEVICE pointers unless said otherwise; the caller owns
+ *     every buffer; nothing is allocated or freed by the library except where a
+ *     function says so;
+ *   - strides are in ELEMENTS of the pointed-to type unless the name ends in
+ *     _bytes;
+ *   - work is enqueued on `stream` (void* = hipStream_t; NULL = default stream)
+ *     and the call returns without synchronising;
+ *   - packed code layouts are the reference's: aither_kvcache/packing.py:13-118
+ *     (4-bit: byte k = idx[2k]<<4 | idx[2k+1]; 2-bit: 4 per byte, first index in
+ *     the top bits; 3-bit: 8 indices -> 24-bit big-endian word, index 0 in bits
+ *     23..21) and aither_kvcache/hybrid_quantizer.py:92-123 for tq35.
+ */
+#ifndef AITHERKV_H
+#define AITHERKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  AKV_OK = 0,
+  AKV_ERR_INVALID = 1,     /* bad argument (null pointer, negative size, bad enum) */
+  AKV_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for          */
+  AKV_ERR_WORKSPACE = 3,   /* workspace missing or too small                       */
+  AKV_ERR_HIP = 4          /* a HIP runtime call failed; see akv_last_error()      */
+} akv_status;
+
+typedef enum { AKV_F16 = 0, AKV_BF16 = 1, AKV_F32 = 2 } akv_dtype;
+typedef enum { AKV_I32 = 0, AKV_I64 = 1 } akv_itype;
+
+/* Library version string (static storage). */
+const char* akv_version(void);
+/* Message for the last non-OK status returned on this host thread (static storage). */
+const char* akv_last_error(void);
+/* Number of compute units of the current device (0 and a status if no device). */
+int akv_device_cu_count(int* cu_count);
+
+/* ---------------------------------------------------------------------------------
+ * Rotation matrix, prepared once per quantizer.
+ * `rotation` is the reference's Pi (row-major [d,d] float32, y = Pi x,
+ * aither_kvcache/rotation.py:20-35, used as x @ Pi.T at quantizer.py:150).  The
+ * kernels want it in several layouts (Pi, Pi^T, and fp16 hi/lo MFMA tiles);
+ * akv_rotation_prepare writes them all into `prep` (device, akv_rotation_prepared_bytes(d)
+ * bytes, 256-byte aligned), which the entry points below take instead of `rotation`.
+ * ------------------------------------------------------------------------------- */
+size_t akv_rotation_prepared_bytes(int d);
+int akv_rotation_prepare(const float* rotation, int d, void* prep, size_t prep_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * Codec primitives -- aither_kvcache/triton_ops.py:220-259
+ * (triton_quantize_4bit/2bit, triton_dequantize_4bit/2bit; 3-bit is a stub there and
+ * real here).  Ties follow the torch path (quantizer.py:203-207): code = #{b : b < y}.
+ * ------------------------------------------------------------------------------- */
+int akv_quantize_pack(const float* y, int64_t n, int d, int64_t y_stride,
+                      const float* boundaries, int bits,
+                      uint8_t* out, int64_t out_stride, void* stream);
+int akv_unpack_lookup(const uint8_t* packed, int64_t n, int d, int64_t packed_stride,
+                      const float* centroids, int bits,
+                      float* out, int64_t out_stride, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * TurboQuant.encode -- aither_kvcache/quantizer.py:122-166.
+ * n vectors of d elements (row stride x_stride): norm, x/(norm+1e-10), rotation,
+ * codebook search, packing.  Writes out_packed[n][packed_size(d,bits)] (row stride
+ * packed_stride bytes) and out_norms[n] (float32).
+ * ------------------------------------------------------------------------------- */
+int akv_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride,
+               const void* rot_prep, const float* boundaries, int bits,
+               uint8_t* out_packed, int64_t packed_stride, float* out_norms, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * fused_tq4_kv_update -- aither_kvcache/fused_kv_update.py:300-405 (semantics of its
+ * torch fallback :220-293), for 4-, 3- and 2-bit.
+ * x[num_tokens][num_kv_heads][d]; slot = slot_mapping[token]; tokens with slot < 0 or
+ * slot / block_size >= max_blocks are skipped; writes
+ *   out_packed[blk*ps_blk + pos*ps_pos + head*ps_head + 0..packed)   (uint8)
+ *   out_norms [blk*ns_blk + pos*ns_pos + head*ns_head]               (float32)
+ * ------------------------------------------------------------------------------- */
+int akv_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads, int d,
+                     int64_t xs_token, int64_t xs_head,
+                     const void* slot_mapping, int slot_itype,
+                     const void* rot_prep, const float* boundaries, int bits,
+                     uint8_t* out_packed, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                     float* out_norms, int64_t ns_blk, int64_t ns_pos, int64_t ns_head,
+                     int block_size, int64_t max_blocks, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * TurboQuant.decode -- aither_kvcache/quantizer.py:168-197:
+ * out[i] = (centroids[codes_i] @ Pi) * norms[i], cast to out_dtype.
+ * ------------------------------------------------------------------------------- */
+int akv_decode(const uint8_t* packed, int64_t packed_stride, const float* norms, int64_t n, int d,
+               const void* rot_prep, const float* centroids, int bits,
+               void* out, int out_dtype, int64_t out_stride, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * TQPagedAttention.forward -- aither_kvcache/fused_attention.py:594-748, with the result
+ * of TQPagedAttentionRef.forward (:91-185).  The query pre-rotation (:659) and the output
+ * inverse rotation (:747) are done inside.
+ *   query        [num_seqs][num_q_heads][d], strides qs_seq / qs_head (last dim contiguous)
+ *   k/v_packed   [blocks][block_size][num_kv_heads][packed] uint8, strides in bytes
+ *   k/v_norms    [blocks][block_size][num_kv_heads] float32, strides in elements
+ *   block_tables [num_seqs][max_blocks_per_seq] (row stride bt_stride); entries at or
+ *                beyond ceil(ctx/block_size) are never read
+ *   context_lens [num_seqs]; 0 gives a zero output row
+ *   out          [num_seqs][num_q_heads][d] in out_dtype, strides os_seq / os_head
+ * kv head of query head h is h / (num_q_heads / num_kv_heads).
+ * `workspace` (device, >= akv_paged_attn_workspace_bytes(...), 256-byte aligned) holds the
+ * rotated queries and the split partials; the caller allocates it once.
+ * ------------------------------------------------------------------------------- */
+size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d);
+int akv_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+                   const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+                   const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
+                   const uint8_t* v_packed, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+                   const float* v_norms, int64_t vns_blk, int64_t vns_pos, int64_t vns_head,
+                   const void* block_tables, int bt_itype, int64_t bt_stride,
+                   const void* context_lens, int cl_itype,
+                   const void* rot_prep, const float* centroids, int bits,
+                   void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+                   int num_seqs, int num_q_heads, int num_kv_heads, int d,
+                   int block_size, int64_t max_blocks_per_seq, float scale,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * HybridTurboQuant, mode tq35 with calibrate_uniform() groups (dims 0..63 at 3-bit MSE,
+ * dims 64..127 at 2-bit MSE, each with a 1-bit QJL residual sketch and fp16 norms inside
+ * the 64-byte row) -- aither_kvcache/hybrid_quantizer.py:616-779 (encode), :785-933 (decode).
+ * `hyb_table` is a device float32[AKV_HYB_TABLE_FLOATS] laid out as
+ *   [0,64)    group-0 Hadamard signs   [64,128)  group-1 Hadamard signs
+ *   [128,192) group-0 QJL signs        [192,256) group-1 QJL signs
+ *   [256,264) group-0 centroids (8)    [264,268) group-1 centroids (4)
+ *   [268,275) group-0 boundaries (7)   [275,278) group-1 boundaries (3)
+ * head_dim is 128.
+ * ------------------------------------------------------------------------------- */
+#define AKV_HYB_TABLE_FLOATS 288
+#define AKV_HYB_PACKED_BYTES 64
+int akv_hybrid_encode(const void* x, int x_dtype, int64_t n, int64_t x_stride,
+                      const float* hyb_table, uint8_t* out, int64_t out_stride_bytes, void* stream);
+/* Paged form: the encode half of tq::hybrid_decode_step, aither_kvcache/vllm/hooks.py:271-284;
+ * same skipping rule as akv_encode_paged. */
+int akv_hybrid_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads,
+                            int64_t xs_token, int64_t xs_head,
+                            const void* slot_mapping, int slot_itype, const float* hyb_table,
+                            uint8_t* out, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                            int block_size, int64_t max_blocks, void* stream);
+int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_bytes, int64_t n,
+                      const float* hyb_table, float* out, int64_t out_stride, void* stream);
+/* Decode attention over a tq35 paged cache.  The reference has no fused kernel for this: its
+ * tq::hybrid_decode_step (aither_kvcache/vllm/hooks.py:240-345) decompresses every addressed
+ * block and runs dense attention; this computes the same softmax(q K^T * scale) V directly on
+ * the packed rows (float32 accumulation).  `scale` is explicit, as at hooks.py:341. */
+size_t akv_hybrid_paged_attn_workspace_bytes(int num_seqs, int num_q_heads);
+int akv_hybrid_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+                          const uint8_t* k_cache, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+                          const uint8_t* v_cache, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+                          const void* block_tables, int bt_itype, int64_t bt_stride,
+                          const void* context_lens, int cl_itype, const float* hyb_table,
+                          void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+                          int num_seqs, int num_q_heads, int num_kv_heads,
+                          int block_size, int64_t max_blocks_per_seq, float scale,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * TriAttention.decode_step -- aither_kvcache/triattention/attention.py:186-280 with
+ * TrigSeriesScorer.score (scorer.py:115-208), int4 coefficients:
+ *   k/v_indices [B][S][KVH][F] uint8, k/v_coeffs [B][S][KVH][F] uint8 (hi nibble = even
+ *   component), k/v_scales [B][S][KVH] fp16, all contiguous; theta [d/2] float32
+ *   (spectral.py:34-51); query [B][QH][d] (contiguous); query_pos [B] or NULL (= S);
+ *   key_positions [B][S] or NULL (= 0..S-1); out [B][QH][d] float32.
+ * ------------------------------------------------------------------------------- */
+size_t akv_tri_decode_workspace_bytes(int batch, int num_q_heads, int d);
+int akv_tri_decode_step(const void* query, int q_dtype,
+                        const uint8_t* k_indices, const uint8_t* k_coeffs, const void* k_scales,
+                        const uint8_t* v_indices, const uint8_t* v_coeffs, const void* v_scales,
+                        const float* theta,
+                        const void* query_pos, int qp_itype,
+                        const void* key_positions, int kp_itype,
+                        float* out, int batch, int64_t seq_len, int num_q_heads, int num_kv_heads,
+                        int d, int num_freqs,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AITHERKV_H */

@@ -1,0 +1,601 @@
+"""CPU oracle for the TurboQuant / tq35 / TriAttention hot path  --  TEST INFRASTRUCTURE ONLY.
+
+This module is a plain numpy restatement of the reference's algorithm for the
+path (encode-on-write -> paged decode attention -> TriAttention decode_step).
+It exists to CHECK the HIP kernels.  Nothing in the shipped package imports it:
+only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may.
+
+Every function cites the reference lines it restates (paths are relative to the
+reference tree).  How each one is pinned:
+
+  pinned by the committed golden vectors (tests/golden/golden_v1.npz, produced
+  by running the reference itself) and by independent brute force / closed forms
+  in tests/test_oracle_*.py:
+      get_codebook, pack_*/unpack_*, pack_multibit/unpack_multibit,
+      encode, decode, kv_update, paged_attention_loop, paged_attention,
+      fwht, structured_hadamard, dimension_aware_codebook,
+      hybrid_encode, hybrid_decode, rope_frequencies, spectral_encode,
+      tri_scores, tri_decode_step
+  derived here (the reference has no such function; it always decompresses
+  tq35 data before attending): hybrid_paged_attention is *defined* as
+  hybrid_decode -> dense f32 softmax attention, i.e. the reference's
+  tq::hybrid_decode_step (vllm/hooks.py:294-345) without its bf16 down-cast.
+
+Inputs that only torch's CPU generator / LAPACK can produce (the rotation matrix
+and the tq35 sign vectors) are arguments here; the tests take them from the
+golden file.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+
+f32 = np.float32
+
+# --------------------------------------------------------------------------------------
+# codebook.py
+# --------------------------------------------------------------------------------------
+# Lloyd-Max centroids of N(0,1) (Max 1960), as tabulated at codebook.py:28-53.
+_STD_CENTROIDS = {
+    1: [-0.798284, 0.798284],
+    2: [-1.510469, -0.452781, 0.452781, 1.510469],
+    3: [-2.152090, -1.344134, -0.756031, -0.245104, 0.245104, 0.756031, 1.344134, 2.152090],
+    4: [-2.733266, -2.069016, -1.618002, -1.256233, -0.942391, -0.656804, -0.388089, -0.128350,
+        0.128350, 0.388089, 0.656804, 0.942391, 1.256233, 1.618002, 2.069016, 2.733266],
+}
+_STD_MSE = {1: 0.363480, 2: 0.117517, 3: 0.034506, 4: 0.009497}
+
+
+def get_codebook(d: int, bits: int):
+    """codebook.py:62-82 + quantizer.py:96-99: centroids/sqrt(d) in float64, boundaries are
+    midpoints, both cast to float32 by the quantizer."""
+    if bits not in _STD_CENTROIDS:
+        raise ValueError(f"Supported bit-widths: {list(_STD_CENTROIDS)}. Got {bits}")
+    c = np.array(_STD_CENTROIDS[bits], dtype=np.float64) * (1.0 / math.sqrt(d))
+    b = (c[:-1] + c[1:]) / 2
+    return c.astype(f32), b.astype(f32), _STD_MSE[bits]
+
+
+def theory_bounds(bits: int):
+    """codebook.py:85-89."""
+    return 1.0 / 4 ** bits, (3 * math.pi / 2) / 4 ** bits
+
+
+# --------------------------------------------------------------------------------------
+# packing.py
+# --------------------------------------------------------------------------------------
+def packed_size(dim: int, bits: int) -> int:
+    """packing.py:121-131."""
+    if bits == 4:
+        return dim // 2
+    if bits == 3:
+        assert dim % 8 == 0
+        return dim * 3 // 8
+    if bits == 2:
+        return dim // 4
+    raise ValueError(f"Unsupported bit-width: {bits}")
+
+
+def pack_4bit(idx):
+    """packing.py:13-23: byte k = idx[2k] << 4 | idx[2k+1]."""
+    idx = np.asarray(idx).astype(np.uint8)
+    return ((idx[..., 0::2] << 4) | idx[..., 1::2]).astype(np.uint8)
+
+
+def unpack_4bit(packed, dim):
+    """packing.py:26-37."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    out = np.empty(packed.shape[:-1] + (dim,), dtype=np.uint8)
+    out[..., 0::2] = (packed >> 4) & 0x0F
+    out[..., 1::2] = packed & 0x0F
+    return out
+
+
+def pack_2bit(idx):
+    """packing.py:40-52: byte k = a<<6 | b<<4 | c<<2 | d for idx[4k..4k+3]."""
+    idx = np.asarray(idx).astype(np.uint8)
+    return ((idx[..., 0::4] << 6) | (idx[..., 1::4] << 4) | (idx[..., 2::4] << 2)
+            | idx[..., 3::4]).astype(np.uint8)
+
+
+def unpack_2bit(packed, dim):
+    """packing.py:55-70."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    out = np.empty(packed.shape[:-1] + (dim,), dtype=np.uint8)
+    for k in range(4):
+        out[..., k::4] = (packed >> (6 - 2 * k)) & 0x03
+    return out
+
+
+def pack_3bit(idx):
+    """packing.py:73-98: 8 values -> one 24-bit big-endian word, value i at bits 23-3i..21-3i."""
+    idx = np.asarray(idx).astype(np.int32)
+    D = idx.shape[-1]
+    assert D % 8 == 0
+    g = idx.reshape(idx.shape[:-1] + (D // 8, 8))
+    bits24 = np.zeros(g.shape[:-1], dtype=np.int32)
+    for i in range(8):
+        bits24 |= (g[..., i] & 0x7) << (21 - 3 * i)
+    b = np.stack([(bits24 >> 16) & 0xFF, (bits24 >> 8) & 0xFF, bits24 & 0xFF], axis=-1)
+    return b.astype(np.uint8).reshape(idx.shape[:-1] + (D // 8 * 3,))
+
+
+def unpack_3bit(packed, dim):
+    """packing.py:101-118."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    g = packed.reshape(packed.shape[:-1] + (dim // 8, 3)).astype(np.int32)
+    bits24 = (g[..., 0] << 16) | (g[..., 1] << 8) | g[..., 2]
+    out = np.empty(g.shape[:-1] + (8,), dtype=np.uint8)
+    for i in range(8):
+        out[..., i] = (bits24 >> (21 - 3 * i)) & 0x7
+    return out.reshape(packed.shape[:-1] + (dim,))
+
+
+_PACK = {2: pack_2bit, 3: pack_3bit, 4: pack_4bit}
+_UNPACK = {2: unpack_2bit, 3: unpack_3bit, 4: unpack_4bit}
+
+
+# --------------------------------------------------------------------------------------
+# quantizer.py
+# --------------------------------------------------------------------------------------
+def quantize(y, boundaries, bits):
+    """quantizer.py:203-207: idx = clamp(searchsorted(bnd, y, right=False)) = #{b : b < y}."""
+    idx = np.searchsorted(np.asarray(boundaries, dtype=f32), np.asarray(y, dtype=f32), side="left")
+    return np.clip(idx, 0, (1 << bits) - 1)
+
+
+def rotate_unit(x, rotation):
+    """quantizer.py:140-150: norms, u = x/(n+1e-10), y = u @ R.T, all float32."""
+    xf = np.ascontiguousarray(np.asarray(x).astype(f32)).reshape(-1, rotation.shape[0])
+    norms = np.sqrt(np.sum(xf * xf, axis=-1, dtype=f32)).astype(f32)
+    u = xf / (norms[:, None] + f32(1e-10))
+    y = u @ np.ascontiguousarray(rotation.T)
+    return y.astype(f32), norms
+
+
+def rotate_unit_f64(x, rotation):
+    """Same quantity as rotate_unit with the dot products carried in float64.  Used to tell a
+    rounding-order difference (rotated value within a few float32 ulps of a decision
+    boundary) from a real defect when two float32 implementations disagree on a code."""
+    xf = np.asarray(x).astype(f32).reshape(-1, rotation.shape[0])
+    norms = np.sqrt(np.sum(xf.astype(np.float64) ** 2, axis=-1))
+    u = (xf / (norms.astype(f32)[:, None] + f32(1e-10))).astype(np.float64)
+    return u @ rotation.astype(np.float64).T
+
+
+def boundary_ulp_distance(y64, boundaries):
+    """Distance from each float64 rotated value to the nearest decision boundary, in units of
+    the float32 ulp at that boundary (spacing of float32 at |b|; at b == 0 the spacing near
+    the values that actually occur, taken at 2**-24 relative to the typical |y|)."""
+    b = np.asarray(boundaries, dtype=np.float64)
+    d = np.abs(y64[..., None] - b)
+    k = np.argmin(d, axis=-1)
+    nearest = b[k]
+    scale = np.maximum(np.abs(nearest), np.abs(y64))
+    ulp = np.spacing(np.maximum(scale, 1e-30).astype(f32)).astype(np.float64)
+    return np.min(d, axis=-1) / ulp
+
+
+def encode(x, rotation, boundaries, bits) -> Tuple[np.ndarray, np.ndarray]:
+    """TurboQuant.encode, quantizer.py:122-166 (torch path :203-207)."""
+    x = np.asarray(x)
+    batch = x.shape[:-1]
+    y, norms = rotate_unit(x, rotation)
+    packed = _PACK[bits](quantize(y, boundaries, bits))
+    return packed.reshape(batch + (packed.shape[-1],)), norms.reshape(batch)
+
+
+def decode(packed, norms, rotation, centroids, bits, out_dtype=np.float16):
+    """TurboQuant.decode, quantizer.py:168-197 (torch path :209-212)."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    norms = np.asarray(norms)
+    D = rotation.shape[0]
+    batch = norms.shape
+    idx = _UNPACK[bits](packed.reshape(-1, packed.shape[-1]), D)
+    y_hat = np.asarray(centroids, dtype=f32)[idx.astype(np.int64)]
+    x_hat = (y_hat @ rotation.astype(f32)) * norms.reshape(-1).astype(f32)[:, None]
+    return x_hat.reshape(batch + (D,)).astype(out_dtype)
+
+
+# --------------------------------------------------------------------------------------
+# fused_kv_update.py (torch fallback = semantics of record)
+# --------------------------------------------------------------------------------------
+def kv_update(x, slot_mapping, out_packed, out_norms, rotation, boundaries, block_size=16,
+              max_blocks=0, bits=4):
+    """_pytorch_tq4_kv_update, fused_kv_update.py:220-293 (generalised over bits): negative
+    slots and blocks >= max_blocks are skipped; writes out_packed[blk, pos], out_norms[blk,
+    pos] in place."""
+    if max_blocks == 0:
+        max_blocks = out_packed.shape[0]
+    slot_mapping = np.asarray(slot_mapping)
+    x = np.asarray(x)
+    valid = slot_mapping >= 0
+    blk = slot_mapping // block_size
+    valid &= blk < max_blocks
+    if not valid.any():
+        return
+    xs = x[valid]
+    N, H, D = xs.shape
+    packed, norms = encode(xs.reshape(N * H, D), rotation, boundaries, bits)
+    b = blk[valid]
+    p = slot_mapping[valid] % block_size
+    out_packed[b, p] = packed.reshape(N, H, -1)
+    out_norms[b, p] = norms.reshape(N, H)
+
+
+# --------------------------------------------------------------------------------------
+# fused_attention.py
+# --------------------------------------------------------------------------------------
+def paged_attention_loop(query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
+                         rotation, centroids, bits, block_size=16, scale=None):
+    """TQPagedAttentionRef.forward, fused_attention.py:91-185, literally: per (seq, q-head) an
+    online softmax over tokens in float32; ctx == 0 leaves zeros; output in query dtype.
+    Pure Python loops: small cases only."""
+    query = np.asarray(query)
+    S, QH, D = query.shape
+    KVH = k_packed.shape[2]
+    gqa = QH // KVH
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    scale = f32(scale)
+    c = np.asarray(centroids, dtype=f32)
+    R = rotation.astype(f32)
+    out = np.zeros_like(query)
+    for s in range(S):
+        ctx = int(context_lens[s])
+        if ctx == 0:
+            continue
+        nblk = math.ceil(ctx / block_size)
+        for qh in range(QH):
+            h = qh // gqa
+            q_rot = R @ query[s, qh].astype(f32)
+            m = f32(-np.inf)
+            l = f32(0)
+            acc = np.zeros(D, dtype=f32)
+            for bi in range(nblk):
+                phys = int(block_tables[s, bi])
+                n_valid = min(block_size, ctx - bi * block_size)
+                for pos in range(n_valid):
+                    k = c[_UNPACK[bits](k_packed[phys, pos, h][None], D)[0].astype(np.int64)]
+                    score = f32(np.dot(q_rot[0::2], k[0::2]) + np.dot(q_rot[1::2], k[1::2]))
+                    score = f32(score * f32(k_norms[phys, pos, h]) * scale)
+                    m_new = max(m, score)
+                    with np.errstate(invalid="ignore"):
+                        alpha = f32(np.exp(f32(m - m_new)))
+                    beta = f32(np.exp(f32(score - m_new)))
+                    l = f32(alpha * l + beta)
+                    v = c[_UNPACK[bits](v_packed[phys, pos, h][None], D)[0].astype(np.int64)]
+                    acc = alpha * acc + f32(beta * f32(v_norms[phys, pos, h])) * v
+                    m = m_new
+            if l > 0:
+                acc = acc / l
+            out[s, qh] = (R.T @ acc).astype(query.dtype)
+    return out
+
+
+def gather_dequant(packed, norms, block_tables, context_lens, centroids, bits, D, block_size,
+                   dtype=f32):
+    """Rotated-domain dequantisation of every token a sequence addresses:
+    yields per sequence an array [ctx, KVH, D] = centroids[idx] * norm (no inverse rotation)."""
+    c = np.asarray(centroids, dtype=dtype)
+    res = []
+    for s in range(len(context_lens)):
+        ctx = int(context_lens[s])
+        nblk = -(-ctx // block_size)
+        blocks = np.asarray(block_tables[s, :nblk], dtype=np.int64)
+        pk = packed[blocks].reshape((nblk * block_size,) + packed.shape[2:])[:ctx]
+        nm = norms[blocks].reshape((nblk * block_size,) + norms.shape[2:])[:ctx]
+        idx = _UNPACK[bits](pk, D).astype(np.int64)
+        res.append(c[idx] * nm[..., None].astype(dtype))
+    return res
+
+
+def paged_attention(query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
+                    rotation, centroids, bits, block_size=16, scale=None, dtype=f32,
+                    cast_output=True):
+    """Vectorised form of the same computation (softmax over all tokens at once instead of the
+    running max/sum of fused_attention.py:141-163 -- equal in exact arithmetic).  `dtype`
+    float64 gives a higher-precision judge for tolerance checks."""
+    query = np.asarray(query)
+    S, QH, D = query.shape
+    KVH = k_packed.shape[2]
+    gqa = QH // KVH
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    R = rotation.astype(dtype)
+    out = np.zeros((S, QH, D), dtype=dtype)
+    kd = gather_dequant(k_packed, k_norms, block_tables, context_lens, centroids, bits, D,
+                        block_size, dtype)
+    vd = gather_dequant(v_packed, v_norms, block_tables, context_lens, centroids, bits, D,
+                        block_size, dtype)
+    for s in range(S):
+        if int(context_lens[s]) == 0:
+            continue
+        q_rot = query[s].astype(dtype) @ R.T                       # [QH, D]
+        q_rot = q_rot.reshape(KVH, gqa, D)
+        sc = np.einsum("hgd,thd->hgt", q_rot, kd[s]) * dtype(scale)
+        sc -= sc.max(axis=-1, keepdims=True)
+        p = np.exp(sc)
+        p /= p.sum(axis=-1, keepdims=True)
+        acc = np.einsum("hgt,thd->hgd", p, vd[s]).reshape(QH, D)
+        out[s] = acc @ R
+    return out.astype(query.dtype) if cast_output else out
+
+
+# --------------------------------------------------------------------------------------
+# hybrid_quantizer.py (tq35, calibrate_uniform)
+# --------------------------------------------------------------------------------------
+def fwht(x):
+    """fwht_pow2, hybrid_quantizer.py:130-151: unnormalised Walsh-Hadamard butterflies over the
+    last axis (power of two)."""
+    x = np.array(x, dtype=f32, copy=True)
+    n = x.shape[-1]
+    h = 1
+    while h < n:
+        v = x.reshape(x.shape[:-1] + (-1, 2 * h))
+        a = v[..., :h].copy()
+        b = v[..., h:].copy()
+        v[..., :h] = a + b
+        v[..., h:] = a - b
+        h *= 2
+    return x
+
+
+def structured_hadamard(x, signs, inverse=False):
+    """structured_hadamard, hybrid_quantizer.py:200-234 with normalized=True."""
+    dim = x.shape[-1]
+    if inverse:
+        y = fwht(x) * signs
+    else:
+        y = fwht(x * signs)
+    return (y / f32(math.sqrt(dim))).astype(f32)
+
+
+def dimension_aware_codebook(dim: int, bits: int):
+    """dimension_aware_codebook, hybrid_quantizer.py:241-303: 200-iteration Lloyd on a
+    10,000-point grid weighted by (1-x^2)^((d-3)/2), float64, cast to float32."""
+    L = 1 << bits
+    n = 10000
+    start, end = -0.999, 0.999
+    step = (end - start) / (n - 1)
+    i = np.arange(n, dtype=np.float64)
+    # torch.linspace fills the upper half from the end point
+    grid = np.where(i < n // 2, start + step * i, end - step * (n - 1 - i))
+    w = (1.0 - grid * grid) ** ((dim - 3) / 2.0)
+    w = w / w.sum()
+    step_c = (grid[-1] - grid[0]) / (L - 1)
+    j = np.arange(L, dtype=np.float64)
+    c = np.where(j < L // 2, grid[0] + step_c * j, grid[-1] - step_c * (L - 1 - j))
+    for _ in range(200):
+        b = (c[:-1] + c[1:]) / 2.0
+        a = np.clip(np.searchsorted(b, grid, side="left"), 0, L - 1)
+        new = c.copy()
+        for k in range(L):
+            m = a == k
+            ws = w[m].sum()
+            if ws > 1e-30:
+                new[k] = (grid[m] * w[m]).sum() / ws
+        done = np.abs(c - new).max() < 1e-10
+        c = new
+        if done:
+            break
+    return c.astype(f32), ((c[:-1] + c[1:]) / 2.0).astype(f32)
+
+
+def pack_multibit(idx, bits):
+    """pack_multibit, hybrid_quantizer.py:310-352: MSB-first bit stream over the last axis."""
+    idx = np.asarray(idx).astype(np.int64)
+    dim = idx.shape[-1]
+    flat = idx.reshape(-1, dim) & ((1 << bits) - 1)
+    nbytes = math.ceil(dim * bits / 8)
+    bitsarr = np.zeros((flat.shape[0], nbytes * 8), dtype=np.uint8)
+    for b in range(bits):
+        bitsarr[:, b:dim * bits:bits] = (flat >> (bits - 1 - b)) & 1
+    return np.packbits(bitsarr, axis=-1, bitorder="big").reshape(idx.shape[:-1] + (nbytes,))
+
+
+def unpack_multibit(packed, dim, bits):
+    """unpack_multibit, hybrid_quantizer.py:355-396."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    flat = packed.reshape(-1, packed.shape[-1])
+    bitsarr = np.unpackbits(flat, axis=-1, bitorder="big")[:, :dim * bits]
+    v = np.zeros((flat.shape[0], dim), dtype=np.uint8)
+    for b in range(bits):
+        v = (v << 1) | bitsarr[:, b::bits]
+    return v.reshape(packed.shape[:-1] + (dim,))
+
+
+class HybridParams:
+    """The constants HybridTurboQuant(head_dim=128, mode='tq35') holds after
+    calibrate_uniform(): hybrid_quantizer.py:52-58,92-123,486-547,590-603.
+    The sign vectors come from torch's CPU generator (seed 42) and are arguments."""
+
+    def __init__(self, g0_had, g1_had, g0_qjl, g1_qjl, head_dim=128, codebooks=None):
+        assert head_dim == 128
+        self.head_dim = head_dim
+        self.g_dim = (64, 64)
+        self.mse_bits = (3, 2)
+        self.had = (np.asarray(g0_had, f32), np.asarray(g1_had, f32))
+        self.qjl = (np.asarray(g0_qjl, f32), np.asarray(g1_qjl, f32))
+        if codebooks is None:
+            codebooks = (dimension_aware_codebook(64, 3), dimension_aware_codebook(64, 2))
+        self.centroids = (codebooks[0][0], codebooks[1][0])
+        self.boundaries = (codebooks[0][1], codebooks[1][1])
+        self.qjl_scale = (math.sqrt(math.pi / 2.0) / 64, math.sqrt(math.pi / 2.0) / 64)
+        # byte layout: [mse | qjl bits | norm fp16 | residual norm fp16] per group
+        self.mse_bytes = (24, 16)
+        self.group_bytes = (24 + 8 + 4, 16 + 8 + 4)
+        self.packed_dim = 64
+
+
+def _hybrid_encode_group(xg, hp: HybridParams, g):
+    """_encode_single_group, hybrid_quantizer.py:706-779."""
+    xg = xg.astype(f32)
+    n = np.sqrt(np.sum(xg * xg, axis=-1, dtype=f32)).astype(f32)
+    unit = xg / (n[:, None] + f32(1e-10))
+    rot = structured_hadamard(unit, hp.had[g])
+    idx = np.clip(np.searchsorted(hp.boundaries[g], rot, side="left"), 0, (1 << hp.mse_bits[g]) - 1)
+    mse_packed = pack_multibit(idx, hp.mse_bits[g])
+    mse_hat = structured_hadamard(hp.centroids[g][idx], hp.had[g], inverse=True)
+    res = (unit - mse_hat).astype(f32)
+    rn = np.sqrt(np.sum(res * res, axis=-1, dtype=f32)).astype(f32)
+    proj = structured_hadamard(res, hp.qjl[g])
+    qjl_packed = pack_multibit((proj >= 0).astype(np.uint8), 1)
+    nb = n.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    rb = rn.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return np.concatenate([mse_packed, qjl_packed, nb, rb], axis=-1)
+
+
+def hybrid_encode(x, hp: HybridParams):
+    """HybridTurboQuant.encode with calibrate_uniform groups (dims 0..63 / 64..127),
+    hybrid_quantizer.py:616-704."""
+    x = np.asarray(x)
+    flat = x.reshape(-1, 128).astype(f32)
+    out = np.concatenate([_hybrid_encode_group(flat[:, :64], hp, 0),
+                          _hybrid_encode_group(flat[:, 64:], hp, 1)], axis=-1)
+    return out.reshape(x.shape[:-1] + (64,))
+
+
+def _hybrid_decode_group(pg, hp: HybridParams, g):
+    """_decode_single_group, hybrid_quantizer.py:876-933."""
+    mb = hp.mse_bytes[g]
+    idx = unpack_multibit(pg[:, :mb], 64, hp.mse_bits[g]).astype(np.int64)
+    mse_hat = structured_hadamard(hp.centroids[g][idx], hp.had[g], inverse=True)
+    sgn = 2.0 * unpack_multibit(pg[:, mb:mb + 8], 64, 1).astype(f32) - 1.0
+    qjl_hat = structured_hadamard((sgn * f32(hp.qjl_scale[g])).astype(f32), hp.qjl[g], inverse=True)
+    n = np.ascontiguousarray(pg[:, mb + 8:mb + 10]).view(np.float16).reshape(-1).astype(f32)
+    rn = np.ascontiguousarray(pg[:, mb + 10:mb + 12]).view(np.float16).reshape(-1).astype(f32)
+    return ((mse_hat + qjl_hat * rn[:, None]) * n[:, None]).astype(f32)
+
+
+def hybrid_decode(packed, hp: HybridParams):
+    """HybridTurboQuant.decode, hybrid_quantizer.py:785-874; returns float32."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    flat = packed.reshape(-1, 64)
+    out = np.concatenate([_hybrid_decode_group(flat[:, :36], hp, 0),
+                          _hybrid_decode_group(flat[:, 36:], hp, 1)], axis=-1)
+    return out.reshape(packed.shape[:-1] + (128,))
+
+
+def dense_attention(query, keys, values, scale, dtype=f32):
+    """softmax(q K^T * scale) V for one sequence with GQA: query [QH,D], keys/values [T,KVH,D]."""
+    QH, D = query.shape
+    KVH = keys.shape[1]
+    g = QH // KVH
+    q = query.astype(dtype).reshape(KVH, g, D)
+    sc = np.einsum("hgd,thd->hgt", q, keys.astype(dtype)) * dtype(scale)
+    sc -= sc.max(axis=-1, keepdims=True)
+    p = np.exp(sc)
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("hgt,thd->hgd", p, values.astype(dtype)).reshape(QH, D)
+
+
+def hybrid_paged_attention(query, k_cache, v_cache, block_tables, context_lens, hp: HybridParams,
+                           scale, block_size=16, dtype=f32):
+    """tq::hybrid_decode_step's attention (vllm/hooks.py:294-345) in float32: decompress every
+    addressed token with hybrid_decode, mask by context length, dense softmax attention.
+    Caches are [blocks, block_size, KVH, 64] uint8.  Returns float32 [S, QH, D]."""
+    query = np.asarray(query)
+    S, QH, D = query.shape
+    out = np.zeros((S, QH, D), dtype=dtype)
+    for s in range(S):
+        ctx = int(context_lens[s])
+        if ctx == 0:
+            continue
+        nblk = -(-ctx // block_size)
+        blocks = np.asarray(block_tables[s, :nblk], dtype=np.int64)
+        kp = k_cache[blocks].reshape((-1,) + k_cache.shape[2:])[:ctx]
+        vp = v_cache[blocks].reshape((-1,) + v_cache.shape[2:])[:ctx]
+        out[s] = dense_attention(query[s], hybrid_decode(kp, hp), hybrid_decode(vp, hp), scale,
+                                 dtype)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# triattention/
+# --------------------------------------------------------------------------------------
+def rope_frequencies(head_dim, base=1_000_000.0):
+    """spectral.py:34-51: theta_i = base ** (-2 i / d), evaluated in float32."""
+    i = np.arange(head_dim // 2, dtype=f32)
+    return np.power(f32(base), (f32(-2.0) * i) / f32(head_dim)).astype(f32)
+
+
+def spectral_encode(x, num_freqs=12):
+    """SpectralKVEncoder.encode for coeff_bits=4, encoder.py:73-133: top-F pairs by energy,
+    indices ascending, per-token max-abs scale (clamped at 1e-8), codes =
+    clamp(round((v/scale + 1) * 7.5), 0, 15), byte = code_even << 4 | code_odd, scale -> fp16."""
+    x = np.asarray(x)
+    D = x.shape[-1]
+    pairs = x.astype(f32).reshape(x.shape[:-1] + (D // 2, 2))
+    en = np.sum(pairs * pairs, axis=-1, dtype=f32)
+    order = np.argsort(-en, axis=-1, kind="stable")[..., :num_freqs]
+    top = np.sort(order, axis=-1)
+    tp = np.take_along_axis(pairs, top[..., None], axis=-2)
+    scales = np.maximum(np.abs(tp).reshape(tp.shape[:-2] + (-1,)).max(axis=-1), f32(1e-8))
+    nrm = tp / scales[..., None, None]
+    q = np.clip(np.round((nrm + f32(1)) * f32(7.5)), 0, 15).astype(np.uint8)
+    packed = ((q[..., 0] << 4) | q[..., 1]).astype(np.uint8)
+    return top.astype(np.uint8), packed, scales.astype(np.float16)
+
+
+def unpack_coefficients(packed, scales):
+    """TrigSeriesScorer._unpack_coefficients (4-bit), scorer.py:84-104."""
+    s = np.asarray(scales).astype(f32)[..., None]
+    v0 = (np.asarray(packed) >> 4).astype(f32)
+    v1 = (np.asarray(packed) & 0x0F).astype(f32)
+    return ((v0 / f32(7.5) - f32(1.0)) * s).astype(f32), ((v1 / f32(7.5) - f32(1.0)) * s).astype(f32)
+
+
+def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_positions=None):
+    """TrigSeriesScorer.score (pre-RoPE), scorer.py:115-208 -> [B, QH, S] float32 logits."""
+    query = np.asarray(query)
+    B, QH, D = query.shape
+    S, KVH = k_idx.shape[1], k_idx.shape[2]
+    gqa = QH // KVH
+    if key_positions is None:
+        key_positions = np.broadcast_to(np.arange(S)[None], (B, S))
+    if query_pos is None:
+        query_pos = np.full((B,), S)
+    k0, k1 = unpack_coefficients(k_packed, k_scales)              # [B,S,KVH,F]
+    hmap = np.arange(QH) // gqa
+    idx = k_idx.astype(np.int64)[:, :, hmap].transpose(0, 2, 1, 3)  # [B,QH,S,F]
+    k0 = k0[:, :, hmap].transpose(0, 2, 1, 3)
+    k1 = k1[:, :, hmap].transpose(0, 2, 1, 3)
+    qf = query.astype(f32)
+    qe = np.take_along_axis(np.broadcast_to(qf[..., 0::2][:, :, None], (B, QH, S, D // 2)), idx, -1)
+    qo = np.take_along_axis(np.broadcast_to(qf[..., 1::2][:, :, None], (B, QH, S, D // 2)), idx, -1)
+    c = qe * k0 + qo * k1
+    s = qo * k0 - qe * k1
+    delta = (np.asarray(key_positions).astype(f32).reshape(B, 1, S, 1)
+             - np.asarray(query_pos).astype(f32).reshape(B, 1, 1, 1))
+    ph = (delta * np.asarray(theta, dtype=f32)[idx]).astype(f32)
+    raw = np.sum(c * np.cos(ph) + s * np.sin(ph), axis=-1, dtype=f32)
+    return (raw * f32(1.0 / math.sqrt(D))).astype(f32)
+
+
+def tri_decode_step(query, k_enc, v_enc, theta, query_pos=None, key_positions=None):
+    """TriAttention.decode_step, attention.py:186-280: scores -> softmax over S -> weighted
+    scatter-add of the value coefficients into even/odd bins -> interleave.  k_enc / v_enc are
+    (indices, packed, scales) triples.  Returns float32 [B, QH, D]."""
+    query = np.asarray(query)
+    B, QH, D = query.shape
+    sc = tri_scores(query, *k_enc, theta, query_pos, key_positions)
+    sc = sc - sc.max(axis=-1, keepdims=True)
+    w = np.exp(sc)
+    w = (w / w.sum(axis=-1, keepdims=True, dtype=f32)).astype(f32)
+    v_idx, v_packed, v_scales = v_enc
+    KVH = v_idx.shape[2]
+    gqa = QH // KVH
+    v0, v1 = unpack_coefficients(v_packed, v_scales)               # [B,S,KVH,F]
+    out = np.zeros((B, QH, D), dtype=f32)
+    for b in range(B):
+        for qh in range(QH):
+            h = qh // gqa
+            ii = v_idx[b, :, h].astype(np.int64).reshape(-1)
+            wv0 = (w[b, qh][:, None] * v0[b, :, h]).reshape(-1)
+            wv1 = (w[b, qh][:, None] * v1[b, :, h]).reshape(-1)
+            np.add.at(out[b, qh], 2 * ii, wv0)
+            np.add.at(out[b, qh], 2 * ii + 1, wv1)
+    return out

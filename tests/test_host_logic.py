@@ -1,0 +1,216 @@
+"""Host-side behaviour that needs no GPU: configuration errors, sizes and layouts, init-time
+tables against the reference's, the C-ABI library's exports, and the loud failure on CPU
+tensors (reference: tests/test_core.py:246-425, tests/test_hybrid_hooks.py:411-442,
+tests/test_triattention.py:62-86)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import aitherkvcache_amd as akv
+from aitherkvcache_amd import _lib
+from aitherkvcache_amd.codebook import get_codebook, get_theory_bounds
+from aitherkvcache_amd.hybrid_quantizer import (HybridTurboQuant, _make_hybrid_layout,
+                                                _lloyd_on_grid, dimension_aware_codebook)
+from aitherkvcache_amd.packing import packed_size
+from aitherkvcache_amd.rotation import (random_orthogonal, hadamard_matrix, random_signs,
+                                        randomized_hadamard_matrix, fast_hadamard_transform)
+from aitherkvcache_amd.triattention import TriAttentionConfig, TriAttention, rope_frequencies
+from aitherkvcache_amd.vllm import resolve_kv_cache_dtype, register_custom_ops
+from aitherkvcache_amd.vllm.kv_cache_dtype import tq_dim_for_head
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- the C ABI -----------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "aitherkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(akv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 18
+    assert os.path.exists(_lib.LIB_PATH), "build the HIP library first (make -C aitherkvcache_amd/csrc)"
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [n for n in names if not hasattr(handle, n)]
+    assert not missing, missing
+    # and the Python binding lists the same set
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_library_loads_and_reports_version():
+    L = _lib.lib()
+    assert b"aitherkv" in L.akv_version()
+    assert L.akv_rotation_prepared_bytes(128) == 4 * 128 * 128 * 4
+    # argument validation happens before any device work
+    rc = L.akv_encode(None, 0, -1, 128, 128, None, None, 4, None, 64, None, None)
+    assert rc == _lib.AKV_ERR_INVALID and b"akv_encode" in L.akv_last_error()
+    rc = L.akv_encode(None, 0, 4, 96, 96, None, None, 4, None, 48, None, None)
+    assert rc == _lib.AKV_ERR_UNSUPPORTED
+    with pytest.raises(NotImplementedError):
+        _lib.check(rc)
+    with pytest.raises(ValueError):
+        _lib.check(_lib.AKV_ERR_INVALID)
+
+
+# ---- TurboQuant surface -------------------------------------------------------------------
+def test_config_errors():
+    with pytest.raises(ValueError, match="Supported bit-widths"):
+        akv.TurboQuant(head_dim=128, bits=5, device="cpu")
+    with pytest.raises(ValueError, match="power of 2"):
+        akv.TurboQuant(head_dim=100, bits=4, device="cpu")
+
+
+@pytest.mark.parametrize("bits,packed,ratio", [(4, 64, 3.8), (3, 48, 4.9), (2, 32, 7.1)])
+def test_sizes_and_ratios(bits, packed, ratio):
+    tq = akv.TurboQuant(head_dim=128, bits=bits, device="cpu")
+    assert tq._packed_dim == packed == packed_size(128, bits)
+    assert abs(tq.compression_ratio() - ratio) < 0.06
+    assert tq.num_levels == 1 << bits
+    assert tq.centroids.dtype == torch.float32 and tq.centroids.numel() == 1 << bits
+    assert tq.boundaries_inner.numel() == (1 << bits) - 1
+    assert "TurboQuant" in repr(tq) and f"bits={bits}" in repr(tq)
+    rep = tq.memory_report(seq_len=1024)
+    assert rep["ratio_vs_fp16"] == pytest.approx(256 / (packed + 4))
+    assert (tq.theory_lower, tq.theory_upper) == get_theory_bounds(bits)
+
+
+def test_cpu_tensors_fail_loudly():
+    tq = akv.TurboQuant(head_dim=128, bits=4, device="cpu")
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        tq.encode(torch.zeros(2, 128))
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        tq.decode(torch.zeros(2, 64, dtype=torch.uint8), torch.zeros(2))
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        akv.fused_tq4_kv_update(torch.zeros(1, 1, 128), torch.zeros(1, dtype=torch.int64),
+                                torch.zeros(1, 16, 1, 64, dtype=torch.uint8), torch.zeros(1, 16, 1),
+                                tq.rotation, tq.boundaries_inner)
+    # an empty update returns before touching anything, like the reference (fused_kv_update.py:340)
+    akv.fused_tq4_kv_update(torch.zeros(0, 1, 128), torch.zeros(0, dtype=torch.int64),
+                            torch.zeros(1, 16, 1, 64, dtype=torch.uint8), torch.zeros(1, 16, 1),
+                            tq.rotation, tq.boundaries_inner)
+    with pytest.raises(ValueError, match="power of 2"):
+        akv.fused_tq4_kv_update(torch.zeros(1, 1, 96), torch.zeros(1, dtype=torch.int64),
+                                torch.zeros(1, 16, 1, 48, dtype=torch.uint8), torch.zeros(1, 16, 1),
+                                tq.rotation, tq.boundaries_inner)
+
+
+# ---- init-time tables against the reference ------------------------------------------------
+def test_rotation_matches_reference(golden):
+    for d in (64, 128):
+        R = random_orthogonal(d, seed=42, device="cpu").numpy()
+        assert R.dtype == np.float32
+        # LAPACK's blocked QR rounds differently with the thread count, so the reference's own
+        # matrix moves by ~1e-6 between runs on different machines
+        assert np.max(np.abs(R - golden[f"rotation_d{d}_seed42"])) < 1e-5
+        assert np.allclose(R @ R.T, np.eye(d), atol=1e-5)
+    assert np.array_equal(random_orthogonal(128, 3, "cpu").numpy(), random_orthogonal(128, 3, "cpu").numpy())
+    assert not np.allclose(random_orthogonal(128, 3, "cpu").numpy(), random_orthogonal(128, 4, "cpu").numpy())
+    nthreads = torch.get_num_threads()
+    try:
+        torch.set_num_threads(1)
+        assert np.array_equal(random_orthogonal(128, 42, "cpu").numpy(), golden["rotation_d128_seed42"])
+    finally:
+        torch.set_num_threads(nthreads)
+
+
+def test_hadamard_helpers():
+    H = hadamard_matrix(16)
+    assert torch.allclose(H @ H.T, torch.eye(16), atol=1e-6)
+    x = torch.randn(3, 16)
+    assert torch.allclose(fast_hadamard_transform(x), x @ (H * 4).T, atol=1e-5)
+    M = randomized_hadamard_matrix(32, device="cpu")
+    assert torch.allclose(M @ M.T, torch.eye(32), atol=1e-5)
+    s = random_signs(64, seed=1, device="cpu")
+    assert set(s.tolist()) <= {-1.0, 1.0} and torch.equal(s, random_signs(64, seed=1, device="cpu"))
+    with pytest.raises(AssertionError):
+        hadamard_matrix(12)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_codebook_matches_reference(golden, bits):
+    c, b, _ = get_codebook(128, bits)
+    assert np.array_equal(c.astype(np.float32), golden[f"centroids_b{bits}"])
+    assert np.array_equal(b.astype(np.float32), golden[f"boundaries_b{bits}"])
+    with pytest.raises(ValueError):
+        get_codebook(128, 5)
+
+
+def test_hybrid_host_state_matches_reference(golden):
+    h = HybridTurboQuant(head_dim=128, mode="tq35", seed=42, device="cpu")
+    for nm in ("g0_had", "g1_had", "g0_qjl", "g1_qjl"):
+        assert np.array_equal(getattr(h, f"_{nm}_signs").numpy(), golden[f"hyb_{nm}_signs"])
+    for g, bits in ((0, 3), (1, 2)):
+        assert np.array_equal(getattr(h, f"_g{g}_centroids").numpy(), golden[f"hyb_centroids_64_{bits}"])
+        assert np.array_equal(getattr(h, f"_g{g}_boundaries").numpy(), golden[f"hyb_boundaries_64_{bits}"])
+        # and the general routine reproduces the tabulated case up to the noise in the middle boundary
+        c, b = _lloyd_on_grid(64, bits)
+        assert np.array_equal(c, golden[f"hyb_centroids_64_{bits}"])
+        assert np.allclose(b, golden[f"hyb_boundaries_64_{bits}"], rtol=0, atol=1e-15)
+    tab = h._table.numpy()
+    assert tab.shape == (_lib.HYB_TABLE_FLOATS,)
+    assert np.array_equal(tab[128:192], golden["hyb_g0_qjl_signs"])
+    assert np.array_equal(tab[256:264], golden["hyb_centroids_64_3"])
+    assert np.array_equal(tab[275:278], golden["hyb_boundaries_64_2"])
+    c, b = dimension_aware_codebook(32, 2)
+    assert c.numel() == 4 and torch.all(c[1:] > c[:-1])
+
+
+def test_hybrid_layout_and_errors():
+    lay = _make_hybrid_layout(128, "tq35")
+    assert (lay.group0.total_bytes, lay.group1.total_bytes, lay.packed_dim) == (36, 28, 64)
+    assert HybridTurboQuant.packed_dim_for_mode(128, "tq35") == 64
+    assert HybridTurboQuant.packed_dim_for_mode(128, "tq25") == 8 + 4 + 4 + 12 + 12 + 4
+    with pytest.raises(ValueError, match="Unsupported mode"):
+        HybridTurboQuant(mode="tq99", device="cpu")
+    h = HybridTurboQuant(device="cpu")
+    with pytest.raises(RuntimeError, match="calibrate"):
+        h.encode(torch.zeros(1, 128))
+    h.calibrate_uniform(num_kv_heads=8)
+    assert h._group0_indices.shape == (8, 64) and int(h._group1_indices[0, 0]) == 64
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        h.encode(torch.zeros(1, 128))
+    assert h.compression_ratio() == 4.0 and "calibrated" in repr(h)
+    t = HybridTurboQuant(mode="tq25", device="cpu")
+    t.calibrate_uniform()
+    with pytest.raises(NotImplementedError):
+        t.encode(torch.zeros(1, 128))
+
+
+def test_tri_config_and_theta(golden):
+    c = TriAttentionConfig()
+    assert c.bytes_per_kv_token == 26 and c.fp16_bytes_per_kv_token == 256 and c.compression_ratio > 9
+    assert TriAttentionConfig(coeff_bits=8).bytes_per_kv_token == 38
+    assert TriAttentionConfig(coeff_bits=16).bytes_per_kv_token == 62
+    with pytest.raises(ValueError, match="head_dim must be even"):
+        TriAttentionConfig(head_dim=127)
+    with pytest.raises(ValueError, match="cannot exceed"):
+        TriAttentionConfig(head_dim=32, num_freqs=20)
+    with pytest.raises(ValueError, match="coeff_bits"):
+        TriAttentionConfig(coeff_bits=6)
+    assert TriAttentionConfig(num_freqs=10, layer_freq_schedule=[16, 14]).freq_budget(1) == 14
+    assert np.array_equal(rope_frequencies(128, 1e6).numpy(), golden["theta_d128_base1e6"])
+    assert np.array_equal(rope_frequencies(32, 1e4).numpy(), golden["theta_d32_base1e4"])
+    tri = TriAttention(c, device="cpu")
+    enc = tri.encoder.encode(torch.from_numpy(golden["tri_keys"].astype(np.float32)))
+    assert np.array_equal(enc.indices.numpy(), golden["tri_k_indices"])
+    assert np.array_equal(enc.packed.numpy(), golden["tri_k_packed"])
+    assert np.array_equal(enc.scales.numpy(), golden["tri_k_scales"])
+
+
+def test_kv_cache_dtype_names_and_ops():
+    assert resolve_kv_cache_dtype("tq-t4nc").bits == 4
+    assert resolve_kv_cache_dtype("TQ-T3NC").bits == 3
+    assert resolve_kv_cache_dtype("tq-t2nc").packed_bytes_d128 == 32
+    assert resolve_kv_cache_dtype("tq35").mode == "tq35"
+    assert tq_dim_for_head(128, resolve_kv_cache_dtype("tq-t4nc")) == 68
+    assert tq_dim_for_head(128, resolve_kv_cache_dtype("tq-t35nc")) == 64
+    with pytest.raises(ValueError):
+        resolve_kv_cache_dtype("fp8")
+    assert register_custom_ops() and register_custom_ops()
+    assert hasattr(torch.ops.tq, "decode_step") and hasattr(torch.ops.tq, "hybrid_decode_step")
