@@ -255,7 +255,9 @@ static int akv_launch_attn_general_gq(const akv_attn_args& a, int grid, hipStrea
     return akv_fail(AKV_ERR_UNSUPPORTED, "paged_attn: num_q_heads*head_dim too large for LDS (%zu bytes)", lds);
   AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_general_kernel<D, BITS, GQ>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  akv_profile_mark_begin(stream);
   akv_attn_general_kernel<D, BITS, GQ><<<grid, 512, lds, stream>>>(a);
+  akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_attn_general_kernel");
   return AKV_OK;
 }

@@ -24,6 +24,35 @@ int akv_cached_cu_count() {
   return cached;
 }
 
+static bool g_profile_on = false;
+static hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
+static bool g_ev_recorded = false;
+
+void akv_profile_mark_begin(hipStream_t s) {
+  if (g_profile_on) (void)hipEventRecord(g_ev_begin, s);
+}
+void akv_profile_mark_end(hipStream_t s) {
+  if (g_profile_on) { (void)hipEventRecord(g_ev_end, s); g_ev_recorded = true; }
+}
+
+extern "C" int akv_profile_enable(int on) {
+  if (on && !g_ev_begin) {
+    AKV_HIP(hipEventCreate(&g_ev_begin));
+    AKV_HIP(hipEventCreate(&g_ev_end));
+  }
+  g_profile_on = on != 0;
+  g_ev_recorded = false;
+  return AKV_OK;
+}
+
+extern "C" int akv_profile_last_ms(float* ms) {
+  AKV_REQUIRE(ms != nullptr, "akv_profile_last_ms: null output");
+  if (!g_ev_recorded) return akv_fail(AKV_ERR_INVALID, "akv_profile_last_ms: nothing recorded");
+  AKV_HIP(hipEventSynchronize(g_ev_end));
+  AKV_HIP(hipEventElapsedTime(ms, g_ev_begin, g_ev_end));
+  return AKV_OK;
+}
+
 extern "C" const char* akv_version(void) { return "aitherkv-hip 0.1 (gfx950)"; }
 extern "C" const char* akv_last_error(void) { return akv_error_buffer(); }
 extern "C" int akv_device_cu_count(int* cu_count) {
@@ -381,7 +410,9 @@ static int akv_launch_gen(K kernel, const char* name, size_t lds, const akv_gen_
   int cus = akv_cached_cu_count();
   int64_t cap = (int64_t)(cus > 0 ? cus : 256) * 2;
   int grid = (int)(tiles < cap ? tiles : cap);
+  akv_profile_mark_begin((hipStream_t)stream);
   kernel<<<grid, 256, lds, (hipStream_t)stream>>>(a);
+  akv_profile_mark_end((hipStream_t)stream);
   AKV_LAUNCH_CHECK(name);
   return AKV_OK;
 }

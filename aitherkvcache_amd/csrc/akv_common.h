@@ -50,6 +50,10 @@ static inline int akv_packed_size(int d, int bits) { return d * bits / 8; }
 
 int akv_cached_cu_count();  // 0 when no device (defined in akv_codec.hip)
 
+// Event pair around the dominant kernel of an entry point (akv_profile_enable).
+void akv_profile_mark_begin(hipStream_t s);
+void akv_profile_mark_end(hipStream_t s);
+
 // Offsets (in floats) into the prepared-rotation buffer.
 //   [0, d*d)        Pi     row-major  (y_i = sum_j Pi[i][j] x_j)
 //   [d*d, 2*d*d)    Pi^T   row-major

@@ -460,7 +460,9 @@ static int hyb_launch_attn(const hyb_attn_args& a, int grid, hipStream_t stream)
   if (lds > 160 * 1024)
     return akv_fail(AKV_ERR_UNSUPPORTED, "hybrid_paged_attn: too many query heads for LDS (%zu bytes)", lds);
   AKV_HIP(hipFuncSetAttribute((const void*)hyb_attn_kernel<GQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  akv_profile_mark_begin(stream);
   hyb_attn_kernel<GQ><<<grid, 512, lds, stream>>>(a);
+  akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("hyb_attn_kernel");
   return AKV_OK;
 }

@@ -234,6 +234,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
   const int gqa = num_q_heads / num_kv_heads;
   dim3 grid(a.nsplit / TRI_WAVES, num_kv_heads, batch);
+  akv_profile_mark_begin(stream);
   if (gqa % 4 == 0) {
     const size_t lds = ((size_t)d / 2 + 4 * d + TRI_WAVES * 4 * d) * sizeof(float);
     tri_decode_kernel<4><<<grid, 256, lds, stream>>>(a);
@@ -241,6 +242,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
     const size_t lds = ((size_t)d / 2 + 1 * d + TRI_WAVES * 1 * d) * sizeof(float);
     tri_decode_kernel<1><<<grid, 256, lds, stream>>>(a);
   }
+  akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("tri_decode_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 64, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");

@@ -1,0 +1,342 @@
+#!/usr/bin/env python3
+"""Benchmark of the TurboQuant hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode4|decode3|decode2|tq35|tri|encode]
+
+A step is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  The default workload is the headline one: paged decode attention over a tq-t4nc cache
+at the Llama-3-8B layer shape (32 query / 8 KV heads, head_dim 128, batch 16, context lengths
+uniform in [1k, 40k], block_size 16, random non-contiguous block tables, seed 2), the cache
+having been written by the encode-on-write kernel.  One JSON line is printed:
+
+  value      algorithmic GB/s of the whole step (prologue + main + reduce kernels)
+  roofline   the dominant kernel alone: algorithmic bytes / its mean duration, measured with HIP
+             events on the launch stream (akv_profile_enable), against the 8 TB/s HBM peak
+  cpu_baseline  the numpy oracle of the same computation timed on this box's host cores on a
+             bounded sample of the same batch
+  encode     the encode-on-write kernel: Mvec/s on 2**20 vectors and the latency of one
+             256-token step (K and V, 8 heads)
+
+Algorithmic bytes per context token = 8 heads x (64 B codes + 4 B norm) x (K and V) = 1088 B
+(104 / 72 / 128 B x 8 for 3-bit / 2-bit / tq35), plus queries, outputs and block tables.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode4",
+                    choices=["decode4", "decode3", "decode2", "tq35", "tri", "encode"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    return ap.parse_args()
+
+
+def lognormal_kv(torch, shape, gen, dev):
+    """fp16 vectors: N(0,1) entries times a lognormal(0, 0.5) scale per vector."""
+    g = torch.randn(shape, device=dev, generator=gen)
+    s = torch.exp(0.5 * torch.randn(shape[:-1], device=dev, generator=gen))
+    return (g * s.unsqueeze(-1)).half()
+
+
+def profile_ms(L):
+    ms = ctypes.c_float()
+    rc = L.akv_profile_last_ms(ctypes.byref(ms))
+    if rc != 0:
+        raise RuntimeError(L.akv_last_error().decode())
+    return ms.value
+
+
+def timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def kernel_ms(torch, L, fn, steps):
+    """Mean duration of the dominant kernel over `steps` calls (HIP events on the launch stream)."""
+    L.akv_profile_enable(1)
+    acc = 0.0
+    for _ in range(steps):
+        fn()
+        acc += profile_ms(L)
+    L.akv_profile_enable(0)
+    return acc / steps
+
+
+# ---------------------------------------------------------------------------------------------
+def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds):
+    tq = akv.TurboQuant(head_dim=128, bits=4, device=str(dev))
+    gen = torch.Generator(device=dev).manual_seed(1)
+    res = {}
+    # (a) one serving step: 256 tokens x 8 heads, K and V, random free slots
+    NB, BS, H, T = 8192, 16, 8, 256
+    kp = torch.zeros(NB, BS, H, 64, dtype=torch.uint8, device=dev)
+    vp = torch.zeros_like(kp)
+    kn = torch.zeros(NB, BS, H, device=dev)
+    vn = torch.zeros_like(kn)
+    perm = torch.randperm(NB * BS, device=dev, generator=gen)
+    k = lognormal_kv(torch, (T, H, 128), gen, dev)
+    v = lognormal_kv(torch, (T, H, 128), gen, dev)
+    slots = perm[:T].contiguous()
+
+    class Cache:
+        pass
+    c = Cache()
+    c.tq, c.block_size, c.max_blocks = tq, BS, NB
+    c.k_packed, c.v_packed, c.k_norms, c.v_norms = kp[None], vp[None], kn[None], vn[None]
+    step_ms = timed(torch, lambda: akv.fused_encode_and_store(c, 0, k, v, slots), steps, warmup)
+    res["step_256tok_us"] = step_ms * 1e3
+    res["step_256tok_bytes"] = 2 * T * H * 324 + T * 8
+    # (b) bandwidth regime
+    n = 1 << 20
+    x = lognormal_kv(torch, (n, 128), gen, dev)
+    ms = timed(torch, lambda: tq.encode(x), max(5, steps // 5), 3)
+    kms = kernel_ms(torch, L, lambda: tq.encode(x), 5)
+    res["vectors"] = n
+    res["mvec_s"] = n / ms / 1e3
+    res["kernel_mvec_s"] = n / kms / 1e3
+    res["kernel_gbs"] = n * 324 / kms / 1e6
+    res["kernel_frac_hbm"] = res["kernel_gbs"] / HBM_PEAK_GBS
+    if cpu:
+        from oracle import tq_oracle as O
+        R = tq.rotation.cpu().numpy()
+        _, b, _ = O.get_codebook(128, 4)
+        xs = x[:65536].cpu().numpy()
+        O.encode(xs[:4096], R, b, 4)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < cpu_seconds / 3 or reps < 2:
+            O.encode(xs, R, b, 4)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_mvec_s"] = 65536 / dt / 1e6
+    return res, tq
+
+
+def decode_workload(torch, akv, dev, tq, bits_or_mode, seed, num_seqs, ctx):
+    """Cache written through the HIP encode kernels + tables + queries."""
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    KVH, QH, BS = 8, 32, 16
+    nblk = -(-ctx // BS)
+    NB = int(nblk.sum())
+    hybrid = bits_or_mode == "tq35"
+    P = 64 if hybrid else tq._packed_dim
+    kp = torch.zeros(NB, BS, KVH, P, dtype=torch.uint8, device=dev)
+    vp = torch.zeros_like(kp)
+    kn = vn = None
+    if not hybrid:
+        kn = torch.zeros(NB, BS, KVH, device=dev)
+        vn = torch.zeros_like(kn)
+    CH = 4096
+    for b0 in range(0, NB, CH):
+        b1 = min(NB, b0 + CH)
+        slots = torch.arange(b0 * BS, b1 * BS, device=dev)
+        for packed, norms in ((kp, kn), (vp, vn)):
+            x = lognormal_kv(torch, ((b1 - b0) * BS, KVH, 128), gen, dev)
+            if hybrid:
+                akv.hybrid_encode_and_store(tq, x, slots, packed, BS)
+            else:
+                akv.fused_kv_update(x, slots, packed, norms, tq.rotation, tq.boundaries_inner, tq.bits, BS)
+    perm = rng.permutation(NB)
+    tables = np.zeros((num_seqs, int(nblk.max())), dtype=np.int32)
+    off = 0
+    for s in range(num_seqs):
+        tables[s, :nblk[s]] = perm[off:off + nblk[s]]
+        off += nblk[s]
+    q = torch.randn(num_seqs, QH, 128, device=dev, generator=gen).half()
+    return dict(kp=kp, kn=kn, vp=vp, vn=vn, tables_np=tables, ctx_np=ctx,
+                tables=torch.from_numpy(tables).to(dev), ctx=torch.from_numpy(ctx.astype(np.int32)).to(dev),
+                q=q, QH=QH, KVH=KVH, BS=BS, NB=NB)
+
+
+def cpu_attention_baseline(w, tq, bits, seconds):
+    """The oracle's vectorised float32 attention on whole sequences of the batch, shortest first,
+    until the time budget is used."""
+    from oracle import tq_oracle as O
+    R = tq.rotation.cpu().numpy()
+    c = tq.centroids.cpu().numpy()
+    order = np.argsort(w["ctx_np"])
+    q = w["q"].cpu().numpy()
+    tokens = 0
+    used = []
+    t0 = time.perf_counter()
+    for s in order:
+        nb = -(-int(w["ctx_np"][s]) // 16)
+        blocks = w["tables"][s, :nb].long()
+        kp = w["kp"][blocks].cpu().numpy()
+        kn = w["kn"][blocks].cpu().numpy()
+        vp = w["vp"][blocks].cpu().numpy()
+        vn = w["vn"][blocks].cpu().numpy()
+        t1 = time.perf_counter()
+        O.paged_attention(q[s:s + 1], kp, kn, vp, vn, np.arange(nb)[None], w["ctx_np"][s:s + 1], R, c, bits)
+        dt = time.perf_counter() - t1
+        tokens += int(w["ctx_np"][s])
+        used.append((int(s), dt))
+        if time.perf_counter() - t0 > seconds:
+            break
+    compute = sum(d for _, d in used)
+    return tokens, compute, [s for s, _ in used]
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: this build has no multi-GPU path (the hot path shards "
+              "without communication by sequence, KV head or layer); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import aitherkvcache_amd as akv
+    from aitherkvcache_amd import _lib
+    from aitherkvcache_amd.triattention import TriAttention, TriAttentionConfig
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a HIP device")
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    cpu = not args.no_cpu
+
+    enc, tq4 = bench_encode(torch, akv, L, dev, args.steps, args.warmup, cpu, args.cpu_seconds)
+    out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "data": "synthetic", "unit": "GB/s"}
+    cpu_obj = None
+
+    if args.workload in ("decode4", "decode3", "decode2", "tq35"):
+        if args.workload == "decode4":
+            rng = np.random.default_rng(2)
+            ctx = rng.integers(1024, 40961, size=16).astype(np.int64)
+            name = "config 2: paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 16, ctx U[1k,40k], block 16, seed 2"
+            bits, per_tok, tq = 4, 1088, tq4
+        else:
+            ctx = np.full(64, 8192, dtype=np.int64)
+            bits = {"decode3": 3, "decode2": 2, "tq35": "tq35"}[args.workload]
+            per_tok = {"decode3": 8 * 104, "decode2": 8 * 72, "tq35": 8 * 128}[args.workload]
+            name = f"config 3: paged decode attention, {args.workload}, 32Q/8KV d=128, batch 64 x 8192, block 16, seed 3"
+            if bits == "tq35":
+                tq = akv.HybridTurboQuant(device=str(dev))
+                tq.calibrate_uniform(8)
+            else:
+                tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
+        seed = 2 if args.workload == "decode4" else 3
+        # two copies of the cache, alternated, so that no step finds its data in the 256 MB
+        # last-level cache left by the previous one
+        ws = [decode_workload(torch, akv, dev, tq, bits, seed + 100 * i, len(ctx), ctx) for i in range(2)]
+        if bits == "tq35":
+            attn = akv.HybridPagedAttention(tq, 32)
+            calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["vp"], w["tables"], w["ctx"], scale=1 / math.sqrt(128))
+                     for w in ws]
+        else:
+            attn = akv.TQPagedAttention(tq, 32)
+            calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["kn"], w["vp"], w["vn"], w["tables"], w["ctx"])
+                     for w in ws]
+        state = {"i": 0}
+
+        def step():
+            calls[state["i"] & 1]()
+            state["i"] += 1
+
+        tokens = int(ctx.sum())
+        algo_bytes = tokens * per_tok + 2 * len(ctx) * 32 * 128 * 2 + ws[0]["tables"].numel() * 4
+        ms = timed(torch, step, args.steps, args.warmup)
+        kms = kernel_ms(torch, L, step, max(10, args.steps // 2))
+        out.update(metric="tq-t4nc paged-decode attn GB/s" if args.workload == "decode4"
+                   else f"{args.workload} paged-decode attn GB/s",
+                   value=algo_bytes / ms / 1e6, ms_per_step=ms, dtype="f32",
+                   config={"workload": name, "context_tokens": tokens, "algorithmic_bytes_per_step": algo_bytes,
+                           "cache_copies_alternated": 2})
+        achieved = tokens * per_tok / kms / 1e6
+        out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                           "kernel": "main decode-attention kernel", "kernel_ms": kms}
+        if cpu and bits != "tq35":
+            toks, secs, seqs = cpu_attention_baseline(ws[0], tq, bits, args.cpu_seconds)
+            cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+                       "sample": f"numpy float32 oracle (gather, unpack, codebook, einsum, softmax, einsum, inverse "
+                                 f"rotation) on whole sequences {seqs} of the batch = {toks} context tokens"}
+    elif args.workload == "tri":
+        cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=8, num_query_heads=32,
+                                 rope_base=1e6)
+        tri = TriAttention(cfg, device=str(dev))
+        gen = torch.Generator(device=dev).manual_seed(4)
+        B, S = 8, 32768
+        std = (torch.arange(64, device=dev) + 1.0) ** -0.75
+        sets = []
+        for _ in range(3):     # three copies alternated: one copy (109 MB) would sit in the last-level cache
+            keys = (torch.randn(B, S, 8, 64, 2, device=dev, generator=gen) * std[:, None]).reshape(B, S, 8, 128).half()
+            vals = torch.randn(B, S, 8, 128, device=dev, generator=gen).half()
+            sets.append(tri.encode_kv(keys, vals))
+            del keys, vals
+        q = torch.randn(B, 32, 128, device=dev, generator=gen)
+        state = {"i": 0}
+
+        def step():
+            k_enc, v_enc = sets[state["i"] % 3]
+            tri.decode_step(q, k_enc, v_enc)
+            state["i"] += 1
+
+        algo_bytes = B * S * 8 * 52
+        ms = timed(torch, step, args.steps, args.warmup)
+        kms = kernel_ms(torch, L, step, max(10, args.steps // 2))
+        out.update(metric="TriAttention decode_step GB/s", value=algo_bytes / ms / 1e6, ms_per_step=ms, dtype="f32",
+                   config={"workload": "config 4: TriAttention decode_step, F=12 int4, 32Q/8KV d=128, batch 8 x 32768, seed 4",
+                           "algorithmic_bytes_per_step": algo_bytes, "cache_copies_alternated": 3})
+        achieved = algo_bytes / kms / 1e6
+        out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "tri_decode_kernel",
+                           "kernel_ms": kms}
+        if cpu:
+            from oracle import tq_oracle as O
+            k_enc, v_enc = sets[0]
+            S_s = 2048
+            ke = tuple(t[:1, :S_s].cpu().numpy() for t in k_enc)
+            ve = tuple(t[:1, :S_s].cpu().numpy() for t in v_enc)
+            th = tri._theta.cpu().numpy()
+            t0 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t0 < args.cpu_seconds or reps < 1:
+                O.tri_decode_step(q[:1].cpu().numpy(), ke, ve, th)
+                reps += 1
+            dt = (time.perf_counter() - t0) / reps
+            cpu_obj = {"value": S_s * 8 * 52 / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+                       "sample": f"numpy oracle of decode_step on batch element 0, first {S_s} tokens"}
+    else:  # encode as the measured step
+        n = enc["vectors"]
+        out.update(metric="tq-t4nc encode GB/s", value=n * 324 / (n / enc["mvec_s"] / 1e3) / 1e6,
+                   ms_per_step=n / enc["mvec_s"] / 1e3, dtype="f32",
+                   config={"workload": "TurboQuant.encode of 2**20 fp16 vectors x 128 (324 B per vector)"})
+        out["roofline"] = {"bound": "hbm", "achieved": enc["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": enc["kernel_frac_hbm"], "traffic": None, "kernel": "encode kernel"}
+        if cpu:
+            cpu_obj = {"value": enc.get("cpu_mvec_s", 0) * 324 / 1e3, "unit": "GB/s", "cores": cores, "kind": "port",
+                       "sample": "numpy oracle encode of 65,536 vectors (config 0)"}
+    out["cpu_baseline"] = cpu_obj
+    out["encode"] = enc
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -51,6 +51,16 @@ const char* akv_last_error(void);
 int akv_device_cu_count(int* cu_count);
 
 /* ---------------------------------------------------------------------------------
+ * Measurement hook (no counterpart in the reference).  While enabled, every entry point
+ * brackets its dominant kernel (the main decode-attention kernel, the encode kernel, the
+ * TriAttention scoring kernel) with a pair of HIP events recorded on the launch stream.
+ * akv_profile_last_ms waits for the pair of the most recent call and returns its elapsed
+ * time in milliseconds.  Meant for benchmarks; leave it off in serving code.
+ * ------------------------------------------------------------------------------- */
+int akv_profile_enable(int on);
+int akv_profile_last_ms(float* ms);
+
+/* ---------------------------------------------------------------------------------
  * Rotation matrix, prepared once per quantizer.
  * `rotation` is the reference's Pi (row-major [d,d] float32, y = Pi x,
  * aither_kvcache/rotation.py:20-35, used as x @ Pi.T at quantizer.py:150).  The

@@ -1,0 +1,263 @@
+"""Paged decode attention over the TurboQuant cache (HIP, through the C ABI) against the
+reference's own outputs and the oracle.  Tolerance: 2e-3 max-abs on fp16 outputs."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import aitherkvcache_amd as akv
+from oracle import tq_oracle as O
+from tests.util import kv_like
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def within_tol(got, ref64):
+    """|got - ref| <= 2e-3, plus the rounding of the fp16 output itself (half an fp16 ulp =
+    2**-11 relative) where |ref| is large enough for that to matter (|out| >= 4)."""
+    got = np.asarray(got, dtype=np.float64)
+    return bool(np.all(np.abs(got - ref64) <= TOL + 2.0 ** -11 * np.abs(ref64)))
+
+
+def make_tq(golden, dev, bits):
+    tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
+    tq.rotation = torch.from_numpy(golden["rotation_d128_seed42"]).to(dev)
+    return tq
+
+
+def t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("itype", [torch.int64, torch.int32])
+def test_golden_outputs(golden, dev, bits, itype):
+    tq = make_tq(golden, dev, bits)
+    attn = akv.TQPagedAttention(tq, num_query_heads=8)
+    tables = golden["attn_tables"]          # holds a 10**6 padding entry that must never be read
+    out = attn.forward(t(golden["attn_q"], dev), t(golden[f"attn_kp_b{bits}"], dev),
+                       t(golden[f"attn_kn_b{bits}"], dev), t(golden[f"attn_vp_b{bits}"], dev),
+                       t(golden[f"attn_vn_b{bits}"], dev), t(tables, dev).to(itype),
+                       t(golden["attn_ctx"], dev).to(itype), block_size=16, num_kv_heads=2)
+    assert out.dtype == torch.float16 and out.shape == (4, 8, 128)
+    got = out.cpu().numpy().astype(np.float32)
+    ref = golden[f"attn_out_b{bits}"].astype(np.float32)
+    assert np.all(got[0] == 0)                                   # ctx == 0 -> zeros
+    err = np.max(np.abs(got - ref))
+    print(f"[attn golden] bits={bits} max|diff|={err:.2e} exact={np.mean(got == ref):.4f}")
+    assert err <= TOL
+
+
+def build_cache(rng, tq, dev, num_blocks, kvh, bits, block_size=16, pad=0):
+    """Random K/V written through the HIP encode-on-write kernel.  Returns device tensors and the
+    host copies the oracle reads."""
+    P = tq._packed_dim
+    T = num_blocks * block_size
+    keys = kv_like(rng, (T, kvh, 128))
+    vals = kv_like(rng, (T, kvh, 128))
+    kp = torch.zeros(num_blocks, block_size, kvh, P + pad, dtype=torch.uint8, device=dev)
+    vp = torch.zeros_like(kp)
+    kn = torch.zeros(num_blocks, block_size, kvh, device=dev)
+    vn = torch.zeros_like(kn)
+    slots = torch.arange(T, device=dev)
+    akv.fused_kv_update(t(keys, dev), slots, kp, kn, tq.rotation, tq.boundaries_inner, bits, block_size)
+    akv.fused_kv_update(t(vals, dev), slots, vp, vn, tq.rotation, tq.boundaries_inner, bits, block_size)
+    return kp, kn, vp, vn
+
+
+def oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, bits, block_size=16, P=None):
+    c, _, _ = O.get_codebook(128, bits)
+    P = P or kp.shape[-1]
+    return O.paged_attention(q, kp.cpu().numpy()[..., :P], kn.cpu().numpy(), vp.cpu().numpy()[..., :P],
+                             vn.cpu().numpy(), tables, ctx, golden["rotation_d128_seed42"], c, bits,
+                             block_size=block_size, dtype=np.float64, cast_output=False)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("qh,kvh", [(32, 8), (8, 8), (6, 2), (16, 2)])
+def test_ragged_batch_vs_oracle(golden, dev, bits, qh, kvh):
+    """Ragged contexts (0, 1, partial block, many blocks), permuted non-contiguous tables, GQA
+    ratios 4 / 1 / 3 / 8."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(200 + bits + qh)
+    NB = 96
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, kvh, bits)
+    ctx = np.array([0, 1, 15, 16, 17, 333, 700, 64], dtype=np.int64)
+    width = 48
+    tables = np.full((len(ctx), width), -7, dtype=np.int64)             # garbage padding
+    for s, c_ in enumerate(ctx):
+        nb = -(-int(c_) // 16)
+        tables[s, :nb] = rng.permutation(NB)[:nb]
+    q = rng.standard_normal((len(ctx), qh, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, num_query_heads=qh)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), block_size=16, num_kv_heads=kvh)
+    ref = oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, bits)
+    got = out.cpu().numpy().astype(np.float64)
+    err = np.max(np.abs(got - ref))
+    print(f"[attn ragged] bits={bits} qh={qh} kvh={kvh} max|diff|={err:.2e} max|out|={np.abs(ref).max():.2f}")
+    assert np.all(got[0] == 0)
+    assert within_tol(got, ref)
+    # float32 queries give float32 outputs, closer still
+    out32 = attn.forward(t(q.astype(np.float32), dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), 16, kvh)
+    assert out32.dtype == torch.float32
+    assert np.max(np.abs(out32.cpu().numpy() - ref)) <= 5e-4
+
+
+def test_serving_layout_strided_views(golden, dev):
+    """K/V as views of one uint8 [blocks, 2, bs, heads, 68] tensor (row pitch 68 bytes) and norms
+    as a slice of a [layers, blocks, bs, heads] tensor."""
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(31)
+    NB, BS, KVH, QH = 40, 16, 8, 32
+    cache = torch.zeros(NB, 2, BS, KVH, 68, dtype=torch.uint8, device=dev)
+    norms = torch.zeros(2, 3, NB, BS, KVH, device=dev)
+    T = NB * BS
+    keys, vals = kv_like(rng, (T, KVH, 128)), kv_like(rng, (T, KVH, 128))
+    slots = torch.arange(T, device=dev)
+    akv.fused_tq4_kv_update(t(keys, dev), slots, cache[:, 0], norms[0, 1], tq.rotation, tq.boundaries_inner)
+    akv.fused_tq4_kv_update(t(vals, dev), slots, cache[:, 1], norms[1, 1], tq.rotation, tq.boundaries_inner)
+    ctx = np.array([640, 100, 37], dtype=np.int32)
+    tables = np.stack([rng.permutation(NB) for _ in range(3)]).astype(np.int32)
+    q = rng.standard_normal((3, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), cache[:, 0][..., :64], norms[0, 1], cache[:, 1][..., :64], norms[1, 1],
+                       t(tables, dev), t(ctx, dev))
+    ref = oracle_out(q, cache[:, 0], norms[0, 1], cache[:, 1], norms[1, 1], tables, ctx, golden, 4, P=64)
+    assert within_tol(out.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("block_size", [8, 32])
+def test_other_block_sizes(golden, dev, block_size):
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(block_size)
+    NB, KVH, QH = 24, 2, 8
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, 4, block_size=block_size)
+    ctx = np.array([block_size * 5 + 3, 2], dtype=np.int64)
+    tables = np.stack([rng.permutation(NB)[:8] for _ in range(2)])
+    q = rng.standard_normal((2, QH, 128)).astype(np.float16)
+    out = akv.TQPagedAttention(tq, QH).forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev),
+                                               block_size=block_size)
+    ref = oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, 4, block_size=block_size)
+    assert within_tol(out.cpu().numpy(), ref)
+
+
+def test_long_context_split_invariants(golden, dev):
+    """Sizes where a sequence is cut across many workgroups: results must not depend on where the
+    cuts fall.  (a) against the float64 oracle; (b) the same sequence alone or inside a batch
+    that shifts every cut; (c) a block-table permutation with the blocks moved accordingly."""
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(99)
+    NB, KVH, QH = 1600, 8, 32
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, 4)
+    ctx = np.array([12000, 1030, 5000, 7531], dtype=np.int64)
+    width = 800
+    tables = np.zeros((4, width), dtype=np.int64)
+    perm = rng.permutation(NB)
+    off = 0
+    for s, c_ in enumerate(ctx):
+        nb = -(-int(c_) // 16)
+        tables[s, :nb] = perm[off:off + nb]
+        off += nb
+    q = rng.standard_normal((4, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).cpu().numpy().astype(np.float64)
+    ref = oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, 4)
+    err = np.max(np.abs(out - ref))
+    print(f"[attn long] max|diff|={err:.2e}")
+    assert within_tol(out, ref)
+    # the invariance checks use float32 queries so that no fp16 output rounding blurs them
+    q32 = t(q.astype(np.float32), dev)
+    full = attn.forward(q32, kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).cpu().numpy()
+    assert np.max(np.abs(full - ref)) <= 3e-4
+    solo = attn.forward(q32[2:3], kp, kn, vp, vn, t(tables[2:3], dev), t(ctx[2:3], dev)).cpu().numpy()
+    assert np.max(np.abs(solo - full[2:3])) <= 2e-5
+    # move every physical block and remap the tables
+    mv = rng.permutation(NB)
+    inv = np.argsort(mv)
+    out2 = attn.forward(q32, kp[t(mv, dev)], kn[t(mv, dev)], vp[t(mv, dev)], vn[t(mv, dev)],
+                        t(inv[tables], dev), t(ctx, dev)).cpu().numpy()
+    assert np.max(np.abs(out2 - full)) <= 2e-5
+
+
+def test_config2_shape_properties(golden, dev):
+    """Llama-3-8B layer shape at benchmark scale (32Q/8KV, batch 16, ctx U[1k, 40k]): too large for
+    the oracle at full size, so: one sequence is checked against the oracle, and the softmax
+    weights must sum to one (uniform values -> output equals the value)."""
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(2)
+    ctx = rng.integers(1024, 40961, size=16).astype(np.int64)
+    nblk = -(-ctx // 16)
+    NB = int(nblk.sum())
+    KVH, QH = 8, 32
+    # K random; V = one fixed vector everywhere -> attention output must be that vector decoded
+    kp = torch.zeros(NB, 16, KVH, 64, dtype=torch.uint8, device=dev)
+    kn = torch.zeros(NB, 16, KVH, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(5)
+    CH = 2048
+    for b0 in range(0, NB, CH):
+        b1 = min(NB, b0 + CH)
+        x = torch.randn((b1 - b0) * 16, KVH, 128, device=dev, generator=gen).half()
+        akv.fused_tq4_kv_update(x, torch.arange(b0 * 16, b1 * 16, device=dev), kp, kn, tq.rotation,
+                                tq.boundaries_inner)
+    v1 = kv_like(rng, (1, KVH, 128))
+    vp1, vn1 = tq.encode(t(v1, dev))
+    vp = vp1.reshape(1, 1, KVH, 64).expand(NB, 16, KVH, 64).contiguous()
+    vn = vn1.reshape(1, 1, KVH).expand(NB, 16, KVH).contiguous()
+    perm = rng.permutation(NB)
+    tables = np.zeros((16, int(nblk.max())), dtype=np.int32)
+    off = 0
+    for s in range(16):
+        tables[s, :nblk[s]] = perm[off:off + nblk[s]]
+        off += nblk[s]
+    q = rng.standard_normal((16, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).float()
+    want = tq.decode(vp1, vn1).float().reshape(KVH, 1, 128).expand(KVH, 4, 128).reshape(1, QH, 128)
+    assert torch.max(torch.abs(out - want)).item() <= TOL
+    # shortest sequence against the oracle with random V
+    s = int(np.argmin(ctx))
+    vp_r, vn_r = kp.roll(5, 0), kn.roll(5, 0)
+    o = attn.forward(t(q[s:s + 1], dev), kp, kn, vp_r, vn_r, t(tables[s:s + 1], dev), t(ctx[s:s + 1], dev))
+    used = np.unique(tables[s, :nblk[s]])
+    remap = {b: i for i, b in enumerate(used)}
+    small_tab = np.array([[remap[b] for b in tables[s, :nblk[s]]]])
+    idx = t(used.astype(np.int64), dev)
+    ref = oracle_out(q[s:s + 1], kp[idx], kn[idx], vp_r[idx], vn_r[idx], small_tab, ctx[s:s + 1], golden, 4)
+    assert within_tol(o.cpu().numpy(), ref)
+
+
+def test_decode_step_custom_op(golden, dev):
+    """tq::decode_step: encode the step's token into the serving cache, attend, write output."""
+    from aitherkvcache_amd.vllm import hooks
+    hooks.reset_state()
+    assert hooks.register_custom_ops()
+    tq = hooks.init_quantizer(128, bits=4, device=str(dev))
+    tq.rotation = torch.from_numpy(golden["rotation_d128_seed42"]).to(dev)
+    rng = np.random.default_rng(55)
+    NB, BS, KVH, QH, L = 12, 16, 2, 8, 2
+    kv_cache = torch.zeros(NB, 2, BS, KVH, 68, dtype=torch.uint8, device=dev)
+    k_norms = torch.zeros(L, NB, BS, KVH, device=dev)
+    v_norms = torch.zeros_like(k_norms)
+    hist = 37                                              # tokens already in the cache per sequence
+    tables = np.stack([np.array([3, 7, 1, 0]), np.array([9, 2, 5, 0])]).astype(np.int32)
+    keys, vals = kv_like(rng, (2, hist + 1, KVH, 128)), kv_like(rng, (2, hist + 1, KVH, 128))
+    for s in range(2):
+        slots = np.array([tables[s, p // BS] * BS + p % BS for p in range(hist)])
+        akv.fused_tq4_kv_update(t(keys[s, :hist], dev), t(slots, dev), kv_cache[:, 0], k_norms[1], tq.rotation, tq.boundaries_inner)
+        akv.fused_tq4_kv_update(t(vals[s, :hist], dev), t(slots, dev), kv_cache[:, 1], v_norms[1], tq.rotation, tq.boundaries_inner)
+    new_slots = np.array([tables[s, hist // BS] * BS + hist % BS for s in range(2)] + [-1], dtype=np.int64)
+    q = rng.standard_normal((3, QH, 128)).astype(np.float16)           # third row is padding
+    key = np.concatenate([keys[:, hist], np.zeros((1, KVH, 128), np.float16)])
+    val = np.concatenate([vals[:, hist], np.zeros((1, KVH, 128), np.float16)])
+    output = torch.zeros(3, QH, 128, dtype=torch.float16, device=dev)
+    seq_lens = np.array([hist + 1, hist + 1], dtype=np.int32)
+    ret = torch.ops.tq.decode_step(t(q, dev), t(key, dev), t(val, dev), kv_cache, output, k_norms, v_norms,
+                                   t(new_slots, dev), t(tables, dev), t(seq_lens, dev), 1, QH, KVH, 128,
+                                   1 / math.sqrt(128), 2)
+    assert torch.equal(ret, output) and torch.all(output[2] == 0)
+    ref = oracle_out(q[:2], kv_cache[:, 0], k_norms[1], kv_cache[:, 1], v_norms[1], tables, seq_lens, golden, 4, P=64)
+    assert within_tol(output[:2].cpu().numpy(), ref)
+    # the new token really was written (its norm is in place), layer 0 untouched
+    assert float(k_norms[1, tables[0, hist // BS], hist % BS, 0]) > 0 and torch.all(k_norms[0] == 0)

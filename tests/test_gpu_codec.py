@@ -1,0 +1,229 @@
+"""HIP codec kernels (through the C ABI) against the oracle and the reference's own vectors."""
+import numpy as np
+import pytest
+import torch
+
+import aitherkvcache_amd as akv
+from aitherkvcache_amd import triton_ops
+from oracle import tq_oracle as O
+from tests.util import kv_like, code_mismatch_report
+
+pytestmark = pytest.mark.gpu
+
+MAX_ULPS = 16       # a code may differ from the float32 oracle only if the float64 rotated value
+                    # lies within this many float32 ulps of a decision boundary
+
+
+def make_tq(golden, dev, bits, d=128):
+    tq = akv.TurboQuant(head_dim=d, bits=bits, device=str(dev))
+    tq.rotation = torch.from_numpy(golden[f"rotation_d{d}_seed42"]).to(dev)   # the reference's matrix
+    return tq
+
+
+def check_codes(packed, norms, x, R, bits, ref_packed=None, ref_norms=None, d=128):
+    """Bit-exact codes modulo the boundary-ulp rule; norms to 1e-6 relative."""
+    _, b, _ = O.get_codebook(d, bits)
+    if ref_packed is None:
+        ref_packed, ref_norms = O.encode(x, R, b, bits)
+    ca = O._UNPACK[bits](packed.reshape(-1, packed.shape[-1]), d)
+    cb = O._UNPACK[bits](ref_packed.reshape(-1, ref_packed.shape[-1]), d)
+    y64 = O.rotate_unit_f64(np.asarray(x).reshape(-1, d), R)
+    n, max_ulps, hist = code_mismatch_report(ca, cb, y64, b, O)
+    total = ca.size
+    print(f"[codes] bits={bits} mismatching={n}/{total} max_ulps={max_ulps:.2f} hist={hist}")
+    assert max_ulps <= MAX_ULPS, hist
+    assert hist.get("max_code_step", 1) == 1
+    assert n <= max(3, total * 2e-5), (n, total)
+    nr = np.asarray(ref_norms).reshape(-1).astype(np.float64)
+    ng = np.asarray(norms).reshape(-1).astype(np.float64)
+    nz = nr > 0
+    assert np.max(np.abs(ng[nz] - nr[nz]) / nr[nz]) < 1e-6
+    assert np.all(ng[~nz] == 0)
+    return n
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_encode_decode_golden(golden, dev, bits):
+    tq = make_tq(golden, dev, bits)
+    x = golden["enc_x"]
+    packed, norms = tq.encode(torch.from_numpy(x).to(dev))
+    assert packed.dtype == torch.uint8 and packed.shape == (96, tq._packed_dim)
+    assert norms.dtype == torch.float32 and norms.shape == (96,)
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, golden["rotation_d128_seed42"], bits,
+                golden[f"enc_packed_b{bits}"], golden[f"enc_norms_b{bits}"])
+    # zero vector: ties at boundary 0.0 go to the lower bin (0x77.. at 4-bit), norm 0
+    mid = (1 << bits) // 2 - 1
+    assert np.all(O._UNPACK[bits](packed[5:6].cpu().numpy(), 128) == mid)
+    dec = tq.decode(torch.from_numpy(golden[f"enc_packed_b{bits}"]).to(dev),
+                    torch.from_numpy(golden[f"enc_norms_b{bits}"]).to(dev))
+    assert dec.dtype == torch.float16
+    ref = golden[f"dec_b{bits}"].astype(np.float32)
+    got = dec.cpu().numpy().astype(np.float32)
+    assert np.max(np.abs(got - ref)) <= 2e-3
+    assert np.mean(got == ref) > 0.995
+
+
+@pytest.mark.parametrize("dtype,key", [(torch.float32, "f32"), (torch.bfloat16, "bf16")])
+def test_encode_other_input_dtypes(golden, dev, dtype, key):
+    tq = make_tq(golden, dev, 4)
+    src = golden["enc_x_f32"] if key == "f32" else golden["enc_x_bf16_as_f32"]
+    x = torch.from_numpy(src).to(dev).to(dtype)
+    packed, norms = tq.encode(x)
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), src, golden["rotation_d128_seed42"], 4,
+                golden[f"enc_packed_{key}_b4"], golden[f"enc_norms_{key}_b4"])
+
+
+def test_head_dim_64(golden, dev):
+    tq = make_tq(golden, dev, 4, d=64)
+    x = golden["enc_x_d64"]
+    packed, norms = tq.encode(torch.from_numpy(x).to(dev))
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, golden["rotation_d64_seed42"], 4,
+                golden["enc_packed_d64_b4"], golden["enc_norms_d64_b4"], d=64)
+    dec = tq.decode(torch.from_numpy(golden["enc_packed_d64_b4"]).to(dev),
+                    torch.from_numpy(golden["enc_norms_d64_b4"]).to(dev)).cpu().numpy()
+    assert np.max(np.abs(dec.astype(np.float32) - golden["dec_d64_b4"].astype(np.float32))) <= 2e-3
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("n", [1, 31, 33, 4097])
+def test_encode_ragged_sizes_vs_oracle(golden, dev, bits, n):
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(1000 + n + bits)
+    x = kv_like(rng, (n, 128))
+    packed, norms = tq.encode(torch.from_numpy(x).to(dev))
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, golden["rotation_d128_seed42"], bits)
+    c, _, _ = O.get_codebook(128, bits)
+    dec = tq.decode(packed, norms).cpu().numpy().astype(np.float32)
+    ref = O.decode(packed.cpu().numpy(), norms.cpu().numpy(), golden["rotation_d128_seed42"], c, bits)
+    assert np.max(np.abs(dec - ref.astype(np.float32))) <= 2e-3 * max(1.0, np.abs(ref).max() / 4)
+
+
+def test_batch_shapes_and_empty(golden, dev):
+    tq = make_tq(golden, dev, 4)
+    x = torch.randn(2, 3, 5, 128, device=dev, dtype=torch.float16)
+    p, n = tq.encode(x)
+    assert p.shape == (2, 3, 5, 64) and n.shape == (2, 3, 5)
+    assert tq.decode(p, n).shape == (2, 3, 5, 128)
+    p1, n1 = tq.encode(x[0, 0, 0])
+    assert p1.shape == (64,) and n1.shape == ()
+    assert torch.equal(p1, p[0, 0, 0]) and torch.equal(n1, n[0, 0, 0])
+    pe, ne = tq.encode(torch.zeros(0, 128, device=dev, dtype=torch.float16))
+    assert pe.shape == (0, 64) and ne.shape == (0,)
+    assert tq.decode(pe, ne).shape == (0, 128)
+    # a strided view (every other row) encodes like its contiguous copy
+    big = torch.randn(64, 256, device=dev, dtype=torch.float16)
+    pv, nv = tq.encode(big[:, :128])
+    pc, nc = tq.encode(big[:, :128].contiguous())
+    assert torch.equal(pv, pc) and torch.equal(nv, nc)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_quantize_pack_and_unpack_lookup_exact(golden, dev, bits):
+    """Given the same rotated values these two are pure integer work: bit-exact."""
+    c, b, _ = O.get_codebook(128, bits)
+    rng = np.random.default_rng(5)
+    y = rng.normal(0, 0.09, size=(257, 128)).astype(np.float32)
+    y[0, :len(b)] = b                               # exact ties
+    y[1, :len(b)] = np.nextafter(b, np.float32(np.inf))
+    y[2] = 0.0
+    got = triton_ops.hip_quantize(torch.from_numpy(y).to(dev), torch.from_numpy(b).to(dev), bits)
+    want = O._PACK[bits](O.quantize(y, b, bits))
+    assert np.array_equal(got.cpu().numpy(), want)
+    back = triton_ops.hip_dequantize(got, torch.from_numpy(c).to(dev), 128, bits).cpu().numpy()
+    assert np.array_equal(back, c[O._UNPACK[bits](want, 128).astype(np.int64)])
+    if bits == 4:
+        assert torch.equal(triton_ops.triton_quantize_4bit(torch.from_numpy(y).to(dev), torch.from_numpy(b).to(dev)), got)
+
+
+@pytest.mark.parametrize("max_blocks,suffix", [(0, ""), (4, "_max4")])
+def test_paged_update_golden(golden, dev, max_blocks, suffix):
+    tq = make_tq(golden, dev, 4)
+    kp = torch.zeros(6, 16, 2, 64, dtype=torch.uint8, device=dev)
+    kn = torch.zeros(6, 16, 2, device=dev)
+    akv.fused_tq4_kv_update(torch.from_numpy(golden["upd_x"]).to(dev),
+                            torch.from_numpy(golden["upd_slots"]).to(dev), kp, kn, tq.rotation,
+                            tq.boundaries_inner, block_size=16, max_blocks=max_blocks)
+    ref_p, ref_n = golden["upd_packed" + suffix], golden["upd_norms" + suffix]
+    assert np.array_equal(kn.cpu().numpy() != 0, ref_n != 0)          # same tokens skipped
+    written = ref_n != 0
+    x = golden["upd_x"]
+    # rows in slot order for the ulp accounting
+    slots = golden["upd_slots"]
+    ok = (slots >= 0) & (slots // 16 < (max_blocks or 6))
+    check_codes(kp.cpu().numpy()[slots[ok] // 16, slots[ok] % 16], kn.cpu().numpy()[slots[ok] // 16, slots[ok] % 16],
+                x[ok], golden["rotation_d128_seed42"], 4,
+                ref_p[slots[ok] // 16, slots[ok] % 16], ref_n[slots[ok] // 16, slots[ok] % 16])
+    assert np.all(kp.cpu().numpy()[~written] == 0)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("itype", [torch.int64, torch.int32])
+def test_paged_update_strided_cache(golden, dev, bits, itype):
+    """The serving layout: uint8 [blocks, 2, bs, heads, packed + 4] with K = [:, 0], V = [:, 1];
+    rows are only 4-byte aligned and norms live in a [layers, blocks, bs, heads] tensor."""
+    tq = make_tq(golden, dev, bits)
+    P = tq._packed_dim
+    NB, BS, H, T = 8, 16, 4, 50
+    rng = np.random.default_rng(77 + bits)
+    cache = torch.full((NB, 2, BS, H, P + 4), 0xAB, dtype=torch.uint8, device=dev)
+    norms = torch.zeros(3, NB, BS, H, device=dev)
+    x = kv_like(rng, (T, H, 128))
+    slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+    slots[::7] = -1
+    akv.fused_kv_update(torch.from_numpy(x).to(dev), torch.from_numpy(slots).to(dev).to(itype),
+                        cache[:, 1], norms[2], tq.rotation, tq.boundaries_inner, bits, block_size=BS)
+    _, b, _ = O.get_codebook(128, bits)
+    ref_p = np.full((NB, BS, H, P + 4), 0xAB, np.uint8)
+    ref_n = np.zeros((NB, BS, H), np.float32)
+    view = ref_p[..., :P]
+    O.kv_update(x, slots, view, ref_n, golden["rotation_d128_seed42"], b, BS, 0, bits)
+    got = cache.cpu().numpy()
+    assert np.all(got[:, 0] == 0xAB)                                   # K half untouched
+    assert np.all(got[:, 1][..., P:] == 0xAB)                          # spare bytes untouched
+    ok = slots >= 0
+    check_codes(got[:, 1][slots[ok] // BS, slots[ok] % BS][..., :P], norms[2].cpu().numpy()[slots[ok] // BS, slots[ok] % BS],
+                x[ok], golden["rotation_d128_seed42"], bits)
+    assert np.array_equal(norms[2].cpu().numpy() != 0, ref_n != 0)
+    assert torch.all(norms[:2] == 0)
+
+
+def test_fused_encode_and_store(golden, dev):
+    class Cache:
+        pass
+    c = Cache()
+    c.tq = make_tq(golden, dev, 4)
+    c.block_size, c.max_blocks = 16, 4
+    c.k_packed = torch.zeros(2, 4, 16, 2, 64, dtype=torch.uint8, device=dev)
+    c.v_packed = torch.zeros_like(c.k_packed)
+    c.k_norms = torch.zeros(2, 4, 16, 2, device=dev)
+    c.v_norms = torch.zeros_like(c.k_norms)
+    k = torch.randn(5, 2, 128, device=dev, dtype=torch.float16)
+    v = torch.randn(5, 2, 128, device=dev, dtype=torch.float16)
+    slots = torch.tensor([3, 17, 40, 63, 64], device=dev)      # 64 -> block 4 >= max_blocks: skipped
+    akv.fused_encode_and_store(c, 1, k, v, slots)
+    kp, kn = c.tq.encode(k[:4])
+    vp, vn = c.tq.encode(v[:4])
+    b, p = (slots[:4] // 16).cpu(), (slots[:4] % 16).cpu()
+    assert torch.equal(c.k_packed[1][b, p].cpu(), kp.cpu()) and torch.equal(c.v_packed[1][b, p].cpu(), vp.cpu())
+    assert torch.equal(c.k_norms[1][b, p].cpu(), kn.cpu()) and torch.equal(c.v_norms[1][b, p].cpu(), vn.cpu())
+    assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
+
+
+def test_config0_round_trip_full_size(golden, dev):
+    """65,536 x 128 fp16, 4-bit: every code accounted for, distortion at the table value."""
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(0)
+    x = kv_like(rng, (65536, 128))
+    xt = torch.from_numpy(x).to(dev)
+    packed, norms = tq.encode(xt)
+    n = check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, golden["rotation_d128_seed42"], 4)
+    print(f"[config0] mismatching codes: {n} of {65536 * 128}")
+    xh = tq.decode(packed, norms).float()
+    xf = xt.float()
+    rel = ((xf - xh).pow(2).sum(-1) / xf.pow(2).sum(-1)).mean().item()
+    assert abs(rel - 0.0095) / 0.0095 < 0.05
+    # idempotence: re-encoding the reconstruction reproduces the codes (same cell) almost everywhere
+    p2, _ = tq.encode(xh)
+    assert (p2 == packed).float().mean().item() > 0.97
+    rep = tq.validate(num_vectors=20000)
+    assert rep["mse_theory_lower"] <= rep["mse"] <= rep["mse_theory_upper"] and rep["hip_active"]

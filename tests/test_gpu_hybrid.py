@@ -1,0 +1,151 @@
+"""tq35 hybrid codec and attention (HIP) against the reference's vectors and the oracle."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import aitherkvcache_amd as akv
+from oracle import tq_oracle as O
+from tests.util import kv_like
+
+pytestmark = pytest.mark.gpu
+
+
+def t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def params(golden):
+    books = tuple((golden[f"hyb_centroids_64_{k}"], golden[f"hyb_boundaries_64_{k}"]) for k in (3, 2))
+    return O.HybridParams(golden["hyb_g0_had_signs"], golden["hyb_g1_had_signs"],
+                          golden["hyb_g0_qjl_signs"], golden["hyb_g1_qjl_signs"], codebooks=books)
+
+
+def compare_rows(got, ref):
+    """Rows must agree byte for byte, except that a norm whose float32 value sits on an fp16
+    rounding boundary may land one fp16 step away (sum order), and a code / sign whose rotated
+    value sits on a decision boundary may flip.  Returns counts of each kind."""
+    got, ref = got.reshape(-1, 64), ref.reshape(-1, 64)
+    bad_rows = np.where(np.any(got != ref, axis=1))[0]
+    stats = {"rows": len(got), "rows_differing": len(bad_rows), "norm_ulp": 0, "code_bytes": 0, "sign_bytes": 0}
+    for r in bad_rows:
+        for lo in (32, 34, 60, 62):
+            a = int(got[r, lo]) | int(got[r, lo + 1]) << 8
+            b = int(ref[r, lo]) | int(ref[r, lo + 1]) << 8
+            if a != b:
+                assert abs(a - b) == 1, (r, lo, a, b)            # one fp16 step at most
+                stats["norm_ulp"] += 1
+        stats["code_bytes"] += int(np.sum(got[r, 0:24] != ref[r, 0:24]) + np.sum(got[r, 36:52] != ref[r, 36:52]))
+        stats["sign_bytes"] += int(np.sum(got[r, 24:32] != ref[r, 24:32]) + np.sum(got[r, 52:60] != ref[r, 52:60]))
+    return stats
+
+
+def test_golden_encode_decode(golden, dev):
+    h = akv.HybridTurboQuant(head_dim=128, mode="tq35", device=str(dev))
+    h.calibrate_uniform()
+    packed = h.encode(t(golden["hyb_x"], dev))
+    assert packed.dtype == torch.uint8 and packed.shape == (40, 64)
+    st = compare_rows(packed.cpu().numpy(), golden["hyb_packed"])
+    print("[hybrid golden]", st)
+    assert st["rows_differing"] <= 1
+    dec = h.decode(t(golden["hyb_packed"], dev))
+    assert dec.dtype == torch.float32
+    assert np.array_equal(dec.cpu().numpy(), golden["hyb_decoded"])            # bit-exact
+    h2 = akv.HybridTurboQuant(device=str(dev))
+    h2.calibrate_uniform(num_kv_heads=2)
+    p2 = h2.encode(t(golden["hyb_x_heads2"], dev))
+    assert p2.shape == (6, 2, 64)
+    assert compare_rows(p2.cpu().numpy(), golden["hyb_packed_heads2"])["rows_differing"] <= 1
+    assert np.array_equal(h2.decode(t(golden["hyb_packed_heads2"], dev)).cpu().numpy(), golden["hyb_decoded_heads2"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_encode_vs_oracle_bulk(golden, dev, dtype):
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform()
+    hp = params(golden)
+    rng = np.random.default_rng(9)
+    x = t(kv_like(rng, (20000, 128), np.float32), dev).to(dtype)
+    packed = h.encode(x).cpu().numpy()
+    ref = O.hybrid_encode(x.float().cpu().numpy(), hp)
+    st = compare_rows(packed, ref)
+    print("[hybrid bulk]", dtype, st)
+    assert st["rows_differing"] <= 0.01 * st["rows"]
+    assert st["code_bytes"] + st["sign_bytes"] <= 0.002 * st["rows"]
+    # decode is exact integer/butterfly work
+    dec = h.decode(t(ref, dev)).cpu().numpy()
+    assert np.array_equal(dec, O.hybrid_decode(ref, hp))
+    assert h.decode(t(ref, dev)[:0]).shape == (0, 128)
+    rep = h.validate(4000)
+    assert rep["cosine_similarity"] > 0.9 and rep["packed_dim_bytes"] == 64
+
+
+def build_cache(rng, h, dev, NB, KVH, BS=16, row=64):
+    kc = torch.zeros(NB, BS, KVH, row, dtype=torch.uint8, device=dev)
+    vc = torch.zeros_like(kc)
+    keys, vals = kv_like(rng, (NB * BS, KVH, 128)), kv_like(rng, (NB * BS, KVH, 128))
+    slots = torch.arange(NB * BS, device=dev)
+    akv.hybrid_encode_and_store(h, t(keys, dev), slots, kc, BS)
+    akv.hybrid_encode_and_store(h, t(vals, dev), slots, vc, BS)
+    return kc, vc, keys, vals
+
+
+@pytest.mark.parametrize("qh,kvh", [(32, 8), (6, 2)])
+def test_paged_attention_vs_oracle(golden, dev, qh, kvh):
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform(num_kv_heads=kvh)
+    hp = params(golden)
+    rng = np.random.default_rng(21 + qh)
+    NB = 64
+    kc, vc, keys, _ = build_cache(rng, h, dev, NB, kvh)
+    # paged write == flat encode of the same vectors
+    assert torch.equal(kc.reshape(-1, kvh, 64), h.encode(t(keys, dev)))
+    ctx = np.array([0, 1, 16, 17, 500, 333], dtype=np.int64)
+    tables = np.full((6, 32), -3, dtype=np.int64)
+    for s, c_ in enumerate(ctx):
+        nb = -(-int(c_) // 16)
+        tables[s, :nb] = rng.permutation(NB)[:nb]
+    q = rng.standard_normal((6, qh, 128)).astype(np.float16)
+    scale = 1 / math.sqrt(128)
+    attn = akv.HybridPagedAttention(h, qh)
+    out = attn.forward(t(q, dev), kc, vc, t(tables, dev), t(ctx, dev), scale=scale)
+    assert out.dtype == torch.float16
+    ref = O.hybrid_paged_attention(q, kc.cpu().numpy(), vc.cpu().numpy(), tables, ctx, hp, scale, dtype=np.float64)
+    err = np.max(np.abs(out.cpu().numpy().astype(np.float64) - ref))
+    print(f"[hybrid attn] qh={qh} max|diff|={err:.2e}")
+    got = out.cpu().numpy().astype(np.float64)
+    # 2e-3 plus half an fp16 ulp of the output itself where outputs are large
+    assert np.all(got[0] == 0) and np.all(np.abs(got - ref) <= 2e-3 + 2.0 ** -11 * np.abs(ref))
+    o32 = attn.forward(t(q.astype(np.float32), dev), kc, vc, t(tables, dev).int(), t(ctx, dev).int(), scale=0.05)
+    ref32 = O.hybrid_paged_attention(q, kc.cpu().numpy(), vc.cpu().numpy(), tables, ctx, hp, 0.05, dtype=np.float64)
+    assert np.max(np.abs(o32.cpu().numpy() - ref32)) <= 2e-4
+
+
+def test_hybrid_decode_step_custom_op(golden, dev):
+    from aitherkvcache_amd.vllm import hooks
+    hooks.reset_state()
+    hooks.register_custom_ops()
+    h = hooks.init_quantizer(128, mode="tq35", device=str(dev), num_kv_heads=2)
+    hp = params(golden)
+    rng = np.random.default_rng(66)
+    NB, BS, KVH, QH = 10, 16, 2, 8
+    kv_cache = torch.zeros(NB, 2, BS, KVH, 64, dtype=torch.uint8, device=dev)
+    hist = 21
+    tables = np.array([[4, 8, 0], [1, 6, 0]], dtype=np.int32)
+    keys, vals = kv_like(rng, (2, hist + 1, KVH, 128)), kv_like(rng, (2, hist + 1, KVH, 128))
+    for s in range(2):
+        slots = t(np.array([tables[s, p // BS] * BS + p % BS for p in range(hist)]), dev)
+        akv.hybrid_encode_and_store(h, t(keys[s, :hist], dev), slots, kv_cache[:, 0], BS)
+        akv.hybrid_encode_and_store(h, t(vals[s, :hist], dev), slots, kv_cache[:, 1], BS)
+    new_slots = np.array([tables[s, hist // BS] * BS + hist % BS for s in range(2)], dtype=np.int64)
+    q = rng.standard_normal((2, QH, 128)).astype(np.float16)
+    output = torch.zeros(2, QH, 128, dtype=torch.float16, device=dev)
+    seq_lens = np.array([hist + 1, hist + 1], dtype=np.int32)
+    scale = 0.09
+    ret = torch.ops.tq.hybrid_decode_step(t(q, dev), t(keys[:, hist], dev), t(vals[:, hist], dev), kv_cache, output,
+                                          t(new_slots, dev), t(tables, dev), t(seq_lens, dev), 0, QH, KVH, 128, scale, 2)
+    assert torch.equal(ret, output)
+    ref = O.hybrid_paged_attention(q, kv_cache[:, 0].cpu().numpy(), kv_cache[:, 1].cpu().numpy(), tables,
+                                   seq_lens, hp, scale, dtype=np.float64)
+    assert np.max(np.abs(output.cpu().numpy().astype(np.float64) - ref)) <= 2e-3

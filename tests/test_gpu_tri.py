@@ -1,0 +1,88 @@
+"""TriAttention decode_step (HIP) against the reference's outputs and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from aitherkvcache_amd.triattention import TriAttention, TriAttentionConfig, SpectralEncoding
+from oracle import tq_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-5     # float32 outputs; differences come from sin/cos last-place and summation order
+
+
+def t(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def enc(golden, nm, dev):
+    return SpectralEncoding(t(golden[f"tri_{nm}_indices"], dev), t(golden[f"tri_{nm}_packed"], dev),
+                            t(golden[f"tri_{nm}_scales"], dev))
+
+
+def test_golden_decode_step(golden, dev):
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=2, num_query_heads=8,
+                             rope_base=1_000_000.0)
+    tri = TriAttention(cfg, device=str(dev))
+    assert np.array_equal(tri._theta.cpu().numpy(), golden["theta_d128_base1e6"])
+    ke, ve = enc(golden, "k", dev), enc(golden, "v", dev)
+    q = t(golden["tri_q"], dev)
+    out = tri.decode_step(q, ke, ve)
+    assert out.dtype == torch.float32 and out.shape == (2, 8, 128)
+    e1 = np.max(np.abs(out.cpu().numpy() - golden["tri_out_default_pos"]))
+    out2 = tri.decode_step(q, ke, ve, t(golden["tri_qpos"], dev), t(golden["tri_kpos"], dev))
+    e2 = np.max(np.abs(out2.cpu().numpy() - golden["tri_out_explicit_pos"]))
+    print(f"[tri golden] default-pos {e1:.2e}, explicit-pos {e2:.2e}")
+    assert e1 <= TOL and e2 <= TOL
+    # int32 positions, fp16 query
+    out3 = tri.decode_step(q.half(), ke, ve, t(golden["tri_qpos"], dev).int(), t(golden["tri_kpos"], dev).int())
+    ref3 = O.tri_decode_step(golden["tri_q"].astype(np.float16), tuple(golden[f"tri_k_{n}"] for n in ("indices", "packed", "scales")),
+                             tuple(golden[f"tri_v_{n}"] for n in ("indices", "packed", "scales")),
+                             golden["theta_d128_base1e6"], golden["tri_qpos"], golden["tri_kpos"])
+    assert np.max(np.abs(out3.cpu().numpy() - ref3)) <= TOL
+
+
+@pytest.mark.parametrize("B,S,QH,KVH,D,F,base", [(3, 1000, 32, 8, 128, 12, 1e6), (2, 333, 6, 2, 32, 4, 1e4),
+                                                 (1, 64, 4, 4, 64, 32, 1e4), (2, 5000, 8, 1, 128, 12, 1e6)])
+def test_vs_oracle_shapes(dev, B, S, QH, KVH, D, F, base):
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=4, num_kv_heads=KVH, num_query_heads=QH, rope_base=base)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(S)
+    pair_std = (np.arange(D // 2) + 1.0) ** -0.75
+    keys = (rng.standard_normal((B, S, KVH, D // 2, 2)) * pair_std[:, None]).reshape(B, S, KVH, D).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    k_enc, v_enc = tri.encode_kv(t(keys, dev), t(vals, dev))
+    # the write side (torch ops on the device) agrees with the oracle's encoder
+    ki, kpk, ks = O.spectral_encode(keys, F)
+    assert np.array_equal(k_enc.indices.cpu().numpy(), ki) and np.array_equal(k_enc.packed.cpu().numpy(), kpk)
+    assert np.array_equal(k_enc.scales.cpu().numpy(), ks)
+    q = rng.standard_normal((B, QH, D)).astype(np.float32)
+    qpos = rng.integers(S, 40000, size=B)
+    kpos = np.sort(rng.integers(0, 32768, size=(B, S)), axis=-1)
+    theta = tri._theta.cpu().numpy()
+    out = tri.decode_step(t(q, dev), k_enc, v_enc, t(qpos, dev), t(kpos, dev)).cpu().numpy()
+    ref = O.tri_decode_step(q, (ki, kpk, ks), tuple(x.cpu().numpy() for x in v_enc), theta, qpos, kpos)
+    err = np.max(np.abs(out - ref))
+    print(f"[tri] B={B} S={S} D={D} F={F} max|diff|={err:.2e} max|out|={np.abs(ref).max():.3f}")
+    assert err <= TOL
+    out_d = tri.decode_step(t(q, dev), k_enc, v_enc).cpu().numpy()
+    ref_d = O.tri_decode_step(q, (ki, kpk, ks), tuple(x.cpu().numpy() for x in v_enc), theta)
+    assert np.max(np.abs(out_d - ref_d)) <= TOL
+
+
+def test_uniform_values_property(dev):
+    """Every token holds the same value row -> the output is that row, whatever the scores
+    (softmax weights sum to one across all splits)."""
+    cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32)
+    tri = TriAttention(cfg, device=str(dev))
+    B, S = 2, 32768
+    g = torch.Generator(device=dev).manual_seed(4)
+    keys = torch.randn(B, S, 8, 128, device=dev, generator=g).half()
+    one = torch.randn(1, 1, 8, 128, device=dev, generator=g).half()
+    k_enc, _ = tri.encode_kv(keys, keys)
+    v1 = tri.encoder.encode(one)
+    v_enc = SpectralEncoding(v1.indices.expand(B, S, 8, 12).contiguous(), v1.packed.expand(B, S, 8, 12).contiguous(),
+                             v1.scales.expand(B, S, 8).contiguous())
+    q = torch.randn(B, 32, 128, device=dev, generator=g)
+    out = tri.decode_step(q, k_enc, v_enc)
+    want = tri.encoder.decode(v1).reshape(1, 8, 1, 128).expand(B, 8, 4, 128).reshape(B, 32, 128)
+    assert torch.max(torch.abs(out - want)).item() <= 1e-5
