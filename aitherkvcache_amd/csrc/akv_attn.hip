@@ -240,12 +240,17 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
 // ----------------------------------------------------------------------------------
 // host entry
 // ----------------------------------------------------------------------------------
-// MFMA main kernel (akv_attn_mfma.hip); AKV_ERR_UNSUPPORTED when it does not apply.
-int akv_attn_mfma_try(const akv_attn_args& a, int d, int bits, int grid, hipStream_t stream);
+// MFMA path (akv_attn_mfma.hip)
+size_t akv_attn_mfma_extra_bytes(int S, int KVH);
+bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits);
+int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
+                      const akv_attn_args& a, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream);
 
 extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
   if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
-  return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, d, akv_attn_grid()).bytes;
+  // the number of kv heads is not known here; it is at most the number of query heads
+  return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, d, akv_attn_grid()).bytes +
+         akv_attn_mfma_extra_bytes(num_seqs, num_q_heads);
 }
 
 template <int D, int BITS, int GQ>
@@ -317,13 +322,11 @@ extern "C" int akv_paged_attn(
   if (workspace_bytes < ws.bytes)
     return akv_fail(AKV_ERR_WORKSPACE, "akv_paged_attn: workspace %zu < %zu bytes", workspace_bytes, ws.bytes);
 
+  if (workspace_bytes < ws.bytes + akv_attn_mfma_extra_bytes(num_seqs, num_q_heads))
+    return akv_fail(AKV_ERR_WORKSPACE, "akv_paged_attn: workspace %zu < %zu bytes", workspace_bytes,
+                    ws.bytes + akv_attn_mfma_extra_bytes(num_seqs, num_q_heads));
   const float* Pi = (const float*)rot_prep;
   const float* PiT = Pi + (size_t)d * d;
-  const int pgrid = num_seqs * num_q_heads + 1;
-#define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot)
-  if (q_dtype == AKV_F16) AKV_PRO(AKV_F16); else if (q_dtype == AKV_BF16) AKV_PRO(AKV_BF16); else AKV_PRO(AKV_F32);
-#undef AKV_PRO
-  AKV_LAUNCH_CHECK("akv_attn_prologue_kernel");
 
   akv_attn_args a;
   a.kp = k_packed; a.kps_blk = kps_blk; a.kps_pos = kps_pos; a.kps_head = kps_head;
@@ -337,8 +340,17 @@ extern "C" int akv_paged_attn(
   a.max_blocks_per_seq = max_blocks_per_seq; a.scale = scale;
   a.prefix = ws.prefix; a.qrot = ws.qrot; a.part_acc = ws.part_acc; a.part_ml = ws.part_ml;
 
-  int rc = akv_attn_mfma_try(a, d, bits, G, stream);
-  if (rc == AKV_ERR_UNSUPPORTED) {
+  int rc;
+  int Gused = G;
+  if (akv_attn_mfma_applicable(a, d, bits)) {
+    Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
+    rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
+  } else {
+    const int pgrid = num_seqs * num_q_heads + 1;
+#define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot)
+    if (q_dtype == AKV_F16) AKV_PRO(AKV_F16); else if (q_dtype == AKV_BF16) AKV_PRO(AKV_BF16); else AKV_PRO(AKV_F32);
+#undef AKV_PRO
+    AKV_LAUNCH_CHECK("akv_attn_prologue_kernel");
     rc = AKV_ERR_UNSUPPORTED;
 #define AKV_CASE(DD, BB) if (d == DD && bits == BB) rc = akv_launch_attn_general<DD, BB>(a, G, stream);
     AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
@@ -347,7 +359,7 @@ extern "C" int akv_paged_attn(
 #undef AKV_CASE
   }
   if (rc) return rc;
-  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
-  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
-  return akv_launch_reduce<256>(out_dtype, a, Pi, G, out, os_seq, os_head, stream);
+  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
+  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
+  return akv_launch_reduce<256>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
 }

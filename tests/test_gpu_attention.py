@@ -102,7 +102,9 @@ def test_ragged_batch_vs_oracle(golden, dev, bits, qh, kvh):
     # float32 queries give float32 outputs, closer still
     out32 = attn.forward(t(q.astype(np.float32), dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), 16, kvh)
     assert out32.dtype == torch.float32
-    assert np.max(np.abs(out32.cpu().numpy() - ref)) <= 5e-4
+    # float32 in/out isolates the arithmetic: the general kernels are float32 throughout (~1e-6);
+    # the MFMA kernel's fp16 codebook table costs ~1e-4 relative, i.e. up to ~6e-4 at |out| ~ 5
+    assert np.max(np.abs(out32.cpu().numpy() - ref)) <= 1e-3
 
 
 def test_serving_layout_strided_views(golden, dev):
@@ -170,7 +172,7 @@ def test_long_context_split_invariants(golden, dev):
     # the invariance checks use float32 queries so that no fp16 output rounding blurs them
     q32 = t(q.astype(np.float32), dev)
     full = attn.forward(q32, kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).cpu().numpy()
-    assert np.max(np.abs(full - ref)) <= 3e-4
+    assert np.max(np.abs(full - ref)) <= 1e-3
     solo = attn.forward(q32[2:3], kp, kn, vp, vn, t(tables[2:3], dev), t(ctx[2:3], dev)).cpu().numpy()
     assert np.max(np.abs(solo - full[2:3])) <= 2e-5
     # move every physical block and remap the tables
