@@ -35,53 +35,94 @@ __global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
 }
 
 // ----------------------------------------------------------------------------------
-// reduce: one wavefront per (sequence, query head)
+// reduce: one workgroup per (sequence, group of 4 query heads).  Wavefront w merges the
+// partials of head 4*group + w; then all 256 threads apply the inverse rotation, one load of
+// Pi[k][j] serving two heads.
 // ----------------------------------------------------------------------------------
 template <int D, int ODT>
-__global__ __launch_bounds__(64) void akv_attn_reduce_kernel(
+__global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
     const float* __restrict__ part_ml, const float* __restrict__ Pi, int S, int QH, int G,
     void* __restrict__ out, int64_t os_seq, int64_t os_head) {
   constexpr int DPL = D / 64;
-  __shared__ float a_lds[D];
-  const int s = blockIdx.x / QH, h = blockIdx.x % QH;
-  const int lane = threadIdx.x;
+  __shared__ float a_lds[4][D];
+  const int groups = (QH + 3) / 4;
+  const int s = blockIdx.x / groups, hg = blockIdx.x % groups;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int h = hg * 4 + wave;
   const int b0 = prefix[s], b1 = prefix[s + 1];
-  const int64_t obase = s * os_seq + h * os_head;
   if (b1 <= b0) {
+    if (h < QH) {
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, obase + lane * DPL + i, 0.f);
+      for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, s * os_seq + h * os_head + lane * DPL + i, 0.f);
+    }
     return;
   }
-  const int total = prefix[S];
-  const int per = (total + G - 1) / G;
-  const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
-  float m = -INFINITY, l = 0.f, acc[DPL];
+  if (h < QH) {
+    const int total = prefix[S];
+    const int per = (total + G - 1) / G;
+    const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
+    // pass 1 (lanes over slots, all loads in flight together): global max and sum
+    float M = -INFINITY;
+    for (int w = w_lo + lane; w <= w_hi; w += 64) M = fmaxf(M, part_ml[((size_t)(w + s) * QH + h) * 2]);
+    M = akv_wave_max(M);
+    float l = 0.f;
+    for (int w = w_lo + lane; w <= w_hi; w += 64) {
+      const size_t slot = (size_t)(w + s) * QH + h;
+      const float ms = part_ml[slot * 2];
+      if (ms > -INFINITY) l += __expf(ms - M) * part_ml[slot * 2 + 1];
+    }
+    l = akv_wave_sum(l);
+    // pass 2: weighted sum of the partial accumulators (independent loads, unrolled)
+    float acc[DPL];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
-  for (int w = w_lo; w <= w_hi; ++w) {
-    const size_t slot = (size_t)(w + s) * QH + h;
-    const float ms = part_ml[slot * 2], ls = part_ml[slot * 2 + 1];
-    float alpha, beta;
-    akv_lse_merge(m, l, ms, ls, alpha, beta);
+    for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+#pragma unroll 4
+    for (int w = w_lo; w <= w_hi; ++w) {
+      const size_t slot = (size_t)(w + s) * QH + h;
+      const float ms = part_ml[slot * 2];
+      const float wgt = ms > -INFINITY ? __expf(ms - M) : 0.f;
 #pragma unroll
-    for (int i = 0; i < DPL; ++i)
-      acc[i] = alpha * acc[i] + beta * part_acc[slot * D + lane * DPL + i];
+      for (int i = 0; i < DPL; ++i) acc[i] = fmaf(wgt, part_acc[slot * D + lane * DPL + i], acc[i]);
+    }
+    const float inv = l > 0.f ? 1.f / l : 1.f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) a_lds[wave][lane * DPL + i] = acc[i] * inv;
+  } else {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) a_lds[wave][lane * DPL + i] = 0.f;
   }
-  const float inv = l > 0.f ? 1.f / l : 1.f;
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) a_lds[lane * DPL + i] = acc[i] * inv;
   __syncthreads();
-  float o[DPL];
+  // inverse rotation: thread t owns coordinates (t % 128) * JP .. of heads 2 * (t / 128) and + 1
+  constexpr int JT = 128;                 // threads along the coordinate axis
+  constexpr int JP = D / JT > 0 ? D / JT : 1;   // coordinates per thread (D=256 -> 2)
+  const int jt = threadIdx.x % JT, pr = threadIdx.x / JT;
+  if (jt * JP < D) {
+    float o[2][JP];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) o[i] = 0.f;
-  for (int k = 0; k < D; ++k) {
-    const float a = a_lds[k];
+    for (int q = 0; q < 2; ++q)
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) o[i] = fmaf(a, Pi[(size_t)k * D + lane * DPL + i], o[i]);
+      for (int i = 0; i < JP; ++i) o[q][i] = 0.f;
+#pragma unroll 16
+    for (int k = 0; k < D; ++k) {
+      const float a0v = a_lds[2 * pr][k], a1v = a_lds[2 * pr + 1][k];
+#pragma unroll
+      for (int i = 0; i < JP; ++i) {
+        const float pv = Pi[(size_t)k * D + jt * JP + i];
+        o[0][i] = fmaf(a0v, pv, o[0][i]);
+        o[1][i] = fmaf(a1v, pv, o[1][i]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int hq = hg * 4 + 2 * pr + q;
+      if (hq < QH) {
+#pragma unroll
+        for (int i = 0; i < JP; ++i)
+          akv_elem<ODT>::store(out, s * os_seq + hq * os_head + jt * JP + i, o[q][i]);
+      }
+    }
   }
-#pragma unroll
-  for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, obase + lane * DPL + i, o[i]);
 }
 
 // ----------------------------------------------------------------------------------
@@ -277,11 +318,11 @@ static int akv_launch_attn_general(const akv_attn_args& a, int grid, hipStream_t
 template <int D>
 static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, int G, void* out,
                              int64_t os_seq, int64_t os_head, hipStream_t stream) {
-  const int grid = a.S * a.QH;
+  const int grid = a.S * ((a.QH + 3) / 4);
   switch (odt) {
-    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
-    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
-    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 64, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
   }
   AKV_LAUNCH_CHECK("akv_attn_reduce_kernel");
   return AKV_OK;

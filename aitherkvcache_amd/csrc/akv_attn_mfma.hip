@@ -37,12 +37,12 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 #ifndef MF_KSPLIT
 #define MF_KSPLIT 1                            // scores use hi + lo table halves (2 MFMA per k-step)
 #endif
-#define MF_ALPHA_CANDIDATES 4096
+#define MF_ALPHA_CANDIDATES 65536
 
 struct akv_mfma_extra {
-  const uint32_t* lut;   // [2][256] fp16 pairs: hi = fp16(alpha c), lo = fp16(alpha c - hi)  (workspace)
+  const uint32_t* lut;   // [2][256] fp16 pairs: hi = fp16(alpha c), lo = fp16(alpha c - hi); then the tag (workspace)
   const float* alpha;    // [1]                         (workspace)
-  const uint4* qop;      // [S][KVH][4 k-steps][64 lanes] half8 as uint4 (workspace)
+  const uint4* qop;      // [S][KVH][4 k-steps x 2 halves][64 lanes] half8 as uint4 (workspace)
 };
 
 // ----------------------------------------------------------------------------------
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
     uint4* __restrict__ qop, uint32_t* __restrict__ lut, float* __restrict__ alpha_out) {
-  __shared__ float q_lds[8][128];
+  __shared__ __align__(16) float q_lds[128][8];   // [input coordinate][query head of the group], zero-padded
   __shared__ float qr_lds[8][128];
   __shared__ int32_t scratch[257];
   __shared__ float best_err[256];
@@ -66,6 +66,15 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     return;
   }
   if ((int)blockIdx.x == nq + 1) {
+    // The table depends on the codebook only.  It is kept in the workspace together with the
+    // centroids it was built from (lut[512..527]) and a marker (lut[528]); when they match, the
+    // search is skipped.
+    __shared__ int stale;
+    if (tid == 0) stale = (lut[528] != 0x7451u) ? 1 : 0;
+    __syncthreads();
+    if (tid < 16 && __float_as_uint(centroids[tid]) != lut[512 + tid]) stale = 1;
+    __syncthreads();
+    if (!stale) return;
     // alpha search: minimise the largest relative fp16 rounding error of alpha * c over the levels
     float c[16];
     for (int v = 0; v < 16; ++v) c[v] = centroids[v];
@@ -96,30 +105,60 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     lut[tid] = (unsigned)__half_as_ushort(h0) | ((unsigned)__half_as_ushort(h1) << 16);
     const __half l0 = __float2half_rn(x0 - __half2float(h0)), l1 = __float2half_rn(x1 - __half2float(h1));
     lut[256 + tid] = (unsigned)__half_as_ushort(l0) | ((unsigned)__half_as_ushort(l1) << 16);
+    if (tid < 16) lut[512 + tid] = __float_as_uint(centroids[tid]);
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) lut[528] = 0x7451u;
     return;
   }
   const int s = blockIdx.x / KVH, h = blockIdx.x % KVH;
   const int gqa = QH / KVH;
-  for (int i = tid; i < gqa * 128; i += 256)
-    q_lds[i >> 7][i & 127] = akv_elem<QDT>::load(query, s * qs_seq + (h * gqa + (i >> 7)) * qs_head + (i & 127));
+  for (int i = tid; i < 8 * 128; i += 256) {
+    const int q = i >> 7, j = i & 127;
+    q_lds[j][q] = q < gqa ? akv_elem<QDT>::load(query, s * qs_seq + (h * gqa + q) * qs_head + j) : 0.f;
+  }
   __syncthreads();
   {
-    const int dim = tid & 127;
-    for (int q = tid >> 7; q < gqa; q += 2) {
-      float acc = 0.f;
-      for (int j = 0; j < 128; ++j) acc = fmaf(PiT[j * 128 + dim], q_lds[q][j], acc);
-      qr_lds[q][dim] = acc;
+    // thread (dim, half): partial dot products over 64 of the 128 input coordinates for every
+    // query head of the group; the 64 matrix loads of a thread are independent and unrolled
+    const int dim = tid & 127, half = tid >> 7;
+    float part[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) part[q] = 0.f;
+#pragma unroll 16
+    for (int jj = 0; jj < 64; ++jj) {
+      const int j = half * 64 + jj;
+      const float pv = PiT[j * 128 + dim];
+      const float4 qa = *(const float4*)&q_lds[j][0];
+      const float4 qc = *(const float4*)&q_lds[j][4];
+      part[0] = fmaf(pv, qa.x, part[0]); part[1] = fmaf(pv, qa.y, part[1]);
+      part[2] = fmaf(pv, qa.z, part[2]); part[3] = fmaf(pv, qa.w, part[3]);
+      part[4] = fmaf(pv, qc.x, part[4]); part[5] = fmaf(pv, qc.y, part[5]);
+      part[6] = fmaf(pv, qc.z, part[6]); part[7] = fmaf(pv, qc.w, part[7]);
+    }
+    if (half == 1) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) qr_lds[q][dim] = part[q];
+    }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) qr_lds[q][dim] += part[q];
     }
   }
   __syncthreads();
-  // operand layout: [k-step st][lane (col, g)][e] = coordinate 32g + 8st + e of column col
-  {
-    const int st = tid >> 6, lane = tid & 63;
+  // operand layout: [k-step st][half u][lane (col, g)][e].  The K operand of (st, u) holds, for
+  // bytes 2u and 2u+1 of dword st of the lane's 16 code bytes, the hi pair then the lo pair of
+  // the table entry: elements (0,1) hi / (2,3) lo of byte 2u, (4,5) hi / (6,7) lo of byte 2u+1.
+  // So element e of the query operand is coordinate 32g + 8st + 4u + 2(e/4) + (e&1).
+  for (int idx = tid; idx < 8 * 64; idx += 256) {
+    const int su = idx >> 6, lane = idx & 63;
+    const int st = su >> 1, u = su & 1;
     const int col = lane & 15, g = lane >> 4;
     unsigned short hbits[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int dim = 32 * g + 8 * st + e;
+      const int dim = 32 * g + 8 * st + 4 * u + 2 * (e >> 2) + (e & 1);
       float v = 0.f;
       if (col < 8) {
         if (col < gqa) v = __half2float(__float2half_rn(qr_lds[col][dim]));
@@ -132,7 +171,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     uint4 o;
     o.x = hbits[0] | (hbits[1] << 16); o.y = hbits[2] | (hbits[3] << 16);
     o.z = hbits[4] | (hbits[5] << 16); o.w = hbits[6] | (hbits[7] << 16);
-    qop[((size_t)(s * KVH + h) * 4 + st) * 64 + lane] = o;
+    qop[((size_t)(s * KVH + h) * 8 + su) * 64 + lane] = o;
   }
 }
 
@@ -145,19 +184,23 @@ struct mf_raw {      // what one wavefront loads for one 32-token chunk
   float kn[8], vn[8];  // norms of tokens 4g+i of tile 0 (i<4) and tile 1
 };
 
-__device__ __forceinline__ uint32_t mf_lut(const unsigned char* lds, uint32_t lane4, uint32_t word, uint32_t sel) {
+typedef __attribute__((address_space(3))) const uint32_t mf_lds_u32;
+
+// The table is the kernel's only LDS object, so it starts at LDS address 0 and a table address
+// can be used as the LDS address itself (saves one add per lookup).
+__device__ __forceinline__ uint32_t mf_lut(const unsigned char*, uint32_t lane4, uint32_t word, uint32_t sel) {
   // address = byte(word, k) * 256 + lane * 4, built by one byte permute:
   // result byte 0 <- lane4 byte 0 (selector 0x00), byte 1 <- word byte k (selector 0x04 + k), rest zero
   const uint32_t addr = __builtin_amdgcn_perm(word, lane4, sel);
-  return *(const uint32_t*)(lds + addr);
+  return *(mf_lds_u32*)(uintptr_t)addr;
 }
 
 // hi and lo halves of an entry in one go (the two loads differ by 128 bytes -> ds_read2_b32)
-__device__ __forceinline__ void mf_lut2(const unsigned char* lds, uint32_t lane4, uint32_t word, uint32_t sel,
+__device__ __forceinline__ void mf_lut2(const unsigned char*, uint32_t lane4, uint32_t word, uint32_t sel,
                                         uint32_t& hi, uint32_t& lo) {
   const uint32_t addr = __builtin_amdgcn_perm(word, lane4, sel);
-  hi = *(const uint32_t*)(lds + addr);
-  lo = *(const uint32_t*)(lds + addr + 128);
+  hi = *(mf_lds_u32*)(uintptr_t)addr;
+  lo = *(mf_lds_u32*)(uintptr_t)(addr + 128);
 }
 
 __device__ __forceinline__ half8 mf_pack(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -177,7 +220,8 @@ __device__ __forceinline__ float mf_from_lo_cols(float v) {
 
 __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
   const int col = lane & 15, g = lane >> 4;
   // replicate the table: dword index i = entry * 64 + half * 32 + copy
   {
@@ -212,13 +256,13 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
 
     for (int h = wave; h < a.KVH; h += MF_WAVES) {
       // query operand of this (sequence, kv head)
-      half8 qb[4];
+      half8 qb[8];
       {
-        const uint4* qp = x.qop + ((size_t)(s * a.KVH + h) * 4) * 64 + lane;
+        const uint4* qp = x.qop + ((size_t)(s * a.KVH + h) * 8) * 64 + lane;
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-          const uint4 u = qp[st * 64];
-          qb[st] = mf_pack(u.x, u.y, u.z, u.w);
+        for (int su = 0; su < 8; ++su) {
+          const uint4 u = qp[su * 64];
+          qb[su] = mf_pack(u.x, u.y, u.z, u.w);
         }
       }
       float4v o[8];
@@ -226,26 +270,43 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
       for (int j = 0; j < 8; ++j) o[j] = (float4v){0.f, 0.f, 0.f, 0.f};
       float m_run = -INFINITY, l_run = 0.f;
 
-      const unsigned char* kbase = a.kp + (int64_t)h * a.kps_head + (int64_t)col * a.kps_pos + 16 * g;
-      const unsigned char* vbase = a.vp + (int64_t)h * a.vps_head + 4 * col;
-      const float* knb = a.kn + (int64_t)h * a.kns_head;
-      const float* vnb = a.vn + (int64_t)h * a.vns_head;
+      // per-lane byte offsets inside a physical block (32-bit), added to a wavefront-uniform base
+      const uint32_t koff = (uint32_t)(h * a.kps_head + col * a.kps_pos + 16 * g);
+      uint32_t voff[4], knoff[4], vnoff[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        voff[i] = (uint32_t)(h * a.vps_head + (4 * g + i) * a.vps_pos + 4 * col);
+        knoff[i] = (uint32_t)((h * a.kns_head + (4 * g + i) * a.kns_pos) * 4);
+        vnoff[i] = (uint32_t)((h * a.vns_head + (4 * g + i) * a.vns_pos) * 4);
+      }
 
+      // physical block ids of the segment: lane i holds the id of block (window start + i); the
+      // window is refreshed every 64 blocks, so the chunk loop itself reads no table entry
+      // (a table load in the loop would make every prefetch wait for all loads before it)
+      int pbwin = 0;
+      auto load_window = [&](int first_blk) {
+        const int bi = min(first_blk + lane, blk_hi - 1);
+        pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
+      };
       auto load_chunk = [&](mf_raw& r, int c) {
-        const int bi0 = blk_lo + 2 * c;
-        const int bi1 = min(bi0 + 1, blk_hi - 1);
+        if ((c & 31) == 0) load_window(blk_lo + 2 * c);
+        const int w0 = (2 * c) & 63;
+        const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
         int64_t pb[2];
-        pb[0] = akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi0);
-        pb[1] = akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi1);
+        pb[0] = __builtin_amdgcn_readlane(pbwin, w0);
+        pb[1] = __builtin_amdgcn_readlane(pbwin, w1);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          r.k[j] = *(const uint4*)(kbase + pb[j] * a.kps_blk);
+          const unsigned char* kb = a.kp + pb[j] * a.kps_blk;
+          const unsigned char* vb = a.vp + pb[j] * a.vps_blk;
+          const unsigned char* knb = (const unsigned char*)(a.kn + pb[j] * a.kns_blk);
+          const unsigned char* vnb = (const unsigned char*)(a.vn + pb[j] * a.vns_blk);
+          r.k[j] = *(const uint4*)(kb + koff);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int pos = 4 * g + i;
-            r.v[4 * j + i] = *(const uint32_t*)(vbase + pb[j] * a.vps_blk + (int64_t)pos * a.vps_pos);
-            r.kn[4 * j + i] = knb[pb[j] * a.kns_blk + (int64_t)pos * a.kns_pos];
-            r.vn[4 * j + i] = vnb[pb[j] * a.vns_blk + (int64_t)pos * a.vns_pos];
+            r.v[4 * j + i] = *(const uint32_t*)(vb + voff[i]);
+            r.kn[4 * j + i] = *(const float*)(knb + knoff[i]);
+            r.vn[4 * j + i] = *(const float*)(vnb + vnoff[i]);
           }
         }
       };
@@ -254,37 +315,42 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
         const int tok0 = (blk_lo + 2 * c) * 16;      // first token of tile 0
         // ---- scores
         float sv[8];
+        {
+          // 16 steps (tile j, dword st, half u); the table reads of step n+1 are issued before
+          // the MFMA of step n
+          const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
+          uint32_t w[2][4];
+          float4v acc[2];
+          acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
+          acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
+          mf_lut2(lut_lane, lane4, kw[0], 0x0c0c0400u, w[0][0], w[0][1]);
+          mf_lut2(lut_lane, lane4, kw[0], 0x0c0c0500u, w[0][2], w[0][3]);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          float4v acc = (float4v){0.f, 0.f, 0.f, 0.f};
-          const uint32_t kw[4] = {r.k[j].x, r.k[j].y, r.k[j].z, r.k[j].w};
-#pragma unroll
-          for (int st = 0; st < 4; ++st) {
-#if MF_KSPLIT
-            uint32_t h[4], lw[4];
-            mf_lut2(lut_lane, lane4, kw[st], 0x0c0c0400u, h[0], lw[0]);
-            mf_lut2(lut_lane, lane4, kw[st], 0x0c0c0500u, h[1], lw[1]);
-            mf_lut2(lut_lane, lane4, kw[st], 0x0c0c0600u, h[2], lw[2]);
-            mf_lut2(lut_lane, lane4, kw[st], 0x0c0c0700u, h[3], lw[3]);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(h[0], h[1], h[2], h[3]), qb[st], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(lw[0], lw[1], lw[2], lw[3]), qb[st], acc, 0, 0, 0);
-#else
-            const half8 ka = mf_pack(mf_lut(lut_lane, lane4, kw[st], 0x0c0c0400u), mf_lut(lut_lane, lane4, kw[st], 0x0c0c0500u),
-                                     mf_lut(lut_lane, lane4, kw[st], 0x0c0c0600u), mf_lut(lut_lane, lane4, kw[st], 0x0c0c0700u));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[st], acc, 0, 0, 0);
-#endif
+          for (int n = 0; n < 16; ++n) {
+            if (n + 1 < 16) {
+              const int n1 = n + 1;
+              const uint32_t word = kw[n1 >> 1];
+              const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (n1 & 1)) << 8);
+              mf_lut2(lut_lane, lane4, word, sel, w[n1 & 1][0], w[n1 & 1][1]);
+              mf_lut2(lut_lane, lane4, word, sel + 0x100u, w[n1 & 1][2], w[n1 & 1][3]);
+            }
+            acc[n >> 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(w[n & 1][0], w[n & 1][1], w[n & 1][2], w[n & 1][3]),
+                                                                 qb[n & 7], acc[n >> 3], 0, 0, 0);
           }
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // columns c and c + 8 carry the hi and lo part of the same query head: both lanes form
-            // the same sum, so the softmax state below is identical in the two
-            // (both cross-lane moves run with all lanes active; only the choice is per lane)
-            const float from_hi = mf_from_hi_cols(acc[i]);
-            const float from_lo = mf_from_lo_cols(acc[i]);
-            const float full = acc[i] + (col < 8 ? from_hi : from_lo);
-            const int tok = tok0 + 16 * j + 4 * g + i;
-            const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
-            sv[4 * j + i] = ok ? full * r.kn[4 * j + i] * sc_mul : -INFINITY;
+          for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              // columns c and c + 8 carry the hi and lo part of the same query head: both lanes form
+              // the same sum, so the softmax state below is identical in the two
+              // (both cross-lane moves run with all lanes active; only the choice is per lane)
+              const float from_hi = mf_from_hi_cols(acc[j][i]);
+              const float from_lo = mf_from_lo_cols(acc[j][i]);
+              const float full = acc[j][i] + (col < 8 ? from_hi : from_lo);
+              const int tok = tok0 + 16 * j + 4 * g + i;
+              const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
+              sv[4 * j + i] = ok ? full * r.kn[4 * j + i] * sc_mul : -INFINITY;
+            }
           }
         }
         // ---- running softmax (per column; rows of 16 lanes hold different tokens)
@@ -303,19 +369,15 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
             for (int i = 0; i < 4; ++i) o[j][i] *= resc;
           m_run = m_new;
         }
-        float pw[8];
+        // weights: hi part in columns [0,8), remainder in columns [8,16)
+        half8 pb;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const float p = __expf(sv[i] - m_run);      // exp(-inf) = 0 for masked tokens
           l_run += p;
-          pw[i] = p * r.vn[i] * inv_alpha;
-        }
-        // hi part in columns [0,8), remainder in columns [8,16)
-        half8 pb;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float hi = __half2float(__float2half_rn(pw[i]));
-          pb[i] = (_Float16)(col < 8 ? hi : pw[i] - hi);
+          const float pw = p * r.vn[i] * inv_alpha;
+          const float hi = __half2float(__float2half_rn(pw));
+          pb[i] = (_Float16)(col < 8 ? hi : pw - hi);
         }
         // ---- values: pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates
         uint32_t xe[4], xo[4];
@@ -325,15 +387,22 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
           xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
           xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
         }
+        {
+          // 8 steps: step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
+          uint32_t w[2][4];
 #pragma unroll
-        for (int bi = 0; bi < 4; ++bi) {               // byte bi of the dword: coordinates 8m + 2bi, 8m + 2bi + 1
-          const uint32_t sel = 0x0c0c0400u + ((uint32_t)bi << 8);
-          const half8 ve = mf_pack(mf_lut(lut_lane, lane4, xe[0], sel), mf_lut(lut_lane, lane4, xe[1], sel),
-                                   mf_lut(lut_lane, lane4, xe[2], sel), mf_lut(lut_lane, lane4, xe[3], sel));
-          o[2 * bi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ve, pb, o[2 * bi], 0, 0, 0);
-          const half8 vo = mf_pack(mf_lut(lut_lane, lane4, xo[0], sel), mf_lut(lut_lane, lane4, xo[1], sel),
-                                   mf_lut(lut_lane, lane4, xo[2], sel), mf_lut(lut_lane, lane4, xo[3], sel));
-          o[2 * bi + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vo, pb, o[2 * bi + 1], 0, 0, 0);
+          for (int p = 0; p < 4; ++p) w[0][p] = mf_lut(lut_lane, lane4, xe[p], 0x0c0c0400u);
+#pragma unroll
+          for (int n = 0; n < 8; ++n) {
+            if (n + 1 < 8) {
+              const int n1 = n + 1;
+              const uint32_t sel = 0x0c0c0400u + ((uint32_t)(n1 >> 1) << 8);
+#pragma unroll
+              for (int p = 0; p < 4; ++p) w[n1 & 1][p] = mf_lut(lut_lane, lane4, (n1 & 1) ? xo[p] : xe[p], sel);
+            }
+            o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(w[n & 1][0], w[n & 1][1], w[n & 1][2], w[n & 1][3]),
+                                                          pb, o[n], 0, 0, 0);
+          }
         }
       };
 
@@ -384,7 +453,7 @@ static bool mfma_disabled() {
 
 // extra workspace the MFMA path needs beyond akv_attn_ws (appended after it)
 size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
-  return akv_align256(2048) + akv_align256(4) + akv_align256((size_t)S * KVH * 4 * 64 * 16);
+  return akv_align256(2304) + akv_align256(4) + akv_align256((size_t)S * KVH * 8 * 64 * 16);
 }
 
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
@@ -409,7 +478,7 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
                       const akv_attn_args& a, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
   akv_mfma_extra x;
   char* p = (char*)extra_ws;
-  x.lut = (const uint32_t*)p; p += akv_align256(2048);
+  x.lut = (const uint32_t*)p; p += akv_align256(2304);
   x.alpha = (const float*)p; p += akv_align256(4);
   x.qop = (const uint4*)p;
   if (q_dtype == AKV_F16) launch_mfma_prologue<AKV_F16>(query, qs_seq, qs_head, PiT, a, prefix, x, stream);

@@ -217,7 +217,8 @@ def test_config2_shape_properties(golden, dev):
     attn = akv.TQPagedAttention(tq, QH)
     out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).float()
     want = tq.decode(vp1, vn1).float().reshape(KVH, 1, 128).expand(KVH, 4, 128).reshape(1, QH, 128)
-    assert torch.max(torch.abs(out - want)).item() <= TOL
+    # both sides are fp16-rounded: allow one fp16 ulp on top of the tolerance
+    assert bool(torch.all(torch.abs(out - want) <= TOL + 2.0 ** -10 * want.abs()))
     # shortest sequence against the oracle with random V
     s = int(np.argmin(ctx))
     vp_r, vn_r = kp.roll(5, 0), kn.roll(5, 0)
