@@ -1,48 +1,70 @@
 // MFMA paged decode attention for the 4-bit cache at head_dim 128, block_size 16.
 //
-// One workgroup = 8 wavefronts, wavefront <-> kv head; tokens are taken 32 at a time (two
-// physical blocks).  Everything is arranged so that no register ever has to be transposed:
+// One workgroup = 16 wavefronts working on one range of (sequence, block) pairs for all kv
+// heads: wavefronts 0-7 are SCORE wavefronts (one per kv head), 8-15 VALUE wavefronts (same
+// heads).  Tokens are taken 32 at a time (two physical blocks).  Per chunk a score wavefront
+// loads the K codes and both norms, forms the scores on the matrix cores, updates the running
+// softmax and leaves the weights (fp16 operand form) plus the rescale factor in LDS; after one
+// workgroup barrier the value wavefront of the same head multiplies them into the value codes
+// it prefetched meanwhile.  The two kinds overlap (the score side works on chunk c+1 while the
+// value side consumes chunk c) and, at under 128 registers each, four wavefronts share a SIMD.
+//
+// Register layouts are chosen so that nothing is ever transposed:
 //
 //   scores   S^T[token, col] = sum_d Khat[token, d] * Qop[d, col]       v_mfma_f32_16x16x32_f16
 //            A = Khat: lane (n = l%16, g = l/16) owns bytes [16g, 16g+16) of token n's code row
-//            (one 16-byte load); k-step s uses its dword s = coordinates 32g + 8s + 0..7.
-//            B = Qop: the rotated queries of the kv head's query heads, in the same coordinate
-//            order, columns [0,8) = fp16 rounding of q', columns [8,16) = fp16 of the remainder
-//            (so the product carries q' to ~22 bits at no extra MFMA).
-//            Result: lane (col, g) holds tokens 4g..4g+3 of the tile for column col.
-//   softmax  running max / sum per column; the weights p * |v| / alpha of a lane are exactly the
-//            k-slice of the B operand of the next product (tokens 4g..4g+3 of both tiles), again
-//            split hi / lo over columns [0,8) / [8,16).
+//            (one 16-byte load).
+//            B = Qop: the rotated, pre-scaled queries of the kv head's query heads, columns [0,8)
+//            = fp16 rounding of q', columns [8,16) = fp16 of the remainder (q' to ~22 bits at no
+//            extra MFMA).  Result: lane (col, g) holds tokens 4g..4g+3 of the tile for column col.
+//   softmax  running max / sum per column in the log2 domain; the weights p * |v| of a lane are
+//            exactly the k-slice of the B operand of the next product (tokens 4g..4g+3 of both
+//            tiles), again split hi / lo over columns [0,8) / [8,16).
 //   values   O^T[coord, col] += sum_token Vhat[token, coord] * P[token, col]
 //            A = Vhat^T: lane (m, g) loads dword m (coordinates 8m..8m+7) of its 8 tokens and
 //            builds, for each of the 8 coordinates, the 8-token k-slice; M-tile j row m is
 //            coordinate 8m + j.
 //
-// Dequantisation goes through a table in LDS indexed by a whole BYTE: entry (a<<4|b) is the
-// fp16 pair (alpha c[a], alpha c[b]).  For K a byte holds two neighbouring coordinates of one
-// token -- already a k-pair.  For V the k axis is the token axis, so bytes are first re-formed
-// from the same nibble position of two neighbouring tokens (two bit-field inserts per 8 codes).
-// The table is replicated 64 times (address = byte * 256 + lane * 4) so that lookups never
-// conflict on an LDS bank.  alpha in [1,2) is chosen per codebook so that alpha*c is almost
-// exactly representable in fp16 (the rounding of the 16 levels would otherwise be the largest
-// error of the whole computation); it is divided out of the scores and of the weights.
+// Dequantisation goes through tables in LDS indexed by a whole BYTE: entry (a<<4|b) is the fp16
+// pair (c[a], c[b]).  For K a byte holds two neighbouring coordinates of one token -- already a
+// k-pair; the K table carries a hi and a lo half (c = hi + lo to ~22 bits) and both go through
+// the matrix core, interleaved in one operand.  For V the k axis is the token axis, so bytes
+// are first re-formed from the same nibble position of two neighbouring tokens (two bit-field
+// inserts per 8 codes); the V table holds fp16(alpha c) with alpha in [1,2) chosen so that the
+// sixteen levels are almost exactly representable, and alpha is divided out at the end.  Every
+// table entry is replicated 32 times (address = entry * 256 + (lane & 31) * 4): the LDS serves
+// 32 lanes per cycle, so lookups never conflict on a bank.
 #include "akv_attn_common.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-#define MF_WAVES 8
-#define MF_LUT_COPIES 32                       // copies of each half of an entry (lane & 31)
-#define MF_LUT_BYTES (256 * 256)               // entry e at e*256: [hi pair x 32][lo pair x 32]
-#ifndef MF_KSPLIT
-#define MF_KSPLIT 1                            // scores use hi + lo table halves (2 MFMA per k-step)
-#endif
+#define MF_HEADS 8                  // kv heads per pass = score wavefronts = value wavefronts
+#define MF_THREADS 1024
+#define MF_WAIT_VM0 0x0f70          // s_waitcnt vmcnt(0), other counters untouched
+#define MF_WIN 30                   // chunks served by one window of 64 block ids (even, <= 31)
+#define MF_LDS_BYTES (128 * 1024)   // two tables of 256 entries x 256 bytes
+// entry e of table A at e*256:          [fp16(alpha c) pairs for V x 32 copies][hi pairs for K x 32 copies]
+// entry e of table B at 65536 + e*256:  [lo pairs for K x 32 copies][128 bytes of exchange buffer]
+// so the lo half of a K lookup sits 65408 bytes after its hi half: reachable by the 16-bit offset of a
+// single LDS read, and impossible to fuse with the hi read into a two-address read (which would need
+// extra register moves to regroup the results for the matrix core)
+#define MF_TABB 65536u
+#define MF_KLO_DIST 65408u
 #define MF_ALPHA_CANDIDATES 65536
+// words of the table block kept in the workspace
+#define MF_W_KHI 0
+#define MF_W_KLO 256
+#define MF_W_VHI 512
+#define MF_W_TAG 768                // 16 centroids the tables were built from
+#define MF_W_MARK 784
+#define MF_W_ALPHA 785
+#define MF_W_WORDS 1024
+#define MF_MARK 0x7452u
 
 struct akv_mfma_extra {
-  const uint32_t* lut;   // [2][256] fp16 pairs: hi = fp16(alpha c), lo = fp16(alpha c - hi); then the tag (workspace)
-  const float* alpha;    // [1]                         (workspace)
-  const uint4* qop;      // [S][KVH][4 k-steps x 2 halves][64 lanes] half8 as uint4 (workspace)
+  const uint32_t* lut;   // table block, MF_W_* (workspace)
+  const uint4* qop;      // [S][KVH][4 k-steps][64 lanes] half8 as uint4 (workspace)
 };
 
 // ----------------------------------------------------------------------------------
@@ -53,7 +75,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
-    uint4* __restrict__ qop, uint32_t* __restrict__ lut, float* __restrict__ alpha_out) {
+    uint4* __restrict__ qop, uint32_t* __restrict__ lut, float qscale) {
   __shared__ __align__(16) float q_lds[128][8];   // [input coordinate][query head of the group], zero-padded
   __shared__ float qr_lds[8][128];
   __shared__ int32_t scratch[257];
@@ -66,13 +88,12 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     return;
   }
   if ((int)blockIdx.x == nq + 1) {
-    // The table depends on the codebook only.  It is kept in the workspace together with the
-    // centroids it was built from (lut[512..527]) and a marker (lut[528]); when they match, the
-    // search is skipped.
+    // The tables depend on the codebook only.  They are kept in the workspace together with
+    // the centroids they were built from and a marker; when those match, nothing is rebuilt.
     __shared__ int stale;
-    if (tid == 0) stale = (lut[528] != 0x7451u) ? 1 : 0;
+    if (tid == 0) stale = (lut[MF_W_MARK] != MF_MARK) ? 1 : 0;
     __syncthreads();
-    if (tid < 16 && __float_as_uint(centroids[tid]) != lut[512 + tid]) stale = 1;
+    if (tid < 16 && __float_as_uint(centroids[tid]) != lut[MF_W_TAG + tid]) stale = 1;
     __syncthreads();
     if (!stale) return;
     // alpha search: minimise the largest relative fp16 rounding error of alpha * c over the levels
@@ -96,19 +117,21 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     if (tid == 0) {
       for (int t = 1; t < 256; ++t)
         if (best_err[t] < best_err[0]) { best_err[0] = best_err[t]; best_alpha[0] = best_alpha[t]; }
-      alpha_out[0] = best_alpha[0];
+      lut[MF_W_ALPHA] = __float_as_uint(best_alpha[0]);
     }
     __syncthreads();
     const float al = best_alpha[0];
-    const float x0 = al * centroids[tid >> 4], x1 = al * centroids[tid & 15];   // pair (first, second)
-    const __half h0 = __float2half_rn(x0), h1 = __float2half_rn(x1);
-    lut[tid] = (unsigned)__half_as_ushort(h0) | ((unsigned)__half_as_ushort(h1) << 16);
-    const __half l0 = __float2half_rn(x0 - __half2float(h0)), l1 = __float2half_rn(x1 - __half2float(h1));
-    lut[256 + tid] = (unsigned)__half_as_ushort(l0) | ((unsigned)__half_as_ushort(l1) << 16);
-    if (tid < 16) lut[512 + tid] = __float_as_uint(centroids[tid]);
+    const float c0 = centroids[tid >> 4], c1 = centroids[tid & 15];   // pair (first, second)
+    const __half k0 = __float2half_rn(c0), k1 = __float2half_rn(c1);
+    lut[MF_W_KHI + tid] = (unsigned)__half_as_ushort(k0) | ((unsigned)__half_as_ushort(k1) << 16);
+    const __half l0 = __float2half_rn(c0 - __half2float(k0)), l1 = __float2half_rn(c1 - __half2float(k1));
+    lut[MF_W_KLO + tid] = (unsigned)__half_as_ushort(l0) | ((unsigned)__half_as_ushort(l1) << 16);
+    const __half v0 = __float2half_rn(al * c0), v1 = __float2half_rn(al * c1);
+    lut[MF_W_VHI + tid] = (unsigned)__half_as_ushort(v0) | ((unsigned)__half_as_ushort(v1) << 16);
+    if (tid < 16) lut[MF_W_TAG + tid] = __float_as_uint(centroids[tid]);
     __threadfence();
     __syncthreads();
-    if (tid == 0) lut[528] = 0x7451u;
+    if (tid == 0) lut[MF_W_MARK] = MF_MARK;
     return;
   }
   const int s = blockIdx.x / KVH, h = blockIdx.x % KVH;
@@ -143,22 +166,18 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     __syncthreads();
     if (half == 0) {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) qr_lds[q][dim] += part[q];
+      for (int q = 0; q < 8; ++q) qr_lds[q][dim] = (qr_lds[q][dim] + part[q]) * qscale;
     }
   }
   __syncthreads();
-  // operand layout: [k-step st][half u][lane (col, g)][e].  The K operand of (st, u) holds, for
-  // bytes 2u and 2u+1 of dword st of the lane's 16 code bytes, the hi pair then the lo pair of
-  // the table entry: elements (0,1) hi / (2,3) lo of byte 2u, (4,5) hi / (6,7) lo of byte 2u+1.
-  // So element e of the query operand is coordinate 32g + 8st + 4u + 2(e/4) + (e&1).
-  for (int idx = tid; idx < 8 * 64; idx += 256) {
-    const int su = idx >> 6, lane = idx & 63;
-    const int st = su >> 1, u = su & 1;
+  // operand layout: [k-step st][lane (col, g)][e] = coordinate 32g + 8st + e of column col
+  {
+    const int st = tid >> 6, lane = tid & 63;
     const int col = lane & 15, g = lane >> 4;
     unsigned short hbits[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int dim = 32 * g + 8 * st + 4 * u + 2 * (e >> 2) + (e & 1);
+      const int dim = 32 * g + 8 * st + e;
       float v = 0.f;
       if (col < 8) {
         if (col < gqa) v = __half2float(__float2half_rn(qr_lds[col][dim]));
@@ -171,36 +190,33 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     uint4 o;
     o.x = hbits[0] | (hbits[1] << 16); o.y = hbits[2] | (hbits[3] << 16);
     o.z = hbits[4] | (hbits[5] << 16); o.w = hbits[6] | (hbits[7] << 16);
-    qop[((size_t)(s * KVH + h) * 8 + su) * 64 + lane] = o;
+    qop[((size_t)(s * KVH + h) * 4 + st) * 64 + lane] = o;
   }
 }
 
 // ----------------------------------------------------------------------------------
 // main kernel
 // ----------------------------------------------------------------------------------
-struct mf_raw {      // what one wavefront loads for one 32-token chunk
-  uint4 k[2];        // K code rows: tile j, token l%16, bytes [16g, 16g+16)
-  uint32_t v[8];     // V codes: token tau(g,e), dword l%16
-  float kn[8], vn[8];  // norms of tokens 4g+i of tile 0 (i<4) and tile 1
-};
+typedef __attribute__((address_space(3))) const uint32_t mf_lds_cu32;
+typedef __attribute__((address_space(3))) uint32_t mf_lds_u32;
+typedef uint32_t mf_u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) mf_u32x4 mf_lds_u128;
 
-typedef __attribute__((address_space(3))) const uint32_t mf_lds_u32;
+// The tables are the kernel's only LDS object, so they start at LDS address 0 and a table offset
+// is the LDS address itself (saves one add per lookup).
+// address = byte k of `word` * 256 + lanebits (the copy (lane & 31) * 4, plus 128 for the K half),
+// built by one byte permute: result byte 0 <- lanebits byte 0, byte 1 <- word byte k (selector 4 + k).
+#define MF_SEL(k) (0x0c0c0400u + ((uint32_t)(k) << 8))
 
-// The table is the kernel's only LDS object, so it starts at LDS address 0 and a table address
-// can be used as the LDS address itself (saves one add per lookup).
-__device__ __forceinline__ uint32_t mf_lut(const unsigned char*, uint32_t lane4, uint32_t word, uint32_t sel) {
-  // address = byte(word, k) * 256 + lane * 4, built by one byte permute:
-  // result byte 0 <- lane4 byte 0 (selector 0x00), byte 1 <- word byte k (selector 0x04 + k), rest zero
-  const uint32_t addr = __builtin_amdgcn_perm(word, lane4, sel);
-  return *(mf_lds_u32*)(uintptr_t)addr;
+__device__ __forceinline__ uint32_t mf_lut(uint32_t lanebits, uint32_t word, uint32_t sel) {
+  const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
+  return *(mf_lds_cu32*)(uintptr_t)addr;
 }
-
-// hi and lo halves of an entry in one go (the two loads differ by 128 bytes -> ds_read2_b32)
-__device__ __forceinline__ void mf_lut2(const unsigned char*, uint32_t lane4, uint32_t word, uint32_t sel,
-                                        uint32_t& hi, uint32_t& lo) {
-  const uint32_t addr = __builtin_amdgcn_perm(word, lane4, sel);
-  hi = *(mf_lds_u32*)(uintptr_t)addr;
-  lo = *(mf_lds_u32*)(uintptr_t)(addr + 128);
+// hi and lo halves of a K lookup: one address, two reads
+__device__ __forceinline__ void mf_lut2(uint32_t lanebits, uint32_t word, uint32_t sel, uint32_t& hi, uint32_t& lo) {
+  const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
+  hi = *(mf_lds_cu32*)(uintptr_t)addr;
+  lo = *(mf_lds_cu32*)(uintptr_t)(addr + MF_KLO_DIST);
 }
 
 __device__ __forceinline__ half8 mf_pack(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -218,21 +234,39 @@ __device__ __forceinline__ float mf_from_lo_cols(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x118 /*row_shr:8*/, 0xf, 0xf, true));
 }
 
-__global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, akv_mfma_extra x) {
-  extern __shared__ __align__(16) unsigned char lds_raw[];
+// workgroup barrier that orders LDS traffic only (outstanding global loads keep flying)
+__device__ __forceinline__ void mf_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+struct mf_kraw {       // score wavefront, one 32-token chunk
+  uint4 k[2];          // K code rows: tile j, token l%16, bytes [16g, 16g+16)
+  float nrm;           // lane < 32: K norm of token l, else V norm of token l - 32
+};
+struct mf_vraw {       // value wavefront
+  uint32_t v[8];       // V codes: token tau(g,e), dword l%16
+};
+
+// One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
+// separate instantiations entered through one uniform branch, so that neither keeps the other's
+// loop-invariant registers alive.
+template <int ROLE>
+__device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
   const int col = lane & 15, g = lane >> 4;
-  // replicate the table: dword index i = entry * 64 + half * 32 + copy
-  {
-    uint32_t* l32 = (uint32_t*)lds_raw;
-    for (int i = threadIdx.x; i < 256 * 64; i += 512) l32[i] = x.lut[((i >> 5) & 1) * 256 + (i >> 6)];
+  const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
+  const uint32_t lane4v = (uint32_t)(lane & 31) * 4u;      // V lookups: first half of table A
+  const uint32_t lane4k = lane4v + 128u;                   // K lookups: second half of table A (+ MF_KLO_DIST)
+  // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
+  //   weights (16 B per lane): entry 16q + lane/8, offset 128 + (lane%8)*16
+  //   rescale (4 B per lane):  entry 16q + 8 + lane/32, offset 128 + (lane%32)*4
+  uint32_t pb_addr[2], rs_addr[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const uint32_t q = (uint32_t)(hs * 2 + b);
+    pb_addr[b] = MF_TABB + (16u * q + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
+    rs_addr[b] = MF_TABB + (16u * q + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
   }
-  const unsigned char* lut_lane = lds_raw;
-  const uint32_t lane4 = (uint32_t)(lane & 31) * 4u;
-  const float alpha = x.alpha[0];
-  const float inv_alpha = 1.f / alpha;
-  __syncthreads();
 
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
@@ -240,7 +274,6 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
   const int g0 = blockIdx.x * per;
   const int g1 = min(total, g0 + per);
   const int gqa = a.QH / a.KVH;
-  const float sc_mul = a.scale * inv_alpha;
 
   int gcur = g0;
   while (gcur < g1) {
@@ -254,189 +287,279 @@ __global__ __launch_bounds__(512) void akv_attn_mfma4_kernel(akv_attn_args a, ak
     const int nblk = blk_hi - blk_lo;
     const int nchunks = (nblk + 1) >> 1;
 
-    for (int h = wave; h < a.KVH; h += MF_WAVES) {
-      // query operand of this (sequence, kv head)
-      half8 qb[8];
-      {
-        const uint4* qp = x.qop + ((size_t)(s * a.KVH + h) * 8) * 64 + lane;
-#pragma unroll
-        for (int su = 0; su < 8; ++su) {
-          const uint4 u = qp[su * 64];
-          qb[su] = mf_pack(u.x, u.y, u.z, u.w);
-        }
-      }
-      float4v o[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = (float4v){0.f, 0.f, 0.f, 0.f};
-      float m_run = -INFINITY, l_run = 0.f;
+    for (int hbase = 0; hbase < a.KVH; hbase += MF_HEADS) {
+      const int h = hbase + hs;
+      const bool active = h < a.KVH;          // inactive wavefronts only keep the barriers company
+      const int hh = active ? h : 0;
 
-      // per-lane byte offsets inside a physical block (32-bit), added to a wavefront-uniform base
-      const uint32_t koff = (uint32_t)(h * a.kps_head + col * a.kps_pos + 16 * g);
-      uint32_t voff[4], knoff[4], vnoff[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        voff[i] = (uint32_t)(h * a.vps_head + (4 * g + i) * a.vps_pos + 4 * col);
-        knoff[i] = (uint32_t)((h * a.kns_head + (4 * g + i) * a.kns_pos) * 4);
-        vnoff[i] = (uint32_t)((h * a.vns_head + (4 * g + i) * a.vns_pos) * 4);
-      }
-
-      // physical block ids of the segment: lane i holds the id of block (window start + i); the
-      // window is refreshed every 64 blocks, so the chunk loop itself reads no table entry
-      // (a table load in the loop would make every prefetch wait for all loads before it)
-      int pbwin = 0;
-      auto load_window = [&](int first_blk) {
-        const int bi = min(first_blk + lane, blk_hi - 1);
+      // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment.
+      // A window of 64 ids serves MF_WIN chunks plus the two-chunk lookahead of the prefetch.  Its
+      // reload drains every outstanding load (once per MF_WIN chunks); the chunk loop itself issues
+      // the same loads on every path, so its waits stay counted waits for the chunk that is due.
+      int pbwin = 0, win_c0 = 0;
+      auto load_window = [&](int c0) {
+        const int bi = min(blk_lo + 2 * c0 + lane, blk_hi - 1);
         pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
+        asm volatile("" : "+v"(pbwin));   // the window is complete here, not "maybe in flight" in the loop
+        win_c0 = c0;
       };
-      auto load_chunk = [&](mf_raw& r, int c) {
-        if ((c & 31) == 0) load_window(blk_lo + 2 * c);
-        const int w0 = (2 * c) & 63;
+      auto chunk_blocks = [&](int c_in, int64_t& p0, int64_t& p1) {
+        const int c = min(c_in, nchunks - 1);      // lookahead past the end re-reads the last chunk
+        const int w0 = 2 * (c - win_c0);
         const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
-        int64_t pb[2];
-        pb[0] = __builtin_amdgcn_readlane(pbwin, w0);
-        pb[1] = __builtin_amdgcn_readlane(pbwin, w1);
+        p0 = __builtin_amdgcn_readlane(pbwin, w0);
+        p1 = __builtin_amdgcn_readlane(pbwin, w1);
+      };
+      if (nchunks > 0) load_window(0);
+
+      if constexpr (ROLE == 0) {
+        // =========================== score wavefront ===========================
+        half8 qb[4];
+        {
+          const uint4* qp = x.qop + ((size_t)(s * a.KVH + hh) * 4) * 64 + lane;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const unsigned char* kb = a.kp + pb[j] * a.kps_blk;
-          const unsigned char* vb = a.vp + pb[j] * a.vps_blk;
-          const unsigned char* knb = (const unsigned char*)(a.kn + pb[j] * a.kns_blk);
-          const unsigned char* vnb = (const unsigned char*)(a.vn + pb[j] * a.vns_blk);
-          r.k[j] = *(const uint4*)(kb + koff);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            r.v[4 * j + i] = *(const uint32_t*)(vb + voff[i]);
-            r.kn[4 * j + i] = *(const float*)(knb + knoff[i]);
-            r.vn[4 * j + i] = *(const float*)(vnb + vnoff[i]);
+          for (int st = 0; st < 4; ++st) {
+            const uint4 u = qp[st * 64];
+            qb[st] = mf_pack(u.x, u.y, u.z, u.w);
           }
         }
-      };
-
-      auto process = [&](const mf_raw& r, int c) {
-        const int tok0 = (blk_lo + 2 * c) * 16;      // first token of tile 0
-        // ---- scores
-        float sv[8];
-        {
-          // 16 steps (tile j, dword st, half u); the table reads of step n+1 are issued before
-          // the MFMA of step n
-          const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
-          uint32_t w[2][4];
-          float4v acc[2];
-          acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
-          acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
-          mf_lut2(lut_lane, lane4, kw[0], 0x0c0c0400u, w[0][0], w[0][1]);
-          mf_lut2(lut_lane, lane4, kw[0], 0x0c0c0500u, w[0][2], w[0][3]);
+        float m_run = -INFINITY, l_run = 0.f;
+        const uint32_t koff = (uint32_t)(hh * a.kps_head + col * a.kps_pos + 16 * g);
+        // norms travel one per lane (lanes [0,32): K norm of token l, lanes [32,64): V norm of token
+        // l - 32), prefetched with the codes, and are spread to the accumulator layout through the
+        // spare halves of table B entries 16q + 10 (K) and 16q + 11 (V)
+        const int ntok = lane & 31;
+        const bool nrm_is_v = lane >= 32;
+        const float* nrm_base = nrm_is_v ? a.vn : a.kn;
+        const int64_t nrm_blk = nrm_is_v ? a.vns_blk : a.kns_blk;
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hh * a.vns_head + (ntok & 15) * a.vns_pos
+                                                     : hh * a.kns_head + (ntok & 15) * a.kns_pos);
+        uint32_t nw_addr[2], nr_addr[2];
 #pragma unroll
-          for (int n = 0; n < 16; ++n) {
-            if (n + 1 < 16) {
-              const int n1 = n + 1;
-              const uint32_t word = kw[n1 >> 1];
-              const uint32_t sel = 0x0c0c0400u + ((uint32_t)(2 * (n1 & 1)) << 8);
-              mf_lut2(lut_lane, lane4, word, sel, w[n1 & 1][0], w[n1 & 1][1]);
-              mf_lut2(lut_lane, lane4, word, sel + 0x100u, w[n1 & 1][2], w[n1 & 1][3]);
+        for (int b = 0; b < 2; ++b) {
+          const uint32_t q = (uint32_t)(hs * 2 + b);
+          nw_addr[b] = MF_TABB + (16u * q + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
+          nr_addr[b] = MF_TABB + (16u * q + 10u) * 256u + 128u + (uint32_t)g * 16u;
+        }
+        auto load_chunk = [&](mf_kraw& r, int c) {
+          int64_t pb[2];
+          chunk_blocks(c, pb[0], pb[1]);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) r.k[j] = *(const uint4*)(a.kp + pb[j] * a.kps_blk + koff);
+          r.nrm = nrm_base[(ntok >= 16 ? pb[1] : pb[0]) * nrm_blk + nrm_off];
+        };
+        auto produce = [&](const mf_kraw& r, int c) {
+          float sv[8];
+          *(mf_lds_u32*)(uintptr_t)nw_addr[c & 1] = __float_as_uint(r.nrm);
+          {
+            // 8 steps (tile j, dword st): 4 table reads (hi and lo of each of the dword's 4 bytes) feed
+            // two MFMAs; the reads of step n+1 are issued before the MFMAs of step n
+            const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
+            uint32_t wh[2][4], wl[2][4];
+            float4v acc[2];
+            acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
+            acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[0], MF_SEL(b), wh[0][b], wl[0][b]);
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+              if (n + 1 < 8) {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n + 1], MF_SEL(b), wh[(n + 1) & 1][b], wl[(n + 1) & 1][b]);
+              }
+              acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  mf_pack(wh[n & 1][0], wh[n & 1][1], wh[n & 1][2], wh[n & 1][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
+              acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  mf_pack(wl[n & 1][0], wl[n & 1][1], wl[n & 1][2], wl[n & 1][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
             }
-            acc[n >> 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(w[n & 1][0], w[n & 1][1], w[n & 1][2], w[n & 1][3]),
-                                                                 qb[n & 7], acc[n >> 3], 0, 0, 0);
+            // columns c and c + 8 carry the hi and lo part of the same query head; only lanes of
+            // columns [0,8) keep a meaningful softmax state (the others see the lo part alone)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              union { mf_u32x4 u; float f[4]; } kn;
+              kn.u = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 64u * j);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
+            }
           }
+          if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
+            const int tok0 = (blk_lo + 2 * c) * 16;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const int tok = tok0 + 16 * j + 4 * g + i;
+                const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
+                if (!ok) sv[4 * j + i] = -INFINITY;
+              }
+          }
+          // running softmax in the log2 domain (scale * log2 e is folded into the query operand)
+          float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float m_new = fmaxf(m_run, mx);
+          const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
+          m_run = m_new;
+          float psum = 0.f;
+          half8 pbv;
+          union { mf_u32x4 u[2]; float f[8]; } vn;
+          vn.u[0] = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 256u);
+          vn.u[1] = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 256u + 64u);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);    // 0 for masked tokens
+            psum += p;
+            const float pw = p * vn.f[i];
+            const float hi = __half2float(__float2half_rn(pw));
+            const float lo_left = mf_from_lo_cols(pw - hi);           // columns [8,16) take the remainder
+            pbv[i] = (_Float16)(col < 8 ? hi : lo_left);
+          }
+          l_run = l_run * resc + psum;
+          const float resc_left = mf_from_lo_cols(resc);
+          const float resc_out = col < 8 ? resc : resc_left;
+          union { half8 h; mf_u32x4 u; } cv;
+          cv.h = pbv;
+          *(mf_lds_u128*)(uintptr_t)pb_addr[c & 1] = cv.u;
+          *(mf_lds_u32*)(uintptr_t)rs_addr[c & 1] = __float_as_uint(resc_out);
+        };
+
+        mf_kraw ra, rb;
+        if (nchunks > 0) load_chunk(ra, 0);
+        // pairs of chunks with the same loads on every path (an early exit from the middle of the
+        // body would make the compiler wait for the newest prefetch at the top of every iteration)
+        int c = 0;
+        for (; c + 1 < nchunks; c += 2) {
+          if (c - win_c0 >= MF_WIN) load_window(c);
+          load_chunk(rb, c + 1);
+          __builtin_amdgcn_sched_barrier(0);   // the prefetch is issued before anything waits
+          produce(ra, c);
+          mf_barrier();
+          load_chunk(ra, c + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          produce(rb, c + 1);
+          mf_barrier();
+        }
+        if (c < nchunks) {      // odd tail, already in ra
+          produce(ra, c);
+          mf_barrier();
+        }
+        __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
+        mf_barrier();   // value side done with the buffers
+        float lsum = l_run;
+        lsum += __shfl_xor(lsum, 16, 64);
+        lsum += __shfl_xor(lsum, 32, 64);
+        if (active && col < gqa && g == 0) {
+          const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
+          a.part_ml[slot * 2] = m_run * 0.6931471805599453f;   // back to the natural-log domain
+          a.part_ml[slot * 2 + 1] = lsum;
+        }
+      } else {
+        // =========================== value wavefront ===========================
+        float4v o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (float4v){0.f, 0.f, 0.f, 0.f};
+        uint32_t voff[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) voff[i] = (uint32_t)(hh * a.vps_head + (4 * g + i) * a.vps_pos + 4 * col);
+        auto load_chunk = [&](mf_vraw& r, int c) {
+          int64_t pb[2];
+          chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
+            const unsigned char* vb = a.vp + pb[j] * a.vps_blk;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              // columns c and c + 8 carry the hi and lo part of the same query head: both lanes form
-              // the same sum, so the softmax state below is identical in the two
-              // (both cross-lane moves run with all lanes active; only the choice is per lane)
-              const float from_hi = mf_from_hi_cols(acc[j][i]);
-              const float from_lo = mf_from_lo_cols(acc[j][i]);
-              const float full = acc[j][i] + (col < 8 ? from_hi : from_lo);
-              const int tok = tok0 + 16 * j + 4 * g + i;
-              const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
-              sv[4 * j + i] = ok ? full * r.kn[4 * j + i] * sc_mul : -INFINITY;
-            }
+            for (int i = 0; i < 4; ++i) r.v[4 * j + i] = *(const uint32_t*)(vb + voff[i]);
           }
-        }
-        // ---- running softmax (per column; rows of 16 lanes hold different tokens)
-        float mx = sv[0];
+        };
+        auto consume = [&](const mf_vraw& r, int c) {
+          // pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates
+          uint32_t xe[4], xo[4];
 #pragma unroll
-        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
-          const float resc = __expf(m_run - m_new);   // 0 on the first chunk (m_run = -inf)
-          l_run *= resc;
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[j][i] *= resc;
-          m_run = m_new;
-        }
-        // weights: hi part in columns [0,8), remainder in columns [8,16)
-        half8 pb;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float p = __expf(sv[i] - m_run);      // exp(-inf) = 0 for masked tokens
-          l_run += p;
-          const float pw = p * r.vn[i] * inv_alpha;
-          const float hi = __half2float(__float2half_rn(pw));
-          pb[i] = (_Float16)(col < 8 ? hi : pw - hi);
-        }
-        // ---- values: pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates
-        uint32_t xe[4], xo[4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          const uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
-          xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
-          xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
-        }
-        {
-          // 8 steps: step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
+          for (int p = 0; p < 4; ++p) {
+            const uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
+            xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
+            xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
+          }
           uint32_t w[2][4];
 #pragma unroll
-          for (int p = 0; p < 4; ++p) w[0][p] = mf_lut(lut_lane, lane4, xe[p], 0x0c0c0400u);
+          for (int p = 0; p < 4; ++p) w[0][p] = mf_lut(lane4v, xe[p], MF_SEL(0));
+          union { half8 h; mf_u32x4 u; } cv;
+          cv.u = *(mf_lds_u128*)(uintptr_t)pb_addr[c & 1];
+          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)rs_addr[c & 1]);
+          if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) o[j][i] *= resc;
+          }
+          // 8 steps: step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
 #pragma unroll
           for (int n = 0; n < 8; ++n) {
             if (n + 1 < 8) {
               const int n1 = n + 1;
-              const uint32_t sel = 0x0c0c0400u + ((uint32_t)(n1 >> 1) << 8);
 #pragma unroll
-              for (int p = 0; p < 4; ++p) w[n1 & 1][p] = mf_lut(lut_lane, lane4, (n1 & 1) ? xo[p] : xe[p], sel);
+              for (int p = 0; p < 4; ++p) w[n1 & 1][p] = mf_lut(lane4v, (n1 & 1) ? xo[p] : xe[p], MF_SEL(n1 >> 1));
             }
             o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(w[n & 1][0], w[n & 1][1], w[n & 1][2], w[n & 1][3]),
-                                                          pb, o[n], 0, 0, 0);
+                                                          cv.h, o[n], 0, 0, 0);
+          }
+        };
+
+        mf_vraw ra, rb;
+        if (nchunks > 0) load_chunk(ra, 0);
+        int c = 0;
+        for (; c + 1 < nchunks; c += 2) {
+          if (c - win_c0 >= MF_WIN) load_window(c);
+          load_chunk(rb, c + 1);
+          __builtin_amdgcn_sched_barrier(0);   // the prefetch is issued before anything waits
+          mf_barrier();
+          consume(ra, c);
+          load_chunk(ra, c + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          mf_barrier();
+          consume(rb, c + 1);
+        }
+        if (c < nchunks) {      // odd tail, already in ra
+          mf_barrier();
+          consume(ra, c);
+        }
+        __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
+        mf_barrier();
+        // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + j
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[j][i] = (o[j][i] + mf_from_hi_cols(o[j][i])) * inv_alpha;
+        if (active && col < gqa) {
+          const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
+          float* dst = a.part_acc + slot * 128 + 32 * g;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            *(float4*)(dst + 8 * i) = make_float4(o[0][i], o[1][i], o[2][i], o[3][i]);
+            *(float4*)(dst + 8 * i + 4) = make_float4(o[4][i], o[5][i], o[6][i], o[7][i]);
           }
         }
-      };
-
-      mf_raw ra, rb;
-      if (nchunks > 0) load_chunk(ra, 0);
-      for (int c = 0; c < nchunks; c += 2) {
-        if (c + 1 < nchunks) load_chunk(rb, c + 1);
-        process(ra, c);
-        if (c + 1 < nchunks) {
-          if (c + 2 < nchunks) load_chunk(ra, c + 2);
-          process(rb, c + 1);
-        }
-      }
-
-      // ---- partial: columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + j
-      float lsum = l_run;
-      lsum += __shfl_xor(lsum, 16, 64);
-      lsum += __shfl_xor(lsum, 32, 64);
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[j][i] += mf_from_hi_cols(o[j][i]);
-      if (col < gqa) {
-        const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
-        float* dst = a.part_acc + slot * 128 + 32 * g;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          *(float4*)(dst + 8 * i) = make_float4(o[0][i], o[1][i], o[2][i], o[3][i]);
-          *(float4*)(dst + 8 * i + 4) = make_float4(o[4][i], o[5][i], o[6][i], o[7][i]);
-        }
-        if (g == 0) { a.part_ml[slot * 2] = m_run; a.part_ml[slot * 2 + 1] = lsum; }
       }
     }
   }
+}
+
+__global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma4_kernel(akv_attn_args a, akv_mfma_extra x) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
+  // ---- tables (layout at MF_LDS_BYTES)
+  {
+    uint32_t* l32 = (uint32_t*)lds_raw;
+    for (int i = threadIdx.x; i < 256 * 64; i += MF_THREADS) {       // table A: dword e*64 + half*32 + copy
+      const int e = i >> 6, half = (i >> 5) & 1;
+      l32[i] = x.lut[(half ? MF_W_KHI : MF_W_VHI) + e];
+    }
+    for (int i = threadIdx.x; i < 256 * 32; i += MF_THREADS)         // table B, first halves
+      l32[16384 + (i >> 5) * 64 + (i & 31)] = x.lut[MF_W_KLO + (i >> 5)];
+  }
+  __syncthreads();
+  if ((wave >> 3) == 0) mf_role_main<0>(a, x, wave & 7);
+  else mf_role_main<1>(a, x, wave & 7);
 }
 
 // ----------------------------------------------------------------------------------
@@ -453,7 +576,7 @@ static bool mfma_disabled() {
 
 // extra workspace the MFMA path needs beyond akv_attn_ws (appended after it)
 size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
-  return akv_align256(2304) + akv_align256(4) + akv_align256((size_t)S * KVH * 8 * 64 * 16);
+  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * KVH * 4 * 64 * 16);
 }
 
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
@@ -465,34 +588,26 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   return true;
 }
 
-template <int QDT>
-static void launch_mfma_prologue(const void* query, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                                 const akv_attn_args& a, int32_t* prefix, const akv_mfma_extra& x,
-                                 hipStream_t stream) {
-  akv_attn_mfma_prologue_kernel<QDT><<<a.S * a.KVH + 2, 256, 0, stream>>>(
-      query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size,
-      a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, (float*)x.alpha);
-}
-
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
                       const akv_attn_args& a, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
   akv_mfma_extra x;
   char* p = (char*)extra_ws;
-  x.lut = (const uint32_t*)p; p += akv_align256(2304);
-  x.alpha = (const float*)p; p += akv_align256(4);
+  x.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
   x.qop = (const uint4*)p;
-  if (q_dtype == AKV_F16) launch_mfma_prologue<AKV_F16>(query, qs_seq, qs_head, PiT, a, prefix, x, stream);
-  else if (q_dtype == AKV_BF16) launch_mfma_prologue<AKV_BF16>(query, qs_seq, qs_head, PiT, a, prefix, x, stream);
-  else launch_mfma_prologue<AKV_F32>(query, qs_seq, qs_head, PiT, a, prefix, x, stream);
+  const float qscale = a.scale * 1.4426950408889634f;   // scores come out in the log2 domain
+  const int pgrid = a.S * a.KVH + 2;
+#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, qscale)
+  if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
+#undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
   static bool configured = false;
   if (!configured) {
     AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                MF_LUT_BYTES));
+                                MF_LDS_BYTES));
     configured = true;
   }
   akv_profile_mark_begin(stream);
-  akv_attn_mfma4_kernel<<<grid, 512, MF_LUT_BYTES, stream>>>(a, x);
+  akv_attn_mfma4_kernel<<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_attn_mfma4_kernel");
   return AKV_OK;

@@ -45,6 +45,9 @@ def parse():
                     choices=["decode4", "decode3", "decode2", "tq35", "tri", "encode"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device-to-device copy (a dispatch of known traffic, to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return ap.parse_args()
 
 
@@ -219,6 +222,14 @@ def main():
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     cpu = not args.no_cpu
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     enc, tq4 = bench_encode(torch, akv, L, dev, args.steps, args.warmup, cpu, args.cpu_seconds)
     out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
