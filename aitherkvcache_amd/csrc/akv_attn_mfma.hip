@@ -50,6 +50,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 // single LDS read, and impossible to fuse with the hi read into a two-address read (which would need
 // extra register moves to regroup the results for the matrix core)
 #define MF_TABB 65536u
+#define MF_XBUF 4096u                // distance of the two exchange buffers of a head slot
 #define MF_KLO_DIST 65408u
 #define MF_ALPHA_CANDIDATES 65536
 // words of the table block kept in the workspace
@@ -234,6 +235,18 @@ __device__ __forceinline__ float mf_from_lo_cols(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x118 /*row_shr:8*/, 0xf, 0xf, true));
 }
 
+// block id x block stride on the scalar unit (a 64-bit product of 64-bit operands would go through
+// the vector unit and drag the whole address into vector registers); strides are below 2^31
+__device__ __forceinline__ uint64_t mf_umul(uint32_t a, uint32_t b) { return (uint64_t)a * (uint64_t)b; }
+
+// Identity the optimiser cannot look through: keeps the widening of a 32-bit lane offset next to
+// the load that uses it, where it folds into the (scalar base + 32-bit lane offset) address form
+// instead of becoming a loop-invariant 64-bit register pair and a 64-bit add per load.
+__device__ __forceinline__ uint32_t mf_here(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // workgroup barrier that orders LDS traffic only (outstanding global loads keep flying)
 __device__ __forceinline__ void mf_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -254,19 +267,15 @@ template <int ROLE>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
-  const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
   const uint32_t lane4v = (uint32_t)(lane & 31) * 4u;      // V lookups: first half of table A
   const uint32_t lane4k = lane4v + 128u;                   // K lookups: second half of table A (+ MF_KLO_DIST)
   // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
   //   weights (16 B per lane): entry 16q + lane/8, offset 128 + (lane%8)*16
   //   rescale (4 B per lane):  entry 16q + 8 + lane/32, offset 128 + (lane%32)*4
-  uint32_t pb_addr[2], rs_addr[2];
-#pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const uint32_t q = (uint32_t)(hs * 2 + b);
-    pb_addr[b] = MF_TABB + (16u * q + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
-    rs_addr[b] = MF_TABB + (16u * q + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
-  }
+  // (buffer 1 lies MF_XBUF bytes after buffer 0; the parity of the chunk is a compile-time constant
+  // at every use, so it folds into the offset field of the LDS instruction)
+  const uint32_t pb_addr = MF_TABB + (32u * hs + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
+  const uint32_t rs_addr = MF_TABB + (32u * hs + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
 
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
@@ -303,12 +312,12 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         asm volatile("" : "+v"(pbwin));   // the window is complete here, not "maybe in flight" in the loop
         win_c0 = c0;
       };
-      auto chunk_blocks = [&](int c_in, int64_t& p0, int64_t& p1) {
+      auto chunk_blocks = [&](int c_in, uint32_t& p0, uint32_t& p1) {
         const int c = min(c_in, nchunks - 1);      // lookahead past the end re-reads the last chunk
         const int w0 = 2 * (c - win_c0);
         const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
-        p0 = __builtin_amdgcn_readlane(pbwin, w0);
-        p1 = __builtin_amdgcn_readlane(pbwin, w1);
+        p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
+        p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
       };
       if (nchunks > 0) load_window(0);
 
@@ -331,53 +340,53 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const int ntok = lane & 31;
         const bool nrm_is_v = lane >= 32;
         const float* nrm_base = nrm_is_v ? a.vn : a.kn;
-        const int64_t nrm_blk = nrm_is_v ? a.vns_blk : a.kns_blk;
+        const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vns_blk : a.kns_blk);
         const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hh * a.vns_head + (ntok & 15) * a.vns_pos
                                                      : hh * a.kns_head + (ntok & 15) * a.kns_pos);
-        uint32_t nw_addr[2], nr_addr[2];
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          const uint32_t q = (uint32_t)(hs * 2 + b);
-          nw_addr[b] = MF_TABB + (16u * q + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
-          nr_addr[b] = MF_TABB + (16u * q + 10u) * 256u + 128u + (uint32_t)g * 16u;
-        }
+        const uint32_t nw_addr = MF_TABB + (32u * hs + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
+        const uint32_t nr_addr = MF_TABB + (32u * hs + 10u) * 256u + 128u + (uint32_t)g * 16u;
         auto load_chunk = [&](mf_kraw& r, int c) {
-          int64_t pb[2];
+          uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
-          for (int j = 0; j < 2; ++j) r.k[j] = *(const uint4*)(a.kp + pb[j] * a.kps_blk + koff);
-          r.nrm = nrm_base[(ntok >= 16 ? pb[1] : pb[0]) * nrm_blk + nrm_off];
+          for (int j = 0; j < 2; ++j) r.k[j] = *(const uint4*)(a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + mf_here(koff));
+          r.nrm = nrm_base[mf_umul(ntok >= 16 ? pb[1] : pb[0], nrm_blk) + nrm_off];
         };
-        auto produce = [&](const mf_kraw& r, int c) {
+        auto produce = [&](mf_kraw& r, int c, const uint32_t par) {
           float sv[8];
-          *(mf_lds_u32*)(uintptr_t)nw_addr[c & 1] = __float_as_uint(r.nrm);
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + MF_XBUF * par) = __float_as_uint(r.nrm);
           {
             // 8 steps (tile j, dword st): 4 table reads (hi and lo of each of the dword's 4 bytes) feed
             // two MFMAs; the reads of step n+1 are issued before the MFMAs of step n
             const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
-            uint32_t wh[2][4], wl[2][4];
+            uint32_t wh[3][4], wl[3][4];      // ring of three steps: two in flight behind the one multiplied
             float4v acc[2];
             acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
             acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[0], MF_SEL(b), wh[0][b], wl[0][b]);
+            for (int n = 0; n < 2; ++n)
+#pragma unroll
+              for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n], MF_SEL(b), wh[n][b], wl[n][b]);
 #pragma unroll
             for (int n = 0; n < 8; ++n) {
-              if (n + 1 < 8) {
+              if (n + 2 < 8) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n + 1], MF_SEL(b), wh[(n + 1) & 1][b], wl[(n + 1) & 1][b]);
+                for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n + 2], MF_SEL(b), wh[(n + 2) % 3][b], wl[(n + 2) % 3][b]);
               }
               acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(wh[n & 1][0], wh[n & 1][1], wh[n & 1][2], wh[n & 1][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
+                  mf_pack(wh[n % 3][0], wh[n % 3][1], wh[n % 3][2], wh[n % 3][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
               acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(wl[n & 1][0], wl[n & 1][1], wl[n & 1][2], wl[n & 1][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
+                  mf_pack(wl[n % 3][0], wl[n % 3][1], wl[n % 3][2], wl[n % 3][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
+            load_chunk(r, c + 2);
+            __builtin_amdgcn_sched_barrier(0);
             // columns c and c + 8 carry the hi and lo part of the same query head; only lanes of
             // columns [0,8) keep a meaningful softmax state (the others see the lo part alone)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               union { mf_u32x4 u; float f[4]; } kn;
-              kn.u = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 64u * j);
+              kn.u = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 64u * j);
 #pragma unroll
               for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
             }
@@ -403,8 +412,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           float psum = 0.f;
           half8 pbv;
           union { mf_u32x4 u[2]; float f[8]; } vn;
-          vn.u[0] = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 256u);
-          vn.u[1] = *(mf_lds_u128*)(uintptr_t)(nr_addr[c & 1] + 256u + 64u);
+          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u);
+          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u + 64u);
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);    // 0 for masked tokens
@@ -419,28 +428,29 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           const float resc_out = col < 8 ? resc : resc_left;
           union { half8 h; mf_u32x4 u; } cv;
           cv.h = pbv;
-          *(mf_lds_u128*)(uintptr_t)pb_addr[c & 1] = cv.u;
-          *(mf_lds_u32*)(uintptr_t)rs_addr[c & 1] = __float_as_uint(resc_out);
+          *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
+          *(mf_lds_u32*)(uintptr_t)(rs_addr + MF_XBUF * par) = __float_as_uint(resc_out);
         };
 
         mf_kraw ra, rb;
-        if (nchunks > 0) load_chunk(ra, 0);
+        if (nchunks > 0) {
+          load_chunk(ra, 0);
+          __builtin_amdgcn_sched_barrier(0);   // queue order = chunk order, as in the loop
+          load_chunk(rb, 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         // pairs of chunks with the same loads on every path (an early exit from the middle of the
         // body would make the compiler wait for the newest prefetch at the top of every iteration)
         int c = 0;
         for (; c + 1 < nchunks; c += 2) {
           if (c - win_c0 >= MF_WIN) load_window(c);
-          load_chunk(rb, c + 1);
-          __builtin_amdgcn_sched_barrier(0);   // the prefetch is issued before anything waits
-          produce(ra, c);
+          produce(ra, c, 0);
           mf_barrier();
-          load_chunk(ra, c + 2);
-          __builtin_amdgcn_sched_barrier(0);
-          produce(rb, c + 1);
+          produce(rb, c + 1, 1);
           mf_barrier();
         }
         if (c < nchunks) {      // odd tail, already in ra
-          produce(ra, c);
+          produce(ra, c, 0);
           mf_barrier();
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
@@ -458,34 +468,39 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         float4v o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = (float4v){0.f, 0.f, 0.f, 0.f};
-        uint32_t voff[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) voff[i] = (uint32_t)(hh * a.vps_head + (4 * g + i) * a.vps_pos + 4 * col);
+        const uint32_t voff = (uint32_t)(hh * a.vps_head + 4 * g * a.vps_pos + 4 * col);   // token 4g of a tile
         auto load_chunk = [&](mf_vraw& r, int c) {
-          int64_t pb[2];
+          uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const unsigned char* vb = a.vp + pb[j] * a.vps_blk;
+            const unsigned char* vb = a.vp + mf_umul(pb[j], (uint32_t)a.vps_blk);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) r.v[4 * j + i] = *(const uint32_t*)(vb + voff[i]);
+            for (int i = 0; i < 4; ++i)      // the token step rides in the uniform base
+              r.v[4 * j + i] = *(const uint32_t*)(vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff));
           }
         };
-        auto consume = [&](const mf_vraw& r, int c) {
-          // pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates
-          uint32_t xe[4], xo[4];
+        uint32_t xe[4], xo[4];
+        // pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates; then
+        // the raw registers take the chunk after next (see the score side)
+        auto regroup = [&](mf_vraw& r, int c) {
 #pragma unroll
           for (int p = 0; p < 4; ++p) {
             const uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
             xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
             xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
           }
+          __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
+          load_chunk(r, c + 2);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        auto consume = [&](int c, const uint32_t par) {
           uint32_t w[2][4];
 #pragma unroll
           for (int p = 0; p < 4; ++p) w[0][p] = mf_lut(lane4v, xe[p], MF_SEL(0));
           union { half8 h; mf_u32x4 u; } cv;
-          cv.u = *(mf_lds_u128*)(uintptr_t)pb_addr[c & 1];
-          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)rs_addr[c & 1]);
+          cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par);
+          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + MF_XBUF * par));
           if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -506,26 +521,31 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
 
         mf_vraw ra, rb;
-        if (nchunks > 0) load_chunk(ra, 0);
+        if (nchunks > 0) {
+          load_chunk(ra, 0);
+          __builtin_amdgcn_sched_barrier(0);   // queue order = chunk order, as in the loop
+          load_chunk(rb, 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         int c = 0;
         for (; c + 1 < nchunks; c += 2) {
           if (c - win_c0 >= MF_WIN) load_window(c);
-          load_chunk(rb, c + 1);
-          __builtin_amdgcn_sched_barrier(0);   // the prefetch is issued before anything waits
+          regroup(ra, c);
           mf_barrier();
-          consume(ra, c);
-          load_chunk(ra, c + 2);
-          __builtin_amdgcn_sched_barrier(0);
+          consume(c, 0);
+          regroup(rb, c + 1);
           mf_barrier();
-          consume(rb, c + 1);
+          consume(c + 1, 1);
         }
         if (c < nchunks) {      // odd tail, already in ra
+          regroup(ra, c);
           mf_barrier();
-          consume(ra, c);
+          consume(c, 0);
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         mf_barrier();
         // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + j
+        const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
 #pragma unroll
@@ -585,6 +605,10 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   const int gqa = a.QH / a.KVH;
   if (gqa > 8) return false;
   if ((((uintptr_t)a.kp | (uintptr_t)a.kps_blk | (uintptr_t)a.kps_pos | (uintptr_t)a.kps_head) & 15) != 0) return false;
+  const int64_t strides[12] = {a.kps_blk, a.kps_pos, a.kps_head, a.kns_blk, a.kns_pos, a.kns_head,
+                               a.vps_blk, a.vps_pos, a.vps_head, a.vns_blk, a.vns_pos, a.vns_head};
+  for (int i = 0; i < 12; ++i)
+    if (strides[i] < 0 || strides[i] >= ((int64_t)1 << 27)) return false;   // 32-bit in-block offsets
   return true;
 }
 
