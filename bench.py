@@ -36,6 +36,18 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
+    summary (counters scaled by a copy kernel of known size); None when no such run is on record."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f).get(workload)
+    except OSError:
+        return None
+    return None if rec is None else rec["fetch_bytes"] + rec["write_bytes"]
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -281,7 +293,7 @@ def main():
                            "cache_copies_alternated": 2})
         achieved = tokens * per_tok / kms / 1e6
         out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
                            "kernel": "main decode-attention kernel", "kernel_ms": kms}
         if cpu and bits != "tq35":
             toks, secs, seqs = cpu_attention_baseline(ws[0], tq, bits, args.cpu_seconds)
