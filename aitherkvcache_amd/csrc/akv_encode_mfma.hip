@@ -7,7 +7,8 @@
 //   Y[v, j] = sum_i X[v, i] * Pi[j, i]                     v_mfma_f32_16x16x32_f16
 //     A = X: lane (row = l%16, g = l/16) holds, for k-step ks, elements i = 32g + 8ks + e (e<8)
 //         of vector `row` -- 64 contiguous bytes of the input row, loaded by four 16-byte loads
-//         that ARE the four A operands.  float16 input is exact in the operand, so the vector is
+//         that ARE the four A operands (measured faster than the layout in which the four lanes
+//         of a row share each load).  float16 input is exact in the operand, so the vector is
 //         not normalised before the product: y = (sum_i Pi[j,i] x_i) * 1/(|x| + 1e-10), with one
 //         correctly rounded reciprocal per vector.
 //     B = Pi: float32 entries split into two float16 terms (hi + lo, scaled by 64 to stay clear
@@ -27,19 +28,28 @@
 // A wavefront encodes 64 vectors per step (four M-tiles share every B operand read from LDS);
 // a workgroup is eight independent wavefronts plus the B operand (64 KB) and the cell table.
 #include "akv_common.h"
+#include <type_traits>
 
 typedef _Float16 em_half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 em_half2 __attribute__((ext_vector_type(2)));
 typedef float em_float4 __attribute__((ext_vector_type(4)));
 
-#define EM_WAVES 8
+#ifndef EM_MT
+#define EM_MT 2                    // M-tiles (16 vectors each) per wavefront step
+#endif
+#define EM_WAVES (32 / EM_MT)      // EM_MT 2: sixteen wavefronts under 128 registers; 4: eight under 256
 #define EM_THREADS (EM_WAVES * 64)
-#define EM_ROWS 64                 // vectors per wavefront step
-#define EM_CELLS 128
+#define EM_ROWS (16 * EM_MT)       // vectors per wavefront step
+#define EM_CELLS 512               // uniform cells over y in [-1.0039, 1.0039)
+#define EM_CELL_S 2040.f           // 8 x cells per unit of y: the cell table is addressed in bytes
+#define EM_CELL_C (8388608.f + 2048.f)   // 2^23 + centre: the sum's mantissa is 8 x the cell coordinate
+#define EM_CELL_MASK 0xff8u
+#define EM_MAX_ROW_NORM 1.0015f    // |y| <= |row of Pi| <= this keeps y inside the table
 #define EM_PSCALE 64.f             // scale of the matrix operand
 #define EM_B_BYTES 65536           // [hi/lo][8 nt][4 ks][64 lanes] x 16 B
-#define EM_LUT_OFF EM_B_BYTES      // EM_CELLS x {uint32 base, float boundary}
-#define EM_PAR_OFF (EM_LUT_OFF + EM_CELLS * 8)   // float inv_w, float off, uint32 bad, pad
+#define EM_LUT_OFF 0               // EM_CELLS x {uint32 base, float boundary}: LDS address = cell byte offset
+#define EM_B_OFF (EM_CELLS * 8)
+#define EM_PAR_OFF (EM_B_OFF + EM_B_BYTES)       // uint32 bad, pad
 #define EM_BND_OFF (EM_PAR_OFF + 16)              // 16 floats: boundaries (fallback search)
 #define EM_WAVE_OFF (EM_BND_OFF + 64)
 #define EM_WAVE_BYTES (EM_ROWS * (8 + 8 + 8 + 4))  // src offset, packed offset, norm offset, 1/(|x|+eps)
@@ -72,26 +82,52 @@ __global__ __launch_bounds__(256) void akv_em_prepare_kernel(const float* __rest
   bop[2048 + t] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
 }
 
+// flag word after the B operand: 1 when some row of the matrix is longer than EM_MAX_ROW_NORM (then
+// a rotated unit vector may leave the range of the cell table and the kernel counts boundaries)
+__global__ __launch_bounds__(128) void akv_em_rownorm_kernel(const float* __restrict__ Pi, uint32_t* __restrict__ flag) {
+  __shared__ uint32_t bad;
+  if (threadIdx.x == 0) bad = 0u;
+  __syncthreads();
+  float ss = 0.f;
+  for (int i = 0; i < 128; ++i) {
+    const float v = Pi[(size_t)threadIdx.x * 128 + i];
+    ss = fmaf(v, v, ss);
+  }
+  if (!(sqrtf(ss) <= EM_MAX_ROW_NORM)) atomicOr(&bad, 1u);
+  __syncthreads();
+  if (threadIdx.x == 0) flag[0] = bad;
+}
+
 int akv_prepare_rotation_mfma(const float* rotation, int d, void* prep, hipStream_t stream) {
   if (d != 128) return AKV_OK;
   uint4* bop = (uint4*)((float*)prep + (size_t)2 * d * d);
   akv_em_prepare_kernel<<<8, 256, 0, stream>>>(rotation, bop);
   AKV_LAUNCH_CHECK("akv_em_prepare_kernel");
+  akv_em_rownorm_kernel<<<1, 128, 0, stream>>>(rotation, (uint32_t*)(bop + EM_B_BYTES / 16));
+  AKV_LAUNCH_CHECK("akv_em_rownorm_kernel");
   return AKV_OK;
 }
 
 // ----------------------------------------------------------------------------------
 // encode kernel
 // ----------------------------------------------------------------------------------
+#ifdef EM_STAMP
+__device__ unsigned long long em_stamps[64 * 16 * 8];
+extern "C" int akv_debug_enc_stamps(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(em_stamps), sizeof(em_stamps)); }
+#define EM_ST(k) do { if (blockIdx.x == 7 && stepno < 16) { unsigned long long t_; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_) :: "memory"); if (lane == 0) em_stamps[(wave * 16 + stepno) * 8 + (k)] = t_; } } while (0)
+#else
+#define EM_ST(k) do { } while (0)
+#endif
 typedef uint32_t em_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t em_u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) em_u32x4 em_lds_u128;
 typedef __attribute__((address_space(3))) em_u32x2 em_lds_u64;
 
-// cell of a value: monotone non-decreasing in y for inv_w > 0
-__device__ __forceinline__ uint32_t em_cell(float y, float inv_w, float off) {
-  const float t = __builtin_amdgcn_fmed3f(fmaf(y, inv_w, off), 0.f, (float)(EM_CELLS - 1));
-  return (uint32_t)t;
+// Byte offset of the cell of y in the table: y * S + (2^23 + centre) has the cell coordinate (x 8)
+// in its mantissa, so one fused multiply-add and one mask replace scale, clamp, convert and shift.
+// Monotone non-decreasing for |y| < 1.0039; NaN lands inside the table like any other pattern.
+__device__ __forceinline__ uint32_t em_cell(float y) {
+  return __float_as_uint(fmaf(y, EM_CELL_S, EM_CELL_C)) & EM_CELL_MASK;
 }
 
 template <int BITS, bool PAGED>
@@ -104,45 +140,37 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 
   // ---- workgroup set-up: B operand, boundaries, cell table
   {
-    uint4* b_lds = (uint4*)lds;
+    uint4* b_lds = (uint4*)(lds + EM_B_OFF);
     for (int i = threadIdx.x; i < EM_B_BYTES / 16; i += EM_THREADS) b_lds[i] = bop[i];
     float* bnd = (float*)(lds + EM_BND_OFF);
+    uint32_t* par = (uint32_t*)(lds + EM_PAR_OFF);
     if (threadIdx.x < 16) bnd[threadIdx.x] = threadIdx.x < NB ? a.table[threadIdx.x] : INFINITY;
+    if (threadIdx.x == 0) par[0] = ((const uint32_t*)(bop + EM_B_BYTES / 16))[0];   // rows of Pi too long for the table
     __syncthreads();
-    float* par = (float*)(lds + EM_PAR_OFF);
     if (threadIdx.x == 0) {
-      const float lo = bnd[0], hi = bnd[NB - 1];
-      const float w = (hi - lo) / (float)(EM_CELLS - 2);
-      const float inv_w = 1.f / w;
-      par[0] = inv_w;
-      par[1] = 1.f - lo * inv_w;       // boundary 0 falls in cell 1
-      // usable only for finite, strictly increasing boundaries
-      bool ok = (w > 0.f) && (inv_w < INFINITY);
+      // the table serves finite, strictly increasing boundaries inside (-1, 1)
+      bool ok = fabsf(bnd[0]) < 1.f && fabsf(bnd[NB - 1]) < 1.f;
       for (int k = 1; k < NB; ++k) ok = ok && (bnd[k] > bnd[k - 1]);
-      ((uint32_t*)par)[2] = ok ? 0u : 1u;
+      if (!ok) par[0] = 1u;
     }
     __syncthreads();
-    const float inv_w = par[0], off = par[1];
-    if (threadIdx.x < EM_CELLS) {
+    for (int c = threadIdx.x; c < EM_CELLS; c += EM_THREADS) {
       uint32_t base = 0, cnt = 0;
       float inside = INFINITY;
       for (int k = 0; k < NB; ++k) {
-        const uint32_t c = em_cell(bnd[k], inv_w, off);
-        if (c < threadIdx.x) ++base;
-        if (c == threadIdx.x) { ++cnt; inside = bnd[k]; }
+        const uint32_t cb = em_cell(bnd[k]) >> 3;
+        if (cb < (uint32_t)c) ++base;
+        if (cb == (uint32_t)c) { ++cnt; inside = bnd[k]; }
       }
       uint32_t* lut = (uint32_t*)(lds + EM_LUT_OFF);
-      lut[2 * threadIdx.x] = base;
-      lut[2 * threadIdx.x + 1] = __float_as_uint(inside);
-      if (cnt > 1) atomicOr((uint32_t*)par + 2, 1u);
+      lut[2 * c] = base;
+      lut[2 * c + 1] = __float_as_uint(inside);
+      if (cnt > 1) atomicOr(par, 1u);
     }
     __syncthreads();
   }
-  const float inv_w = ((const float*)(lds + EM_PAR_OFF))[0];
-  const float off = ((const float*)(lds + EM_PAR_OFF))[1];
-  const bool linear_search = ((const uint32_t*)(lds + EM_PAR_OFF))[2] != 0;   // uniform
+  const bool linear_search = ((const uint32_t*)(lds + EM_PAR_OFF))[0] != 0;   // uniform
   const float* bnd = (const float*)(lds + EM_BND_OFF);
-  const uint32_t lut_addr = EM_LUT_OFF;
 
   unsigned char* wl = lds + EM_WAVE_OFF + wave * EM_WAVE_BYTES;
   int64_t* src_off = (int64_t*)wl;                    // element offset of the vector in x, or -1
@@ -151,16 +179,56 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   float* rinv = (float*)(wl + EM_ROWS * 24);          // 1/(|x| + 1e-10), scaled back by 1/EM_PSCALE; NaN rows flagged
 
   const int64_t steps = (a.n + EM_ROWS - 1) / EM_ROWS;
-  for (int64_t step = (int64_t)blockIdx.x * EM_WAVES + wave; step < steps; step += (int64_t)gridDim.x * EM_WAVES) {
+  const int64_t stride = (int64_t)gridDim.x * EM_WAVES;
+
+  // A operands of one step straight from memory (zeros past the end): lane l resolves the source
+  // row of vector base + l, the lanes of an M-tile pick the rows up through LDS
+  auto fetch = [&](em_half8 (&A)[EM_MT][4], int64_t step) {
+    const int64_t n = step * EM_ROWS + lane;
+    int64_t so = -1;
+    if (step < steps && n < a.n && lane < EM_ROWS) {
+      if (PAGED) {
+        const int64_t tok = n / a.heads, head = n - tok * a.heads;
+        so = tok * a.xs0 + head * a.xs1;
+      } else {
+        so = n * a.xs0;
+      }
+    }
+    if (lane < EM_ROWS) src_off[lane] = so;
+#pragma unroll
+    for (int mt = 0; mt < EM_MT; ++mt) {
+      const int64_t ro = src_off[16 * mt + (lane & 15)];
+      if (ro >= 0) {
+        const uint4* p = (const uint4*)((const __half*)a.x + ro + 32 * g);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          union { uint4 u; em_half8 h; } cv;
+          cv.u = p[ks];
+          A[mt][ks] = cv.h;
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) A[mt][ks] = (em_half8){0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  };
+
+  int stepno = 0;
+  (void)stepno;
+  auto encode_step = [&](auto linear_tag, int64_t step) {
+    constexpr bool LINEAR = decltype(linear_tag)::value;
+    em_half8 A[EM_MT][4];
+    EM_ST(0);
+    fetch(A, step);
+    EM_ST(1);
     const int64_t base = step * EM_ROWS;
-    // ---- lane l resolves the addresses of vector base + l
+    // ---- lane l resolves the destination of vector base + l
     {
       const int64_t n = base + lane;
-      int64_t so = -1, dp = -1, dn = 0;
-      if (n < a.n) {
+      int64_t dp = -1, dn = 0;
+      if (n < a.n && lane < EM_ROWS) {
         if (PAGED) {
           const int64_t tok = n / a.heads, head = n - tok * a.heads;
-          so = tok * a.xs0 + head * a.xs1;
           const int64_t slot = akv_load_index(a.slots, a.slot_itype, tok);
           if (slot >= 0) {
             const int64_t blk = slot / a.block_size, pos = slot - blk * a.block_size;
@@ -170,37 +238,20 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
             }
           }
         } else {
-          so = n * a.xs0;
           dp = n * a.ps0;
           dn = n;
         }
       }
-      src_off[lane] = so;
-      dst_p[lane] = dp;
-      dst_n[lane] = dn;
-    }
-    // ---- A operands straight from memory; squared norms
-    em_half8 A[4][4];
-    float ss[4];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      const int64_t so = src_off[16 * mt + (lane & 15)];
-      ss[mt] = 0.f;
-      if (so >= 0) {
-        const uint4* p = (const uint4*)((const __half*)a.x + so + 32 * g);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          union { uint4 u; em_half8 h; em_half2 h2[4]; } cv;
-          cv.u = p[ks];
-          A[mt][ks] = cv.h;
-        }
-      } else {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) A[mt][ks] = (em_half8){0, 0, 0, 0, 0, 0, 0, 0};
+      if (lane < EM_ROWS) {
+        dst_p[lane] = dp;
+        dst_n[lane] = dn;
       }
     }
+    float ss[EM_MT];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < EM_MT; ++mt) ss[mt] = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < EM_MT; ++mt) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         union { em_half8 h; em_half2 h2[4]; } cv;
@@ -208,74 +259,139 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 #pragma unroll
         for (int q = 0; q < 4; ++q) ss[mt] = __builtin_amdgcn_fdot2(cv.h2[q], cv.h2[q], ss[mt], false);
       }
-      ss[mt] += __shfl_xor(ss[mt], 16, 64);
-      ss[mt] += __shfl_xor(ss[mt], 32, 64);
     }
-    // lane (row, g = mt) finishes vector 16 mt + row: norm out, reciprocal to LDS
+    // lane l < EM_ROWS finishes vector l = 16 mt + row: transpose-reduce the partial sums over the
+    // four lanes of a row
     {
-      float mine = ss[0];
-      if (g == 1) mine = ss[1];
-      if (g == 2) mine = ss[2];
-      if (g == 3) mine = ss[3];
+      const bool g1 = (g & 1) != 0;
+#if EM_MT == 4
+      const bool g2 = (g & 2) != 0;
+      const float a01 = (g1 ? ss[1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[1], 16, 64);
+      const float a23 = (g1 ? ss[3] : ss[2]) + __shfl_xor(g1 ? ss[2] : ss[3], 16, 64);
+      const float mine = (g2 ? a23 : a01) + __shfl_xor(g2 ? a01 : a23, 32, 64);
+#else
+      const float a01 = (g1 ? ss[1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[1], 16, 64);
+      const float mine = a01 + __shfl_xor(a01, 32, 64);     // lanes g and g + 2 both hold M-tile g & 1
+#endif
       const float nrm = sqrtf(mine);
       const float r = (1.f / (nrm + 1e-10f)) * (1.f / EM_PSCALE);
       // a vector with a NaN or an infinity rotates to NaN everywhere: every code is the last level
-      rinv[lane] = (nrm < INFINITY) ? r : __uint_as_float(0x7fc00000u);
-      if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
+      if (lane < EM_ROWS) {
+        rinv[lane] = (nrm < INFINITY) ? r : __uint_as_float(0x7fc00000u);
+        if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
+      }
     }
+    EM_ST(2);
     // ---- rotate, search, pack
-    uint32_t packed[4][4];
+    uint32_t packed[EM_MT][4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < EM_MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) packed[mt][i] = 0u;
-    em_float4 rv[4];
+    em_float4 rv[EM_MT];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < EM_MT; ++mt) {
       union { em_u32x4 u; em_float4 f; } cv;
       cv.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_WAVE_OFF + wave * EM_WAVE_BYTES + EM_ROWS * 24 + (16 * mt + 4 * g) * 4);
       rv[mt] = cv.f;
     }
+    // N-tiles are software-pipelined: the matrix-core work of tile nt + 1 is issued together with
+    // the search of tile nt (independent instruction streams in one basic block), so the vector
+    // unit works in the shadow of the MFMAs.  The loop stays rolled (two tiles per pass): unrolled,
+    // the scheduler would want every B operand in registers at once.
+    auto mfma_tile = [&](int nt, em_float4 (&acc)[EM_MT]) {
 #pragma unroll
-    for (int nt = 0; nt < 8; ++nt) {
-      em_float4 acc[4];
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) acc[mt] = (em_float4){0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < EM_MT; ++mt) acc[mt] = (em_float4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         union { em_u32x4 u; em_half8 h; } bh, bl;
-        bh.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(((nt * 4 + ks) * 64 + lane) * 16);
-        bl.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(32768 + ((nt * 4 + ks) * 64 + lane) * 16);
+        bh.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_B_OFF + ((nt * 4 + ks) * 64 + lane) * 16);
+        bl.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_B_OFF + 32768 + ((nt * 4 + ks) * 64 + lane) * 16);
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < EM_MT; ++mt) {
+#if defined(EM_EXP) && (EM_EXP == 2 || EM_EXP == 3)
+          acc[mt][ks] += (float)A[mt][ks][0] * (float)bh.h[0] + (float)bl.h[1];
+#else
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bh.h, acc[mt], 0, 0, 0);
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bl.h, acc[mt], 0, 0, 0);
+#endif
         }
       }
-      // output coordinate 8 col + nt of rows 4g + i
+    };
+    auto search_tile = [&](int nt, const em_float4 (&acc)[EM_MT]) {
+      // output coordinate 8 col + nt of rows 4g + i; position of code nt inside the lane's packed
+      // group of eight codes
+      const int sh = BITS == 4 ? 8 * (nt >> 1) + ((nt & 1) ? 0 : 4)
+                   : BITS == 3 ? 21 - 3 * nt
+                               : 8 * (nt >> 2) + 6 - 2 * (nt & 3);
+      float y[EM_MT][4];
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < EM_MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float y = acc[mt][i] * rv[mt][i];
-          uint32_t code;
-          if (!linear_search) {
-            const uint32_t c = em_cell(y, inv_w, off);
-            const em_u32x2 e = *(em_lds_u64*)(uintptr_t)(lut_addr + c * 8u);
-            code = e.x + ((__uint_as_float(e.y) < y) ? 1u : 0u);
-          } else {
-            code = akv_search<BITS>(y, bnd);
+        for (int i = 0; i < 4; ++i) y[mt][i] = acc[mt][i] * rv[mt][i];
+#if defined(EM_EXP) && (EM_EXP == 1 || EM_EXP == 3)
+      if constexpr (true) {
+#pragma unroll
+        for (int mt = 0; mt < EM_MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) packed[mt][i] |= (__float_as_uint(y[mt][i]) & 15u) << sh;
+      } else
+#endif
+      if constexpr (!LINEAR) {
+        em_u32x2 e[EM_MT][4];
+#pragma unroll
+        for (int mt = 0; mt < EM_MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            e[mt][i] = *(em_lds_u64*)(uintptr_t)em_cell(y[mt][i]);
+#pragma unroll
+        for (int mt = 0; mt < EM_MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t code = e[mt][i].x + ((__uint_as_float(e[mt][i].y) < y[mt][i]) ? 1u : 0u);
+            packed[mt][i] |= code << sh;
           }
-          // position of code nt inside the lane's packed group of eight codes
-          const int sh = BITS == 4 ? 8 * (nt >> 1) + ((nt & 1) ? 0 : 4)
-                       : BITS == 3 ? 21 - 3 * nt
-                                   : 8 * (nt >> 2) + 6 - 2 * (nt & 3);
-          packed[mt][i] |= code << sh;
-        }
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < EM_MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            uint32_t code = 0;
+#pragma unroll 1
+            for (int k = 0; k < NB; ++k) code += (bnd[k] < y[mt][i]) ? 1u : 0u;
+            packed[mt][i] |= code << sh;
+          }
+      }
+    };
+    em_float4 accA[EM_MT], accB[EM_MT];
+    mfma_tile(0, accA);
+#pragma unroll 1
+    for (int nt = 0; nt < 6; nt += 2) {
+      mfma_tile(nt + 1, accB);
+      search_tile(nt, accA);
+      mfma_tile(nt + 2, accA);
+      search_tile(nt + 1, accB);
+      // issue order of the pass: one MFMA, then the vector and LDS work that fits in its shadow
+#pragma unroll
+      for (int q = 0; q < 16 * EM_MT; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+      }
     }
+    mfma_tile(7, accB);
+    search_tile(6, accA);
+#pragma unroll
+    for (int q = 0; q < 8 * EM_MT; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    search_tile(7, accB);
+    EM_ST(3);
     // ---- store: lane (col, g) writes group col of rows 4g + i
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < EM_MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int row = 16 * mt + 4 * g + i;
@@ -294,6 +410,15 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           *(uint16_t*)(prow + 2 * col) = (uint16_t)v;
         }
       }
+    EM_ST(4);
+    ++stepno;
+  };
+
+  // (two wavefronts share a SIMD: one computes while the other waits for its rows)
+  if (__builtin_expect(!linear_search, 1)) {
+    for (int64_t step = (int64_t)blockIdx.x * EM_WAVES + wave; step < steps; step += stride) encode_step(std::false_type{}, step);
+  } else {
+    for (int64_t step = (int64_t)blockIdx.x * EM_WAVES + wave; step < steps; step += stride) encode_step(std::true_type{}, step);
   }
 }
 
