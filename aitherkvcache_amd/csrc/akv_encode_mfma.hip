@@ -18,15 +18,18 @@
 //         8col..8col+7 of a vector: one dword of a 4-bit row, three bytes of a 3-bit row, one
 //         halfword of a 2-bit row -- sixteen lanes write one packed row contiguously.
 //
-// Codebook search: code = #{b < y}.  A table of EM_CELLS uniform cells over the boundary range
+// Codebook search: code = #{b < y}.  A table of EM_CELLS uniform cells over y in (-1.004, 1.004)
 // maps cell -> (number of boundaries in lower cells, the one boundary inside the cell or +inf);
 // the cell index is a monotone function of y evaluated by the same instructions for y and, when
-// the table is built, for the boundaries, so base + (boundary < y) is exact for every float.
-// If two boundaries share a cell (no such codebook is produced by the library) the kernel falls
-// back to counting all boundaries.
+// the table is built, for the boundaries, so base + (boundary < y) is exact for every float in
+// range.  |y| <= (longest row of Pi) x |unit vector|, and the prepare step records whether every
+// row is short enough; if not, or if two boundaries share a cell or lie outside (-1, 1) (no such
+// codebook is produced by the library), the kernel counts all boundaries instead.
 //
-// A wavefront encodes 64 vectors per step (four M-tiles share every B operand read from LDS);
-// a workgroup is eight independent wavefronts plus the B operand (64 KB) and the cell table.
+// A wavefront encodes EM_ROWS vectors per step (its M-tiles share every B operand read from LDS);
+// a workgroup is EM_WAVES independent wavefronts plus the B operand (64 KB) and the cell table.
+// Vector-unit and matrix-core time add up on a SIMD here (measured), so the search is kept to six
+// vector instructions per value: multiply, fma, mask, compare, add-with-carry, shift-or.
 #include "akv_common.h"
 #include <type_traits>
 
