@@ -34,14 +34,47 @@ __device__ __forceinline__ float tri_dequant(uint32_t code, float scale) {
   return __fmul_rn(__fsub_rn(__fdiv_rn((float)code, 7.5f), 1.0f), scale);
 }
 
-template <int GQ>
+// sin and cos of a float32 angle of any size reached by positions x frequencies (|x| < ~1e5):
+// quadrant k = rint(x * 2/pi), remainder by a three-constant Cody-Waite subtraction carried by
+// fused multiply-adds (each step is exact before its single rounding), then the classic degree-7 /
+// degree-8 minimax polynomials on [-pi/4, pi/4].  Absolute error ~1e-7, the accuracy the float32
+// library routine has, at a fraction of its cost for large arguments (no table-driven reduction).
+__device__ __forceinline__ void tri_sincos(float x, float& sn, float& cs) {
+  const float k = rintf(x * 0.636619772367581343f);
+  float r = fmaf(k, -1.57079637050628662109375f, x);
+  r = fmaf(k, 4.37113900018624283e-8f, r);
+  r = fmaf(k, 1.71512451370281e-15f, r);
+  const float r2 = r * r;
+  float ps = fmaf(r2, -1.9515295891e-4f, 8.3321608736e-3f);
+  ps = fmaf(ps, r2, -1.6666654611e-1f);
+  const float s0 = fmaf(ps * r2, r, r);
+  float pc = fmaf(r2, 2.443315711809948e-5f, -1.388731625493765e-3f);
+  pc = fmaf(pc, r2, 4.166664568298827e-2f);
+  const float c0 = fmaf(pc * r2, r2, fmaf(r2, -0.5f, 1.0f));
+  const int q = (int)k;
+  const float a = (q & 1) ? c0 : s0;
+  const float b = (q & 1) ? s0 : c0;
+  sn = __uint_as_float(__float_as_uint(a) ^ ((uint32_t)(q & 2) << 30));
+  cs = __uint_as_float(__float_as_uint(b) ^ ((uint32_t)((q + 1) & 2) << 30));
+}
+
+template <int GQ, bool F12, bool DENSE>
 __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   float* theta = (float*)lds_raw;                         // [D/2]
   float* q_lds = theta + a.D / 2;                         // [GQ][D]   (per workgroup pass)
-  float* acc_base = q_lds + GQ * a.D;                     // [TRI_WAVES][GQ][D]
+  float* dq = q_lds + GQ * a.D;                           // [16]: code / 7.5 - 1 with the reference's roundings
+  float* acc_base = dq + 16;                              // [TRI_WAVES][GQ][D]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* acc = acc_base + (size_t)wave * GQ * a.D;
+  // DENSE (head_dim 128): instead of bins updated by LDS atomics (which serialise when many tokens
+  // retain the same pair -- the usual case), each wavefront has a 16-token x 128-coordinate tile
+  // and a 64 x GQ weight table; a lane owns one coordinate pair and its sums stay in registers
+  float* tile = acc_base + (size_t)wave * (16 * 128 + 64 * GQ);
+  float* wtab = tile + 16 * 128;
+  if (DENSE) {
+    for (int i = lane; i < 16 * 128; i += 64) tile[i] = 0.f;   // every use leaves the tile zero again
+  }
   const int D = a.D, F = a.F;
   const int gqa = a.QH / a.KVH;
   const int b = blockIdx.z, h = blockIdx.y;
@@ -49,6 +82,7 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
   const float inv_sqrt_d = 1.0f / sqrtf((float)D);
 
   for (int i = threadIdx.x; i < D / 2; i += 256) theta[i] = a.theta[i];
+  if (threadIdx.x < 16) dq[threadIdx.x] = __fsub_rn(__fdiv_rn((float)threadIdx.x, 7.5f), 1.0f);
 
   const int64_t per = (a.S + a.nsplit - 1) / a.nsplit;
   const int64_t s0 = min(a.S, (int64_t)split * per);
@@ -60,14 +94,20 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
     for (int i = threadIdx.x; i < GQ * D; i += 256) {
       const int q = i / D, d = i % D;
       const int64_t off = ((int64_t)b * a.QH + (h * gqa + qg + q)) * D + d;
+      const int slot = ((d >> 1) * GQ + q) * 2 + (d & 1);   // [pair][q][even, odd]: one pair index serves all GQ heads
       float v;
       if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
       else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
       else v = akv_elem<AKV_F32>::load(a.query, off);
-      q_lds[i] = v;
+      q_lds[slot] = v;
     }
-    for (int i = lane; i < GQ * D; i += 64) acc[i] = 0.f;
+    if (!DENSE) {
+      for (int i = lane; i < GQ * D; i += 64) acc[i] = 0.f;
+    }
     __syncthreads();
+    float o[GQ][2];
+#pragma unroll
+    for (int q = 0; q < GQ; ++q) o[q][0] = o[q][1] = 0.f;
 
     float m[GQ], l[GQ];
 #pragma unroll
@@ -84,16 +124,25 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       float sc[GQ];
 #pragma unroll
       for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+      uint32_t ki[3], kc[3];
+      if (F12) {   // the token's 12 index bytes and 12 coefficient bytes as three dwords each
+        const uint32_t* pi = (const uint32_t*)(a.k_idx + row * 12);
+        const uint32_t* pc = (const uint32_t*)(a.k_cf + row * 12);
+#pragma unroll
+        for (int w = 0; w < 3; ++w) { ki[w] = pi[w]; kc[w] = pc[w]; }
+      }
+#pragma unroll 4
       for (int f = 0; f < F; ++f) {
-        const uint32_t idx = a.k_idx[row * F + f];
-        const uint32_t cf = a.k_cf[row * F + f];
-        const float k0 = tri_dequant(cf >> 4, ksc), k1 = tri_dequant(cf & 15u, ksc);
+        const uint32_t idx = F12 ? (ki[f >> 2] >> (8 * (f & 3))) & 255u : a.k_idx[row * F + f];
+        const uint32_t cf = F12 ? (kc[f >> 2] >> (8 * (f & 3))) & 255u : a.k_cf[row * F + f];
+        const float k0 = __fmul_rn(dq[cf >> 4], ksc), k1 = __fmul_rn(dq[cf & 15u], ksc);
         const float ph = __fmul_rn(delta, theta[idx]);
         float sn, cs;
-        sincosf(ph, &sn, &cs);
+        tri_sincos(ph, sn, cs);
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float qe = q_lds[q * D + 2 * idx], qo = q_lds[q * D + 2 * idx + 1];
+          const float2 qq = *(const float2*)(q_lds + (idx * GQ + q) * 2);
+          const float qe = qq.x, qo = qq.y;
           const float c = qe * k0 + qo * k1;
           const float s = qo * k0 - qe * k1;
           sc[q] += c * cs + s * sn;
@@ -112,6 +161,61 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
         l[q] = l[q] * alpha[q] + p[q];
         m[q] = mn;
       }
+      if (DENSE) {
+        if (rescale) {  // wavefront-uniform: m is the same in every lane
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) { o[q][0] *= alpha[q]; o[q][1] *= alpha[q]; }
+        }
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) wtab[lane * GQ + q] = p[q];
+        float vsc = 0.f;
+        uint32_t vi[3] = {0, 0, 0}, vc[3] = {0, 0, 0};
+        if (valid) {
+          vsc = __half2float(a.v_sc[row]);
+          if (F12) {
+            const uint32_t* pi = (const uint32_t*)(a.v_idx + row * 12);
+            const uint32_t* pc = (const uint32_t*)(a.v_cf + row * 12);
+#pragma unroll
+            for (int w = 0; w < 3; ++w) { vi[w] = pi[w]; vc[w] = pc[w]; }
+          }
+        }
+        float* my_row = tile + (lane & 15) * 128;
+#pragma unroll 1
+        for (int sub = 0; sub < 4; ++sub) {
+          const bool mine = valid && (lane >> 4) == sub;
+          if (mine) {
+#pragma unroll 4
+            for (int f = 0; f < F; ++f) {
+              const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+              const uint32_t cf = F12 ? (vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+              *(float2*)(my_row + 2 * idx) = make_float2(__fmul_rn(dq[cf >> 4], vsc), __fmul_rn(dq[cf & 15u], vsc));
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 4
+          for (int t = 0; t < 16; ++t) {
+            const float2 v = *(const float2*)(tile + t * 128 + 2 * lane);
+#pragma unroll
+            for (int q = 0; q < GQ; ++q) {
+              const float w = wtab[(16 * sub + t) * GQ + q];
+              o[q][0] = fmaf(w, v.x, o[q][0]);
+              o[q][1] = fmaf(w, v.y, o[q][1]);
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          if (mine) {
+#pragma unroll 4
+            for (int f = 0; f < F; ++f) {
+              const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+              *(float2*)(my_row + 2 * idx) = make_float2(0.f, 0.f);
+            }
+          }
+        }
+      } else {
       if (rescale) {  // wavefront-uniform: m is the same in every lane
 #pragma unroll
         for (int q = 0; q < GQ; ++q)
@@ -122,10 +226,18 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       }
       if (valid) {
         const float vsc = __half2float(a.v_sc[row]);
+        uint32_t vi[3], vc[3];
+        if (F12) {
+          const uint32_t* pi = (const uint32_t*)(a.v_idx + row * 12);
+          const uint32_t* pc = (const uint32_t*)(a.v_cf + row * 12);
+#pragma unroll
+          for (int w = 0; w < 3; ++w) { vi[w] = pi[w]; vc[w] = pc[w]; }
+        }
+#pragma unroll 4
         for (int f = 0; f < F; ++f) {
-          const uint32_t idx = a.v_idx[row * F + f];
-          const uint32_t cf = a.v_cf[row * F + f];
-          const float v0 = tri_dequant(cf >> 4, vsc), v1 = tri_dequant(cf & 15u, vsc);
+          const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+          const uint32_t cf = F12 ? (vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+          const float v0 = __fmul_rn(dq[cf >> 4], vsc), v1 = __fmul_rn(dq[cf & 15u], vsc);
 #pragma unroll
           for (int q = 0; q < GQ; ++q) {
             atomicAdd(&acc[q * D + 2 * idx], p[q] * v0);
@@ -136,37 +248,49 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
     }
     if (split < a.nsplit) {
 #pragma unroll
       for (int q = 0; q < GQ; ++q) {
         const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
         const float lsum = akv_wave_sum(l[q]);
-        for (int i = lane; i < D; i += 64) a.part_acc[slot * D + i] = acc[q * D + i];
+        if (DENSE) *(float2*)(a.part_acc + slot * D + 2 * lane) = make_float2(o[q][0], o[q][1]);
+        else for (int i = lane; i < D; i += 64) a.part_acc[slot * D + i] = acc[q * D + i];
         if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
       }
     }
   }
 }
 
-__global__ __launch_bounds__(64) void tri_reduce_kernel(const float* __restrict__ part_acc,
-                                                        const float* __restrict__ part_ml,
-                                                        int nsplit, int D, float* __restrict__ out) {
+// one workgroup per (batch, query head): split weights once, then one thread per coordinate
+__global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict__ part_acc,
+                                                         const float* __restrict__ part_ml,
+                                                         int nsplit, int D, float* __restrict__ out) {
+  __shared__ float w[TRI_MAX_SPLITS];
+  __shared__ float red[2];
   const size_t pair = blockIdx.x;  // b * QH + qh
-  const int lane = threadIdx.x;
-  float m = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, part_ml[(pair * nsplit + s) * 2]);
-  float l = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = part_ml[(pair * nsplit + s) * 2];
-    if (ms > -INFINITY) l += __expf(ms - m) * part_ml[(pair * nsplit + s) * 2 + 1];
+  if (threadIdx.x < 64) {
+    float m = -INFINITY;
+    for (int s = threadIdx.x; s < nsplit; s += 64) m = fmaxf(m, part_ml[(pair * nsplit + s) * 2]);
+    m = akv_wave_max(m);
+    float l = 0.f;
+    for (int s = threadIdx.x; s < nsplit; s += 64) {
+      const float ms = part_ml[(pair * nsplit + s) * 2];
+      const float ws = ms > -INFINITY ? __expf(ms - m) : 0.f;
+      w[s] = ws;
+      l += ws * part_ml[(pair * nsplit + s) * 2 + 1];
+    }
+    l = akv_wave_sum(l);
+    if (threadIdx.x == 0) red[0] = l > 0.f ? 1.f / l : 0.f;
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  for (int i = lane; i < D; i += 64) {
+  __syncthreads();
+  const float inv = red[0];
+  for (int i = threadIdx.x; i < D; i += 128) {
     float acc = 0.f;
     for (int s = 0; s < nsplit; ++s) {
-      const float ms = part_ml[(pair * nsplit + s) * 2];
-      if (ms > -INFINITY) acc += __expf(ms - m) * part_acc[(pair * nsplit + s) * D + i];
+      const float ws = w[s];
+      if (ws != 0.f) acc = fmaf(ws, part_acc[(pair * nsplit + s) * D + i], acc);
     }
     out[pair * D + i] = acc * inv;
   }
@@ -235,16 +359,24 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   const int gqa = num_q_heads / num_kv_heads;
   dim3 grid(a.nsplit / TRI_WAVES, num_kv_heads, batch);
   akv_profile_mark_begin(stream);
-  if (gqa % 4 == 0) {
-    const size_t lds = ((size_t)d / 2 + 4 * d + TRI_WAVES * 4 * d) * sizeof(float);
-    tri_decode_kernel<4><<<grid, 256, lds, stream>>>(a);
-  } else {
-    const size_t lds = ((size_t)d / 2 + 1 * d + TRI_WAVES * 1 * d) * sizeof(float);
-    tri_decode_kernel<1><<<grid, 256, lds, stream>>>(a);
-  }
+  // rows of 12 bytes can be read as dwords when the arrays are 4-byte aligned
+  const bool f12 = num_freqs == 12 &&
+                   ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
+  const bool dense = d == 128;
+#define TRI_LAUNCH(GQV)                                                                                   \
+  do {                                                                                                    \
+    const size_t per_wave = dense ? (size_t)(16 * 128 + 64 * GQV) : (size_t)GQV * d;                      \
+    const size_t lds = ((size_t)d / 2 + (size_t)GQV * d + 16 + TRI_WAVES * per_wave) * sizeof(float);     \
+    if (dense && f12) tri_decode_kernel<GQV, true, true><<<grid, 256, lds, stream>>>(a);                  \
+    else if (dense) tri_decode_kernel<GQV, false, true><<<grid, 256, lds, stream>>>(a);                   \
+    else if (f12) tri_decode_kernel<GQV, true, false><<<grid, 256, lds, stream>>>(a);                     \
+    else tri_decode_kernel<GQV, false, false><<<grid, 256, lds, stream>>>(a);                             \
+  } while (0)
+  if (gqa % 4 == 0) TRI_LAUNCH(4); else TRI_LAUNCH(1);
+#undef TRI_LAUNCH
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("tri_decode_kernel");
-  tri_reduce_kernel<<<batch * num_q_heads, 64, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
+  tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
   return AKV_OK;
 }
