@@ -247,6 +247,24 @@ __device__ __forceinline__ uint32_t mf_here(uint32_t v) {
   return v;
 }
 
+// Reductions over the four 16-lane rows of a wavefront (every lane gets the result for its column)
+// by the row-swap instructions: v_permlane32_swap exchanges rows {2,3} of its first operand with
+// rows {0,1} of the second, v_permlane16_swap rows {1,3} with rows {0,2}; fed the same value twice
+// they leave (rows 0,1,0,1 | rows 2,3,2,3) and (rows 0,0,2,2 | rows 1,1,3,3).  Two vector
+// instructions per step, no trip through the LDS crossbar.
+__device__ __forceinline__ float mf_rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float mf_rows_sum(float v) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // workgroup barrier that orders LDS traffic only (outstanding global loads keep flying)
 __device__ __forceinline__ void mf_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -404,8 +422,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           }
           // running softmax in the log2 domain (scale * log2 e is folded into the query operand)
           float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          mx = mf_rows_max(mx);
           const float m_new = fmaxf(m_run, mx);
           const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
           m_run = m_new;
@@ -456,8 +473,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
         mf_barrier();   // value side done with the buffers
         float lsum = l_run;
-        lsum += __shfl_xor(lsum, 16, 64);
-        lsum += __shfl_xor(lsum, 32, 64);
+        lsum = mf_rows_sum(lsum);
         if (active && col < gqa && g == 0) {
           const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
           a.part_ml[slot * 2] = m_run * 0.6931471805599453f;   // back to the natural-log domain
