@@ -419,9 +419,9 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 
   // (two wavefronts share a SIMD: one computes while the other waits for its rows)
   if (__builtin_expect(!linear_search, 1)) {
-    for (int64_t step = (int64_t)blockIdx.x * EM_WAVES + wave; step < steps; step += stride) encode_step(std::false_type{}, step);
+    for (int64_t step = (int64_t)wave * gridDim.x + blockIdx.x; step < steps; step += stride) encode_step(std::false_type{}, step);
   } else {
-    for (int64_t step = (int64_t)blockIdx.x * EM_WAVES + wave; step < steps; step += stride) encode_step(std::true_type{}, step);
+    for (int64_t step = (int64_t)wave * gridDim.x + blockIdx.x; step < steps; step += stride) encode_step(std::true_type{}, step);
   }
 }
 
@@ -443,8 +443,9 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   if (((uintptr_t)a.packed | (uintptr_t)a.ps0 | (uintptr_t)a.ps1 | (uintptr_t)a.ps2) & amask) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const float*)rot_prep + (size_t)2 * d * d);
   const int64_t steps = (a.n + EM_ROWS - 1) / EM_ROWS;
-  const int64_t wgs = (steps + EM_WAVES - 1) / EM_WAVES;
-  const int grid = (int)(wgs < akv_cached_cu_count() ? wgs : akv_cached_cu_count());
+  // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
+  // over as many CUs as it has steps instead of filling the wavefronts of a few
+  const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
 #define EM_LAUNCH(BB, PG)                                                                            \
   do {                                                                                               \
     static bool configured = false;                                                                  \
