@@ -1,4 +1,5 @@
-// MFMA encode (norm -> rotate -> codebook search -> pack -> store) for float16 input at head_dim 128.
+// MFMA encode (norm -> rotate -> codebook search -> pack -> store) for float16 and bfloat16 input
+// at head_dim 128.
 //
 // The rotation is the only heavy arithmetic of the encode path (128 x 128 multiply-adds per
 // vector), so it runs on the matrix cores; everything else is arranged so that the matrix-core
@@ -36,6 +37,7 @@
 typedef _Float16 em_half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 em_half2 __attribute__((ext_vector_type(2)));
 typedef float em_float4 __attribute__((ext_vector_type(4)));
+typedef unsigned short em_us2 __attribute__((ext_vector_type(2)));
 
 #ifndef EM_MT
 #define EM_MT 2                    // M-tiles (16 vectors each) per wavefront step
@@ -133,7 +135,7 @@ __device__ __forceinline__ uint32_t em_cell(float y) {
   return __float_as_uint(fmaf(y, EM_CELL_S, EM_CELL_C)) & EM_CELL_MASK;
 }
 
-template <int BITS, bool PAGED>
+template <int BITS, bool PAGED, int XDT>
 __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   constexpr int NB = (1 << BITS) - 1;
@@ -253,14 +255,68 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     float ss[EM_MT];
 #pragma unroll
     for (int mt = 0; mt < EM_MT; ++mt) ss[mt] = 0.f;
+    uint32_t unscale[EM_MT];     // float bits of the power of two taken out of each M-tile's rows
+    bool nonfinite[EM_MT];       // bfloat16 only: the row holds an infinity or a NaN
+    if constexpr (XDT == AKV_F16) {
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt) {
+      for (int mt = 0; mt < EM_MT; ++mt) {
+        unscale[mt] = 0x3f800000u;
+        nonfinite[mt] = false;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        union { em_half8 h; em_half2 h2[4]; } cv;
-        cv.h = A[mt][ks];
+        for (int ks = 0; ks < 4; ++ks) {
+          union { em_half8 h; em_half2 h2[4]; } cv;
+          cv.h = A[mt][ks];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) ss[mt] = __builtin_amdgcn_fdot2(cv.h2[q], cv.h2[q], ss[mt], false);
+          for (int q = 0; q < 4; ++q) ss[mt] = __builtin_amdgcn_fdot2(cv.h2[q], cv.h2[q], ss[mt], false);
+        }
+      }
+    } else {
+      // bfloat16 rows: squared norm from the exact float32 values; then each row is scaled by the
+      // power of two that brings its largest element into [1, 2) and converted to float16 -- exact
+      // for every element within 2^14 of the largest (8 significant bits fit in 11), and off by at
+      // most 2^-25 of the largest otherwise, far below the resolution of the codebook search
+#pragma unroll
+      for (int mt = 0; mt < EM_MT; ++mt) {
+        em_us2 mx2 = {0, 0};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          union { em_half8 h; uint32_t w[4]; } cv;
+          cv.h = A[mt][ks];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            union { uint32_t u; em_us2 v; } mm;
+            mm.u = cv.w[q] & 0x7fff7fffu;
+            mx2 = __builtin_elementwise_max(mx2, mm.v);
+            const float lo = __uint_as_float(cv.w[q] << 16), hi = __uint_as_float(cv.w[q] & 0xffff0000u);
+            ss[mt] = fmaf(lo, lo, ss[mt]);
+            ss[mt] = fmaf(hi, hi, ss[mt]);
+          }
+        }
+        uint32_t mx = max((uint32_t)mx2[0], (uint32_t)mx2[1]);
+        {   // largest magnitude of the row over its four lanes
+          auto r1 = __builtin_amdgcn_permlane32_swap(mx, mx, false, false);
+          mx = max(r1[0], r1[1]);
+          auto r2 = __builtin_amdgcn_permlane16_swap(mx, mx, false, false);
+          mx = max(r2[0], r2[1]);
+        }
+        uint32_t ef = mx >> 7;                       // exponent field of the largest element
+        nonfinite[mt] = ef == 255u;
+        if (ef == 0u || ef == 255u) ef = 127u;       // all (sub)zero, or not finite (flagged)
+        if (ef == 254u) ef = 253u;                   // keep the scale a normal number
+        const float sc = __uint_as_float((254u - ef) << 23);     // 2^(127 - ef)
+        unscale[mt] = ef << 23;                                   // 2^(ef - 127)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          union { em_half8 h; uint32_t w[4]; em_half2 h2[4]; } cv;
+          cv.h = A[mt][ks];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float lo = __uint_as_float(cv.w[q] << 16) * sc, hi = __uint_as_float(cv.w[q] & 0xffff0000u) * sc;
+            auto pk = __builtin_amdgcn_cvt_pkrtz(lo, hi);
+            cv.h2[q] = (em_half2){(_Float16)pk[0], (_Float16)pk[1]};
+          }
+          A[mt][ks] = cv.h;
+        }
       }
     }
     // lane l < EM_ROWS finishes vector l = 16 mt + row: transpose-reduce the partial sums over the
@@ -277,10 +333,24 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       const float mine = a01 + __shfl_xor(a01, 32, 64);     // lanes g and g + 2 both hold M-tile g & 1
 #endif
       const float nrm = sqrtf(mine);
-      const float r = (1.f / (nrm + 1e-10f)) * (1.f / EM_PSCALE);
-      // a vector with a NaN or an infinity rotates to NaN everywhere: every code is the last level
+#if EM_MT == 4
+      const uint32_t my_unscale = g == 0 ? unscale[0] : g == 1 ? unscale[1] : g == 2 ? unscale[2] : unscale[3];
+#else
+      const uint32_t my_unscale = g1 ? unscale[1] : unscale[0];
+#endif
+      const float r = (1.f / (nrm + 1e-10f)) * (1.f / EM_PSCALE) * __uint_as_float(my_unscale);
+      // a vector with a NaN or an infinity rotates to NaN everywhere: every code is the last level.
+      // (float16 squares cannot overflow, so there an infinite norm means an infinite element; a
+      // finite bfloat16 row whose squares overflow has norm inf, unit vector 0 and y = 0 like the
+      // reference: r is 0 and the scaled products are finite.)
+#if EM_MT == 4
+      const bool my_nonfinite = g == 0 ? nonfinite[0] : g == 1 ? nonfinite[1] : g == 2 ? nonfinite[2] : nonfinite[3];
+#else
+      const bool my_nonfinite = g1 ? nonfinite[1] : nonfinite[0];
+#endif
+      const bool nan_row = XDT == AKV_F16 ? !(nrm < INFINITY) : (my_nonfinite || nrm != nrm);
       if (lane < EM_ROWS) {
-        rinv[lane] = (nrm < INFINITY) ? r : __uint_as_float(0x7fc00000u);
+        rinv[lane] = nan_row ? __uint_as_float(0x7fc00000u) : r;
         if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
       }
     }
@@ -436,7 +506,7 @@ static bool em_disabled() {
 
 int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, int bits,
                         const void* rot_prep, hipStream_t stream) {
-  if (em_disabled() || d != 128 || x_dtype != AKV_F16) return AKV_ERR_UNSUPPORTED;
+  if (em_disabled() || d != 128 || (x_dtype != AKV_F16 && x_dtype != AKV_BF16)) return AKV_ERR_UNSUPPORTED;
   // 16-byte loads of the input rows; aligned stores of the packed groups
   if (((uintptr_t)a.x & 15) || (a.xs0 & 7) || (paged && (a.xs1 & 7))) return AKV_ERR_UNSUPPORTED;
   const int64_t amask = bits == 4 ? 3 : bits == 2 ? 1 : 0;
@@ -446,23 +516,25 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
-#define EM_LAUNCH(BB, PG)                                                                            \
+#define EM_LAUNCH(BB, PG, DT)                                                                        \
   do {                                                                                               \
     static bool configured = false;                                                                  \
     if (!configured) {                                                                               \
-      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG>,                       \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT>,                   \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, EM_LDS_BYTES));        \
       configured = true;                                                                             \
     }                                                                                                \
     akv_profile_mark_begin(stream);                                                                  \
-    akv_encode_mfma_kernel<BB, PG><<<grid, EM_THREADS, EM_LDS_BYTES, stream>>>(a, bop);              \
+    akv_encode_mfma_kernel<BB, PG, DT><<<grid, EM_THREADS, EM_LDS_BYTES, stream>>>(a, bop);          \
     akv_profile_mark_end(stream);                                                                    \
   } while (0)
+#define EM_LAUNCH_DT(BB, PG) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16); else EM_LAUNCH(BB, PG, AKV_BF16); } while (0)
   if (paged) {
-    if (bits == 4) EM_LAUNCH(4, true); else if (bits == 3) EM_LAUNCH(3, true); else EM_LAUNCH(2, true);
+    if (bits == 4) EM_LAUNCH_DT(4, true); else if (bits == 3) EM_LAUNCH_DT(3, true); else EM_LAUNCH_DT(2, true);
   } else {
-    if (bits == 4) EM_LAUNCH(4, false); else if (bits == 3) EM_LAUNCH(3, false); else EM_LAUNCH(2, false);
+    if (bits == 4) EM_LAUNCH_DT(4, false); else if (bits == 3) EM_LAUNCH_DT(3, false); else EM_LAUNCH_DT(2, false);
   }
+#undef EM_LAUNCH_DT
 #undef EM_LAUNCH
   AKV_LAUNCH_CHECK("akv_encode_mfma_kernel");
   return AKV_OK;

@@ -73,6 +73,31 @@ def test_encode_other_input_dtypes(golden, dev, dtype, key):
                 golden[f"enc_packed_{key}_b4"], golden[f"enc_norms_{key}_b4"])
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_encode_bfloat16_wide_range_vs_oracle(golden, dev, bits):
+    """bfloat16 rows go through a per-row power-of-two scaling: rows of very large, very small and
+    mixed magnitudes must give the oracle's codes (the oracle sees the same bfloat16 values)."""
+    rng = np.random.default_rng(77 + bits)
+    n = 2048 + 17
+    x = rng.standard_normal((n, 128)).astype(np.float32)
+    scale = np.exp2(rng.integers(-40, 40, size=n)).astype(np.float32)         # rows from 2^-40 to 2^40
+    x *= scale[:, None]
+    x[::7] *= np.exp2(rng.integers(-20, 1, size=(len(x[::7]), 128))).astype(np.float32)   # wide range inside a row
+    x[3] = 0.0
+    xb = torch.from_numpy(x).to(torch.bfloat16)
+    tq = make_tq(golden, dev, bits)
+    packed, norms = tq.encode(xb.to(dev))
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), xb.float().numpy(), golden["rotation_d128_seed42"], bits)
+    # squares that overflow float32: norm inf, unit vector 0, every code is #{b < 0}; an infinite
+    # element makes the rotated vector NaN: every code is the last level (searchsorted puts NaN last)
+    y = torch.full((2, 128), 2.0 ** 70, dtype=torch.bfloat16)
+    y[1, 5] = float("inf")
+    packed, norms = tq.encode(y.to(dev))
+    codes = O._UNPACK[bits](packed.cpu().numpy(), 128)
+    assert np.all(codes[0] == (1 << bits) // 2 - 1) and np.all(codes[1] == (1 << bits) - 1)
+    assert np.all(np.isinf(norms.cpu().numpy()))
+
+
 def test_head_dim_64(golden, dev):
     tq = make_tq(golden, dev, 4, d=64)
     x = golden["enc_x_d64"]
