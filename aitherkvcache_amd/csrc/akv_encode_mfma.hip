@@ -135,7 +135,7 @@ __device__ __forceinline__ uint32_t em_cell(float y) {
   return __float_as_uint(fmaf(y, EM_CELL_S, EM_CELL_C)) & EM_CELL_MASK;
 }
 
-template <int BITS, bool PAGED, int XDT>
+template <int BITS, bool PAGED, int XDT, bool DIRECT>
 __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   constexpr int NB = (1 << BITS) - 1;
@@ -189,6 +189,27 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   // A operands of one step straight from memory (zeros past the end): lane l resolves the source
   // row of vector base + l, the lanes of an M-tile pick the rows up through LDS
   auto fetch = [&](em_half8 (&A)[EM_MT][4], int64_t step) {
+    if constexpr (DIRECT) {
+      // contiguous rows whose byte offsets fit 31 bits: every lane forms its rows' addresses itself
+      // (scalar base + 32-bit lane offset), no exchange through LDS
+#pragma unroll
+      for (int mt = 0; mt < EM_MT; ++mt) {
+        const uint32_t n = (uint32_t)step * EM_ROWS + 16 * mt + (lane & 15);
+        if (n < (uint32_t)a.n) {
+          const uint4* p = (const uint4*)((const char*)a.x + (n * (uint32_t)a.xs0 + 32u * g) * 2u);
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+            union { uint4 u; em_half8 h; } cv;
+            cv.u = p[ks];
+            A[mt][ks] = cv.h;
+          }
+        } else {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) A[mt][ks] = (em_half8){0, 0, 0, 0, 0, 0, 0, 0};
+        }
+      }
+      return;
+    }
     const int64_t n = step * EM_ROWS + lane;
     int64_t so = -1;
     if (step < steps && n < a.n && lane < EM_ROWS) {
@@ -228,7 +249,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     EM_ST(1);
     const int64_t base = step * EM_ROWS;
     // ---- lane l resolves the destination of vector base + l
-    {
+    if constexpr (!DIRECT) {
       const int64_t n = base + lane;
       int64_t dp = -1, dn = 0;
       if (n < a.n && lane < EM_ROWS) {
@@ -351,7 +372,11 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       const bool nan_row = XDT == AKV_F16 ? !(nrm < INFINITY) : (my_nonfinite || nrm != nrm);
       if (lane < EM_ROWS) {
         rinv[lane] = nan_row ? __uint_as_float(0x7fc00000u) : r;
-        if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
+        if constexpr (DIRECT) {
+          if ((uint32_t)base + lane < (uint32_t)a.n) a.norms[(uint32_t)base + lane] = nrm;
+        } else {
+          if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
+        }
       }
     }
     EM_ST(2);
@@ -468,11 +493,18 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int row = 16 * mt + 4 * g + i;
-        const int64_t dp = dst_p[row];
-        if (dp < 0) continue;
+        uint8_t* prow;
+        if constexpr (DIRECT) {
+          const uint32_t n = (uint32_t)base + row;
+          if (n >= (uint32_t)a.n) continue;
+          prow = a.packed + n * (uint32_t)a.ps0;
+        } else {
+          const int64_t dp = dst_p[row];
+          if (dp < 0) continue;
+          prow = a.packed + dp;
+        }
         uint32_t v = packed[mt][i];
         if (!(rv[mt][i] == rv[mt][i])) v = 0xffffffffu;     // NaN vector: last level everywhere
-        uint8_t* prow = a.packed + dp;
         if (BITS == 4) {
           *(uint32_t*)(prow + 4 * col) = v;
         } else if (BITS == 3) {
@@ -516,23 +548,27 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
-#define EM_LAUNCH(BB, PG, DT)                                                                        \
+#define EM_LAUNCH(BB, PG, DT, DR)                                                                       \
   do {                                                                                               \
     static bool configured = false;                                                                  \
     if (!configured) {                                                                               \
-      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT>,                   \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT, DR>,                 \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, EM_LDS_BYTES));        \
       configured = true;                                                                             \
     }                                                                                                \
     akv_profile_mark_begin(stream);                                                                  \
-    akv_encode_mfma_kernel<BB, PG, DT><<<grid, EM_THREADS, EM_LDS_BYTES, stream>>>(a, bop);          \
+    akv_encode_mfma_kernel<BB, PG, DT, DR><<<grid, EM_THREADS, EM_LDS_BYTES, stream>>>(a, bop);      \
     akv_profile_mark_end(stream);                                                                    \
   } while (0)
-#define EM_LAUNCH_DT(BB, PG) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16); else EM_LAUNCH(BB, PG, AKV_BF16); } while (0)
+#define EM_LAUNCH_DT(BB, PG, DR) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16, DR); else EM_LAUNCH(BB, PG, AKV_BF16, DR); } while (0)
+  // flat rows whose byte offsets stay below 2^31 take the variant with 32-bit lane offsets
+  const bool direct = !paged && a.n < ((int64_t)1 << 31) / (2 * a.xs0 > a.ps0 ? 2 * a.xs0 : a.ps0);
   if (paged) {
-    if (bits == 4) EM_LAUNCH_DT(4, true); else if (bits == 3) EM_LAUNCH_DT(3, true); else EM_LAUNCH_DT(2, true);
+    if (bits == 4) EM_LAUNCH_DT(4, true, false); else if (bits == 3) EM_LAUNCH_DT(3, true, false); else EM_LAUNCH_DT(2, true, false);
+  } else if (direct) {
+    if (bits == 4) EM_LAUNCH_DT(4, false, true); else if (bits == 3) EM_LAUNCH_DT(3, false, true); else EM_LAUNCH_DT(2, false, true);
   } else {
-    if (bits == 4) EM_LAUNCH_DT(4, false); else if (bits == 3) EM_LAUNCH_DT(3, false); else EM_LAUNCH_DT(2, false);
+    if (bits == 4) EM_LAUNCH_DT(4, false, false); else if (bits == 3) EM_LAUNCH_DT(3, false, false); else EM_LAUNCH_DT(2, false, false);
   }
 #undef EM_LAUNCH_DT
 #undef EM_LAUNCH
