@@ -82,6 +82,8 @@ __global__ void akv_prepare_rotation_kernel(const float* __restrict__ R, float* 
 }
 
 int akv_prepare_rotation_mfma(const float* rotation, int d, void* prep, hipStream_t stream);
+int akv_prepare_decode_mfma(const float* rotation, int d, void* prep, hipStream_t stream);
+int akv_decode_mfma_try(const akv_gen_args& a, int d, int bits, int out_dtype, const void* rot_prep, hipStream_t stream);
 
 extern "C" size_t akv_rotation_prepared_bytes(int d) { return akv_prep_floats(d) * sizeof(float); }
 
@@ -94,7 +96,11 @@ extern "C" int akv_rotation_prepare(const float* rotation, int d, void* prep, si
   dim3 grid(d / 32, d / 32);
   akv_prepare_rotation_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rotation, (float*)prep, d);
   AKV_LAUNCH_CHECK("akv_prepare_rotation_kernel");
-  if (d == 128) return akv_prepare_rotation_mfma(rotation, d, prep, (hipStream_t)stream);
+  if (d == 128) {
+    int rc = akv_prepare_rotation_mfma(rotation, d, prep, (hipStream_t)stream);
+    if (rc) return rc;
+    return akv_prepare_decode_mfma(rotation, d, prep, (hipStream_t)stream);
+  }
   return AKV_OK;
 }
 
@@ -524,6 +530,8 @@ extern "C" int akv_decode(const uint8_t* packed, int64_t packed_stride, const fl
   a.packed = const_cast<uint8_t*>(packed); a.ps0 = packed_stride;
   a.norms = const_cast<float*>(norms);
   a.out = out; a.os0 = out_stride;
+  rc = akv_decode_mfma_try(a, d, bits, out_dtype, rot_prep, (hipStream_t)stream);
+  if (rc != AKV_ERR_UNSUPPORTED) return rc;
 #define AKV_CASE(DD, BB) \
   if (d == DD && bits == BB) return akv_decode_dispatch_dtype<DD, BB>(out_dtype, a, stream);
   AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)

@@ -57,8 +57,10 @@ void akv_profile_mark_end(hipStream_t s);
 // Offsets (in floats) into the prepared-rotation buffer.
 //   [0, d*d)        Pi     row-major  (y_i = sum_j Pi[i][j] x_j)
 //   [d*d, 2*d*d)    Pi^T   row-major
-//   [2*d*d, 4*d*d)  fp16 hi / scaled-lo operand tiles for the MFMA encode kernel
-static inline size_t akv_prep_floats(int d) { return (size_t)4 * d * d; }
+//   [2*d*d, ...)    d = 128 only: float16 hi/lo operand tiles of the MFMA encode kernel (64 KB),
+//                   a flag word (256 B reserved), the same for the MFMA decode kernel (64 KB)
+static inline size_t akv_prep_floats(int d) { return (size_t)4 * d * d + 1024; }
+#define AKV_PREP_DECODE_OFFSET(d) ((size_t)2 * (d) * (d) * 4 + 65536 + 256)
 
 // Arguments of the encode / decode kernels (flat and paged forms share one struct).
 struct akv_gen_args {
