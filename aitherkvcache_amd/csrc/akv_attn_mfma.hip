@@ -496,9 +496,13 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
               r.v[4 * j + i] = *(const uint32_t*)(vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff));
           }
         };
+        // Everything that does not need the weights happens BEFORE the barrier, while the score side
+        // is still working: pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd)
+        // coordinates, the raw registers take the chunk after next (see the score side), and all 32
+        // table lookups of the chunk are issued.  After the barrier only the weights are read and
+        // the eight MFMAs run back to back.
+        uint32_t wv[4][4];    // step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
         uint32_t xe[4], xo[4];
-        // pairs of tokens (2p, 2p+1) of this lane's eight -> bytes of (even | odd) coordinates; then
-        // the raw registers take the chunk after next (see the score side)
         auto regroup = [&](mf_vraw& r, int c) {
 #pragma unroll
           for (int p = 0; p < 4; ++p) {
@@ -507,13 +511,20 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
           }
           __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
-          load_chunk(r, c + 2);
+          load_chunk(r, c + 1);                // a whole chunk period ahead of its use
           __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int n = 0; n < 4; ++n)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? xo[p] : xe[p], MF_SEL(n >> 1));
         };
         auto consume = [&](int c, const uint32_t par) {
-          uint32_t w[2][4];
+          // second half of the lookups: in flight while the weights arrive and the first four MFMAs run
+          uint32_t wl[4][4];
 #pragma unroll
-          for (int p = 0; p < 4; ++p) w[0][p] = mf_lut(lane4v, xe[p], MF_SEL(0));
+          for (int n = 4; n < 8; ++n)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) wl[n - 4][p] = mf_lut(lane4v, (n & 1) ? xo[p] : xe[p], MF_SEL(n >> 1));
           union { half8 h; mf_u32x4 u; } cv;
           cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par);
           const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + MF_XBUF * par));
@@ -523,40 +534,21 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 #pragma unroll
               for (int i = 0; i < 4; ++i) o[j][i] *= resc;
           }
-          // 8 steps: step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
 #pragma unroll
-          for (int n = 0; n < 8; ++n) {
-            if (n + 1 < 8) {
-              const int n1 = n + 1;
+          for (int n = 0; n < 4; ++n)
+            o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cv.h, o[n], 0, 0, 0);
 #pragma unroll
-              for (int p = 0; p < 4; ++p) w[n1 & 1][p] = mf_lut(lane4v, (n1 & 1) ? xo[p] : xe[p], MF_SEL(n1 >> 1));
-            }
-            o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(w[n & 1][0], w[n & 1][1], w[n & 1][2], w[n & 1][3]),
-                                                          cv.h, o[n], 0, 0, 0);
-          }
+          for (int n = 4; n < 8; ++n)
+            o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wl[n - 4][0], wl[n - 4][1], wl[n - 4][2], wl[n - 4][3]), cv.h, o[n], 0, 0, 0);
         };
 
-        mf_vraw ra, rb;
-        if (nchunks > 0) {
-          load_chunk(ra, 0);
-          __builtin_amdgcn_sched_barrier(0);   // queue order = chunk order, as in the loop
-          load_chunk(rb, 1);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        int c = 0;
-        for (; c + 1 < nchunks; c += 2) {
+        mf_vraw ra;
+        if (nchunks > 0) load_chunk(ra, 0);
+        for (int c = 0; c < nchunks; ++c) {
           if (c - win_c0 >= MF_WIN) load_window(c);
           regroup(ra, c);
           mf_barrier();
-          consume(c, 0);
-          regroup(rb, c + 1);
-          mf_barrier();
-          consume(c + 1, 1);
-        }
-        if (c < nchunks) {      // odd tail, already in ra
-          regroup(ra, c);
-          mf_barrier();
-          consume(c, 0);
+          consume(c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         mf_barrier();

@@ -116,13 +116,6 @@ int akv_prepare_rotation_mfma(const float* rotation, int d, void* prep, hipStrea
 // ----------------------------------------------------------------------------------
 // encode kernel
 // ----------------------------------------------------------------------------------
-#ifdef EM_STAMP
-__device__ unsigned long long em_stamps[64 * 16 * 8];
-extern "C" int akv_debug_enc_stamps(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(em_stamps), sizeof(em_stamps)); }
-#define EM_ST(k) do { if (blockIdx.x == 7 && stepno < 16) { unsigned long long t_; asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_) :: "memory"); if (lane == 0) em_stamps[(wave * 16 + stepno) * 8 + (k)] = t_; } } while (0)
-#else
-#define EM_ST(k) do { } while (0)
-#endif
 typedef uint32_t em_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t em_u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) em_u32x4 em_lds_u128;
@@ -239,14 +232,10 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     }
   };
 
-  int stepno = 0;
-  (void)stepno;
   auto encode_step = [&](auto linear_tag, int64_t step) {
     constexpr bool LINEAR = decltype(linear_tag)::value;
     em_half8 A[EM_MT][4];
-    EM_ST(0);
     fetch(A, step);
-    EM_ST(1);
     const int64_t base = step * EM_ROWS;
     // ---- lane l resolves the destination of vector base + l
     if constexpr (!DIRECT) {
@@ -379,7 +368,6 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         }
       }
     }
-    EM_ST(2);
     // ---- rotate, search, pack
     uint32_t packed[EM_MT][4];
 #pragma unroll
@@ -407,12 +395,8 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         bl.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_B_OFF + 32768 + ((nt * 4 + ks) * 64 + lane) * 16);
 #pragma unroll
         for (int mt = 0; mt < EM_MT; ++mt) {
-#if defined(EM_EXP) && (EM_EXP == 2 || EM_EXP == 3)
-          acc[mt][ks] += (float)A[mt][ks][0] * (float)bh.h[0] + (float)bl.h[1];
-#else
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bh.h, acc[mt], 0, 0, 0);
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bl.h, acc[mt], 0, 0, 0);
-#endif
         }
       }
     };
@@ -427,14 +411,6 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       for (int mt = 0; mt < EM_MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) y[mt][i] = acc[mt][i] * rv[mt][i];
-#if defined(EM_EXP) && (EM_EXP == 1 || EM_EXP == 3)
-      if constexpr (true) {
-#pragma unroll
-        for (int mt = 0; mt < EM_MT; ++mt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) packed[mt][i] |= (__float_as_uint(y[mt][i]) & 15u) << sh;
-      } else
-#endif
       if constexpr (!LINEAR) {
         em_u32x2 e[EM_MT][4];
 #pragma unroll
@@ -486,7 +462,6 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     search_tile(7, accB);
-    EM_ST(3);
     // ---- store: lane (col, g) writes group col of rows 4g + i
 #pragma unroll
     for (int mt = 0; mt < EM_MT; ++mt)
@@ -515,8 +490,6 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           *(uint16_t*)(prow + 2 * col) = (uint16_t)v;
         }
       }
-    EM_ST(4);
-    ++stepno;
   };
 
   // (two wavefronts share a SIMD: one computes while the other waits for its rows)
