@@ -265,6 +265,25 @@ __device__ __forceinline__ float mf_rows_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// Pairwise hand-off between the score and the value wavefront of a head slot: two counters in LDS,
+// `ready` (chunks whose weights are written) and `done` (chunks whose weights have been read), both
+// counted from the start of the kernel.  LDS operations of a wavefront are executed in order, so a
+// counter written after the data is seen after the data.  Waiting polls the counter with a short
+// sleep; the wait is bounded (a logic error shows up as a wrong result in the tests, never as a
+// wavefront that does not finish).
+#define MF_SPIN_LIMIT (1 << 16)
+__device__ __forceinline__ void mf_wait_ge(uint32_t addr, uint32_t need) {
+  for (int spin = 0; spin < MF_SPIN_LIMIT; ++spin) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+    if ((int32_t)((uint32_t)__builtin_amdgcn_readfirstlane((int)v) - need) >= 0) return;
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+__device__ __forceinline__ void mf_publish(uint32_t addr, uint32_t value) {
+  asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(value) : "memory");
+}
+
 // workgroup barrier that orders LDS traffic only (outstanding global loads keep flying)
 __device__ __forceinline__ void mf_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -295,6 +314,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   const uint32_t pb_addr = MF_TABB + (32u * hs + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
   const uint32_t rs_addr = MF_TABB + (32u * hs + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
 
+  const uint32_t fl_addr = MF_TABB + (32u * hs + 12u) * 256u + 128u;   // ready at +0, done at +4
+  uint32_t T = 0;        // chunks of this head slot finished in earlier segments (same on both sides)
+
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
   const int per = (total + G - 1) / G;
@@ -316,8 +338,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 
     for (int hbase = 0; hbase < a.KVH; hbase += MF_HEADS) {
       const int h = hbase + hs;
-      const bool active = h < a.KVH;          // inactive wavefronts only keep the barriers company
-      const int hh = active ? h : 0;
+      const bool active = h < a.KVH;
+      if (!active) continue;                  // both wavefronts of an unused head slot skip the pass
+      const int hh = h;
 
       // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment.
       // A window of 64 ids serves MF_WIN chunks plus the two-chunk lookahead of the prefetch.  Its
@@ -445,8 +468,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           const float resc_out = col < 8 ? resc : resc_left;
           union { half8 h; mf_u32x4 u; } cv;
           cv.h = pbv;
+          // the buffer was last read for chunk c - 2 (or, for the first two chunks, in the previous segment)
+          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T);
           *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + MF_XBUF * par) = __float_as_uint(resc_out);
+          mf_publish(fl_addr, T + (uint32_t)c + 1u);
         };
 
         mf_kraw ra, rb;
@@ -462,16 +488,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         for (; c + 1 < nchunks; c += 2) {
           if (c - win_c0 >= MF_WIN) load_window(c);
           produce(ra, c, 0);
-          mf_barrier();
           produce(rb, c + 1, 1);
-          mf_barrier();
         }
-        if (c < nchunks) {      // odd tail, already in ra
-          produce(ra, c, 0);
-          mf_barrier();
-        }
+        if (c < nchunks) produce(ra, c, 0);      // odd tail, already in ra
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
-        mf_barrier();   // value side done with the buffers
+        T += (uint32_t)nchunks;
         float lsum = l_run;
         lsum = mf_rows_sum(lsum);
         if (active && col < gqa && g == 0) {
@@ -528,6 +549,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           union { half8 h; mf_u32x4 u; } cv;
           cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par);
           const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + MF_XBUF * par));
+          mf_publish(fl_addr + 4u, T + (uint32_t)c + 1u);     // queued behind the two reads
           if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -547,11 +569,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         for (int c = 0; c < nchunks; ++c) {
           if (c - win_c0 >= MF_WIN) load_window(c);
           regroup(ra, c);
-          mf_barrier();
+          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
           consume(c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
-        mf_barrier();
+        T += (uint32_t)nchunks;
         // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + j
         const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
 #pragma unroll
@@ -585,6 +607,7 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma4_kernel(akv_attn_arg
     for (int i = threadIdx.x; i < 256 * 32; i += MF_THREADS)         // table B, first halves
       l32[16384 + (i >> 5) * 64 + (i & 31)] = x.lut[MF_W_KLO + (i >> 5)];
   }
+  if (threadIdx.x < 8) *(uint2*)(lds_raw + MF_TABB + (32u * threadIdx.x + 12u) * 256u + 128u) = make_uint2(0u, 0u);
   __syncthreads();
   if ((wave >> 3) == 0) mf_role_main<0>(a, x, wave & 7);
   else mf_role_main<1>(a, x, wave & 7);
