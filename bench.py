@@ -141,6 +141,17 @@ def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds):
     res["kernel_mvec_s"] = n / kms / 1e3
     res["kernel_gbs"] = n * 324 / kms / 1e6
     res["kernel_frac_hbm"] = res["kernel_gbs"] / HBM_PEAK_GBS
+    # decode of the same vectors (68 B in, 256 B out per vector)
+    coded = [tq.encode(v) for v in xs]
+
+    def dec_step():
+        pk, nr = coded[st["i"] & 1]
+        tq.decode(pk, nr)
+        st["i"] += 1
+    dms = timed(torch, dec_step, max(6, steps // 5), 4)
+    res["decode_mvec_s"] = n / dms / 1e3
+    res["decode_gbs"] = n * 324 / dms / 1e6
+    del coded
     if cpu:
         from oracle import tq_oracle as O
         R = tq.rotation.cpu().numpy()
