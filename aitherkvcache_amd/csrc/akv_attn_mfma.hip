@@ -450,24 +450,33 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
           m_run = m_new;
           float psum = 0.f;
-          half8 pbv;
           union { mf_u32x4 u[2]; float f[8]; } vn;
           vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u);
           vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u + 64u);
+          float pw[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);    // 0 for masked tokens
             psum += p;
-            const float pw = p * vn.f[i];
-            const float hi = __half2float(__float2half_rn(pw));
-            const float lo_left = mf_from_lo_cols(pw - hi);           // columns [8,16) take the remainder
-            pbv[i] = (_Float16)(col < 8 ? hi : lo_left);
+            pw[i] = p * vn.f[i];
+          }
+          // weights as float16 hi + lo, two at a time: hi = pw truncated to float16, lo = pw - hi (exact
+          // in float32, then truncated); columns [0,8) keep hi, columns [8,16) take the lo pair of the
+          // column eight to their left (one row shift per packed pair)
+          union { mf_u32x4 u; uint32_t w[4]; } cv;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q], pw[2 * q + 1]);
+            auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q] - (float)h2[0], pw[2 * q + 1] - (float)h2[1]);
+            union { decltype(h2) h; uint32_t u; } hb, lb;
+            hb.h = h2;
+            lb.h = l2;
+            const uint32_t lo_left = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)lb.u, 0x118 /*row_shr:8*/, 0xf, 0xf, true);
+            cv.w[q] = col < 8 ? hb.u : lo_left;
           }
           l_run = l_run * resc + psum;
           const float resc_left = mf_from_lo_cols(resc);
           const float resc_out = col < 8 ? resc : resc_left;
-          union { half8 h; mf_u32x4 u; } cv;
-          cv.h = pbv;
           // the buffer was last read for chunk c - 2 (or, for the first two chunks, in the previous segment)
           mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T);
           *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
