@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     float acc[DPL];
 #pragma unroll
     for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
-#pragma unroll 4
+#pragma unroll 8
     for (int w = w_lo; w <= w_hi; ++w) {
       const size_t slot = (size_t)(w + s) * QH + h;
       const float ms = part_ml[slot * 2];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     for (int q = 0; q < 2; ++q)
 #pragma unroll
       for (int i = 0; i < JP; ++i) o[q][i] = 0.f;
-#pragma unroll 16
+#pragma unroll 64
     for (int k = 0; k < D; ++k) {
       const float a0v = a_lds[2 * pr][k], a1v = a_lds[2 * pr + 1][k];
 #pragma unroll

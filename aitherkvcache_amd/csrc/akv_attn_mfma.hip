@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     float part[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) part[q] = 0.f;
-#pragma unroll 16
+#pragma unroll
     for (int jj = 0; jj < 64; ++jj) {
       const int j = half * 64 + jj;
       const float pv = PiT[j * 128 + dim];
