@@ -83,7 +83,8 @@ __global__ void akv_prepare_rotation_kernel(const float* __restrict__ R, float* 
 
 int akv_prepare_rotation_mfma(const float* rotation, int d, void* prep, hipStream_t stream);
 int akv_prepare_decode_mfma(const float* rotation, int d, void* prep, hipStream_t stream);
-int akv_decode_mfma_try(const akv_gen_args& a, int d, int bits, int out_dtype, const void* rot_prep, hipStream_t stream);
+int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int out_dtype, const void* rot_prep,
+                        hipStream_t stream);
 
 extern "C" size_t akv_rotation_prepared_bytes(int d) { return akv_prep_floats(d) * sizeof(float); }
 
@@ -333,7 +334,21 @@ __global__ __launch_bounds__(256) void akv_encode_general_kernel(akv_gen_args a)
   }
 }
 
-template <int D, int BITS, int ODT>
+// Row n of a block-wise decode is (listed block n / (block_size*heads), position, head); false
+// when the listed block id is outside the cache.  Offsets: packed in bytes, norms / output in elements.
+__device__ __forceinline__ bool akv_block_row(const akv_gen_args& a, int64_t n, int64_t& po, int64_t& no, int64_t& oo) {
+  const int64_t per_blk = (int64_t)a.block_size * a.heads;
+  const int64_t li = n / per_blk, rem = n - li * per_blk;
+  const int64_t pos = rem / a.heads, head = rem - pos * a.heads;
+  const int64_t blk = akv_load_index(a.slots, a.slot_itype, li);
+  if (blk < 0 || blk >= a.max_blocks) return false;
+  po = blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+  no = blk * a.ns0 + pos * a.ns1 + head * a.ns2;
+  oo = blk * a.os0 + pos * a.os1 + head * a.os2;
+  return true;
+}
+
+template <int D, int BITS, int ODT, bool BLOCKS>
 __global__ __launch_bounds__(256) void akv_decode_general_kernel(akv_gen_args a) {
   constexpr int DPL = D / 64;
   constexpr int KT = akv_gen_cfg<D>::KT;
@@ -357,14 +372,24 @@ __global__ __launch_bounds__(256) void akv_decode_general_kernel(akv_gen_args a)
 
   for (int64_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
     const int64_t base = tile * tile_vecs + wave * AKV_GEN_VPW;
+    bool live[AKV_GEN_VPW];
+    int64_t noff[AKV_GEN_VPW], ooff[AKV_GEN_VPW];
 #pragma unroll
     for (int v = 0; v < AKV_GEN_VPW; ++v) {
       const int64_t n = base + v;
-      const uint8_t* prow = a.packed + (n < a.n ? n : 0) * a.ps0;
+      int64_t poff = 0;
+      live[v] = n < a.n;
+      if constexpr (BLOCKS) {
+        noff[v] = ooff[v] = 0;
+        if (live[v]) live[v] = akv_block_row(a, n, poff, noff[v], ooff[v]);
+      } else {
+        poff = (live[v] ? n : 0) * a.ps0; noff[v] = n; ooff[v] = n * a.os0;
+      }
+      const uint8_t* prow = a.packed + poff;
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         float val = 0.f;
-        if (n < a.n) {
+        if (live[v]) {
           const uint32_t c = akv_stream_code<BITS>(lane * DPL + i, [&](int o) { return (uint32_t)prow[o]; });
           val = cen[c];
         }
@@ -390,12 +415,11 @@ __global__ __launch_bounds__(256) void akv_decode_general_kernel(akv_gen_args a)
     }
 #pragma unroll
     for (int v = 0; v < AKV_GEN_VPW; ++v) {
-      const int64_t n = base + v;
-      if (n >= a.n) continue;
-      const float nv = a.norms[n];
+      if (!live[v]) continue;
+      const float nv = a.norms[noff[v]];
 #pragma unroll
       for (int i = 0; i < DPL; ++i)
-        akv_elem<ODT>::store(a.out, n * a.os0 + lane * DPL + i, acc[v][i] * nv);
+        akv_elem<ODT>::store(a.out, ooff[v] + lane * DPL + i, acc[v][i] * nv);
     }
     __syncthreads();
   }
@@ -503,14 +527,25 @@ extern "C" int akv_encode_paged(const void* x, int x_dtype, int64_t num_tokens, 
   return akv_encode_dispatch<true>(d, bits, x_dtype, a, stream);
 }
 
-template <int D, int BITS>
+template <int D, int BITS, bool BLOCKS>
 static int akv_decode_dispatch_dtype(int dt, const akv_gen_args& a, void* stream) {
   const size_t lds = akv_gen_cfg<D>::lds_bytes;
   switch (dt) {
-    case AKV_F16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F16>, "akv_decode_general_kernel", lds, a, stream);
-    case AKV_BF16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_BF16>, "akv_decode_general_kernel", lds, a, stream);
-    default: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F32>, "akv_decode_general_kernel", lds, a, stream);
+    case AKV_F16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F16, BLOCKS>, "akv_decode_general_kernel", lds, a, stream);
+    case AKV_BF16: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_BF16, BLOCKS>, "akv_decode_general_kernel", lds, a, stream);
+    default: return akv_launch_gen(akv_decode_general_kernel<D, BITS, AKV_F32, BLOCKS>, "akv_decode_general_kernel", lds, a, stream);
   }
+}
+
+template <bool BLOCKS>
+static int akv_decode_dispatch(int d, int bits, int out_dtype, const akv_gen_args& a, void* stream) {
+#define AKV_CASE(DD, BB) \
+  if (d == DD && bits == BB) return akv_decode_dispatch_dtype<DD, BB, BLOCKS>(out_dtype, a, stream);
+  AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
+  AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
+  AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+#undef AKV_CASE
+  return akv_fail(AKV_ERR_UNSUPPORTED, "decode: no kernel for head_dim=%d bits=%d", d, bits);
 }
 
 extern "C" int akv_decode(const uint8_t* packed, int64_t packed_stride, const float* norms,
@@ -530,13 +565,36 @@ extern "C" int akv_decode(const uint8_t* packed, int64_t packed_stride, const fl
   a.packed = const_cast<uint8_t*>(packed); a.ps0 = packed_stride;
   a.norms = const_cast<float*>(norms);
   a.out = out; a.os0 = out_stride;
-  rc = akv_decode_mfma_try(a, d, bits, out_dtype, rot_prep, (hipStream_t)stream);
+  rc = akv_decode_mfma_try(a, false, d, bits, out_dtype, rot_prep, (hipStream_t)stream);
   if (rc != AKV_ERR_UNSUPPORTED) return rc;
-#define AKV_CASE(DD, BB) \
-  if (d == DD && bits == BB) return akv_decode_dispatch_dtype<DD, BB>(out_dtype, a, stream);
-  AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
-  AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
-  AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
-#undef AKV_CASE
-  return akv_fail(AKV_ERR_UNSUPPORTED, "decode: no kernel for head_dim=%d bits=%d", d, bits);
+  return akv_decode_dispatch<false>(d, bits, out_dtype, a, stream);
+}
+
+// Decode of whole cache blocks in place of the reference's gather + decode + scatter
+// (aither_kvcache/vllm/backend.py:1040-1091): every block id in `block_ids` that lies in
+// [0, num_blocks) is decoded from the packed cache into the block of the same index of `out`.
+extern "C" int akv_decode_blocks(const uint8_t* packed, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                                 const float* norms, int64_t ns_blk, int64_t ns_pos, int64_t ns_head,
+                                 const void* block_ids, int ids_itype, int64_t num_ids, int64_t num_blocks,
+                                 int block_size, int num_kv_heads, int d, const void* rot_prep,
+                                 const float* centroids, int bits, void* out, int out_dtype, int64_t os_blk,
+                                 int64_t os_pos, int64_t os_head, void* stream) {
+  AKV_REQUIRE(num_ids >= 0 && num_blocks >= 0 && block_size > 0 && num_kv_heads > 0, "akv_decode_blocks: bad sizes");
+  AKV_REQUIRE(akv_valid_dtype(out_dtype) && akv_valid_itype(ids_itype), "akv_decode_blocks: bad dtype");
+  int rc = akv_check_codec_args("akv_decode_blocks", d, bits);
+  if (rc) return rc;
+  if (num_ids == 0 || num_blocks == 0) return AKV_OK;
+  AKV_REQUIRE(packed && norms && block_ids && rot_prep && centroids && out, "akv_decode_blocks: null pointer");
+  akv_gen_args a = {};
+  a.n = num_ids * block_size * num_kv_heads;
+  a.heads = num_kv_heads; a.block_size = block_size; a.max_blocks = num_blocks;
+  a.slots = block_ids; a.slot_itype = ids_itype;
+  a.mat = (const float*)rot_prep;
+  a.table = centroids;
+  a.packed = const_cast<uint8_t*>(packed); a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
+  a.norms = const_cast<float*>(norms); a.ns0 = ns_blk; a.ns1 = ns_pos; a.ns2 = ns_head;
+  a.out = out; a.os0 = os_blk; a.os1 = os_pos; a.os2 = os_head;
+  rc = akv_decode_mfma_try(a, true, d, bits, out_dtype, rot_prep, (hipStream_t)stream);
+  if (rc != AKV_ERR_UNSUPPORTED) return rc;
+  return akv_decode_dispatch<true>(d, bits, out_dtype, a, stream);
 }

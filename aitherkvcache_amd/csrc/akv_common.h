@@ -82,7 +82,7 @@ struct akv_gen_args {
   int64_t ns0, ns1, ns2;
   // decode output
   void* out;
-  int64_t os0;
+  int64_t os0, os1, os2;  // flat: os0 = row stride; block-wise decode: blk, pos, head strides (elements)
 };
 
 // ----------------------------------------------------------------------------------

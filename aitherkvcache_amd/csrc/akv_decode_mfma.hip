@@ -31,7 +31,8 @@ typedef __attribute__((address_space(3))) const uint32_t dm_lds_cu32;
 #define DM_PSCALE 64.f
 #define DM_LUT_OFF 0                 // 256 entries x 256 B: [hi pair x 32 copies][lo pair x 32 copies]
 #define DM_B_OFF 65536               // [hi/lo][8 nt][4 ks][64 lanes] x 16 B
-#define DM_LDS_BYTES (131072)
+#define DM_ROW_OFF 131072            // per wavefront: DM_ROWS x {packed offset, norm offset, output offset} (block-wise decode)
+#define DM_LDS_BYTES (131072 + DM_WAVES * DM_ROWS * 24)
 #define DM_SEL(k) (0x0c0c0400u + ((uint32_t)(k) << 8))
 
 // B operand of the decode kernel, stored after the encode operand in the prepared-rotation buffer
@@ -66,6 +67,11 @@ int akv_prepare_decode_mfma(const float* rotation, int d, void* prep, hipStream_
   return AKV_OK;
 }
 
+// BLOCKS = false: n contiguous rows (TurboQuant.decode).  BLOCKS = true: the rows are the
+// (position, head) entries of the cache blocks listed in a.slots; every listed block that exists is
+// decoded into the block of the same index of the output buffer (the batch decompress of
+// aither_kvcache/vllm/backend.py:1040-1091 without its gather / unique / scatter passes).
+template <bool BLOCKS>
 __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
@@ -102,15 +108,46 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
     // ---- packed rows and norms
     uint4 pk[2];
     float4 nr[2];
+    int64_t* row_p = (int64_t*)(lds + DM_ROW_OFF + wave * DM_ROWS * 24);   // packed byte offset, or -1
+    int64_t* row_n = row_p + DM_ROWS;                                      // norm element offset
+    int64_t* row_o = row_n + DM_ROWS;                                      // output element offset
+    if constexpr (BLOCKS) {
+      if (lane < DM_ROWS) {   // lane l resolves row base + l = (listed block, position, head)
+        const int64_t n = base + lane;
+        int64_t po = -1, no = 0, oo = 0;
+        if (n < a.n) {
+          const int64_t per_blk = (int64_t)a.block_size * a.heads;
+          const int64_t li = n / per_blk, rem = n - li * per_blk;
+          const int64_t pos = rem / a.heads, head = rem - pos * a.heads;
+          const int64_t blk = akv_load_index(a.slots, a.slot_itype, li);
+          if (blk >= 0 && blk < a.max_blocks) {
+            po = blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+            no = blk * a.ns0 + pos * a.ns1 + head * a.ns2;
+            oo = blk * a.os0 + pos * a.os1 + head * a.os2;
+          }
+        }
+        row_p[lane] = po; row_n[lane] = no; row_o[lane] = oo;
+      }
+    }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
-      const int64_t n = base + 16 * mt + (lane & 15);
-      pk[mt] = n < a.n ? *(const uint4*)(a.packed + n * a.ps0 + 16 * g) : make_uint4(0, 0, 0, 0);
       float nv[4];
+      if constexpr (BLOCKS) {
+        const int64_t po = row_p[16 * mt + (lane & 15)];
+        pk[mt] = po >= 0 ? *(const uint4*)(a.packed + po + 16 * g) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int64_t r = base + 16 * mt + 4 * g + i;
-        nv[i] = r < a.n ? a.norms[r] : 0.f;
+        for (int i = 0; i < 4; ++i) {
+          const int r = 16 * mt + 4 * g + i;
+          nv[i] = row_p[r] >= 0 ? a.norms[row_n[r]] : 0.f;
+        }
+      } else {
+        const int64_t n = base + 16 * mt + (lane & 15);
+        pk[mt] = n < a.n ? *(const uint4*)(a.packed + n * a.ps0 + 16 * g) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int64_t r = base + 16 * mt + 4 * g + i;
+          nv[i] = r < a.n ? a.norms[r] : 0.f;
+        }
       }
       nr[mt] = make_float4(nv[0], nv[1], nv[2], nv[3]);
     }
@@ -159,8 +196,16 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
       const float nv[4] = {nr[mt].x, nr[mt].y, nr[mt].z, nr[mt].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int64_t r = base + 16 * mt + 4 * g + i;
-        if (r >= a.n) continue;
+        __half* orow;
+        if constexpr (BLOCKS) {
+          const int r = 16 * mt + 4 * g + i;
+          if (row_p[r] < 0) continue;
+          orow = (__half*)a.out + row_o[r];
+        } else {
+          const int64_t r = base + 16 * mt + 4 * g + i;
+          if (r >= a.n) continue;
+          orow = (__half*)a.out + r * a.os0;
+        }
         union { dm_half8 h; uint4 u; } o;
 #pragma unroll
         for (int nt = 0; nt < 8; ++nt) {
@@ -168,7 +213,7 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
           const float v = __fmul_rn(acc[mt][nt][i] * (1.f / DM_PSCALE), nv[i]);
           o.h[nt] = (_Float16)v;
         }
-        *(uint4*)((__half*)a.out + r * a.os0 + 8 * col) = o.u;
+        *(uint4*)(orow + 8 * col) = o.u;
       }
     }
   }
@@ -184,19 +229,24 @@ static bool dm_disabled() {
 }
 
 // returns AKV_ERR_UNSUPPORTED when the fast path does not apply (the caller then uses the general kernel)
-int akv_decode_mfma_try(const akv_gen_args& a, int d, int bits, int out_dtype, const void* rot_prep, hipStream_t stream) {
+int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int out_dtype, const void* rot_prep,
+                        hipStream_t stream) {
   if (dm_disabled() || d != 128 || bits != 4 || out_dtype != AKV_F16) return AKV_ERR_UNSUPPORTED;
-  if ((((uintptr_t)a.packed | (uintptr_t)a.ps0) & 15) || (((uintptr_t)a.out) & 15) || (a.os0 & 7)) return AKV_ERR_UNSUPPORTED;
+  if (((uintptr_t)a.packed | (uintptr_t)a.ps0 | (uintptr_t)a.out) & 15) return AKV_ERR_UNSUPPORTED;
+  if (a.os0 & 7) return AKV_ERR_UNSUPPORTED;
+  if (blocks && (((uintptr_t)a.ps1 | (uintptr_t)a.ps2) & 15 || ((a.os1 | a.os2) & 7))) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(d));
   const int64_t steps = (a.n + DM_ROWS - 1) / DM_ROWS;
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
   static bool configured = false;
   if (!configured) {
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));
     configured = true;
   }
   akv_profile_mark_begin(stream);
-  akv_decode_mfma_kernel<<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);
+  if (blocks) akv_decode_mfma_kernel<true><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);
+  else akv_decode_mfma_kernel<false><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_decode_mfma_kernel");
   return AKV_OK;

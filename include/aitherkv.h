@@ -118,6 +118,26 @@ int akv_decode(const uint8_t* packed, int64_t packed_stride, const float* norms,
                void* out, int out_dtype, int64_t out_stride, void* stream);
 
 /* ---------------------------------------------------------------------------------
+ * TurboQuantImpl._batch_decompress_active_blocks -- aither_kvcache/vllm/backend.py:1040-1091
+ * (unique block ids -> gather packed rows and norms -> TurboQuant.decode -> scatter), as
+ * one pass with no gather, unique or scatter step: for every i < num_ids whose
+ * b = block_ids[i] lies in [0, num_blocks), all block_size * num_kv_heads rows of cache
+ * block b are decoded into block b of `out`.  Ids outside the cache are skipped (the
+ * reference filters them, :1063); an id listed twice writes the same values twice.
+ *   packed  [num_blocks][block_size][num_kv_heads][>= packed bytes], byte strides ps_*
+ *   norms   [num_blocks][block_size][num_kv_heads] float32, element strides ns_*
+ *   out     [num_blocks][block_size][num_kv_heads][d], element strides os_*, last dim contiguous
+ * block_ids may be the flattened block table itself (padding entries negative).
+ * ------------------------------------------------------------------------------- */
+int akv_decode_blocks(const uint8_t* packed, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                      const float* norms, int64_t ns_blk, int64_t ns_pos, int64_t ns_head,
+                      const void* block_ids, int ids_itype, int64_t num_ids, int64_t num_blocks,
+                      int block_size, int num_kv_heads, int d,
+                      const void* rot_prep, const float* centroids, int bits,
+                      void* out, int out_dtype, int64_t os_blk, int64_t os_pos, int64_t os_head,
+                      void* stream);
+
+/* ---------------------------------------------------------------------------------
  * TQPagedAttention.forward -- aither_kvcache/fused_attention.py:594-748, with the result
  * of TQPagedAttentionRef.forward (:91-185).  The query pre-rotation (:659) and the output
  * inverse rotation (:747) are done inside.

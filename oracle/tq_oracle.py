@@ -13,6 +13,8 @@ reference tree).  How each one is pinned:
   in tests/test_oracle_*.py:
       get_codebook, pack_*/unpack_*, pack_multibit/unpack_multibit,
       encode, decode, kv_update, paged_attention_loop, paged_attention,
+      batch_decompress_active_blocks (its decode by the golden vectors; its block
+      selection and scatter by a per-block loop in tests/test_oracle_pins.py),
       fwht, structured_hadamard, dimension_aware_codebook,
       hybrid_encode, hybrid_decode, rope_frequencies, spectral_encode,
       tri_scores, tri_decode_step
@@ -197,6 +199,24 @@ def decode(packed, norms, rotation, centroids, bits, out_dtype=np.float16):
     y_hat = np.asarray(centroids, dtype=f32)[idx.astype(np.int64)]
     x_hat = (y_hat @ rotation.astype(f32)) * norms.reshape(-1).astype(f32)[:, None]
     return x_hat.reshape(batch + (D,)).astype(out_dtype)
+
+
+def batch_decompress_active_blocks(cache, norms, buf, block_table, num_blocks, rotation, centroids,
+                                   bits, packed_dim):
+    """One of the two (K, V) halves of TurboQuantImpl._batch_decompress_active_blocks,
+    vllm/backend.py:1040-1091: unique ids of the block table inside [0, num_blocks) (:1061-1063),
+    gather packed[:, :, :, :packed_dim] and norms (:1069-1075), one flat decode (:1083-1087),
+    scatter into buf with a cast to its dtype (:1090-1091).  buf is written in place; blocks
+    not listed keep their contents."""
+    active = np.unique(np.asarray(block_table).reshape(-1))
+    active = active[(active >= 0) & (active < num_blocks)]
+    if active.size == 0:
+        return
+    A, (bs, H) = active.shape[0], cache.shape[1:3]
+    flat_p = cache[active][:, :, :, :packed_dim].reshape(A * bs * H, packed_dim)
+    flat_n = norms[active].reshape(A * bs * H)
+    dec = decode(flat_p, flat_n, rotation, centroids, bits)       # float16, as tq.decode returns
+    buf[active] = dec.reshape(A, bs, H, -1).astype(buf.dtype)
 
 
 # --------------------------------------------------------------------------------------

@@ -236,6 +236,64 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+@pytest.mark.parametrize("bits,out_dtype,extra", [(4, torch.float16, 0), (4, torch.float16, 16), (4, torch.bfloat16, 0),
+                                                  (3, torch.float16, 0), (2, torch.float32, 4)])
+@pytest.mark.parametrize("itype", [torch.int32, torch.int64])
+def test_batch_decompress_active_blocks_vs_oracle(golden, dev, bits, out_dtype, extra, itype):
+    from aitherkvcache_amd.vllm import batch_decompress_active_blocks
+    tq = make_tq(golden, dev, bits)
+    R = golden["rotation_d128_seed42"]
+    c, b, _ = O.get_codebook(128, bits)
+    rng = np.random.default_rng(bits * 10 + extra)
+    B, bs, H, pd = 23, 16, 3, tq._packed_dim
+    caches, norms = [], []
+    for _ in range(2):
+        p, n = O.encode(kv_like(rng, (B, bs, H, 128)), R, b, bits)
+        caches.append(np.concatenate([p, rng.integers(0, 256, (B, bs, H, extra), dtype=np.uint8)], axis=-1))
+        norms.append(n)
+    table = np.full((5, 6), -1, dtype=np.int64)
+    table[0, :3] = [4, 9, 2]
+    table[1, :6] = [9, 21, 22, 0, 17, 30]          # 9 shared; 21, 22 and 30 are outside num_blocks
+    table[3, :1] = [20]
+    num_blocks = 21
+    ref = [np.full((B, bs, H, 128), 3.0, dtype=np.float32) for _ in range(2)]
+    for i in range(2):
+        O.batch_decompress_active_blocks(caches[i], norms[i], ref[i], table, num_blocks, R, c, bits, pd)
+    bufs = [torch.full((B, bs, H, 128), 3.0, dtype=out_dtype, device=dev) for _ in range(2)]
+    batch_decompress_active_blocks(
+        torch.from_numpy(caches[0]).to(dev), torch.from_numpy(caches[1]).to(dev), bufs[0], bufs[1], tq, pd,
+        torch.from_numpy(table).to(dev).to(itype), num_blocks,
+        torch.from_numpy(norms[0]).to(dev), torch.from_numpy(norms[1]).to(dev))
+    touched = np.zeros(B, dtype=bool)
+    touched[[0, 2, 4, 9, 17, 20]] = True
+    for i in range(2):
+        got = bufs[i].float().cpu().numpy()
+        assert np.all(got[~touched] == 3.0)                       # unlisted blocks untouched
+        # the oracle rounds to float16 as tq.decode does: allow half an ulp of the coarser of the two formats
+        rel = {torch.float16: 0.0, torch.bfloat16: 2.0 ** -8, torch.float32: 2.0 ** -11}[out_dtype]
+        tol = 2e-3 + np.abs(ref[i][touched]) * rel
+        assert np.all(np.abs(got[touched] - ref[i][touched]) <= tol)
+        if out_dtype == torch.float16:
+            assert np.mean(got[touched] == ref[i][touched]) > 0.995
+
+
+def test_batch_decompress_empty_and_errors(golden, dev):
+    from aitherkvcache_amd.vllm import decode_blocks
+    tq = make_tq(golden, dev, 4)
+    cache = torch.zeros(4, 16, 2, 64, dtype=torch.uint8, device=dev)
+    norms = torch.ones(4, 16, 2, device=dev)
+    buf = torch.full((4, 16, 2, 128), 5.0, dtype=torch.float16, device=dev)
+    decode_blocks(cache, norms, buf, tq, torch.empty(0, dtype=torch.int64, device=dev), 4)
+    decode_blocks(cache, norms, buf, tq, torch.tensor([-1, 7], device=dev), 4)
+    assert torch.all(buf == 5.0)
+    with pytest.raises(ValueError):
+        decode_blocks(cache, norms, buf, tq, torch.tensor([0], device=dev), 5)
+    with pytest.raises(ValueError):
+        decode_blocks(cache[..., :32], norms, buf, tq, torch.tensor([0], device=dev), 4)
+    with pytest.raises(RuntimeError):
+        decode_blocks(cache.cpu(), norms.cpu(), buf.cpu(), tq, torch.tensor([0]), 4)
+
+
 def test_config0_round_trip_full_size(golden, dev):
     """65,536 x 128 fp16, 4-bit: every code accounted for, distortion at the table value."""
     tq = make_tq(golden, dev, 4)

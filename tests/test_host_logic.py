@@ -46,7 +46,7 @@ def test_library_exports_every_declared_symbol():
 def test_library_loads_and_reports_version():
     L = _lib.lib()
     assert b"aitherkv" in L.akv_version()
-    assert L.akv_rotation_prepared_bytes(128) == 4 * 128 * 128 * 4
+    assert L.akv_rotation_prepared_bytes(128) >= 4 * 128 * 128 * 4      # four d x d float32 planes + tables
     # argument validation happens before any device work
     rc = L.akv_encode(None, 0, -1, 128, 128, None, None, 4, None, 64, None, None)
     assert rc == _lib.AKV_ERR_INVALID and b"akv_encode" in L.akv_last_error()

@@ -165,6 +165,28 @@ def test_paged_attention_equals_decompress_then_dense(golden, bits):
 
 
 # ---- hybrid ------------------------------------------------------------------------------
+def test_batch_decompress_touches_exactly_the_listed_blocks(golden):
+    # per-block loop: a listed block inside the cache equals decode() of that block alone, every
+    # other block of the buffer keeps its sentinel; duplicates, negatives and ids past the cache
+    rng = np.random.default_rng(5)
+    R = golden["rotation_d128_seed42"]
+    c, b, _ = O.get_codebook(128, 4)
+    B, bs, H = 12, 4, 2
+    x = rng.standard_normal((B, bs, H, 128)).astype(np.float32)
+    packed, norms = O.encode(x, R, b, 4)
+    cache = np.concatenate([packed, rng.integers(0, 256, (B, bs, H, 8), dtype=np.uint8)], axis=-1)
+    table = np.array([[3, 7, -1, -1], [7, 0, 11, 10], [9, 40, -1, -1]])
+    num_blocks = 10                                     # 10, 11 and 40 are outside the cache
+    buf = np.full((B, bs, H, 128), 77, dtype=np.float16)
+    O.batch_decompress_active_blocks(cache, norms, buf, table, num_blocks, R, c, 4, 64)
+    for blk in range(B):
+        if blk in (0, 3, 7, 9):
+            one = O.decode(packed[blk], norms[blk], R, c, 4).astype(np.float32)   # BLAS sums in another order
+            assert np.max(np.abs(buf[blk].astype(np.float32) - one)) <= 2e-3
+        else:
+            assert np.all(buf[blk] == 77)
+
+
 def test_fwht_is_the_hadamard_matrix():
     H = np.array([[1.0]])
     while H.shape[0] < 64:
