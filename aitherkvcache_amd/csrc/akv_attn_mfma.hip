@@ -13,10 +13,13 @@
 //
 //   scores   S^T[token, col] = sum_d Khat[token, d] * Qop[d, col]       v_mfma_f32_16x16x32_f16
 //            A = Khat: lane (n = l%16, g = l/16) owns bytes [16g, 16g+16) of token n's code row
-//            (one 16-byte load).
-//            B = Qop: the rotated, pre-scaled queries of the kv head's query heads, columns [0,8)
-//            = fp16 rounding of q', columns [8,16) = fp16 of the remainder (q' to ~22 bits at no
-//            extra MFMA).  Result: lane (col, g) holds tokens 4g..4g+3 of the tile for column col.
+//            (one 16-byte load).  The k-slice of one MFMA is two code bytes = four coordinates,
+//            each as (hi pair, lo pair): elements [hi c0, hi c1, lo c0, lo c1, hi c2, hi c3, lo c2,
+//            lo c3], exactly two 8-byte table entries side by side.
+//            B = Qop: the rotated, pre-scaled queries of the kv head's query heads with every
+//            coordinate pair repeated to face the hi and the lo half; columns [0,8) = fp16 rounding
+//            of q', columns [8,16) = fp16 of the remainder (q' to ~22 bits at no extra MFMA).
+//            Result: lane (col, g) holds tokens 4g..4g+3 of the tile for column col.
 //   softmax  running max / sum per column in the log2 domain; the weights p * |v| of a lane are
 //            exactly the k-slice of the B operand of the next product (tokens 4g..4g+3 of both
 //            tiles), again split hi / lo over columns [0,8) / [8,16).
@@ -27,13 +30,14 @@
 //
 // Dequantisation goes through tables in LDS indexed by a whole BYTE: entry (a<<4|b) is the fp16
 // pair (c[a], c[b]).  For K a byte holds two neighbouring coordinates of one token -- already a
-// k-pair; the K table carries a hi and a lo half (c = hi + lo to ~22 bits) and both go through
-// the matrix core, interleaved in one operand.  For V the k axis is the token axis, so bytes
+// k-pair; a K entry is 8 bytes, the hi pair and the lo pair (c = hi + lo to ~22 bits), fetched by
+// ONE LDS read (the LDS issues about one wavefront read per three to five cycles whatever its
+// width, so an 8-byte read costs little more than a 4-byte one).  For V the k axis is the token axis, so bytes
 // are first re-formed from the same nibble position of two neighbouring tokens (two bit-field
 // inserts per 8 codes); the V table holds fp16(alpha c) with alpha in [1,2) chosen so that the
 // sixteen levels are almost exactly representable, and alpha is divided out at the end.  Every
-// table entry is replicated 32 times (address = entry * 256 + (lane & 31) * 4): the LDS serves
-// 32 lanes per cycle, so lookups never conflict on a bank.
+// table entry is replicated 32 times (address = entry * 256 + (lane & 31) * entry size), so lookups
+// never conflict on a bank.
 #include "akv_attn_common.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -44,14 +48,10 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 #define MF_WAIT_VM0 0x0f70          // s_waitcnt vmcnt(0), other counters untouched
 #define MF_WIN 30                   // chunks served by one window of 64 block ids (even, <= 31)
 #define MF_LDS_BYTES (128 * 1024)   // two tables of 256 entries x 256 bytes
-// entry e of table A at e*256:          [fp16(alpha c) pairs for V x 32 copies][hi pairs for K x 32 copies]
-// entry e of table B at 65536 + e*256:  [lo pairs for K x 32 copies][128 bytes of exchange buffer]
-// so the lo half of a K lookup sits 65408 bytes after its hi half: reachable by the 16-bit offset of a
-// single LDS read, and impossible to fuse with the hi read into a two-address read (which would need
-// extra register moves to regroup the results for the matrix core)
+// entry e of table A at e*256:          [(hi pair, lo pair) for K x 32 copies]
+// entry e of table B at 65536 + e*256:  [fp16(alpha c) pairs for V x 32 copies][128 bytes of exchange buffer]
 #define MF_TABB 65536u
 #define MF_XBUF 4096u                // distance of the two exchange buffers of a head slot
-#define MF_KLO_DIST 65408u
 #define MF_ALPHA_CANDIDATES 65536
 // words of the table block kept in the workspace
 #define MF_W_KHI 0
@@ -65,7 +65,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 
 struct akv_mfma_extra {
   const uint32_t* lut;   // table block, MF_W_* (workspace)
-  const uint4* qop;      // [S][KVH][4 k-steps][64 lanes] half8 as uint4 (workspace)
+  const uint4* qop;      // [S][KVH][8 k-steps][64 lanes] half8 as uint4 (workspace)
 };
 
 // ----------------------------------------------------------------------------------
@@ -171,14 +171,15 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     }
   }
   __syncthreads();
-  // operand layout: [k-step st][lane (col, g)][e] = coordinate 32g + 8st + e of column col
-  {
-    const int st = tid >> 6, lane = tid & 63;
+  // operand layout: [k-step n][lane (col, g)][e] = coordinate 32g + 4n + 2(e/4) + e%2 of column col
+  // (elements 2,3 and 6,7 repeat 0,1 and 4,5: they face the lo halves of the K table entries)
+  for (int n = tid >> 6; n < 8; n += 4) {
+    const int lane = tid & 63;
     const int col = lane & 15, g = lane >> 4;
     unsigned short hbits[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int dim = 32 * g + 8 * st + e;
+      const int dim = 32 * g + 4 * n + 2 * (e >> 2) + (e & 1);
       float v = 0.f;
       if (col < 8) {
         if (col < gqa) v = __half2float(__float2half_rn(qr_lds[col][dim]));
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     uint4 o;
     o.x = hbits[0] | (hbits[1] << 16); o.y = hbits[2] | (hbits[3] << 16);
     o.z = hbits[4] | (hbits[5] << 16); o.w = hbits[6] | (hbits[7] << 16);
-    qop[((size_t)(s * KVH + h) * 4 + st) * 64 + lane] = o;
+    qop[((size_t)(s * KVH + h) * 8 + n) * 64 + lane] = o;
   }
 }
 
@@ -205,19 +206,21 @@ typedef __attribute__((address_space(3))) mf_u32x4 mf_lds_u128;
 
 // The tables are the kernel's only LDS object, so they start at LDS address 0 and a table offset
 // is the LDS address itself (saves one add per lookup).
-// address = byte k of `word` * 256 + lanebits (the copy (lane & 31) * 4, plus 128 for the K half),
-// built by one byte permute: result byte 0 <- lanebits byte 0, byte 1 <- word byte k (selector 4 + k).
-#define MF_SEL(k) (0x0c0c0400u + ((uint32_t)(k) << 8))
+// address = byte k of `word` * 256 + lanebits, built by one byte permute: result byte 0 <- lanebits
+// byte 0 (the copy: (lane & 31) * entry size), byte 1 <- word byte k (selector 4 + k), byte 2 <-
+// lanebits byte 2 (1 for the V table, which lies 65536 bytes up).
+#define MF_SEL(k) (0x0c020400u + ((uint32_t)(k) << 8))
+typedef uint32_t mf_u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const mf_u32x2 mf_lds_cu64;
 
 __device__ __forceinline__ uint32_t mf_lut(uint32_t lanebits, uint32_t word, uint32_t sel) {
   const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
   return *(mf_lds_cu32*)(uintptr_t)addr;
 }
-// hi and lo halves of a K lookup: one address, two reads
-__device__ __forceinline__ void mf_lut2(uint32_t lanebits, uint32_t word, uint32_t sel, uint32_t& hi, uint32_t& lo) {
+// K lookup: (hi pair, lo pair) of one code byte
+__device__ __forceinline__ mf_u32x2 mf_lut2(uint32_t lanebits, uint32_t word, uint32_t sel) {
   const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
-  hi = *(mf_lds_cu32*)(uintptr_t)addr;
-  lo = *(mf_lds_cu32*)(uintptr_t)(addr + MF_KLO_DIST);
+  return *(mf_lds_cu64*)(uintptr_t)addr;
 }
 
 __device__ __forceinline__ half8 mf_pack(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -304,8 +307,8 @@ template <int ROLE>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
-  const uint32_t lane4v = (uint32_t)(lane & 31) * 4u;      // V lookups: first half of table A
-  const uint32_t lane4k = lane4v + 128u;                   // K lookups: second half of table A (+ MF_KLO_DIST)
+  const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * 4u;   // V lookups: first halves of table B entries
+  const uint32_t lane4k = (uint32_t)(lane & 31) * 8u;             // K lookups: table A
   // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
   //   weights (16 B per lane): entry 16q + lane/8, offset 128 + (lane%8)*16
   //   rescale (4 B per lane):  entry 16q + 8 + lane/32, offset 128 + (lane%32)*4
@@ -339,7 +342,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
     for (int hbase = 0; hbase < a.KVH; hbase += MF_HEADS) {
       const int h = hbase + hs;
       const bool active = h < a.KVH;
-      if (!active) continue;                  // both wavefronts of an unused head slot skip the pass
+      // both wavefronts of an unused head slot skip the pass.  (A segment always has a chunk; saying so
+      // here leaves ONE path into the chunk loops: were the first loads conditional, the compiler would
+      // have to assume that the loads issued before them are the newest outstanding ones and would wait
+      // for ALL loads, prefetches included, wherever the loop first touches their registers.)
+      if (!active || nchunks <= 0) continue;
       const int hh = h;
 
       // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment.
@@ -360,15 +367,15 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
         p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
       };
-      if (nchunks > 0) load_window(0);
+      load_window(0);
 
       if constexpr (ROLE == 0) {
         // =========================== score wavefront ===========================
-        half8 qb[4];
+        half8 qb[8];
         {
-          const uint4* qp = x.qop + ((size_t)(s * a.KVH + hh) * 4) * 64 + lane;
+          const uint4* qp = x.qop + ((size_t)(s * a.KVH + hh) * 8) * 64 + lane;
 #pragma unroll
-          for (int st = 0; st < 4; ++st) {
+          for (int st = 0; st < 8; ++st) {
             const uint4 u = qp[st * 64];
             qb[st] = mf_pack(u.x, u.y, u.z, u.w);
           }
@@ -398,26 +405,26 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           *(mf_lds_u32*)(uintptr_t)(nw_addr + MF_XBUF * par) = __float_as_uint(r.nrm);
           {
             // 8 steps (tile j, dword st): 4 table reads (hi and lo of each of the dword's 4 bytes) feed
-            // two MFMAs; the reads of step n+1 are issued before the MFMAs of step n
+            // two MFMAs (bytes 0,1 and bytes 2,3); the reads of step n+2 are issued before the MFMAs of step n
             const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
-            uint32_t wh[3][4], wl[3][4];      // ring of three steps: two in flight behind the one multiplied
+            mf_u32x2 w[3][4];      // ring of three steps: two in flight behind the one multiplied
             float4v acc[2];
             acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
             acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int n = 0; n < 2; ++n)
 #pragma unroll
-              for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n], MF_SEL(b), wh[n][b], wl[n][b]);
+              for (int b = 0; b < 4; ++b) w[n][b] = mf_lut2(lane4k, kw[n], MF_SEL(b));
 #pragma unroll
             for (int n = 0; n < 8; ++n) {
               if (n + 2 < 8) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) mf_lut2(lane4k, kw[n + 2], MF_SEL(b), wh[(n + 2) % 3][b], wl[(n + 2) % 3][b]);
+                for (int b = 0; b < 4; ++b) w[(n + 2) % 3][b] = mf_lut2(lane4k, kw[n + 2], MF_SEL(b));
               }
               acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(wh[n % 3][0], wh[n % 3][1], wh[n % 3][2], wh[n % 3][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
+                  mf_pack(w[n % 3][0].x, w[n % 3][0].y, w[n % 3][1].x, w[n % 3][1].y), qb[2 * (n & 3)], acc[n >> 2], 0, 0, 0);
               acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(wl[n % 3][0], wl[n % 3][1], wl[n % 3][2], wl[n % 3][3]), qb[n & 3], acc[n >> 2], 0, 0, 0);
+                  mf_pack(w[n % 3][2].x, w[n % 3][2].y, w[n % 3][3].x, w[n % 3][3].y), qb[2 * (n & 3) + 1], acc[n >> 2], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
             load_chunk(r, c + 2);
@@ -485,12 +492,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
 
         mf_kraw ra, rb;
-        if (nchunks > 0) {
-          load_chunk(ra, 0);
-          __builtin_amdgcn_sched_barrier(0);   // queue order = chunk order, as in the loop
-          load_chunk(rb, 1);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+        __builtin_amdgcn_sched_barrier(0);     // the query operand is requested before the chunks
+        load_chunk(ra, 0);
+        __builtin_amdgcn_sched_barrier(0);     // queue order = chunk order, as in the loop
+        load_chunk(rb, 1);
+        __builtin_amdgcn_sched_barrier(0);
         // pairs of chunks with the same loads on every path (an early exit from the middle of the
         // body would make the compiler wait for the newest prefetch at the top of every iteration)
         int c = 0;
@@ -573,13 +579,16 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wl[n - 4][0], wl[n - 4][1], wl[n - 4][2], wl[n - 4][3]), cv.h, o[n], 0, 0, 0);
         };
 
+        auto step = [&](mf_vraw& r, int c, const uint32_t par) {
+          regroup(r, c);
+          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
+          consume(c, par);
+        };
         mf_vraw ra;
-        if (nchunks > 0) load_chunk(ra, 0);
+        load_chunk(ra, 0);
         for (int c = 0; c < nchunks; ++c) {
           if (c - win_c0 >= MF_WIN) load_window(c);
-          regroup(ra, c);
-          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
-          consume(c, (uint32_t)(c & 1));
+          step(ra, c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         T += (uint32_t)nchunks;
@@ -606,15 +615,17 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma4_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
-  // ---- tables (layout at MF_LDS_BYTES)
+  // ---- tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) reads the entry's three words once
+  // and writes 8 of its 32 copies with 16-byte stores
   {
-    uint32_t* l32 = (uint32_t*)lds_raw;
-    for (int i = threadIdx.x; i < 256 * 64; i += MF_THREADS) {       // table A: dword e*64 + half*32 + copy
-      const int e = i >> 6, half = (i >> 5) & 1;
-      l32[i] = x.lut[(half ? MF_W_KHI : MF_W_VHI) + e];
-    }
-    for (int i = threadIdx.x; i < 256 * 32; i += MF_THREADS)         // table B, first halves
-      l32[16384 + (i >> 5) * 64 + (i & 31)] = x.lut[MF_W_KLO + (i >> 5)];
+    const int e = threadIdx.x >> 2, qt = threadIdx.x & 3;
+    const uint32_t khi = x.lut[MF_W_KHI + e], klo = x.lut[MF_W_KLO + e], vhi = x.lut[MF_W_VHI + e];
+    uint4* ka = (uint4*)(lds_raw + e * 256 + qt * 64);                  // K copies 8qt .. 8qt+7 (8 bytes each)
+    uint4* va = (uint4*)(lds_raw + MF_TABB + e * 256 + qt * 32);        // V copies 8qt .. 8qt+7 (4 bytes each)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ka[i] = make_uint4(khi, klo, khi, klo);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) va[i] = make_uint4(vhi, vhi, vhi, vhi);
   }
   if (threadIdx.x < 8) *(uint2*)(lds_raw + MF_TABB + (32u * threadIdx.x + 12u) * 256u + 128u) = make_uint2(0u, 0u);
   __syncthreads();
@@ -636,7 +647,7 @@ static bool mfma_disabled() {
 
 // extra workspace the MFMA path needs beyond akv_attn_ws (appended after it)
 size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
-  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * KVH * 4 * 64 * 16);
+  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * KVH * 8 * 64 * 16);
 }
 
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
