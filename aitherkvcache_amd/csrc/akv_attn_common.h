@@ -86,30 +86,35 @@ __device__ __forceinline__ int64_t akv_seq_tokens(const void* context_lens, int 
 // One workgroup (256 threads) writes prefix[0..S].
 __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, int cl_itype, int S,
                                                       int block_size, int64_t max_blocks_per_seq,
-                                                      int32_t* prefix, int32_t* scratch /*[257] LDS*/) {
+                                                      int32_t* prefix, int32_t* scratch /*[>= 4] LDS*/) {
   const int tid = threadIdx.x;
   const int chunk = (S + 255) / 256;
   const int lo = min(S, tid * chunk), hi = min(S, lo + chunk);
   int sum = 0;
   for (int s = lo; s < hi; ++s) sum += akv_seq_blocks(context_lens, cl_itype, s, block_size, max_blocks_per_seq);
-  scratch[tid] = sum;
-  __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int t = 0; t < 256; ++t) {
-      const int v = scratch[t];
-      scratch[t] = run;
-      run += v;
-    }
-    scratch[256] = run;
+  // exclusive scan over the 256 threads: inclusive scan inside each wavefront by lane shifts, then
+  // the four wavefront totals through LDS
+  const int lane = tid & 63, wave = tid >> 6;
+  int inc = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(inc, d, 64);
+    if (lane >= d) inc += up;
   }
+  if (lane == 63) scratch[wave] = inc;
   __syncthreads();
-  int run = scratch[tid];
+  int base = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int t = scratch[w];
+    if (w < wave) base += t;
+  }
+  int run = base + inc - sum;
   for (int s = lo; s < hi; ++s) {
     prefix[s] = run;
     run += akv_seq_blocks(context_lens, cl_itype, s, block_size, max_blocks_per_seq);
   }
-  if (tid == 0) prefix[S] = scratch[256];
+  if (tid == 255) prefix[S] = base + inc;
 }
 
 // largest s with prefix[s] <= g  (prefix non-decreasing, prefix[0] = 0, g < prefix[S])
