@@ -285,7 +285,7 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
 size_t akv_attn_mfma_extra_bytes(int S, int KVH);
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits);
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                      const akv_attn_args& a, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream);
+                      const akv_attn_args& a, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream);
 
 extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
   if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
@@ -385,7 +385,7 @@ extern "C" int akv_paged_attn(
   int Gused = G;
   if (akv_attn_mfma_applicable(a, d, bits)) {
     Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
-    rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
+    rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
   } else {
     const int pgrid = num_seqs * num_q_heads + 1;
 #define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot)

@@ -1,4 +1,4 @@
-// MFMA paged decode attention for the 4-bit cache at head_dim 128, block_size 16.
+// MFMA paged decode attention for the 4-, 3- and 2-bit caches at head_dim 128, block_size 16.
 //
 // One workgroup = 16 wavefronts working on one range of (sequence, block) pairs for all kv
 // heads: wavefronts 0-7 are SCORE wavefronts (one per kv head), 8-15 VALUE wavefronts (same
@@ -38,6 +38,12 @@
 // sixteen levels are almost exactly representable, and alpha is divided out at the end.  Every
 // table entry is replicated 32 times (address = entry * 256 + (lane & 31) * entry size), so lookups
 // never conflict on a bank.
+//
+// The 3-bit and 2-bit caches go through the same tables and the same products: their packed rows
+// are first spread to one code per NIBBLE in registers (a handful of shifts and masks per eight
+// codes, in whatever nibble order is cheapest), and the order is undone for free -- on the K side by
+// building the query operand in the same coordinate order, on the V side by the order in which the
+// accumulators are written out.
 #include "akv_attn_common.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -69,6 +75,43 @@ struct akv_mfma_extra {
 };
 
 // ----------------------------------------------------------------------------------
+// code order after spreading.  K side: transcoded dword st (0..3) of lane g, byte b, nibble `lo`
+// (0 = high nibble) -> coordinate inside the lane's 32.  V side: M-tile n of the value product <->
+// coordinate inside the lane's 8.
+// ----------------------------------------------------------------------------------
+template <int BITS>
+__host__ __device__ constexpr int mf_kcoord(int st, int b, int lo) {
+  if (BITS == 4) return 8 * st + 2 * b + lo;
+  if (BITS == 2) return 16 * (st >> 1) + 4 * b + ((st & 1) ? 2 * lo : 1 + 2 * lo);   // W & 0x33.. | (W >> 2) & 0x33..
+  // 3-bit: bytes (c6,c7) (c3,c5) (c1,c2) (c0,c4) of each group of eight codes (see mf_spread3)
+  constexpr int hi3[4] = {6, 3, 1, 0}, lo3[4] = {7, 5, 2, 4};
+  return 8 * st + (lo ? lo3[b] : hi3[b]);
+}
+template <int BITS>
+__host__ __device__ constexpr int mf_vtile_of_coord(int k) {
+  if (BITS == 4) return k;
+  if (BITS == 2) { constexpr int inv[8] = {2, 3, 0, 1, 6, 7, 4, 5}; return inv[k]; }
+  constexpr int inv[8] = {6, 4, 5, 2, 7, 3, 0, 1};
+  return inv[k];
+}
+// eight 3-bit codes c0..c7 (c0 in bits 23:21 of w) -> nibbles [c7 c6 c5 c3 c2 c1 c4 c0] from bit 0 up
+__device__ __forceinline__ uint32_t mf_spread3(uint32_t w) {
+  uint32_t t = w & 0x7007u;
+  t = ((w << 1) & 0x70070u) | t;
+  t = ((w << 2) & 0x700700u) | t;
+  t = ((w << 15) & 0x07000000u) | t;
+  t = ((w << 7) & 0x70000000u) | t;
+  return t;
+}
+// eight 2-bit codes in a halfword (byte 0 = c0..c3 from the top bits) -> bytes (c2,c3) (c0,c1) (c6,c7) (c4,c5)
+__device__ __forceinline__ uint32_t mf_spread2(uint32_t h) {
+  uint32_t t = (h | (h << 8)) & 0x00FF00FFu;
+  t = (t | (t << 4)) & 0x0F0F0F0Fu;
+  t = (t | (t << 2)) & 0x33333333u;
+  return t;
+}
+
+// ----------------------------------------------------------------------------------
 // prologue: q' = Pi q in MFMA operand layout, block prefix, byte-pair table
 // ----------------------------------------------------------------------------------
 template <int QDT>
@@ -76,7 +119,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
-    uint4* __restrict__ qop, uint32_t* __restrict__ lut, float qscale) {
+    uint4* __restrict__ qop, uint32_t* __restrict__ lut, float qscale, int bits) {
   __shared__ __align__(16) float q_lds[128][8];   // [input coordinate][query head of the group], zero-padded
   __shared__ float qr_lds[8][128];
   __shared__ int32_t scratch[257];
@@ -92,14 +135,15 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     // The tables depend on the codebook only.  They are kept in the workspace together with
     // the centroids they were built from and a marker; when those match, nothing is rebuilt.
     __shared__ int stale;
-    if (tid == 0) stale = (lut[MF_W_MARK] != MF_MARK) ? 1 : 0;
+    const int levels = 1 << bits;
+    if (tid == 0) stale = (lut[MF_W_MARK] != MF_MARK + (uint32_t)bits) ? 1 : 0;
     __syncthreads();
-    if (tid < 16 && __float_as_uint(centroids[tid]) != lut[MF_W_TAG + tid]) stale = 1;
+    if (tid < levels && __float_as_uint(centroids[tid]) != lut[MF_W_TAG + tid]) stale = 1;
     __syncthreads();
     if (!stale) return;
     // alpha search: minimise the largest relative fp16 rounding error of alpha * c over the levels
     float c[16];
-    for (int v = 0; v < 16; ++v) c[v] = centroids[v];
+    for (int v = 0; v < 16; ++v) c[v] = centroids[v & (levels - 1)];
     float berr = 1e30f, balpha = 1.f;
     for (int k = 0; k < MF_ALPHA_CANDIDATES / 256; ++k) {
       const float al = 1.f + (float)(tid * (MF_ALPHA_CANDIDATES / 256) + k) / (float)MF_ALPHA_CANDIDATES;
@@ -122,17 +166,18 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     }
     __syncthreads();
     const float al = best_alpha[0];
-    const float c0 = centroids[tid >> 4], c1 = centroids[tid & 15];   // pair (first, second)
+    // pair (high nibble, low nibble); nibble values above the top level do not occur
+    const float c0 = centroids[(tid >> 4) & (levels - 1)], c1 = centroids[tid & 15 & (levels - 1)];
     const __half k0 = __float2half_rn(c0), k1 = __float2half_rn(c1);
     lut[MF_W_KHI + tid] = (unsigned)__half_as_ushort(k0) | ((unsigned)__half_as_ushort(k1) << 16);
     const __half l0 = __float2half_rn(c0 - __half2float(k0)), l1 = __float2half_rn(c1 - __half2float(k1));
     lut[MF_W_KLO + tid] = (unsigned)__half_as_ushort(l0) | ((unsigned)__half_as_ushort(l1) << 16);
     const __half v0 = __float2half_rn(al * c0), v1 = __float2half_rn(al * c1);
     lut[MF_W_VHI + tid] = (unsigned)__half_as_ushort(v0) | ((unsigned)__half_as_ushort(v1) << 16);
-    if (tid < 16) lut[MF_W_TAG + tid] = __float_as_uint(centroids[tid]);
+    if (tid < levels) lut[MF_W_TAG + tid] = __float_as_uint(centroids[tid]);
     __threadfence();
     __syncthreads();
-    if (tid == 0) lut[MF_W_MARK] = MF_MARK;
+    if (tid == 0) lut[MF_W_MARK] = MF_MARK + (uint32_t)bits;
     return;
   }
   const int s = blockIdx.x / KVH, h = blockIdx.x % KVH;
@@ -171,15 +216,17 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     }
   }
   __syncthreads();
-  // operand layout: [k-step n][lane (col, g)][e] = coordinate 32g + 4n + 2(e/4) + e%2 of column col
-  // (elements 2,3 and 6,7 repeat 0,1 and 4,5: they face the lo halves of the K table entries)
+  // operand layout: [k-step n][lane (col, g)][e]: bytes 2(n%2) + e/4 of transcoded dword n/2, nibble e%2
+  // (4-bit: coordinate 32g + 4n + 2(e/4) + e%2); elements 2,3 and 6,7 repeat 0,1 and 4,5: they face
+  // the lo halves of the K table entries
   for (int n = tid >> 6; n < 8; n += 4) {
     const int lane = tid & 63;
     const int col = lane & 15, g = lane >> 4;
     unsigned short hbits[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int dim = 32 * g + 4 * n + 2 * (e >> 2) + (e & 1);
+      const int st = n >> 1, b = 2 * (n & 1) + (e >> 2), lo = e & 1;
+      const int dim = 32 * g + (bits == 4 ? mf_kcoord<4>(st, b, lo) : bits == 3 ? mf_kcoord<3>(st, b, lo) : mf_kcoord<2>(st, b, lo));
       float v = 0.f;
       if (col < 8) {
         if (col < gqa) v = __half2float(__float2half_rn(qr_lds[col][dim]));
@@ -293,17 +340,18 @@ __device__ __forceinline__ void mf_barrier() {
 }
 
 struct mf_kraw {       // score wavefront, one 32-token chunk
-  uint4 k[2];          // K code rows: tile j, token l%16, bytes [16g, 16g+16)
+  uint4 k[2];          // K code rows: tile j, token l%16, the lane's quarter of the row (16 / 12 / 8 bytes)
   float nrm;           // lane < 32: K norm of token l, else V norm of token l - 32
 };
+typedef uint32_t mf_u32x3 __attribute__((ext_vector_type(3)));
 struct mf_vraw {       // value wavefront
-  uint32_t v[8];       // V codes: token tau(g,e), dword l%16
+  uint32_t v[8];       // V codes: token tau(g,e), the eight codes 8(l%16) .. 8(l%16)+7 (4 / 3 / 2 bytes)
 };
 
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
 // separate instantiations entered through one uniform branch, so that neither keeps the other's
 // loop-invariant registers alive.
-template <int ROLE>
+template <int ROLE, int BITS>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
@@ -381,7 +429,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           }
         }
         float m_run = -INFINITY, l_run = 0.f;
-        const uint32_t koff = (uint32_t)(hh * a.kps_head + col * a.kps_pos + 16 * g);
+        const uint32_t koff = (uint32_t)(hh * a.kps_head + col * a.kps_pos + (BITS == 4 ? 16 : BITS == 3 ? 12 : 8) * g);
         // norms travel one per lane (lanes [0,32): K norm of token l, lanes [32,64): V norm of token
         // l - 32), prefetched with the codes, and are spread to the accumulator layout through the
         // spare halves of table B entries 16q + 10 (K) and 16q + 11 (V)
@@ -397,7 +445,18 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
-          for (int j = 0; j < 2; ++j) r.k[j] = *(const uint4*)(a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + mf_here(koff));
+          for (int j = 0; j < 2; ++j) {
+            const unsigned char* kr = a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + mf_here(koff);
+            if constexpr (BITS == 4) {
+              r.k[j] = *(const uint4*)kr;
+            } else if constexpr (BITS == 3) {
+              const mf_u32x3 t = *(const mf_u32x3*)kr;
+              r.k[j].x = t.x; r.k[j].y = t.y; r.k[j].z = t.z;
+            } else {
+              const uint2 t = *(const uint2*)kr;
+              r.k[j].x = t.x; r.k[j].y = t.y;
+            }
+          }
           r.nrm = nrm_base[mf_umul(ntok >= 16 ? pb[1] : pb[0], nrm_blk) + nrm_off];
         };
         auto produce = [&](mf_kraw& r, int c, const uint32_t par) {
@@ -406,7 +465,23 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           {
             // 8 steps (tile j, dword st): 4 table reads (hi and lo of each of the dword's 4 bytes) feed
             // two MFMAs (bytes 0,1 and bytes 2,3); the reads of step n+2 are issued before the MFMAs of step n
-            const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
+            uint32_t kw[8];       // one code per nibble, two codes per byte
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              if constexpr (BITS == 4) {
+                kw[4 * j] = r.k[j].x; kw[4 * j + 1] = r.k[j].y; kw[4 * j + 2] = r.k[j].z; kw[4 * j + 3] = r.k[j].w;
+              } else if constexpr (BITS == 2) {
+                kw[4 * j] = r.k[j].x & 0x33333333u; kw[4 * j + 1] = (r.k[j].x >> 2) & 0x33333333u;
+                kw[4 * j + 2] = r.k[j].y & 0x33333333u; kw[4 * j + 3] = (r.k[j].y >> 2) & 0x33333333u;
+              } else {
+                // group q = bytes 3q .. 3q+2 of the lane's twelve, as one big-endian 24-bit word
+                const uint32_t d0 = r.k[j].x, d1 = r.k[j].y, d2 = r.k[j].z;
+                kw[4 * j] = mf_spread3(__builtin_amdgcn_perm(d0, d0, 0x0c000102u));
+                kw[4 * j + 1] = mf_spread3(__builtin_amdgcn_perm(d1, d0, 0x0c030405u));
+                kw[4 * j + 2] = mf_spread3(__builtin_amdgcn_perm(d2, d1, 0x0c020304u));
+                kw[4 * j + 3] = mf_spread3(__builtin_amdgcn_perm(d2, d2, 0x0c010203u));
+              }
+            }
             mf_u32x2 w[3][4];      // ring of three steps: two in flight behind the one multiplied
             float4v acc[2];
             acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
@@ -520,7 +595,12 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         float4v o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = (float4v){0.f, 0.f, 0.f, 0.f};
-        const uint32_t voff = (uint32_t)(hh * a.vps_head + 4 * g * a.vps_pos + 4 * col);   // token 4g of a tile
+        // token 4g of a tile; the eight codes of coordinates 8 col .. 8 col + 7: one dword, three bytes
+        // (taken from the aligned dword holding the first of them and, where they run over, from the
+        // neighbour lane's dword), or one halfword
+        const uint32_t voff = (uint32_t)(hh * a.vps_head + 4 * g * a.vps_pos + (BITS == 4 ? 4 * col : BITS == 3 ? ((3 * col) & ~3) : 2 * col));
+        const uint32_t o3 = (uint32_t)(3 * col) & 3u;
+        const uint32_t sel3 = 0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u);   // big-endian 24-bit word
         auto load_chunk = [&](mf_vraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
@@ -528,8 +608,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           for (int j = 0; j < 2; ++j) {
             const unsigned char* vb = a.vp + mf_umul(pb[j], (uint32_t)a.vps_blk);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)      // the token step rides in the uniform base
-              r.v[4 * j + i] = *(const uint32_t*)(vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff));
+            for (int i = 0; i < 4; ++i) {    // the token step rides in the uniform base
+              const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff);
+              if constexpr (BITS == 2) r.v[4 * j + i] = *(const uint16_t*)vr;
+              else r.v[4 * j + i] = *(const uint32_t*)vr;
+            }
           }
         };
         // Everything that does not need the weights happens BEFORE the barrier, while the score side
@@ -542,7 +625,16 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         auto regroup = [&](mf_vraw& r, int c) {
 #pragma unroll
           for (int p = 0; p < 4; ++p) {
-            const uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
+            uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
+            if constexpr (BITS == 3) {
+              const uint32_t na = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wa, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
+              const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wb, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
+              wa = mf_spread3(__builtin_amdgcn_perm(na, wa, sel3));
+              wb = mf_spread3(__builtin_amdgcn_perm(nb, wb, sel3));
+            } else if constexpr (BITS == 2) {
+              wa = mf_spread2(wa);
+              wb = mf_spread2(wb);
+            }
             xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
             xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
           }
@@ -592,7 +684,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         T += (uint32_t)nchunks;
-        // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + j
+        // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + (coordinate of M-tile j)
         const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
 #pragma unroll
         for (int j = 0; j < 8; ++j)
@@ -603,8 +695,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           float* dst = a.part_acc + slot * 128 + 32 * g;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            *(float4*)(dst + 8 * i) = make_float4(o[0][i], o[1][i], o[2][i], o[3][i]);
-            *(float4*)(dst + 8 * i + 4) = make_float4(o[4][i], o[5][i], o[6][i], o[7][i]);
+            *(float4*)(dst + 8 * i) = make_float4(o[mf_vtile_of_coord<BITS>(0)][i], o[mf_vtile_of_coord<BITS>(1)][i],
+                                                  o[mf_vtile_of_coord<BITS>(2)][i], o[mf_vtile_of_coord<BITS>(3)][i]);
+            *(float4*)(dst + 8 * i + 4) = make_float4(o[mf_vtile_of_coord<BITS>(4)][i], o[mf_vtile_of_coord<BITS>(5)][i],
+                                                      o[mf_vtile_of_coord<BITS>(6)][i], o[mf_vtile_of_coord<BITS>(7)][i]);
           }
         }
       }
@@ -612,7 +706,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   }
 }
 
-__global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma4_kernel(akv_attn_args a, akv_mfma_extra x) {
+template <int BITS>
+__global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
   // ---- tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) reads the entry's three words once
@@ -629,8 +724,8 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma4_kernel(akv_attn_arg
   }
   if (threadIdx.x < 8) *(uint2*)(lds_raw + MF_TABB + (32u * threadIdx.x + 12u) * 256u + 128u) = make_uint2(0u, 0u);
   __syncthreads();
-  if ((wave >> 3) == 0) mf_role_main<0>(a, x, wave & 7);
-  else mf_role_main<1>(a, x, wave & 7);
+  if ((wave >> 3) == 0) mf_role_main<0, BITS>(a, x, wave & 7);
+  else mf_role_main<1, BITS>(a, x, wave & 7);
 }
 
 // ----------------------------------------------------------------------------------
@@ -652,10 +747,13 @@ size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
 
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   if (mfma_disabled()) return false;
-  if (d != 128 || bits != 4 || a.block_size != 16) return false;
+  if (d != 128 || bits < 2 || bits > 4 || a.block_size != 16) return false;
   const int gqa = a.QH / a.KVH;
   if (gqa > 8) return false;
-  if ((((uintptr_t)a.kp | (uintptr_t)a.kps_blk | (uintptr_t)a.kps_pos | (uintptr_t)a.kps_head) & 15) != 0) return false;
+  // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword
+  const uintptr_t kalign = bits == 4 ? 15 : bits == 3 ? 3 : 7, valign = bits == 2 ? 1 : 3;
+  if ((((uintptr_t)a.kp | (uintptr_t)a.kps_blk | (uintptr_t)a.kps_pos | (uintptr_t)a.kps_head) & kalign) != 0) return false;
+  if ((((uintptr_t)a.vp | (uintptr_t)a.vps_blk | (uintptr_t)a.vps_pos | (uintptr_t)a.vps_head) & valign) != 0) return false;
   const int64_t strides[12] = {a.kps_blk, a.kps_pos, a.kps_head, a.kns_blk, a.kns_pos, a.kns_head,
                                a.vps_blk, a.vps_pos, a.vps_head, a.vns_blk, a.vns_pos, a.vns_head};
   for (int i = 0; i < 12; ++i)
@@ -664,26 +762,29 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
 }
 
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                      const akv_attn_args& a, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
+                      const akv_attn_args& a, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
   akv_mfma_extra x;
   char* p = (char*)extra_ws;
   x.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
   x.qop = (const uint4*)p;
   const float qscale = a.scale * 1.4426950408889634f;   // scores come out in the log2 domain
   const int pgrid = a.S * a.KVH + 2;
-#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, qscale)
+#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, qscale, bits)
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
   static bool configured = false;
   if (!configured) {
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                MF_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
     configured = true;
   }
   akv_profile_mark_begin(stream);
-  akv_attn_mfma4_kernel<<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
+  if (bits == 4) akv_attn_mfma_kernel<4><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
+  else if (bits == 3) akv_attn_mfma_kernel<3><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
+  else akv_attn_mfma_kernel<2><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
   akv_profile_mark_end(stream);
-  AKV_LAUNCH_CHECK("akv_attn_mfma4_kernel");
+  AKV_LAUNCH_CHECK("akv_attn_mfma_kernel");
   return AKV_OK;
 }
