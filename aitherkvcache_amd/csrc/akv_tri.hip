@@ -380,3 +380,82 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
   return AKV_OK;
 }
+
+// ----------------------------------------------------------------------------------
+// SpectralKVEncoder.encode, int4 coefficients (aither_kvcache/triattention/encoder.py:73-133):
+// one wavefront per vector, lane = RoPE pair.  A pair's rank is the number of pairs with larger
+// energy (equal energies: lower index first; a NaN energy ranks above everything, as in
+// torch.topk); pairs of rank < F are kept, their position in the ascending index order is the
+// number of kept lanes below them.  Arithmetic follows the reference operation by operation
+// (separately rounded squares and sum, true division by the scale, round half to even).
+// ----------------------------------------------------------------------------------
+template <int XDT>
+__global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict__ x, int64_t n, int d, int64_t xs,
+                                                         int F, uint8_t* __restrict__ indices,
+                                                         uint8_t* __restrict__ coeffs, __half* __restrict__ scales) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int P = d >> 1;
+  const bool have = lane < P;
+  for (int64_t v = (int64_t)blockIdx.x * 4 + wave; v < n; v += (int64_t)gridDim.x * 4) {
+    float x0 = 0.f, x1 = 0.f;
+    if (have) {
+      x0 = akv_elem<XDT>::load(x, v * xs + 2 * lane);
+      x1 = akv_elem<XDT>::load(x, v * xs + 2 * lane + 1);
+    }
+    const float e = __fadd_rn(__fmul_rn(x0, x0), __fmul_rn(x1, x1));
+    // non-negative floats and NaNs order like their bit patterns; lanes beyond the last pair sort last
+    const uint32_t key = have ? (__float_as_uint(e) & 0x7fffffffu) + 1u : 0u;
+    int rank = 0;
+#pragma unroll 16
+    for (int q = 0; q < 64; ++q) {
+      const uint32_t kq = (uint32_t)__builtin_amdgcn_readlane((int)key, q);
+      rank += (kq > key || (kq == key && q < lane)) ? 1 : 0;
+    }
+    const bool keep = have && rank < F;
+    const uint64_t mask = __ballot(keep);
+    const int pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    float amax = keep ? fmaxf(fabsf(x0), fabsf(x1)) : 0.f;
+    if (keep && (x0 != x0 || x1 != x1)) amax = __uint_as_float(0x7fc00000u);   // torch.amax propagates NaN
+    // wave maximum that keeps a NaN
+    float m = amax;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float o = __shfl_xor(m, off, 64);
+      m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
+    }
+    const float scale = (m != m) ? m : fmaxf(m, 1e-8f);
+    if (keep) {
+      const float c0 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x0, scale), 1.0f), 7.5f));
+      const float c1 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x1, scale), 1.0f), 7.5f));
+      // clamp(0, 15) then the cast to uint8; a NaN becomes 0 as in torch's float -> uint8 conversion on the CPU
+      const uint32_t q0 = c0 != c0 ? 0u : (uint32_t)fminf(fmaxf(c0, 0.f), 15.f);
+      const uint32_t q1 = c1 != c1 ? 0u : (uint32_t)fminf(fmaxf(c1, 0.f), 15.f);
+      indices[v * F + pos] = (uint8_t)lane;
+      coeffs[v * F + pos] = (uint8_t)((q0 << 4) | q1);
+    }
+    if (lane == 0) scales[v] = __float2half_rn(scale);
+  }
+}
+
+extern "C" int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
+                              uint8_t* indices, uint8_t* coeffs, void* scales, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  AKV_REQUIRE(n >= 0, "akv_tri_encode: n=%lld", (long long)n);
+  AKV_REQUIRE(akv_valid_dtype(x_dtype), "akv_tri_encode: bad dtype");
+  AKV_REQUIRE(d > 0 && d % 2 == 0, "akv_tri_encode: head_dim=%d must be even", d);
+  AKV_REQUIRE(num_freqs > 0 && num_freqs <= d / 2, "akv_tri_encode: num_freqs=%d out of range", num_freqs);
+  if (d > 128) return akv_fail(AKV_ERR_UNSUPPORTED, "akv_tri_encode: head_dim=%d above 128 (one lane per pair)", d);
+  if (n == 0) return AKV_OK;
+  AKV_REQUIRE(x && indices && coeffs && scales, "akv_tri_encode: null pointer");
+  AKV_REQUIRE(x_stride >= d, "akv_tri_encode: stride smaller than row");
+  const int64_t want = (n + 3) / 4;
+  const int cap = akv_cached_cu_count() * 32;
+  const int grid = (int)(want < cap ? want : cap);
+  switch (x_dtype) {
+    case AKV_F16: tri_encode_kernel<AKV_F16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
+    case AKV_BF16: tri_encode_kernel<AKV_BF16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
+    default: tri_encode_kernel<AKV_F32><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
+  }
+  AKV_LAUNCH_CHECK("tri_encode_kernel");
+  return AKV_OK;
+}

@@ -2,13 +2,14 @@
 
 Keeps the F RoPE pairs (dims 2i, 2i+1) of largest energy per token, ascending by index, and
 quantises their 2F values to 4 bits against the token's max-abs scale (reference:
-aither_kvcache/triattention/encoder.py:73-133).  This write side is expressed with torch ops on
-the device the input lives on; only the read side (decode_step) is a hand-written kernel.
+aither_kvcache/triattention/encoder.py:73-133).  On an MI355X tensor with head_dim <= 128 this is one
+HIP kernel (akv_tri_encode); host tensors and wider heads take the same steps as torch ops.
 """
 from typing import NamedTuple, Optional
 
 import torch
 
+from .. import _lib
 from .config import TriAttentionConfig
 
 
@@ -30,6 +31,19 @@ class SpectralKVEncoder:
 
     def encode(self, x: torch.Tensor, num_freqs: Optional[int] = None) -> SpectralEncoding:
         F = num_freqs or self.num_freqs
+        if x.is_cuda and self.head_dim <= 128 and x.dtype in (torch.float16, torch.bfloat16, torch.float32):
+            batch = list(x.shape[:-1])
+            xf = x.reshape(-1, self.head_dim)
+            if xf.stride(-1) != 1:
+                xf = xf.contiguous()
+            n = xf.shape[0]
+            idx = torch.empty(n, F, dtype=torch.uint8, device=x.device)
+            cf = torch.empty(n, F, dtype=torch.uint8, device=x.device)
+            sc = torch.empty(n, dtype=torch.float16, device=x.device)
+            _lib.check(_lib.lib().akv_tri_encode(
+                xf.data_ptr(), _lib.dtype_code(xf), n, self.head_dim, xf.stride(0) if n else self.head_dim, F,
+                idx.data_ptr(), cf.data_ptr(), sc.data_ptr(), _lib.stream_ptr(x.device)))
+            return SpectralEncoding(idx.reshape(batch + [F]), cf.reshape(batch + [F]), sc.reshape(batch))
         pairs = x.reshape(*x.shape[:-1], self.num_pairs, 2).float()
         energy = pairs.pow(2).sum(-1)
         keep = energy.topk(F, dim=-1).indices.sort(dim=-1).values

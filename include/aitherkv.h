@@ -224,6 +224,19 @@ int akv_tri_decode_step(const void* query, int q_dtype,
                         int d, int num_freqs,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------
+ * SpectralKVEncoder.encode, coeff_bits = 4 -- aither_kvcache/triattention/encoder.py:73-133
+ * (the write side of TriAttention; TriAttention.encode_kv, attention.py:160-184, calls it for
+ * keys and values): per vector the num_freqs RoPE pairs (dims 2i, 2i+1) of largest energy,
+ * indices ascending; scale = max |kept coefficient| clamped at 1e-8; code =
+ * clamp(round((v / scale + 1) * 7.5), 0, 15); byte = code(even) << 4 | code(odd).
+ *   x [n][d] (row stride x_stride elements); indices, coeffs [n][num_freqs] uint8; scales [n] fp16.
+ * Pairs of exactly equal energy are kept lowest index first (torch.topk leaves that open).
+ * head_dim above 128 returns AKV_ERR_UNSUPPORTED.
+ * ------------------------------------------------------------------------------- */
+int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
+                   uint8_t* indices, uint8_t* coeffs, void* scales, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

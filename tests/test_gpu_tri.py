@@ -86,3 +86,39 @@ def test_uniform_values_property(dev):
     out = tri.decode_step(q, k_enc, v_enc)
     want = tri.encoder.decode(v1).reshape(1, 8, 1, 128).expand(B, 8, 4, 128).reshape(B, 32, 128)
     assert torch.max(torch.abs(out - want)).item() <= 1e-5
+
+
+def test_spectral_encode_golden(golden, dev):
+    """The write-side kernel reproduces the reference's encodings of the golden keys and values byte for byte."""
+    tri = TriAttention(TriAttentionConfig(num_kv_heads=2, num_query_heads=8), device=str(dev))
+    for nm, src in (("k", "tri_keys"), ("v", "tri_vals")):
+        e = tri.encoder.encode(t(golden[src], dev))
+        assert e.indices.dtype == torch.uint8 and e.packed.dtype == torch.uint8 and e.scales.dtype == torch.float16
+        assert np.array_equal(e.indices.cpu().numpy(), golden[f"tri_{nm}_indices"])
+        assert np.array_equal(e.packed.cpu().numpy(), golden[f"tri_{nm}_packed"])
+        assert np.array_equal(e.scales.cpu().numpy(), golden[f"tri_{nm}_scales"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("D,F", [(128, 12), (64, 7), (32, 16)])
+def test_spectral_encode_vs_oracle(dev, dtype, D, F):
+    rng = np.random.default_rng(D + F)
+    n = 5000
+    x = (rng.standard_normal((n, D)) * rng.lognormal(0, 1.0, (n, 1))).astype(np.float32)
+    x[7] = 0.0                                  # all energies equal: the lowest indices are kept, scale 1e-8 -> fp16 0
+    x[8, 2:] = 0.0                              # fewer non-zero pairs than F
+    x[9] *= 1e-6
+    xt = torch.from_numpy(x).to(dev).to(dtype)
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=F, num_kv_heads=1, num_query_heads=1)
+    tri = TriAttention(cfg, device=str(dev))
+    e = tri.encoder.encode(xt)
+    ri, rp, rs = O.spectral_encode(xt.float().cpu().numpy(), F)
+    assert np.array_equal(e.indices.cpu().numpy(), ri)
+    assert np.array_equal(e.packed.cpu().numpy(), rp)
+    assert np.array_equal(e.scales.cpu().numpy(), rs)
+    # batch shapes and the empty batch
+    e2 = tri.encoder.encode(xt[:24].reshape(2, 3, 4, D))
+    assert e2.indices.shape == (2, 3, 4, F) and e2.scales.shape == (2, 3, 4)
+    assert torch.equal(e2.indices.reshape(24, F), e.indices[:24])
+    e0 = tri.encoder.encode(xt[:0])
+    assert e0.indices.shape == (0, F)
