@@ -61,8 +61,12 @@ class TQPagedAttention:
         if num_kv_heads is None:
             num_kv_heads = k_packed.shape[2]
         if self._block_selector is not None:
-            raise NotImplementedError("sparse block selection is not part of this build; pass "
-                                      "already-filtered block_tables/context_lens instead")
+            # as in the reference (:659-668): even / odd coordinates of the rotated query score the blocks,
+            # the kernel then walks the filtered table
+            q_rot = torch.matmul(query.float(), self.rotation.T)
+            block_tables, context_lens = self._block_selector.select(
+                q_rot[..., 0::2].contiguous(), q_rot[..., 1::2].contiguous(), block_tables, context_lens,
+                query.shape[1] // num_kv_heads, block_size)
         dev = _lib.require_gpu(query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens)
         num_seqs, num_q_heads, head_dim = query.shape
         if head_dim != self.head_dim or num_q_heads != self.num_query_heads:

@@ -237,6 +237,49 @@ int akv_tri_decode_step(const void* query, int q_dtype,
 int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
                    uint8_t* indices, uint8_t* coeffs, void* scales, void* stream);
 
+/* ---------------------------------------------------------------------------------
+ * Block selection for sparse decode attention -- aither_kvcache/block_selector.py.
+ * The attention entry points take the filtered table and context lengths as they are.
+ *
+ * akv_block_rep_update: BlockSelector.update_reps (:282-292) = BlockRepresentativeCache.update
+ *   (:66-101) + finalize of the touched blocks (:103-118).  For each of the n new tokens and each
+ *   kv head, norm * centroids[high nibble] is added to acc_even[block][head][byte] and
+ *   norm * centroids[low nibble] to acc_odd, the block's count goes up by one; then, unless
+ *   rep_even/rep_odd are NULL, rep = acc / max(count, 1) for the blocks listed.  Block ids
+ *   outside [0, max_blocks) are skipped.  4-bit codes.  counts is int32 (the reference keeps
+ *   int16).  k_packed [n][kv_heads][packed_dim] with byte strides, k_norms [n][kv_heads] with
+ *   element strides; acc_* / rep_* [max_blocks][kv_heads][packed_dim] float32, contiguous.
+ * akv_block_rep_finalize: finalize (:103-118) for the blocks listed, or for all when
+ *   block_indices is NULL.
+ * akv_block_scores: score_blocks (:129-179).  q_even / q_odd [seqs][q_heads][half_d] float32
+ *   (even / odd coordinates of the rotated query), scores [seqs][max_blocks_per_seq] float32;
+ *   table columns at or beyond ceil(context / block_size) get -inf, table entries are clamped
+ *   into [0, num_blocks).
+ * akv_block_select: select_blocks (:182-236).  filtered_block_tables [seqs][max_selected] in the
+ *   table's integer type: sink and recent columns, then the best-scoring ones, k =
+ *   min(max_selected, max_blocks_per_seq) in all, in column order, zero padding behind;
+ *   filtered_context_lens = min(context, k * block_size).  Equal scores: lower column first.
+ * ------------------------------------------------------------------------------- */
+int akv_block_rep_update(const void* block_indices, int idx_itype, int64_t n,
+                         const uint8_t* k_packed, int64_t ps_tok, int64_t ps_head,
+                         const float* k_norms, int64_t ns_tok, int64_t ns_head, const float* centroids,
+                         float* acc_even, float* acc_odd, int32_t* counts, float* rep_even, float* rep_odd,
+                         int64_t max_blocks, int num_kv_heads, int packed_dim, void* stream);
+int akv_block_rep_finalize(const void* block_indices, int idx_itype, int64_t n,
+                           const float* acc_even, const float* acc_odd, const int32_t* counts,
+                           float* rep_even, float* rep_odd,
+                           int64_t max_blocks, int num_kv_heads, int packed_dim, void* stream);
+int akv_block_scores(const float* q_even, const float* q_odd, const float* rep_even, const float* rep_odd,
+                     const void* block_tables, int bt_itype, int64_t bt_stride,
+                     const void* context_lens, int cl_itype,
+                     int num_seqs, int num_q_heads, int num_kv_heads, int half_d,
+                     int64_t max_blocks_per_seq, int block_size, int64_t num_blocks,
+                     float* scores, void* stream);
+int akv_block_select(const float* scores, const void* block_tables, int bt_itype, int64_t bt_stride,
+                     const void* context_lens, int cl_itype, int num_seqs, int64_t max_blocks_per_seq,
+                     int block_size, int max_selected, int num_sink_blocks, int num_recent_blocks,
+                     void* filtered_block_tables, void* filtered_context_lens, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

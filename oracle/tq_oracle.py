@@ -13,6 +13,8 @@ reference tree).  How each one is pinned:
   in tests/test_oracle_*.py:
       get_codebook, pack_*/unpack_*, pack_multibit/unpack_multibit,
       encode, decode, kv_update, paged_attention_loop, paged_attention,
+      block_rep_update, block_rep_finalize, block_scores, block_select (golden vectors in
+      tests/golden/golden_block_selector.npz, written by the reference itself),
       batch_decompress_active_blocks (its decode by the golden vectors; its block
       selection and scatter by a per-block loop in tests/test_oracle_pins.py),
       fwht, structured_hadamard, dimension_aware_codebook,
@@ -342,6 +344,75 @@ def paged_attention(query, k_packed, k_norms, v_packed, v_norms, block_tables, c
         acc = np.einsum("hgt,thd->hgd", p, vd[s]).reshape(QH, D)
         out[s] = acc @ R
     return out.astype(query.dtype) if cast_output else out
+
+
+# --------------------------------------------------------------------------------------
+# block_selector.py
+# --------------------------------------------------------------------------------------
+def block_rep_update(acc_even, acc_odd, counts, block_indices, k_packed, k_norms, centroids):
+    """BlockRepresentativeCache.update, block_selector.py:66-101: per new token and kv head the
+    norm-weighted centroids of the high / low nibbles are added to the block's accumulators and
+    the block's count goes up by one.  In place."""
+    kp = np.asarray(k_packed).astype(np.int64)
+    c = np.asarray(centroids, dtype=f32)
+    kn = np.asarray(k_norms, dtype=f32)[..., None]
+    we = kn * c[(kp >> 4) & 0xF]
+    wo = kn * c[kp & 0xF]
+    bi = np.asarray(block_indices)
+    np.add.at(acc_even, bi, we)
+    np.add.at(acc_odd, bi, wo)
+    np.add.at(counts, bi, 1)
+
+
+def block_rep_finalize(acc_even, acc_odd, counts, rep_even, rep_odd, block_indices=None):
+    """BlockRepresentativeCache.finalize, block_selector.py:103-118: rep = acc / max(count, 1)
+    for the given blocks (all when None).  In place."""
+    sel = slice(None) if block_indices is None else np.asarray(block_indices)
+    safe = np.maximum(counts[sel], 1)[..., None].astype(f32)
+    rep_even[sel] = acc_even[sel] / safe
+    rep_odd[sel] = acc_odd[sel] / safe
+
+
+def block_scores(q_even, q_odd, rep_even, rep_odd, block_tables, context_lens, gqa_ratio, block_size):
+    """score_blocks, block_selector.py:129-179: mean query of each GQA group against the
+    representatives of the table's blocks (ids clamped at 0), summed over kv heads and
+    coordinates; columns at or beyond ceil(ctx / block_size) are -inf."""
+    S, QH, HD = q_even.shape
+    KV = QH // gqa_ratio
+    qe = q_even.reshape(S, KV, gqa_ratio, HD).mean(axis=2, dtype=f32)
+    qo = q_odd.reshape(S, KV, gqa_ratio, HD).mean(axis=2, dtype=f32)
+    bt = np.maximum(np.asarray(block_tables), 0)
+    ge, go = rep_even[bt], rep_odd[bt]                            # [S, B, KV, HD]
+    sc = (qe[:, None] * ge).sum(axis=(-1, -2), dtype=f32) + (qo[:, None] * go).sum(axis=(-1, -2), dtype=f32)
+    nb = (np.asarray(context_lens) + block_size - 1) // block_size
+    sc = sc.astype(f32)
+    sc[np.arange(bt.shape[1])[None, :] >= nb[:, None]] = -np.inf
+    return sc
+
+
+def block_select(scores, block_tables, context_lens, block_size, max_selected, num_sink_blocks=2,
+                 num_recent_blocks=2):
+    """select_blocks, block_selector.py:182-236: sink and recent columns forced in, top-k of the
+    rest (k = min(max_selected, table width)), kept in column order, physical ids gathered,
+    zero padding up to max_selected; context = min(ctx, k * block_size).  Among equal scores the
+    lower column wins here (torch.topk leaves that open)."""
+    scores = np.asarray(scores, dtype=f32)
+    S, B = scores.shape
+    ctx = np.asarray(context_lens)
+    nb = (ctx + block_size - 1) // block_size
+    col = np.arange(B)[None, :]
+    valid = col < nb[:, None]
+    mandatory = ((col < num_sink_blocks) | (col >= nb[:, None] - num_recent_blocks)) & valid
+    sel = scores.copy()
+    sel[mandatory] = np.inf
+    sel[~valid] = -np.inf
+    k = min(max_selected, B)
+    top = np.sort(np.argsort(-sel, axis=1, kind="stable")[:, :k], axis=1)
+    fbt = np.take_along_axis(np.asarray(block_tables), top, axis=1)
+    if k < max_selected:
+        fbt = np.concatenate([fbt, np.zeros((S, max_selected - k), dtype=fbt.dtype)], axis=1)
+    fcl = np.minimum(ctx, k * block_size).astype(ctx.dtype)
+    return fbt, fcl
 
 
 # --------------------------------------------------------------------------------------

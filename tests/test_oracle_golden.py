@@ -1,4 +1,6 @@
 """The numpy oracle against the vectors the reference itself produced (CPU only)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -127,3 +129,50 @@ def test_tri_matches_reference(golden):
     assert np.max(np.abs(o1 - golden["tri_out_default_pos"])) < 1e-6
     o2 = O.tri_decode_step(golden["tri_q"], ke, ve, th, golden["tri_qpos"], golden["tri_kpos"])
     assert np.max(np.abs(o2 - golden["tri_out_explicit_pos"])) < 1e-6
+
+
+# ---- block selector (vectors written by tests/golden/make_golden_block_selector.py) -------------
+@pytest.fixture(scope="module")
+def bsel():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_block_selector.npz"))
+
+
+def test_block_representatives_golden(bsel):
+    MB, H, PD = 12, 2, 64
+    acc_e = np.zeros((MB, H, PD), np.float32); acc_o = np.zeros_like(acc_e)
+    rep_e = np.zeros_like(acc_e); rep_o = np.zeros_like(acc_e)
+    counts = np.zeros((MB, H), np.int16)
+    for call in range(3):
+        bi = bsel[f"rep_bi_{call}"]
+        O.block_rep_update(acc_e, acc_o, counts, bi, bsel[f"rep_kp_{call}"], bsel[f"rep_kn_{call}"], bsel["centroids"])
+        O.block_rep_finalize(acc_e, acc_o, counts, rep_e, rep_o, np.unique(bi))
+        assert np.array_equal(counts, bsel[f"rep_counts_after_{call}"])
+        # the reference adds in torch's scatter order, the oracle in input order: a few ulps of a sum
+        np.testing.assert_allclose(rep_e, bsel[f"rep_even_after_{call}"], rtol=2e-6, atol=1e-7)
+        np.testing.assert_allclose(rep_o, bsel[f"rep_odd_after_{call}"], rtol=2e-6, atol=1e-7)
+    assert np.all(bsel["rep_counts_after_2"][10:] == 0) and np.all(bsel["rep_even_after_2"][10:] == 0)
+
+
+def test_block_scores_and_selection_golden(bsel):
+    sc = O.block_scores(bsel["sel_q_even"], bsel["sel_q_odd"], bsel["sel_rep_even"], bsel["sel_rep_odd"],
+                        bsel["sel_bt"], bsel["sel_ctx"], 4, 16)
+    ref = bsel["sel_scores"]
+    assert np.array_equal(np.isneginf(sc), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    assert np.max(np.abs(sc[fin] - ref[fin])) <= 2e-5
+    nb = (bsel["sel_ctx"] + 15) // 16
+    for tag, ms, sinks, recents in (("10", 10, 2, 2), ("40", 40, 2, 2), ("120", 120, 2, 2), ("12_s1r3", 12, 1, 3)):
+        fbt, fcl = O.block_select(ref, bsel["sel_bt"], bsel["sel_ctx"], 16, ms, sinks, recents)
+        rbt, rcl = bsel[f"sel_fbt_{tag}"], bsel[f"sel_fcl_{tag}"]
+        assert np.array_equal(fcl, rcl) and fbt.shape == rbt.shape
+        k = min(ms, bsel["sel_bt"].shape[1])
+        for s in range(fbt.shape[0]):
+            m = min(k, int(nb[s]))          # beyond the valid blocks the reference's choice among -inf columns is arbitrary
+            assert np.array_equal(fbt[s, :m], rbt[s, :m])
+        assert np.all(fbt[:, k:] == 0) and np.all(rbt[:, k:] == 0)
+    assert int(bsel["cls_max_selected"]) == 30
+    fbt, fcl = O.block_select(ref, bsel["sel_bt"], bsel["sel_ctx"], 16, 30)
+    assert np.array_equal(fcl, bsel["cls_fcl"])
+    for s in range(3):
+        m = min(30, int(nb[s]))
+        assert np.array_equal(fbt[s, :m], bsel["cls_fbt"][s, :m])
