@@ -30,12 +30,13 @@ def test_representatives_golden(bsel, dev):
         cache.update(idx, t(bsel[f"rep_pos_{call}"], dev), t(bsel[f"rep_kp_{call}"], dev), t(bsel[f"rep_kn_{call}"], dev))
         cache.finalize(t(np.unique(bi), dev))
         assert np.array_equal(cache._counts.cpu().numpy(), bsel[f"rep_counts_after_{call}"])
-        np.testing.assert_allclose(cache.rep_even.cpu().numpy(), bsel[f"rep_even_after_{call}"], rtol=3e-6, atol=1e-7)
-        np.testing.assert_allclose(cache.rep_odd.cpu().numpy(), bsel[f"rep_odd_after_{call}"], rtol=3e-6, atol=1e-7)
+        # sums of up to ~10 terms of size ~10 in the order the atomics land: absolute slack for cancelling terms
+        np.testing.assert_allclose(cache.rep_even.cpu().numpy(), bsel[f"rep_even_after_{call}"], rtol=3e-6, atol=5e-6)
+        np.testing.assert_allclose(cache.rep_odd.cpu().numpy(), bsel[f"rep_odd_after_{call}"], rtol=3e-6, atol=5e-6)
     cache.clear_blocks(torch.tensor([3, 4], device=dev))
     cache.finalize()
     assert np.array_equal(cache._counts.cpu().numpy(), bsel["rep_counts_cleared"])
-    np.testing.assert_allclose(cache.rep_even.cpu().numpy(), bsel["rep_even_cleared"], rtol=3e-6, atol=1e-7)
+    np.testing.assert_allclose(cache.rep_even.cpu().numpy(), bsel["rep_even_cleared"], rtol=3e-6, atol=5e-6)
     # ids outside the cache are skipped, an empty update is a no-op
     before = cache._acc_even.clone()
     cache.update(torch.tensor([-1, 99], device=dev), torch.zeros(2, dtype=torch.long, device=dev),
