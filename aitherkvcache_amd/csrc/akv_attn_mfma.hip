@@ -45,6 +45,7 @@
 // building the query operand in the same coordinate order, on the V side by the order in which the
 // accumulators are written out.
 #include "akv_attn_common.h"
+#include "akv_nibble.h"
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -73,43 +74,6 @@ struct akv_mfma_extra {
   const uint32_t* lut;   // table block, MF_W_* (workspace)
   const uint4* qop;      // [S][KVH][8 k-steps][64 lanes] half8 as uint4 (workspace)
 };
-
-// ----------------------------------------------------------------------------------
-// code order after spreading.  K side: transcoded dword st (0..3) of lane g, byte b, nibble `lo`
-// (0 = high nibble) -> coordinate inside the lane's 32.  V side: M-tile n of the value product <->
-// coordinate inside the lane's 8.
-// ----------------------------------------------------------------------------------
-template <int BITS>
-__host__ __device__ constexpr int mf_kcoord(int st, int b, int lo) {
-  if (BITS == 4) return 8 * st + 2 * b + lo;
-  if (BITS == 2) return 16 * (st >> 1) + 4 * b + ((st & 1) ? 2 * lo : 1 + 2 * lo);   // W & 0x33.. | (W >> 2) & 0x33..
-  // 3-bit: bytes (c6,c7) (c3,c5) (c1,c2) (c0,c4) of each group of eight codes (see mf_spread3)
-  constexpr int hi3[4] = {6, 3, 1, 0}, lo3[4] = {7, 5, 2, 4};
-  return 8 * st + (lo ? lo3[b] : hi3[b]);
-}
-template <int BITS>
-__host__ __device__ constexpr int mf_vtile_of_coord(int k) {
-  if (BITS == 4) return k;
-  if (BITS == 2) { constexpr int inv[8] = {2, 3, 0, 1, 6, 7, 4, 5}; return inv[k]; }
-  constexpr int inv[8] = {6, 4, 5, 2, 7, 3, 0, 1};
-  return inv[k];
-}
-// eight 3-bit codes c0..c7 (c0 in bits 23:21 of w) -> nibbles [c7 c6 c5 c3 c2 c1 c4 c0] from bit 0 up
-__device__ __forceinline__ uint32_t mf_spread3(uint32_t w) {
-  uint32_t t = w & 0x7007u;
-  t = ((w << 1) & 0x70070u) | t;
-  t = ((w << 2) & 0x700700u) | t;
-  t = ((w << 15) & 0x07000000u) | t;
-  t = ((w << 7) & 0x70000000u) | t;
-  return t;
-}
-// eight 2-bit codes in a halfword (byte 0 = c0..c3 from the top bits) -> bytes (c2,c3) (c0,c1) (c6,c7) (c4,c5)
-__device__ __forceinline__ uint32_t mf_spread2(uint32_t h) {
-  uint32_t t = (h | (h << 8)) & 0x00FF00FFu;
-  t = (t | (t << 4)) & 0x0F0F0F0Fu;
-  t = (t | (t << 2)) & 0x33333333u;
-  return t;
-}
 
 // ----------------------------------------------------------------------------------
 // prologue: q' = Pi q in MFMA operand layout, block prefix, byte-pair table
@@ -468,19 +432,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             uint32_t kw[8];       // one code per nibble, two codes per byte
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-              if constexpr (BITS == 4) {
-                kw[4 * j] = r.k[j].x; kw[4 * j + 1] = r.k[j].y; kw[4 * j + 2] = r.k[j].z; kw[4 * j + 3] = r.k[j].w;
-              } else if constexpr (BITS == 2) {
-                kw[4 * j] = r.k[j].x & 0x33333333u; kw[4 * j + 1] = (r.k[j].x >> 2) & 0x33333333u;
-                kw[4 * j + 2] = r.k[j].y & 0x33333333u; kw[4 * j + 3] = (r.k[j].y >> 2) & 0x33333333u;
-              } else {
-                // group q = bytes 3q .. 3q+2 of the lane's twelve, as one big-endian 24-bit word
-                const uint32_t d0 = r.k[j].x, d1 = r.k[j].y, d2 = r.k[j].z;
-                kw[4 * j] = mf_spread3(__builtin_amdgcn_perm(d0, d0, 0x0c000102u));
-                kw[4 * j + 1] = mf_spread3(__builtin_amdgcn_perm(d1, d0, 0x0c030405u));
-                kw[4 * j + 2] = mf_spread3(__builtin_amdgcn_perm(d2, d1, 0x0c020304u));
-                kw[4 * j + 3] = mf_spread3(__builtin_amdgcn_perm(d2, d2, 0x0c010203u));
-              }
+              const uint32_t raw[4] = {r.k[j].x, r.k[j].y, r.k[j].z, r.k[j].w};
+              uint32_t sp[4];
+              mf_spread_row<BITS>(raw, sp);
+#pragma unroll
+              for (int d = 0; d < 4; ++d) kw[4 * j + d] = sp[d];
             }
             mf_u32x2 w[3][4];      // ring of three steps: two in flight behind the one multiplied
             float4v acc[2];

@@ -1,5 +1,5 @@
-// MFMA decode (unpack -> centroid lookup -> inverse rotation -> x norm -> float16) for the 4-bit
-// codec at head_dim 128: TurboQuant.decode, aither_kvcache/quantizer.py:168-197.
+// MFMA decode (unpack -> centroid lookup -> inverse rotation -> x norm -> float16) for the 4-, 3- and
+// 2-bit codecs at head_dim 128: TurboQuant.decode, aither_kvcache/quantizer.py:168-197.
 //
 //   X[v, i] = n_v * sum_j c[code[v, j]] * Pi[j, i]              v_mfma_f32_16x16x32_f16
 //     A = centroids of the codes: lane (row = l%16, g = l/16) loads bytes [16g, 16g+16) of the
@@ -15,9 +15,14 @@
 //     k-steps are the outer loop (A operands of one k-step live in registers, all 8 x 2
 //     accumulator tiles stay resident).
 //
+// 3-bit and 2-bit rows are spread to one code per nibble in registers (akv_nibble.h) and then take the
+// same table and products; the coordinate order that the spreading leaves is matched by the order in
+// which the rows of the B operand are copied into LDS.
+//
 // A wavefront decodes 32 vectors per step; a workgroup is eight independent wavefronts plus the
 // B operand (64 KB) and the byte table (64 KB).
 #include "akv_common.h"
+#include "akv_nibble.h"
 
 typedef _Float16 dm_half8 __attribute__((ext_vector_type(8)));
 typedef float dm_float4 __attribute__((ext_vector_type(4)));
@@ -34,6 +39,20 @@ typedef __attribute__((address_space(3))) const uint32_t dm_lds_cu32;
 #define DM_ROW_OFF 131072            // per wavefront: DM_ROWS x {packed offset, norm offset, output offset} (block-wise decode)
 #define DM_LDS_BYTES (131072 + DM_WAVES * DM_ROWS * 24)
 #define DM_SEL(k) (0x0c0c0400u + ((uint32_t)(k) << 8))
+
+// the lane's quarter of a packed row: 16 / 12 / 8 bytes
+template <int BITS>
+__device__ __forceinline__ uint4 dm_load_quarter(const uint8_t* row, int g) {
+  if constexpr (BITS == 4) {
+    return *(const uint4*)(row + 16 * g);
+  } else if constexpr (BITS == 3) {
+    const uint32_t* p = (const uint32_t*)(row + 12 * g);
+    return make_uint4(p[0], p[1], p[2], 0u);
+  } else {
+    const uint2 t = *(const uint2*)(row + 8 * g);
+    return make_uint4(t.x, t.y, 0u, 0u);
+  }
+}
 
 // B operand of the decode kernel, stored after the encode operand in the prepared-rotation buffer
 __global__ __launch_bounds__(256) void akv_dm_prepare_kernel(const float* __restrict__ Pi, uint4* __restrict__ bop) {
@@ -71,21 +90,33 @@ int akv_prepare_decode_mfma(const float* rotation, int d, void* prep, hipStream_
 // (position, head) entries of the cache blocks listed in a.slots; every listed block that exists is
 // decoded into the block of the same index of the output buffer (the batch decompress of
 // aither_kvcache/vllm/backend.py:1040-1091 without its gather / unique / scatter passes).
-template <bool BLOCKS>
+template <bool BLOCKS, int BITS>
 __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
   {
-    uint4* b_lds = (uint4*)(lds + DM_B_OFF);
-    for (int i = threadIdx.x; i < 65536 / 16; i += DM_THREADS) b_lds[i] = bop[i];
+    if constexpr (BITS == 4) {
+      uint4* b_lds = (uint4*)(lds + DM_B_OFF);
+      for (int i = threadIdx.x; i < 65536 / 16; i += DM_THREADS) b_lds[i] = bop[i];
+    } else {
+      // element e of k-step ks of a lane faces the coordinate that the spread code stream holds there
+      const uint16_t* src = (const uint16_t*)bop;
+      uint16_t* b_lds = (uint16_t*)(lds + DM_B_OFF);
+      for (int i = threadIdx.x; i < 65536 / 2; i += DM_THREADS) {
+        const int e = i & 7, ln = (i >> 3) & 63, ks = (i >> 9) & 3, rest = i >> 11;   // rest = (hi | lo, nt)
+        const int c = mf_kcoord<BITS>(ks, e >> 1, e & 1);
+        b_lds[i] = src[((rest * 4 + (c >> 3)) * 64 + ln) * 8 + (c & 7)];
+      }
+    }
     // byte table: entry (hi nibble, lo nibble) -> (c[hi nibble], c[lo nibble]): the code of the
     // even coordinate is the high nibble (packing.py:13-23) and goes to the low half of the pair
     uint32_t* lut = (uint32_t*)(lds + DM_LUT_OFF);
     for (int i = threadIdx.x; i < 256 * 64; i += DM_THREADS) {
       const int e = i >> 6, half = (i >> 5) & 1;
-      const float c0 = a.table[e >> 4], c1 = a.table[e & 15];
+      constexpr int LM = (1 << BITS) - 1;      // nibble values above the top level do not occur
+      const float c0 = a.table[(e >> 4) & LM], c1 = a.table[e & 15 & LM];
       const __half h0 = __float2half_rn(c0), h1 = __float2half_rn(c1);
       uint32_t w;
       if (half == 0) {
@@ -134,7 +165,7 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
       float nv[4];
       if constexpr (BLOCKS) {
         const int64_t po = row_p[16 * mt + (lane & 15)];
-        pk[mt] = po >= 0 ? *(const uint4*)(a.packed + po + 16 * g) : make_uint4(0, 0, 0, 0);
+        pk[mt] = po >= 0 ? dm_load_quarter<BITS>(a.packed + po, g) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int r = 16 * mt + 4 * g + i;
@@ -142,7 +173,7 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
         }
       } else {
         const int64_t n = base + 16 * mt + (lane & 15);
-        pk[mt] = n < a.n ? *(const uint4*)(a.packed + n * a.ps0 + 16 * g) : make_uint4(0, 0, 0, 0);
+        pk[mt] = n < a.n ? dm_load_quarter<BITS>(a.packed + n * a.ps0, g) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int64_t r = base + 16 * mt + 4 * g + i;
@@ -150,6 +181,12 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
         }
       }
       nr[mt] = make_float4(nv[0], nv[1], nv[2], nv[3]);
+    }
+    uint32_t kw[2][4];      // one code per nibble
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const uint32_t raw[4] = {pk[mt].x, pk[mt].y, pk[mt].z, pk[mt].w};
+      mf_spread_row<BITS>(raw, kw[mt]);
     }
     dm_float4 acc[2][8];
 #pragma unroll
@@ -162,7 +199,7 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
       dm_half8 ah[2], al[2];
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
-        const uint32_t w = ks == 0 ? pk[mt].x : ks == 1 ? pk[mt].y : ks == 2 ? pk[mt].z : pk[mt].w;
+        const uint32_t w = kw[mt][ks];
         union { uint32_t u[4]; dm_half8 h; } ch, cl;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
@@ -231,22 +268,28 @@ static bool dm_disabled() {
 // returns AKV_ERR_UNSUPPORTED when the fast path does not apply (the caller then uses the general kernel)
 int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int out_dtype, const void* rot_prep,
                         hipStream_t stream) {
-  if (dm_disabled() || d != 128 || bits != 4 || out_dtype != AKV_F16) return AKV_ERR_UNSUPPORTED;
-  if (((uintptr_t)a.packed | (uintptr_t)a.ps0 | (uintptr_t)a.out) & 15) return AKV_ERR_UNSUPPORTED;
+  if (dm_disabled() || d != 128 || bits < 2 || bits > 4 || out_dtype != AKV_F16) return AKV_ERR_UNSUPPORTED;
+  const uintptr_t palign = bits == 4 ? 15 : bits == 3 ? 3 : 7;      // a lane reads 16 / 12 / 8 bytes of a row
+  if ((((uintptr_t)a.packed | (uintptr_t)a.ps0) & palign) || ((uintptr_t)a.out & 15)) return AKV_ERR_UNSUPPORTED;
   if (a.os0 & 7) return AKV_ERR_UNSUPPORTED;
-  if (blocks && (((uintptr_t)a.ps1 | (uintptr_t)a.ps2) & 15 || ((a.os1 | a.os2) & 7))) return AKV_ERR_UNSUPPORTED;
+  if (blocks && (((uintptr_t)a.ps1 | (uintptr_t)a.ps2) & palign || ((a.os1 | a.os2) & 7))) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(d));
   const int64_t steps = (a.n + DM_ROWS - 1) / DM_ROWS;
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
-  static bool configured = false;
-  if (!configured) {
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));
-    configured = true;
-  }
-  akv_profile_mark_begin(stream);
-  if (blocks) akv_decode_mfma_kernel<true><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);
-  else akv_decode_mfma_kernel<false><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);
+#define DM_GO(BL, BB)                                                                                          \
+  do {                                                                                                       \
+    static bool configured = false;                                                                          \
+    if (!configured) {                                                                                       \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<BL, BB>,                               \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));                \
+      configured = true;                                                                                     \
+    }                                                                                                        \
+    akv_profile_mark_begin(stream);                                                                          \
+    akv_decode_mfma_kernel<BL, BB><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);                      \
+  } while (0)
+  if (blocks) { if (bits == 4) DM_GO(true, 4); else if (bits == 3) DM_GO(true, 3); else DM_GO(true, 2); }
+  else { if (bits == 4) DM_GO(false, 4); else if (bits == 3) DM_GO(false, 3); else DM_GO(false, 2); }
+#undef DM_GO
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_decode_mfma_kernel");
   return AKV_OK;

@@ -236,6 +236,22 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("n", [1, 33, 4097])
+def test_decode_random_codes_vs_oracle(golden, dev, bits, n):
+    """Every byte value occurs: the code spreading and the table lookups of the matrix-core decode."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(100 * bits + n)
+    packed = rng.integers(0, 256, (n, tq._packed_dim), dtype=np.uint8)
+    norms = rng.lognormal(1.0, 1.0, n).astype(np.float32)
+    c, _, _ = O.get_codebook(128, bits)
+    ref = O.decode(packed, norms, golden["rotation_d128_seed42"], c, bits).astype(np.float32)
+    got = tq.decode(torch.from_numpy(packed).to(dev), torch.from_numpy(norms).to(dev)).cpu().numpy().astype(np.float32)
+    tol = 2e-3 + np.abs(ref) * 2.0 ** -11          # half a float16 ulp of the output
+    assert np.all(np.abs(got - ref) <= tol)
+    assert np.mean(got == ref) > 0.99
+
+
 @pytest.mark.parametrize("bits,out_dtype,extra", [(4, torch.float16, 0), (4, torch.float16, 16), (4, torch.bfloat16, 0),
                                                   (3, torch.float16, 0), (2, torch.float32, 4)])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
