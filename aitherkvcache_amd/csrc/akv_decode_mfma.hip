@@ -1,4 +1,4 @@
-// MFMA decode (unpack -> centroid lookup -> inverse rotation -> x norm -> float16) for the 4-, 3- and
+// MFMA decode (unpack -> centroid lookup -> inverse rotation -> x norm -> cast) for the 4-, 3- and
 // 2-bit codecs at head_dim 128: TurboQuant.decode, aither_kvcache/quantizer.py:168-197.
 //
 //   X[v, i] = n_v * sum_j c[code[v, j]] * Pi[j, i]              v_mfma_f32_16x16x32_f16
@@ -90,7 +90,7 @@ int akv_prepare_decode_mfma(const float* rotation, int d, void* prep, hipStream_
 // (position, head) entries of the cache blocks listed in a.slots; every listed block that exists is
 // decoded into the block of the same index of the output buffer (the batch decompress of
 // aither_kvcache/vllm/backend.py:1040-1091 without its gather / unique / scatter passes).
-template <bool BLOCKS, int BITS>
+template <bool BLOCKS, int BITS, int ODT>
 __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
@@ -233,24 +233,36 @@ __global__ __launch_bounds__(DM_THREADS) void akv_decode_mfma_kernel(akv_gen_arg
       const float nv[4] = {nr[mt].x, nr[mt].y, nr[mt].z, nr[mt].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        __half* orow;
+        typedef typename akv_elem<ODT>::type out_t;
+        out_t* orow;
         if constexpr (BLOCKS) {
           const int r = 16 * mt + 4 * g + i;
           if (row_p[r] < 0) continue;
-          orow = (__half*)a.out + row_o[r];
+          orow = (out_t*)a.out + row_o[r];
         } else {
           const int64_t r = base + 16 * mt + 4 * g + i;
           if (r >= a.n) continue;
-          orow = (__half*)a.out + r * a.os0;
+          orow = (out_t*)a.out + r * a.os0;
         }
-        union { dm_half8 h; uint4 u; } o;
+        // the reference multiplies the float32 rotated vector by the norm and then casts
+        float v[8];
 #pragma unroll
-        for (int nt = 0; nt < 8; ++nt) {
-          // the reference multiplies the float32 rotated vector by the norm and then casts
-          const float v = __fmul_rn(acc[mt][nt][i] * (1.f / DM_PSCALE), nv[i]);
-          o.h[nt] = (_Float16)v;
+        for (int nt = 0; nt < 8; ++nt) v[nt] = __fmul_rn(acc[mt][nt][i] * (1.f / DM_PSCALE), nv[i]);
+        if constexpr (ODT == AKV_F32) {
+          *(float4*)(orow + 8 * col) = make_float4(v[0], v[1], v[2], v[3]);
+          *(float4*)(orow + 8 * col + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        } else {
+          uint32_t w[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if constexpr (ODT == AKV_F16) {
+              w[q] = (uint32_t)__half_as_ushort(__float2half_rn(v[2 * q])) | ((uint32_t)__half_as_ushort(__float2half_rn(v[2 * q + 1])) << 16);
+            } else {
+              w[q] = (uint32_t)akv_float_to_bf16_bits(v[2 * q]) | ((uint32_t)akv_float_to_bf16_bits(v[2 * q + 1]) << 16);
+            }
+          }
+          *(uint4*)(orow + 8 * col) = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        *(uint4*)(orow + 8 * col) = o.u;
       }
     }
   }
@@ -268,27 +280,34 @@ static bool dm_disabled() {
 // returns AKV_ERR_UNSUPPORTED when the fast path does not apply (the caller then uses the general kernel)
 int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int out_dtype, const void* rot_prep,
                         hipStream_t stream) {
-  if (dm_disabled() || d != 128 || bits < 2 || bits > 4 || out_dtype != AKV_F16) return AKV_ERR_UNSUPPORTED;
+  if (dm_disabled() || d != 128 || bits < 2 || bits > 4) return AKV_ERR_UNSUPPORTED;
   const uintptr_t palign = bits == 4 ? 15 : bits == 3 ? 3 : 7;      // a lane reads 16 / 12 / 8 bytes of a row
   if ((((uintptr_t)a.packed | (uintptr_t)a.ps0) & palign) || ((uintptr_t)a.out & 15)) return AKV_ERR_UNSUPPORTED;
-  if (a.os0 & 7) return AKV_ERR_UNSUPPORTED;
+  if (a.os0 & 7) return AKV_ERR_UNSUPPORTED;      // rows of the output are written 8 elements (16 or 32 bytes) per lane
   if (blocks && (((uintptr_t)a.ps1 | (uintptr_t)a.ps2) & palign || ((a.os1 | a.os2) & 7))) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(d));
   const int64_t steps = (a.n + DM_ROWS - 1) / DM_ROWS;
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
-#define DM_GO(BL, BB)                                                                                          \
+#define DM_GO(BL, BB, OD)                                                                                      \
   do {                                                                                                       \
     static bool configured = false;                                                                          \
     if (!configured) {                                                                                       \
-      AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<BL, BB>,                               \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_decode_mfma_kernel<BL, BB, OD>,                           \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));                \
       configured = true;                                                                                     \
     }                                                                                                        \
     akv_profile_mark_begin(stream);                                                                          \
-    akv_decode_mfma_kernel<BL, BB><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);                      \
+    akv_decode_mfma_kernel<BL, BB, OD><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);                  \
   } while (0)
-  if (blocks) { if (bits == 4) DM_GO(true, 4); else if (bits == 3) DM_GO(true, 3); else DM_GO(true, 2); }
-  else { if (bits == 4) DM_GO(false, 4); else if (bits == 3) DM_GO(false, 3); else DM_GO(false, 2); }
+#define DM_GO_DT(BL, BB)                                                                                       \
+  do {                                                                                                       \
+    if (out_dtype == AKV_F16) DM_GO(BL, BB, AKV_F16);                                                        \
+    else if (out_dtype == AKV_BF16) DM_GO(BL, BB, AKV_BF16);                                                 \
+    else DM_GO(BL, BB, AKV_F32);                                                                             \
+  } while (0)
+  if (blocks) { if (bits == 4) DM_GO_DT(true, 4); else if (bits == 3) DM_GO_DT(true, 3); else DM_GO_DT(true, 2); }
+  else { if (bits == 4) DM_GO_DT(false, 4); else if (bits == 3) DM_GO_DT(false, 3); else DM_GO_DT(false, 2); }
+#undef DM_GO_DT
 #undef DM_GO
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_decode_mfma_kernel");

@@ -252,6 +252,27 @@ def test_decode_random_codes_vs_oracle(golden, dev, bits, n):
     assert np.mean(got == ref) > 0.99
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_other_output_dtypes_vs_oracle(golden, dev, bits, dtype):
+    tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev), dtype=dtype)
+    tq.rotation = torch.from_numpy(golden["rotation_d128_seed42"]).to(dev)
+    rng = np.random.default_rng(7 * bits)
+    n = 1031
+    packed = rng.integers(0, 256, (n, tq._packed_dim), dtype=np.uint8)
+    norms = rng.lognormal(1.0, 1.0, n).astype(np.float32)
+    c, _, _ = O.get_codebook(128, bits)
+    ref = O.decode(packed, norms, golden["rotation_d128_seed42"], c, bits, out_dtype=np.float32)
+    out = tq.decode(torch.from_numpy(packed).to(dev), torch.from_numpy(norms).to(dev))
+    assert out.dtype == dtype
+    got = out.float().cpu().numpy()
+    scale = np.abs(ref).max(axis=1, keepdims=True)
+    if dtype == torch.float32:
+        assert np.all(np.abs(got - ref) <= 4e-6 * scale + 1e-7)       # float32 sums in another order
+    else:
+        assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -8 + 4e-6 * scale)   # half a bfloat16 ulp
+
+
 @pytest.mark.parametrize("bits,out_dtype,extra", [(4, torch.float16, 0), (4, torch.float16, 16), (4, torch.bfloat16, 0),
                                                   (3, torch.float16, 0), (2, torch.float32, 4)])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
