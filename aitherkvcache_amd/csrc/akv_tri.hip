@@ -8,13 +8,32 @@
 // with delta = float(key_pos) - float(query_pos) and the phase formed by ONE float32 multiply
 // as the reference does (phases reach ~3e4 rad, so the argument must match to the last bit
 // before sin/cos).  The phases are shared by the GQ query heads of the kv head.  A running
-// softmax is kept per wavefront; the weighted value coefficients are scatter-added into the
-// wavefront's private LDS bins (D floats per query head).  A second kernel merges the NSPLIT
-// partials with the log-sum-exp rule and writes float32.
+// softmax is kept per wavefront.  The weighted sum of the sparse value rows is formed, at
+// head_dim 128 (DENSE), on the matrix cores: the 64 tokens of a chunk scatter their retained
+// coefficients into a dense [pair][token][even, odd] float16 tile in LDS (an int4 code c stands for
+// (2c - 15)/15, and 2c - 15 is exact in float16), the softmax weights times the value scale go
+// through LDS into the operand layout as float16 hi + lo, and sixteen v_mfma_f32_16x16x32_f16
+// multiply them (rows = pairs, columns = (query head, even/odd, hi/lo), k = (token, even/odd) with
+// zeros where the parities differ).  To keep the weights inside float16 the running maximum is
+// taken over score + ln(value scale), so weight x scale <= 1.  Other head dims scatter-add into
+// LDS bins with atomics.  A second kernel merges the NSPLIT partials with the log-sum-exp rule
+// and writes float32.
 #include "akv_common.h"
 
 #define TRI_MAX_SPLITS 128
 #define TRI_WAVES 4
+// DENSE value tile of a wavefront: 64 pairs x (64 tokens x 4 bytes + 16 bytes of padding, so that the
+// sixteen pairs read by one operand load fall into different banks), then the weight table
+// [8 = hi/lo x 4 query heads] x (64 tokens x 2 bytes + 8)
+#define TRI_VT_PITCH 272
+#define TRI_WT_PITCH 136
+#define TRI_VT_BYTES (64 * TRI_VT_PITCH)
+#define TRI_DENSE_WAVE_BYTES (TRI_VT_BYTES + 8 * TRI_WT_PITCH)
+#define TRI_WSCALE 16384.f          // weights are carried as float16 of (weight x scale) x 2^14
+
+typedef _Float16 tri_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 tri_half2 __attribute__((ext_vector_type(2)));
+typedef float tri_float4 __attribute__((ext_vector_type(4)));
 
 struct tri_args {
   const void* query; int q_dtype;
@@ -70,12 +89,20 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
   // DENSE (head_dim 128): instead of bins updated by LDS atomics (which serialise when many tokens
   // retain the same pair -- the usual case), each wavefront has a 16-token x 128-coordinate tile
   // and a 64 x GQ weight table; a lane owns one coordinate pair and its sums stay in registers
-  float* tile = acc_base + (size_t)wave * (16 * 128 + 64 * GQ);
-  float* wtab = tile + 16 * 128;
-  if (DENSE) {
-    for (int i = lane; i < 16 * 128; i += 64) tile[i] = 0.f;   // every use leaves the tile zero again
+  unsigned char* vt = (unsigned char*)acc_base + (size_t)wave * TRI_DENSE_WAVE_BYTES;
+  unsigned char* wt = vt + TRI_VT_BYTES;
+  if (DENSE) {   // every use leaves the tile zero again; weight rows of absent query heads stay zero
+    for (int i = lane; i < TRI_DENSE_WAVE_BYTES / 4; i += 64) ((uint32_t*)vt)[i] = 0u;
   }
+  // operand roles of the lane: column n = q + 4 e + 8 hl of the weight operand, row m of a 16-pair tile
+  const int col_n = lane & 15, grp = lane >> 4;
+  const int col_q = col_n & 3, col_e = (col_n >> 2) & 1;
+  const uint32_t sel_lo = col_e ? 0x01000c0cu : 0x0c0c0100u;   // first token of a dword into the lane's parity slot
+  const uint32_t sel_hi = col_e ? 0x03020c0cu : 0x0c0c0302u;   // second token
+  const unsigned char* wt_rd = wt + (4 * (col_n >> 3) + col_q) * TRI_WT_PITCH + 8 * grp;
+  const unsigned char* vt_rd = vt + col_n * TRI_VT_PITCH + 16 * grp;
   const int D = a.D, F = a.F;
+  constexpr int FU = F12 ? 12 : 4;   // pair loops: all twelve steps unrolled (static register indices), else four
   const int gqa = a.QH / a.KVH;
   const int b = blockIdx.z, h = blockIdx.y;
   const int split = blockIdx.x * TRI_WAVES + wave;
@@ -105,56 +132,87 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       for (int i = lane; i < GQ * D; i += 64) acc[i] = 0.f;
     }
     __syncthreads();
-    float o[GQ][2];
+    tri_float4 oacc[4];     // DENSE: pairs 16 mt + 4 grp + i of column col_n
 #pragma unroll
-    for (int q = 0; q < GQ; ++q) o[q][0] = o[q][1] = 0.f;
+    for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
 
     float m[GQ], l[GQ];
 #pragma unroll
     for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
 
+    // One chunk of 64 tokens is fetched while the chunk before it is worked on: the token's position,
+    // both scales and (F = 12, aligned arrays) its index and coefficient bytes as three dwords each.
+    // Tokens past the end of the range re-read its last token (never out of bounds; S >= 1 here).
+    // (Everything is kept as loaded -- raw halfwords, the position as two dwords -- and converted where
+    // it is used, so that no load has to be waited for at the point of the fetch.)
+    struct tri_raw { uint32_t ki[3], kc[3], vi[3], vc[3]; uint32_t kp_lo, kp_hi; unsigned short ksc, vsc; };
+    const bool kp_wide = a.kpos && a.kp_itype == AKV_I64;
+    const unsigned char* kp_base = a.kpos ? (const unsigned char*)a.kpos : (const unsigned char*)a.theta;
+    auto fetch = [&](tri_raw& r, int64_t c0) {
+      const int64_t tc = max((int64_t)0, min(c0 + lane, s1 - 1));
+      const int64_t row = ((int64_t)b * a.S + tc) * a.KVH + h;
+      // position: low dword, and the high dword of a 64-bit entry (the low one again otherwise); without
+      // an array of positions the loads read the first frequency and the value is not used
+      const int64_t pe = a.kpos ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
+      r.kp_lo = *(const uint32_t*)(kp_base + pe);
+      r.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
+      r.ksc = ((const unsigned short*)a.k_sc)[row];
+      r.vsc = ((const unsigned short*)a.v_sc)[row];
+      if (F12) {
+        const uint32_t* p0 = (const uint32_t*)(a.k_idx + row * 12);
+        const uint32_t* p1 = (const uint32_t*)(a.k_cf + row * 12);
+        const uint32_t* p2 = (const uint32_t*)(a.v_idx + row * 12);
+        const uint32_t* p3 = (const uint32_t*)(a.v_cf + row * 12);
+#pragma unroll
+        for (int w = 0; w < 3; ++w) { r.ki[w] = p0[w]; r.kc[w] = p1[w]; r.vi[w] = p2[w]; r.vc[w] = p3[w]; }
+      }
+    };
+    tri_raw cur;
+    fetch(cur, s0);
     for (int64_t c0 = s0; c0 < s1; c0 += 64) {
       const int64_t t = c0 + lane;
       const bool valid = t < s1;
       const int64_t tc = valid ? t : s1 - 1;
       const int64_t row = ((int64_t)b * a.S + tc) * a.KVH + h;
-      const float kp = a.kpos ? (float)akv_load_index(a.kpos, a.kp_itype, (int64_t)b * a.S + tc) : (float)tc;
+      tri_raw nxt;
+      fetch(nxt, c0 + 64);
+      const float kp = !a.kpos ? (float)tc
+                       : kp_wide ? (float)(int64_t)(((uint64_t)cur.kp_hi << 32) | cur.kp_lo) : (float)(int32_t)cur.kp_lo;
       const float delta = __fsub_rn(kp, qp);
-      const float ksc = __half2float(a.k_sc[row]);
+      const float ksc = __half2float(__ushort_as_half(cur.ksc));
       float sc[GQ];
 #pragma unroll
       for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
-      uint32_t ki[3], kc[3];
-      if (F12) {   // the token's 12 index bytes and 12 coefficient bytes as three dwords each
-        const uint32_t* pi = (const uint32_t*)(a.k_idx + row * 12);
-        const uint32_t* pc = (const uint32_t*)(a.k_cf + row * 12);
-#pragma unroll
-        for (int w = 0; w < 3; ++w) { ki[w] = pi[w]; kc[w] = pc[w]; }
-      }
-#pragma unroll 4
-      for (int f = 0; f < F; ++f) {
-        const uint32_t idx = F12 ? (ki[f >> 2] >> (8 * (f & 3))) & 255u : a.k_idx[row * F + f];
-        const uint32_t cf = F12 ? (kc[f >> 2] >> (8 * (f & 3))) & 255u : a.k_cf[row * F + f];
+#pragma unroll FU
+      for (int f = 0; f < (F12 ? 12 : F); ++f) {
+        const uint32_t idx = F12 ? (cur.ki[f >> 2] >> (8 * (f & 3))) & 255u : a.k_idx[row * F + f];
+        const uint32_t cf = F12 ? (cur.kc[f >> 2] >> (8 * (f & 3))) & 255u : a.k_cf[row * F + f];
         const float k0 = __fmul_rn(dq[cf >> 4], ksc), k1 = __fmul_rn(dq[cf & 15u], ksc);
         const float ph = __fmul_rn(delta, theta[idx]);
         float sn, cs;
         tri_sincos(ph, sn, cs);
+        // q_e (k0 cos - k1 sin) + q_o (k1 cos + k0 sin): the key pair is turned once for all query heads
+        const float ka = k0 * cs - k1 * sn;
+        const float kb = k1 * cs + k0 * sn;
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
           const float2 qq = *(const float2*)(q_lds + (idx * GQ + q) * 2);
-          const float qe = qq.x, qo = qq.y;
-          const float c = qe * k0 + qo * k1;
-          const float s = qo * k0 - qe * k1;
-          sc[q] += c * cs + s * sn;
+          sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
         }
       }
       float p[GQ];
       bool rescale = false;
       float alpha[GQ];
+      // DENSE: the value scale enters the running maximum, so that p x scale <= 1 (float16 operand)
+      float vsc = 0.f, bias = 0.f;
+      if (DENSE) {
+        vsc = __half2float(__ushort_as_half(cur.vsc));
+        bias = __logf(fmaxf(vsc, 5.9604645e-8f));
+      }
 #pragma unroll
       for (int q = 0; q < GQ; ++q) {
         const float sv = valid ? sc[q] * inv_sqrt_d : -INFINITY;
-        const float mn = fmaxf(m[q], akv_wave_max(sv));
+        const float mn = fmaxf(m[q], akv_wave_max(sv + bias));
         alpha[q] = __expf(m[q] - mn);
         rescale |= (mn != m[q]);
         p[q] = valid ? __expf(sv - mn) : 0.f;
@@ -163,56 +221,60 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       }
       if (DENSE) {
         if (rescale) {  // wavefront-uniform: m is the same in every lane
+          float asel = alpha[0];
+          if (GQ == 4) asel = col_q == 1 ? alpha[1 % GQ] : col_q == 2 ? alpha[2 % GQ] : col_q == 3 ? alpha[3 % GQ] : asel;
 #pragma unroll
-          for (int q = 0; q < GQ; ++q) { o[q][0] *= alpha[q]; o[q][1] *= alpha[q]; }
+          for (int mt = 0; mt < 4; ++mt) oacc[mt] *= asel;
         }
+        // weights: float16 hi (truncated) + lo of p x scale x 2^14, one halfword per (column, token)
 #pragma unroll
-        for (int q = 0; q < GQ; ++q) wtab[lane * GQ + q] = p[q];
-        float vsc = 0.f;
-        uint32_t vi[3] = {0, 0, 0}, vc[3] = {0, 0, 0};
+        for (int q = 0; q < GQ; ++q) {
+          const float w = p[q] * vsc * TRI_WSCALE;
+          auto h2 = __builtin_amdgcn_cvt_pkrtz(w, 0.f);
+          auto l2 = __builtin_amdgcn_cvt_pkrtz(w - (float)h2[0], 0.f);
+          union { decltype(h2) h; uint32_t u; } hb, lb;
+          hb.h = h2; lb.h = l2;
+          *(uint16_t*)(wt + q * TRI_WT_PITCH + 2 * lane) = (uint16_t)hb.u;
+          *(uint16_t*)(wt + (4 + q) * TRI_WT_PITCH + 2 * lane) = (uint16_t)lb.u;
+        }
         if (valid) {
-          vsc = __half2float(a.v_sc[row]);
-          if (F12) {
-            const uint32_t* pi = (const uint32_t*)(a.v_idx + row * 12);
-            const uint32_t* pc = (const uint32_t*)(a.v_cf + row * 12);
-#pragma unroll
-            for (int w = 0; w < 3; ++w) { vi[w] = pi[w]; vc[w] = pc[w]; }
+#pragma unroll FU
+          for (int f = 0; f < (F12 ? 12 : F); ++f) {
+            const uint32_t idx = F12 ? (cur.vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+            const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+            // (2a - 15, 2b - 15) as a float16 pair: 0x6400 + n is float16(1024 + n), minus 1039 is exact
+            union { uint32_t u; tri_half2 h; } cv;
+            cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+            cv.h = cv.h - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+            *(uint32_t*)(vt + (idx & 63u) * TRI_VT_PITCH + 4 * lane) = cv.u;
           }
         }
-        float* my_row = tile + (lane & 15) * 128;
-#pragma unroll 1
-        for (int sub = 0; sub < 4; ++sub) {
-          const bool mine = valid && (lane >> 4) == sub;
-          if (mine) {
-#pragma unroll 4
-            for (int f = 0; f < F; ++f) {
-              const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
-              const uint32_t cf = F12 ? (vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
-              *(float2*)(my_row + 2 * idx) = make_float2(__fmul_rn(dq[cf >> 4], vsc), __fmul_rn(dq[cf & 15u], vsc));
-            }
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll 4
-          for (int t = 0; t < 16; ++t) {
-            const float2 v = *(const float2*)(tile + t * 128 + 2 * lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int q = 0; q < GQ; ++q) {
-              const float w = wtab[(16 * sub + t) * GQ + q];
-              o[q][0] = fmaf(w, v.x, o[q][0]);
-              o[q][1] = fmaf(w, v.y, o[q][1]);
-            }
+        for (int ks = 0; ks < 4; ++ks) {     // 16 tokens per step: k = 2 x token + parity
+          const uint2 wr = *(const uint2*)(wt_rd + 32 * ks);
+          union { uint32_t u[4]; tri_half8 h; } bw;
+          bw.u[0] = __builtin_amdgcn_perm(wr.x, wr.x, sel_lo);
+          bw.u[1] = __builtin_amdgcn_perm(wr.x, wr.x, sel_hi);
+          bw.u[2] = __builtin_amdgcn_perm(wr.y, wr.y, sel_lo);
+          bw.u[3] = __builtin_amdgcn_perm(wr.y, wr.y, sel_hi);
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) {
+            union { uint4 u; tri_half8 h; } av;
+            av.u = *(const uint4*)(vt_rd + mt * 16 * TRI_VT_PITCH + 64 * ks);
+            oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.h, bw.h, oacc[mt], 0, 0, 0);
           }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          if (mine) {
-#pragma unroll 4
-            for (int f = 0; f < F; ++f) {
-              const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
-              *(float2*)(my_row + 2 * idx) = make_float2(0.f, 0.f);
-            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (valid) {
+#pragma unroll FU
+          for (int f = 0; f < (F12 ? 12 : F); ++f) {
+            const uint32_t idx = F12 ? (cur.vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+            *(uint32_t*)(vt + (idx & 63u) * TRI_VT_PITCH + 4 * lane) = 0u;
           }
         }
       } else {
@@ -225,19 +287,12 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       }
       if (valid) {
-        const float vsc = __half2float(a.v_sc[row]);
-        uint32_t vi[3], vc[3];
-        if (F12) {
-          const uint32_t* pi = (const uint32_t*)(a.v_idx + row * 12);
-          const uint32_t* pc = (const uint32_t*)(a.v_cf + row * 12);
-#pragma unroll
-          for (int w = 0; w < 3; ++w) { vi[w] = pi[w]; vc[w] = pc[w]; }
-        }
-#pragma unroll 4
-        for (int f = 0; f < F; ++f) {
-          const uint32_t idx = F12 ? (vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
-          const uint32_t cf = F12 ? (vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
-          const float v0 = __fmul_rn(dq[cf >> 4], vsc), v1 = __fmul_rn(dq[cf & 15u], vsc);
+        const float vs = __half2float(__ushort_as_half(cur.vsc));
+#pragma unroll FU
+        for (int f = 0; f < (F12 ? 12 : F); ++f) {
+          const uint32_t idx = F12 ? (cur.vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
+          const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+          const float v0 = __fmul_rn(dq[cf >> 4], vs), v1 = __fmul_rn(dq[cf & 15u], vs);
 #pragma unroll
           for (int q = 0; q < GQ; ++q) {
             atomicAdd(&acc[q * D + 2 * idx], p[q] * v0);
@@ -249,14 +304,27 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       }
+      cur = nxt;
     }
     if (split < a.nsplit) {
 #pragma unroll
       for (int q = 0; q < GQ; ++q) {
         const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
         const float lsum = akv_wave_sum(l[q]);
-        if (DENSE) *(float2*)(a.part_acc + slot * D + 2 * lane) = make_float2(o[q][0], o[q][1]);
-        else for (int i = lane; i < D; i += 64) a.part_acc[slot * D + i] = acc[q * D + i];
+        if (DENSE) {
+          // hi column + lo column (eight lanes to the right), then the lanes of column (q, parity) store
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float hi = oacc[mt][i];
+              const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
+              if (col_n < 8 && col_q == q)
+                a.part_acc[slot * D + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
+            }
+        } else {
+          for (int i = lane; i < D; i += 64) a.part_acc[slot * D + i] = acc[q * D + i];
+        }
         if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
       }
     }
@@ -365,8 +433,18 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   const bool dense = d == 128;
 #define TRI_LAUNCH(GQV)                                                                                   \
   do {                                                                                                    \
-    const size_t per_wave = dense ? (size_t)(16 * 128 + 64 * GQV) : (size_t)GQV * d;                      \
+    const size_t per_wave = dense ? (size_t)(TRI_DENSE_WAVE_BYTES / 4) : (size_t)GQV * d;                 \
     const size_t lds = ((size_t)d / 2 + (size_t)GQV * d + 16 + TRI_WAVES * per_wave) * sizeof(float);     \
+    if (dense) {   /* more than 64 KB of dynamic LDS has to be allowed once per kernel */               \
+      static bool configured = false;                                                                     \
+      if (!configured) {                                                                                  \
+        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, true, true>,                      \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
+        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, false, true>,                     \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
+        configured = true;                                                                                \
+      }                                                                                                   \
+    }                                                                                                     \
     if (dense && f12) tri_decode_kernel<GQV, true, true><<<grid, 256, lds, stream>>>(a);                  \
     else if (dense) tri_decode_kernel<GQV, false, true><<<grid, 256, lds, stream>>>(a);                   \
     else if (f12) tri_decode_kernel<GQV, true, false><<<grid, 256, lds, stream>>>(a);                     \
