@@ -331,6 +331,257 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
   }
 }
 
+// ----------------------------------------------------------------------------------
+// head_dim 128, F = 12, up to 8 kv heads: one workgroup takes a token range for ALL kv heads
+// ----------------------------------------------------------------------------------
+// In the cache a token's rows of the kv heads lie side by side (12 bytes each), so a wavefront that
+// follows one head reads 12 bytes out of every 12 x kv_heads and touches a cache line per lane.
+// Here wavefront h still works on head h, but the chunk of 64 tokens x kv_heads rows is fetched by
+// the whole workgroup as the contiguous run of bytes it is (thread i <-> row i: one dwordx3 load per
+// array covers 768 contiguous bytes per wavefront), one chunk ahead, and passes through LDS:
+// [array][head][token] entries of 16 bytes -- the row's 12 bytes and, in the fourth dword of the
+// index entries, the row's scale -- written and read by one 16-byte LDS operation each (a head's
+// tokens lie 32 bytes apart from the next head's, which spreads the writes of a token's heads over
+// the banks).  Two workgroup barriers per chunk
+// (staging written -> read, read -> overwritten).  The dense value tile takes 32 tokens at a time.
+#define TRH_HEAD_PITCH (64 * 16 + 32)
+#define TRH_VT_PITCH 144            // 32 tokens x 4 bytes + 16
+#define TRH_VT_BYTES (64 * TRH_VT_PITCH)
+#define TRH_WT_PITCH (64 * 4 + 64)    // [4 query heads] x (64 tokens x (hi, lo) + 64: heads 16 banks apart)
+#define TRH_WAVE_BYTES (TRH_VT_BYTES + 4 * TRH_WT_PITCH)
+
+__device__ __forceinline__ float tri_row16_max(float v) {
+  // maximum over the lane's row of 16 by row rotations (data-parallel primitives, no LDS crossbar)
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128 /*row_ror:8*/, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124 /*row_ror:4*/, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122 /*row_ror:2*/, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121 /*row_ror:1*/, 0xf, 0xf, false)));
+  return v;
+}
+__device__ __forceinline__ float tri_wave_max(float v) {
+  v = tri_row16_max(v);
+  // the four rows: v_permlane32_swap / v_permlane16_swap fed the same value twice leave
+  // (rows 0,1,0,1 | 2,3,2,3) and (rows 0,0,2,2 | 1,1,3,3)
+  auto x = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(x[0]), __uint_as_float(x[1]));
+  auto y = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(y[0]), __uint_as_float(y[1]));
+}
+
+static size_t tri_heads_lds_bytes(int kvh, int gqa_pass) {
+  return 64 * sizeof(float) + (size_t)kvh * gqa_pass * 128 * sizeof(float) + 64 +
+         4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRH_WAVE_BYTES;
+}
+
+template <int GQ>
+__global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int KVH = a.KVH;
+  float* theta = (float*)lds_raw;                               // [64]
+  float* q_lds = theta + 64;                                    // [KVH][64 pairs][GQ][even, odd]
+  unsigned char* stage = (unsigned char*)(q_lds + (size_t)KVH * GQ * 128 + 16);   // [4 arrays][KVH] x TRH_HEAD_PITCH
+  unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
+  const int tid = threadIdx.x, lane = tid & 63, h = tid >> 6;   // wavefront = kv head
+  unsigned char* vt = tiles + (size_t)h * TRH_WAVE_BYTES;
+  unsigned char* wt = vt + TRH_VT_BYTES;
+  for (int i = lane; i < TRH_WAVE_BYTES / 4; i += 64) ((uint32_t*)vt)[i] = 0u;
+  const int col_n = lane & 15, grp = lane >> 4;
+  const int col_q = col_n & 3, col_e = (col_n >> 2) & 1;
+  // a weight dword is (hi | lo << 16) of one token: the lane takes its half into its parity slot
+  const uint32_t sel_w = (col_n >> 3) ? (col_e ? 0x03020c0cu : 0x0c0c0302u) : (col_e ? 0x01000c0cu : 0x0c0c0100u);
+  const unsigned char* wt_rd = wt + col_q * TRH_WT_PITCH + 16 * grp;
+  const unsigned char* vt_rd = vt + col_n * TRH_VT_PITCH + 16 * grp;
+  const int gqa = a.QH / KVH;
+  const int b = blockIdx.y, split = blockIdx.x;
+  const float inv_sqrt_d = 1.0f / sqrtf(128.f);
+  if (tid < 64) theta[tid] = a.theta[tid];
+
+  const int64_t per = (a.S + a.nsplit - 1) / a.nsplit;
+  const int64_t s0 = min(a.S, (int64_t)split * per);
+  const int64_t s1 = min(a.S, s0 + per);
+  const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)a.S;
+  const bool kp_wide = a.kpos && a.kp_itype == AKV_I64;
+  const unsigned char* kp_base = a.kpos ? (const unsigned char*)a.kpos : (const unsigned char*)a.theta;
+
+  // the thread's row of a chunk: token tid / KVH, head tid % KVH
+  const int my_t = tid / KVH, my_h = tid - my_t * KVH;
+  unsigned char* st_wr = stage + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
+  const unsigned char* st_rd = stage + (size_t)h * TRH_HEAD_PITCH + lane * 16;
+  const size_t arr = (size_t)KVH * TRH_HEAD_PITCH;
+  const int64_t last_row = ((int64_t)b * a.S + max(s1, (int64_t)1)) * KVH - 1;
+
+  struct tri_rows { uint32_t x[4][3]; unsigned short ksc, vsc; uint32_t kp_lo, kp_hi; };
+  auto fetch = [&](tri_rows& r, int64_t c0) {
+    const int64_t row = min(((int64_t)b * a.S + c0) * KVH + tid, last_row);   // rows past the range: its last row
+    const uint32_t* p0 = (const uint32_t*)(a.k_idx + row * 12);
+    const uint32_t* p1 = (const uint32_t*)(a.k_cf + row * 12);
+    const uint32_t* p2 = (const uint32_t*)(a.v_idx + row * 12);
+    const uint32_t* p3 = (const uint32_t*)(a.v_cf + row * 12);
+#pragma unroll
+    for (int w = 0; w < 3; ++w) { r.x[0][w] = p0[w]; r.x[1][w] = p1[w]; r.x[2][w] = p2[w]; r.x[3][w] = p3[w]; }
+    r.ksc = ((const unsigned short*)a.k_sc)[row];
+    r.vsc = ((const unsigned short*)a.v_sc)[row];
+    // the wavefront's own token positions (lane = token), as two dwords
+    const int64_t tc = max((int64_t)0, min(c0 + lane, s1 - 1));
+    const int64_t pe = a.kpos ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
+    r.kp_lo = *(const uint32_t*)(kp_base + pe);
+    r.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
+  };
+
+  for (int qg = 0; qg < gqa; qg += GQ) {
+    __syncthreads();
+    for (int i = tid; i < KVH * GQ * 128; i += blockDim.x) {
+      const int hh = i / (GQ * 128), rem = i - hh * (GQ * 128);
+      const int q = rem >> 7, d = rem & 127;
+      const int64_t off = ((int64_t)b * a.QH + (hh * gqa + qg + q)) * 128 + d;
+      float v;
+      if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
+      else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
+      else v = akv_elem<AKV_F32>::load(a.query, off);
+      q_lds[(size_t)hh * GQ * 128 + ((d >> 1) * GQ + q) * 2 + (d & 1)] = v;
+    }
+    const float* qh = q_lds + (size_t)h * GQ * 128;
+    tri_float4 oacc[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
+    float m[GQ], l[GQ];
+#pragma unroll
+    for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
+
+    tri_rows nxt;
+    fetch(nxt, s0);
+    for (int64_t c0 = s0; c0 < s1; c0 += 64) {
+      // the chunk fetched during the previous step goes to the staging area, the next one is requested
+#pragma unroll
+      for (int A = 0; A < 4; ++A)
+        *(uint4*)(st_wr + A * arr) = make_uint4(nxt.x[A][0], nxt.x[A][1], nxt.x[A][2], A == 0 ? nxt.ksc : nxt.vsc);
+      const uint32_t kp_lo = nxt.kp_lo, kp_hi = nxt.kp_hi;
+      __syncthreads();
+      fetch(nxt, c0 + 64);
+      const uint4 e0 = *(const uint4*)(st_rd), e1 = *(const uint4*)(st_rd + arr);
+      const uint4 e2 = *(const uint4*)(st_rd + 2 * arr), e3 = *(const uint4*)(st_rd + 3 * arr);
+      __syncthreads();
+      const uint32_t ki[3] = {e0.x, e0.y, e0.z}, kc[3] = {e1.x, e1.y, e1.z};
+      const uint32_t vi[3] = {e2.x, e2.y, e2.z}, vc[3] = {e3.x, e3.y, e3.z};
+      const float ksc = __half2float(__ushort_as_half((unsigned short)e0.w));
+      const float vsc = __half2float(__ushort_as_half((unsigned short)e2.w));
+
+      const int64_t t = c0 + lane;
+      const bool valid = t < s1;
+      const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
+                       : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
+      const float delta = __fsub_rn(kp, qp);
+      const float ksc15 = ksc * (1.f / 15.f);
+      float sc[GQ];
+#pragma unroll
+      for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+#pragma unroll
+      for (int f = 0; f < 12; ++f) {
+        const uint32_t idx = (ki[f >> 2] >> (8 * (f & 3))) & 63u;
+        const uint32_t cf = (kc[f >> 2] >> (8 * (f & 3))) & 255u;
+        // (2c - 15)/15 for the reference's fl(fl(c/7.5) - 1): equal to a relative 1e-7
+        const float k0 = (float)(int)(2 * (cf >> 4) - 15) * ksc15, k1 = (float)(int)(2 * (cf & 15u) - 15) * ksc15;
+        const float ph = __fmul_rn(delta, theta[idx]);
+        float sn, cs;
+        tri_sincos(ph, sn, cs);
+        const float ka = k0 * cs - k1 * sn;
+        const float kb = k1 * cs + k0 * sn;
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) {
+          const float2 qq = *(const float2*)(qh + (idx * GQ + q) * 2);
+          sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+        }
+      }
+      float p[GQ], alpha[GQ];
+      bool rescale = false;
+      const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
+#pragma unroll
+      for (int q = 0; q < GQ; ++q) {
+        const float sv = valid ? sc[q] * inv_sqrt_d : -INFINITY;
+        const float mn = fmaxf(m[q], tri_wave_max(sv + bias));
+        alpha[q] = __expf(m[q] - mn);
+        rescale |= (mn != m[q]);
+        p[q] = valid ? __expf(sv - mn) : 0.f;
+        l[q] = l[q] * alpha[q] + p[q];
+        m[q] = mn;
+      }
+      if (rescale) {  // wavefront-uniform: m is the same in every lane
+        float asel = alpha[0];
+        if (GQ == 4) asel = col_q == 1 ? alpha[1 % GQ] : col_q == 2 ? alpha[2 % GQ] : col_q == 3 ? alpha[3 % GQ] : asel;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) oacc[mt] *= asel;
+      }
+#pragma unroll
+      for (int q = 0; q < GQ; ++q) {
+        const float w = p[q] * vsc * TRI_WSCALE;
+        auto h2 = __builtin_amdgcn_cvt_pkrtz(w, 0.f);
+        auto l2 = __builtin_amdgcn_cvt_pkrtz(w - (float)h2[0], 0.f);
+        union { decltype(h2) hv; uint32_t u; } hb, lb;
+        hb.hv = h2; lb.hv = l2;
+        *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = (hb.u & 0xffffu) | (lb.u << 16);
+      }
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {      // the tile holds 32 tokens
+        const bool mine = valid && (lane >> 5) == pass;
+        if (mine) {
+#pragma unroll
+          for (int f = 0; f < 12; ++f) {
+            const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
+            const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
+            union { uint32_t u; tri_half2 hv; } cv;
+            cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+            cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+            *(uint32_t*)(vt + idx * TRH_VT_PITCH + 4 * (lane & 31)) = cv.u;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const uint4 wr = *(const uint4*)(wt_rd + 64 * (2 * pass + ks));
+          union { uint32_t u[4]; tri_half8 hv; } bw;
+          bw.u[0] = __builtin_amdgcn_perm(wr.x, wr.x, sel_w);
+          bw.u[1] = __builtin_amdgcn_perm(wr.y, wr.y, sel_w);
+          bw.u[2] = __builtin_amdgcn_perm(wr.z, wr.z, sel_w);
+          bw.u[3] = __builtin_amdgcn_perm(wr.w, wr.w, sel_w);
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) {
+            union { uint4 u; tri_half8 hv; } av;
+            av.u = *(const uint4*)(vt_rd + mt * 16 * TRH_VT_PITCH + 64 * ks);
+            oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.hv, bw.hv, oacc[mt], 0, 0, 0);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (mine) {
+#pragma unroll
+          for (int f = 0; f < 12; ++f) {
+            const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
+            *(uint32_t*)(vt + idx * TRH_VT_PITCH + 4 * (lane & 31)) = 0u;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < GQ; ++q) {
+      const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
+      const float lsum = akv_wave_sum(l[q]);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float hi = oacc[mt][i];
+          const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
+          if (col_n < 8 && col_q == q)
+            a.part_acc[slot * 128 + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
+        }
+      if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
+    }
+  }
+}
+
 // one workgroup per (batch, query head): split weights once, then one thread per coordinate
 __global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict__ part_acc,
                                                          const float* __restrict__ part_ml,
@@ -425,12 +676,44 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
   const int gqa = num_q_heads / num_kv_heads;
-  dim3 grid(a.nsplit / TRI_WAVES, num_kv_heads, batch);
-  akv_profile_mark_begin(stream);
   // rows of 12 bytes can be read as dwords when the arrays are 4-byte aligned
   const bool f12 = num_freqs == 12 &&
                    ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
   const bool dense = d == 128;
+  if (dense && f12 && num_kv_heads <= 8) {
+    // one workgroup per (token range, batch element), a wavefront per kv head
+    const int gq = gqa % 4 == 0 ? 4 : 1;
+    const size_t lds = tri_heads_lds_bytes(num_kv_heads, gq);
+    if (lds <= 160 * 1024) {
+      int cus = akv_cached_cu_count();
+      if (cus <= 0) cus = 256;
+      int64_t n = (cus + batch - 1) / batch;
+      const int64_t by_len = (seq_len + 63) / 64;
+      if (n > by_len) n = by_len;
+      if (n > TRI_MAX_SPLITS) n = TRI_MAX_SPLITS;
+      if (n < 1) n = 1;
+      a.nsplit = (int)n;
+      a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
+      static size_t configured4 = 0, configured1 = 0;
+      size_t& configured = gq == 4 ? configured4 : configured1;
+      if (configured < lds) {
+        if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        configured = lds;
+      }
+      dim3 hgrid(a.nsplit, batch);
+      akv_profile_mark_begin(stream);
+      if (gq == 4) tri_decode_heads_kernel<4><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+      else tri_decode_heads_kernel<1><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+      akv_profile_mark_end(stream);
+      AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
+      tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
+      AKV_LAUNCH_CHECK("tri_reduce_kernel");
+      return AKV_OK;
+    }
+  }
+  dim3 grid(a.nsplit / TRI_WAVES, num_kv_heads, batch);
+  akv_profile_mark_begin(stream);
 #define TRI_LAUNCH(GQV)                                                                                   \
   do {                                                                                                    \
     const size_t per_wave = dense ? (size_t)(TRI_DENSE_WAVE_BYTES / 4) : (size_t)GQV * d;                 \
