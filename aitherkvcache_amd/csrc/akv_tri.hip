@@ -471,24 +471,36 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
                        : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
       const float delta = __fsub_rn(kp, qp);
-      const float ksc15 = ksc * (1.f / 15.f);
+      const float kscale = ksc * (inv_sqrt_d / 15.f);
       float sc[GQ];
 #pragma unroll
       for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+      // Per word of four pairs: the index bytes times 4 (a pair index is below 64, so the shift stays
+      // inside its byte) and the two nibbles of every coefficient byte in bytes of their own; a byte
+      // then becomes a float by one conversion.  A code c stands for (2c - 15)/15 x scale -- equal to
+      // the reference's fl(fl(c/7.5) - 1) x scale to a relative 1e-7 -- and scale/15 multiplies the
+      // finished sum instead of every coefficient.
+      uint32_t ki4[3], chi[3], clo[3];
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        ki4[w] = (ki[w] & 0x3f3f3f3fu) << 2;
+        chi[w] = (kc[w] >> 4) & 0x0f0f0f0fu;
+        clo[w] = kc[w] & 0x0f0f0f0fu;
+      }
 #pragma unroll
       for (int f = 0; f < 12; ++f) {
-        const uint32_t idx = (ki[f >> 2] >> (8 * (f & 3))) & 63u;
-        const uint32_t cf = (kc[f >> 2] >> (8 * (f & 3))) & 255u;
-        // (2c - 15)/15 for the reference's fl(fl(c/7.5) - 1): equal to a relative 1e-7
-        const float k0 = (float)(int)(2 * (cf >> 4) - 15) * ksc15, k1 = (float)(int)(2 * (cf & 15u) - 15) * ksc15;
-        const float ph = __fmul_rn(delta, theta[idx]);
+        const uint32_t idx4 = (ki4[f >> 2] >> (8 * (f & 3))) & 255u;          // byte offset of theta[idx]
+        const float k0 = fmaf((float)((chi[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
+        const float k1 = fmaf((float)((clo[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
+        const float ph = __fmul_rn(delta, *(const float*)((const unsigned char*)theta + idx4));
         float sn, cs;
         tri_sincos(ph, sn, cs);
         const float ka = k0 * cs - k1 * sn;
         const float kb = k1 * cs + k0 * sn;
+        const unsigned char* qrow = (const unsigned char*)qh + idx4 * (2 * GQ);   // idx x GQ x 8 bytes
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float2 qq = *(const float2*)(qh + (idx * GQ + q) * 2);
+          const float2 qq = *(const float2*)(qrow + 8 * q);
           sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
         }
       }
@@ -497,7 +509,7 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
 #pragma unroll
       for (int q = 0; q < GQ; ++q) {
-        const float sv = valid ? sc[q] * inv_sqrt_d : -INFINITY;
+        const float sv = valid ? sc[q] * kscale : -INFINITY;
         const float mn = fmaxf(m[q], tri_wave_max(sv + bias));
         alpha[q] = __expf(m[q] - mn);
         rescale |= (mn != m[q]);
@@ -520,19 +532,26 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
         hb.hv = h2; lb.hv = l2;
         *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = (hb.u & 0xffffu) | (lb.u << 16);
       }
+      // tile entries of the lane's token: address and (2a - 15, 2b - 15) as a float16 pair, formed once
+      // (0x6400 + n is float16(1024 + n); minus 1039 is exact)
+      uint32_t voff[12];
+      uint32_t vval[12];
+#pragma unroll
+      for (int f = 0; f < 12; ++f) {
+        const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
+        const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
+        union { uint32_t u; tri_half2 hv; } cv;
+        cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+        cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+        vval[f] = cv.u;
+        voff[f] = idx * TRH_VT_PITCH + 4 * (lane & 31);
+      }
 #pragma unroll
       for (int pass = 0; pass < 2; ++pass) {      // the tile holds 32 tokens
         const bool mine = valid && (lane >> 5) == pass;
         if (mine) {
 #pragma unroll
-          for (int f = 0; f < 12; ++f) {
-            const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
-            const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
-            union { uint32_t u; tri_half2 hv; } cv;
-            cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
-            cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
-            *(uint32_t*)(vt + idx * TRH_VT_PITCH + 4 * (lane & 31)) = cv.u;
-          }
+          for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = vval[f];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -557,10 +576,7 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if (mine) {
 #pragma unroll
-          for (int f = 0; f < 12; ++f) {
-            const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
-            *(uint32_t*)(vt + idx * TRH_VT_PITCH + 4 * (lane & 31)) = 0u;
-          }
+          for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = 0u;
         }
       }
     }
