@@ -53,28 +53,18 @@ __device__ __forceinline__ float tri_dequant(uint32_t code, float scale) {
   return __fmul_rn(__fsub_rn(__fdiv_rn((float)code, 7.5f), 1.0f), scale);
 }
 
-// sin and cos of a float32 angle of any size reached by positions x frequencies (|x| < ~1e5):
-// quadrant k = rint(x * 2/pi), remainder by a three-constant Cody-Waite subtraction carried by
-// fused multiply-adds (each step is exact before its single rounding), then the classic degree-7 /
-// degree-8 minimax polynomials on [-pi/4, pi/4].  Absolute error ~1e-7, the accuracy the float32
-// library routine has, at a fraction of its cost for large arguments (no table-driven reduction).
+// sin and cos of a float32 angle of any size reached by positions x frequencies (|x| < ~1e6):
+// k = rint(x / 2 pi), remainder r = x - k 2 pi by two fused multiply-adds (2 pi = C1 + C2 with C1 the
+// nearest float: k C1 is exact inside the first one, and its result is exact too), then the hardware
+// sine and cosine, which take their argument in revolutions and are good to 1.3e-7 absolute on
+// [-1/2, 1/2] (measured against double precision over 2^22 arguments).
 __device__ __forceinline__ void tri_sincos(float x, float& sn, float& cs) {
-  const float k = rintf(x * 0.636619772367581343f);
-  float r = fmaf(k, -1.57079637050628662109375f, x);
-  r = fmaf(k, 4.37113900018624283e-8f, r);
-  r = fmaf(k, 1.71512451370281e-15f, r);
-  const float r2 = r * r;
-  float ps = fmaf(r2, -1.9515295891e-4f, 8.3321608736e-3f);
-  ps = fmaf(ps, r2, -1.6666654611e-1f);
-  const float s0 = fmaf(ps * r2, r, r);
-  float pc = fmaf(r2, 2.443315711809948e-5f, -1.388731625493765e-3f);
-  pc = fmaf(pc, r2, 4.166664568298827e-2f);
-  const float c0 = fmaf(pc * r2, r2, fmaf(r2, -0.5f, 1.0f));
-  const int q = (int)k;
-  const float a = (q & 1) ? c0 : s0;
-  const float b = (q & 1) ? s0 : c0;
-  sn = __uint_as_float(__float_as_uint(a) ^ ((uint32_t)(q & 2) << 30));
-  cs = __uint_as_float(__float_as_uint(b) ^ ((uint32_t)((q + 1) & 2) << 30));
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(k, -6.2831854820251465f, x);
+  r = fmaf(k, 1.7484555e-07f, r);
+  const float f = r * 0.15915494309189535f;
+  sn = __builtin_amdgcn_sinf(f);
+  cs = __builtin_amdgcn_cosf(f);
 }
 
 template <int GQ, bool F12, bool DENSE>
@@ -344,6 +334,8 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 // tokens lie 32 bytes apart from the next head's, which spreads the writes of a token's heads over
 // the banks).  Two workgroup barriers per chunk
 // (staging written -> read, read -> overwritten).  The dense value tile takes 32 tokens at a time.
+#define TRH_Q_PAD 16                // a pair's row of the query table: GQ x (even, odd) floats + 16 bytes, so that
+                                    // rows start at sixteen different bank positions (eight without)
 #define TRH_HEAD_PITCH (64 * 16 + 32)
 #define TRH_VT_PITCH 144            // 32 tokens x 4 bytes + 16
 #define TRH_VT_BYTES (64 * TRH_VT_PITCH)
@@ -369,7 +361,7 @@ __device__ __forceinline__ float tri_wave_max(float v) {
 }
 
 static size_t tri_heads_lds_bytes(int kvh, int gqa_pass) {
-  return 64 * sizeof(float) + (size_t)kvh * gqa_pass * 128 * sizeof(float) + 64 +
+  return 64 * sizeof(float) + (size_t)kvh * 64 * (gqa_pass * 8 + TRH_Q_PAD) + 64 +
          4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRH_WAVE_BYTES;
 }
 
@@ -379,7 +371,8 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   const int KVH = a.KVH;
   float* theta = (float*)lds_raw;                               // [64]
   float* q_lds = theta + 64;                                    // [KVH][64 pairs][GQ][even, odd]
-  unsigned char* stage = (unsigned char*)(q_lds + (size_t)KVH * GQ * 128 + 16);   // [4 arrays][KVH] x TRH_HEAD_PITCH
+  constexpr int QROW = GQ * 8 + TRH_Q_PAD;                      // bytes of one pair's row of the query table
+  unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // [4 arrays][KVH] x TRH_HEAD_PITCH
   unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
   const int tid = threadIdx.x, lane = tid & 63, h = tid >> 6;   // wavefront = kv head
   unsigned char* vt = tiles + (size_t)h * TRH_WAVE_BYTES;
@@ -438,9 +431,9 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
       else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
       else v = akv_elem<AKV_F32>::load(a.query, off);
-      q_lds[(size_t)hh * GQ * 128 + ((d >> 1) * GQ + q) * 2 + (d & 1)] = v;
+      *(float*)((unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW + (q * 2 + (d & 1)) * 4) = v;
     }
-    const float* qh = q_lds + (size_t)h * GQ * 128;
+    const unsigned char* qh = (const unsigned char*)q_lds + (size_t)h * 64 * QROW;
     tri_float4 oacc[4];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
@@ -497,7 +490,7 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
         tri_sincos(ph, sn, cs);
         const float ka = k0 * cs - k1 * sn;
         const float kb = k1 * cs + k0 * sn;
-        const unsigned char* qrow = (const unsigned char*)qh + idx4 * (2 * GQ);   // idx x GQ x 8 bytes
+        const unsigned char* qrow = qh + idx4 * (QROW / 4);
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
           const float2 qq = *(const float2*)(qrow + 8 * q);
