@@ -347,7 +347,8 @@ def main():
                            "algorithmic_bytes_per_step": algo_bytes, "cache_copies_alternated": 3})
         achieved = algo_bytes / kms / 1e6
         out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "tri_decode_kernel",
+                           "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic("tri"),
+                           "kernel": "tri_decode_heads_kernel<4>",
                            "kernel_ms": kms}
         if cpu:
             from oracle import tq_oracle as O
