@@ -775,13 +775,20 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
     const float e = __fadd_rn(__fmul_rn(x0, x0), __fmul_rn(x1, x1));
     // non-negative floats and NaNs order like their bit patterns; lanes beyond the last pair sort last
     const uint32_t key = have ? (__float_as_uint(e) & 0x7fffffffu) + 1u : 0u;
-    int rank = 0;
-#pragma unroll 16
-    for (int q = 0; q < 64; ++q) {
-      const uint32_t kq = (uint32_t)__builtin_amdgcn_readlane((int)key, q);
-      rank += (kq > key || (kq == key && q < lane)) ? 1 : 0;
+    // The F-th largest key by a bitwise search (largest T with at least F keys >= T: one compare and a
+    // population count per bit), then everything above it plus, of the keys equal to it, the lowest
+    // lanes -- the order torch.topk's result has once it is sorted by index with ties to the lower index.
+    uint32_t T = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = T | (1u << bit);
+      if (__popcll(__ballot(key >= cand)) >= F) T = cand;
     }
-    const bool keep = have && rank < F;
+    const bool above = key > T, equal = key == T;
+    const int need = F - __popcll(__ballot(above));
+    const uint64_t eqm = __ballot(equal);
+    const int eq_pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(eqm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)eqm, 0u));
+    const bool keep = have && (above || (equal && eq_pos < need));
     const uint64_t mask = __ballot(keep);
     const int pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
     float amax = keep ? fmaxf(fabsf(x0), fabsf(x1)) : 0.f;
