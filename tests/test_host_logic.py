@@ -214,3 +214,31 @@ def test_kv_cache_dtype_names_and_ops():
         resolve_kv_cache_dtype("fp8")
     assert register_custom_ops() and register_custom_ops()
     assert hasattr(torch.ops.tq, "decode_step") and hasattr(torch.ops.tq, "hybrid_decode_step")
+
+
+def test_primary_cache_layout_arithmetic():
+    """Page size, power-of-two page alignment and the PRIMARY uint8 layout
+    (reference: aither_kvcache/vllm/engine.py:110-154, 340-375)."""
+    from aitherkvcache_amd.vllm import tq_page_size_bytes, align_page_size, reshape_primary, primary_views
+    f4, f3, fh = (resolve_kv_cache_dtype(n) for n in ("tq-t4nc", "tq-t3nc", "tq35"))
+    assert tq_page_size_bytes(16, 8, 128, f4) == 2 * 16 * 8 * 68 == 17408
+    assert tq_page_size_bytes(16, 8, 128, f3) == 2 * 16 * 8 * 52
+    assert tq_page_size_bytes(16, 8, 128, fh) == 2 * 16 * 8 * 64 == 16384
+    assert [align_page_size(v) for v in (0, -3, 1, 2, 3, 17408, 16384, 16385)] == [0, -3, 1, 2, 4, 32768, 16384, 32768]
+    page = align_page_size(tq_page_size_bytes(16, 8, 128, f4))
+    raw = torch.arange(3 * page, dtype=torch.int64).to(torch.uint8)      # three padded pages, as bytes
+    kv = reshape_primary(raw, 3, 16, 8, 128, f4)
+    assert kv.shape == (3, 2, 16, 8, 68) and kv.dtype == torch.uint8
+    assert kv.data_ptr() == raw.data_ptr()                               # a view, nothing copied
+    k, v = primary_views(kv, 128, f4)
+    assert k.shape == v.shape == (3, 16, 8, 64)
+    assert k.stride() == (2 * 16 * 8 * 68, 8 * 68, 68, 1)
+    assert v.data_ptr() - k.data_ptr() == 16 * 8 * 68
+    assert int(k[1, 2, 3, 5]) == (1 * 2 * 16 * 8 * 68 + (2 * 8 + 3) * 68 + 5) % 256
+    with pytest.raises(ValueError):
+        reshape_primary(raw[:100], 3, 16, 8, 128, f4)
+    with pytest.raises(ValueError):
+        primary_views(kv, 128, fh)
+    kh = reshape_primary(torch.zeros(2 * 16384, dtype=torch.uint8), 2, 16, 8, 128, fh)
+    a, b = primary_views(kh, 128, fh)
+    assert a.shape == (2, 16, 8, 64) and b.stride(2) == 64
