@@ -44,6 +44,10 @@ struct tri_args {
   const void* kpos; int kp_itype;
   int B; int64_t S; int QH, KVH, D, F;
   int nsplit;
+  // paged cache (arrays are [num_blocks][block_size][KVH][...]; S = max_blocks_per_seq * block_size)
+  const void* block_tables; int bt_itype; int64_t bt_stride;
+  const void* context_lens; int cl_itype;
+  int block_size; int64_t num_blocks;
   float* part_acc;  // [B][QH][nsplit][D]
   float* part_ml;   // [B][QH][nsplit][2]
 };
@@ -365,7 +369,11 @@ static size_t tri_heads_lds_bytes(int kvh, int gqa_pass) {
          4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRH_WAVE_BYTES;
 }
 
-template <int GQ>
+// PAGED: the arrays are a block pool, batch element b reads its tokens through row b of the block
+// table up to its own context length (SpectralKVCache.fetch_sequence,
+// aither_kvcache/triattention/cache.py:163-198, fused into the load; a chunk of 64 tokens is then
+// four runs of contiguous bytes instead of one); key positions are 0..ctx-1, query_pos defaults to ctx.
+template <int GQ, bool PAGED>
 __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int KVH = a.KVH;
@@ -389,10 +397,12 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   const float inv_sqrt_d = 1.0f / sqrtf(128.f);
   if (tid < 64) theta[tid] = a.theta[tid];
 
-  const int64_t per = (a.S + a.nsplit - 1) / a.nsplit;
-  const int64_t s0 = min(a.S, (int64_t)split * per);
-  const int64_t s1 = min(a.S, s0 + per);
-  const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)a.S;
+  // tokens of this batch element; ranges start on multiples of 64 (PAGED: of the block size too)
+  const int64_t S = PAGED ? max((int64_t)0, min(akv_load_index(a.context_lens, a.cl_itype, b), a.S)) : a.S;
+  const int64_t per = PAGED ? (((S + a.nsplit - 1) / a.nsplit + 63) & ~(int64_t)63) : (a.S + a.nsplit - 1) / a.nsplit;
+  const int64_t s0 = min(S, (int64_t)split * per);
+  const int64_t s1 = min(S, s0 + per);
+  const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)S;
   const bool kp_wide = a.kpos && a.kp_itype == AKV_I64;
   const unsigned char* kp_base = a.kpos ? (const unsigned char*)a.kpos : (const unsigned char*)a.theta;
 
@@ -405,7 +415,16 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
 
   struct tri_rows { uint32_t x[4][3]; unsigned short ksc, vsc; uint32_t kp_lo, kp_hi; };
   auto fetch = [&](tri_rows& r, int64_t c0) {
-    const int64_t row = min(((int64_t)b * a.S + c0) * KVH + tid, last_row);   // rows past the range: its last row
+    int64_t row;
+    if (PAGED) {
+      const int64_t tcl = max((int64_t)0, min(c0 + my_t, s1 - 1));           // tokens past the range: its last token
+      const int64_t blk = tcl / a.block_size;
+      int64_t phys = akv_load_index(a.block_tables, a.bt_itype, (int64_t)b * a.bt_stride + blk);
+      phys = max((int64_t)0, min(phys, a.num_blocks - 1));                   // (an empty sequence reads a padding entry)
+      row = ((phys * a.block_size) + (tcl - blk * a.block_size)) * KVH + my_h;
+    } else {
+      row = min(((int64_t)b * a.S + c0) * KVH + tid, last_row);              // rows past the range: its last row
+    }
     const uint32_t* p0 = (const uint32_t*)(a.k_idx + row * 12);
     const uint32_t* p1 = (const uint32_t*)(a.k_cf + row * 12);
     const uint32_t* p2 = (const uint32_t*)(a.v_idx + row * 12);
@@ -681,6 +700,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.theta = theta; a.qpos = query_pos; a.qp_itype = qp_itype; a.kpos = key_positions; a.kp_itype = kp_itype;
   a.B = batch; a.S = seq_len; a.QH = num_q_heads; a.KVH = num_kv_heads; a.D = d; a.F = num_freqs;
   a.nsplit = tri_pick_splits(batch, num_kv_heads, seq_len);
+  a.block_tables = nullptr; a.bt_itype = AKV_I32; a.bt_stride = 0; a.context_lens = nullptr; a.cl_itype = AKV_I32;
+  a.block_size = 0; a.num_blocks = 0;
   float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
@@ -706,14 +727,14 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
       static size_t configured4 = 0, configured1 = 0;
       size_t& configured = gq == 4 ? configured4 : configured1;
       if (configured < lds) {
-        if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         configured = lds;
       }
       dim3 hgrid(a.nsplit, batch);
       akv_profile_mark_begin(stream);
-      if (gq == 4) tri_decode_heads_kernel<4><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
-      else tri_decode_heads_kernel<1><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+      if (gq == 4) tri_decode_heads_kernel<4, false><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+      else tri_decode_heads_kernel<1, false><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
       akv_profile_mark_end(stream);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
@@ -746,6 +767,76 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
 #undef TRI_LAUNCH
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("tri_decode_kernel");
+  tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
+  AKV_LAUNCH_CHECK("tri_reduce_kernel");
+  return AKV_OK;
+}
+
+extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_t* k_indices,
+                                    const uint8_t* k_coeffs, const void* k_scales,
+                                    const uint8_t* v_indices, const uint8_t* v_coeffs,
+                                    const void* v_scales, const float* theta, const void* query_pos,
+                                    int qp_itype, const void* block_tables, int bt_itype,
+                                    int64_t bt_stride, const void* context_lens, int cl_itype,
+                                    float* out, int batch, int64_t num_blocks, int block_size,
+                                    int64_t max_blocks_per_seq, int num_q_heads, int num_kv_heads,
+                                    int d, int num_freqs, void* workspace, size_t workspace_bytes,
+                                    void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  AKV_REQUIRE(batch >= 0 && num_blocks > 0 && block_size > 0 && max_blocks_per_seq >= 0 && num_q_heads > 0 &&
+              num_kv_heads > 0, "akv_tri_decode_paged: bad sizes");
+  AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_tri_decode_paged: num_q_heads %% num_kv_heads != 0");
+  AKV_REQUIRE(akv_valid_dtype(q_dtype), "akv_tri_decode_paged: bad dtype");
+  AKV_REQUIRE(akv_valid_itype(bt_itype) && akv_valid_itype(cl_itype), "akv_tri_decode_paged: bad index type");
+  AKV_REQUIRE(!query_pos || akv_valid_itype(qp_itype), "akv_tri_decode_paged: bad query_pos type");
+  const bool aligned = ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
+  const int gqa = num_q_heads / num_kv_heads;
+  const int gq = gqa % 4 == 0 ? 4 : 1;
+  const size_t lds = tri_heads_lds_bytes(num_kv_heads, gq);
+  if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024)
+    return akv_fail(AKV_ERR_UNSUPPORTED,
+                    "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads and 4-byte "
+                    "aligned arrays");
+  if (batch == 0) return AKV_OK;
+  AKV_REQUIRE(query && out && theta && block_tables && context_lens, "akv_tri_decode_paged: null pointer");
+  AKV_REQUIRE(k_indices && k_coeffs && k_scales && v_indices && v_coeffs && v_scales,
+              "akv_tri_decode_paged: null cache pointer");
+  AKV_REQUIRE(workspace != nullptr, "akv_tri_decode_paged: null workspace");
+  if (workspace_bytes < akv_tri_decode_workspace_bytes(batch, num_q_heads, d))
+    return akv_fail(AKV_ERR_WORKSPACE, "akv_tri_decode_paged: workspace %zu < %zu bytes", workspace_bytes,
+                    akv_tri_decode_workspace_bytes(batch, num_q_heads, d));
+  tri_args a;
+  a.query = query; a.q_dtype = q_dtype;
+  a.k_idx = k_indices; a.k_cf = k_coeffs; a.k_sc = (const __half*)k_scales;
+  a.v_idx = v_indices; a.v_cf = v_coeffs; a.v_sc = (const __half*)v_scales;
+  a.theta = theta; a.qpos = query_pos; a.qp_itype = qp_itype; a.kpos = nullptr; a.kp_itype = AKV_I32;
+  a.B = batch; a.S = max_blocks_per_seq * block_size; a.QH = num_q_heads; a.KVH = num_kv_heads; a.D = d; a.F = num_freqs;
+  a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
+  a.context_lens = context_lens; a.cl_itype = cl_itype; a.block_size = block_size; a.num_blocks = num_blocks;
+  int cus = akv_cached_cu_count();
+  if (cus <= 0) cus = 256;
+  int64_t n = (cus + batch - 1) / batch;
+  const int64_t by_len = (a.S + 63) / 64;
+  if (n > by_len) n = by_len;
+  if (n > TRI_MAX_SPLITS) n = TRI_MAX_SPLITS;
+  if (n < 1) n = 1;
+  a.nsplit = (int)n;
+  float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  a.part_acc = wsf;
+  a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
+  static size_t configured4 = 0, configured1 = 0;
+  size_t& configured = gq == 4 ? configured4 : configured1;
+  if (configured < lds) {
+    if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    configured = lds;
+  }
+  dim3 hgrid(a.nsplit, batch);
+  akv_profile_mark_begin(stream);
+  if (gq == 4) tri_decode_heads_kernel<4, true><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+  else tri_decode_heads_kernel<1, true><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
+  akv_profile_mark_end(stream);
+  AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
   return AKV_OK;

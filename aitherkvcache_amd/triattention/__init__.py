@@ -2,7 +2,8 @@
 from .config import TriAttentionConfig
 from .encoder import SpectralEncoding, SpectralKVEncoder
 from .attention import TriAttention
+from .cache import SpectralKVCache
 from .spectral import rope_frequencies
 
 __all__ = ["TriAttentionConfig", "SpectralEncoding", "SpectralKVEncoder", "TriAttention",
-           "rope_frequencies"]
+           "SpectralKVCache", "rope_frequencies"]

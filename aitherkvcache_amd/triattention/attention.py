@@ -91,3 +91,64 @@ class TriAttention:
             out.data_ptr(), B, S, QH, KVH, D, F,
             self._workspace.data_ptr(), self._workspace.numel(), _lib.stream_ptr(dev)))
         return out
+
+    def decode_step_paged(self, query: torch.Tensor, cache, block_tables: torch.Tensor,
+                          context_lens: torch.Tensor, query_pos: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """One decode step for a batch of sequences held in a SpectralKVCache: sequence b reads its
+        first context_lens[b] tokens through block_tables[b] (what the reference does per sequence
+        with cache.fetch_sequence, cache.py:163-198, followed by decode_step).  query [B, QH, D];
+        block_tables [B, max_blocks_per_seq] int32/int64; context_lens [B]; key positions are
+        0..ctx-1 and query_pos defaults to ctx -> float32 [B, QH, D] (zeros where ctx == 0)."""
+        if not self.config.pre_rope:
+            raise NotImplementedError("post-RoPE scoring is not built")
+        dev = _lib.require_gpu(query, cache.k_indices, cache.k_packed, cache.k_scales, cache.v_indices,
+                               cache.v_packed, cache.v_scales, block_tables, context_lens, query_pos)
+        if self._theta.device != dev:
+            self._theta = self._theta.to(dev)
+        B, QH, D = query.shape
+        NB, BS, KVH, F = cache.k_indices.shape
+        if D != self.head_dim or QH % KVH != 0:
+            raise ValueError(f"query shape {tuple(query.shape)} does not fit head_dim={self.head_dim}, kv_heads={KVH}")
+        if block_tables.dim() != 2 or block_tables.shape[0] != B or context_lens.numel() != B:
+            raise ValueError("block_tables must be [B, max_blocks_per_seq] and context_lens [B]")
+        q = query if query.dtype in (torch.float16, torch.bfloat16, torch.float32) else query.float()
+        q = q.contiguous()
+        for t in (cache.k_indices, cache.k_packed, cache.k_scales, cache.v_indices, cache.v_packed, cache.v_scales):
+            if not t.is_contiguous():
+                raise ValueError("the cache tensors must be contiguous")
+        bt = block_tables if block_tables.dtype in (torch.int32, torch.int64) else block_tables.long()
+        if bt.stride(1) != 1:
+            bt = bt.contiguous()
+        cl = context_lens if context_lens.dtype in (torch.int32, torch.int64) else context_lens.long()
+        cl = cl.contiguous()
+        qp = None
+        if query_pos is not None:
+            qp = query_pos if query_pos.dtype in (torch.int32, torch.int64) else query_pos.long()
+            qp = qp.expand((B,)).contiguous()
+        out = torch.empty(B, QH, D, dtype=torch.float32, device=dev)
+        L = _lib.lib()
+        need = L.akv_tri_decode_workspace_bytes(B, QH, D)
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != dev:
+            self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        rc = L.akv_tri_decode_paged(
+            q.data_ptr(), _lib.dtype_code(q), cache.k_indices.data_ptr(), cache.k_packed.data_ptr(),
+            cache.k_scales.data_ptr(), cache.v_indices.data_ptr(), cache.v_packed.data_ptr(),
+            cache.v_scales.data_ptr(), self._theta.data_ptr(),
+            _lib.ptr(qp), _lib.itype_code(qp) if qp is not None else 0,
+            bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
+            out.data_ptr(), B, NB, BS, bt.shape[1], QH, KVH, D, F,
+            self._workspace.data_ptr(), self._workspace.numel(), _lib.stream_ptr(dev))
+        if rc == _lib.AKV_ERR_UNSUPPORTED:
+            # shapes the paged kernel does not take: gather each sequence and use the dense-layout kernels
+            lens = cl.tolist()
+            for b in range(B):
+                if lens[b] <= 0:
+                    out[b].zero_()
+                    continue
+                k_enc, v_enc = cache.fetch_sequence(bt[b], lens[b])
+                add = lambda e: SpectralEncoding(*(t.unsqueeze(0) for t in e))
+                out[b] = self.decode_step(q[b:b + 1], add(k_enc), add(v_enc),
+                                          None if qp is None else qp[b:b + 1])[0]
+            return out
+        _lib.check(rc)
+        return out

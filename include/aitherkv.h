@@ -225,6 +225,31 @@ int akv_tri_decode_step(const void* query, int q_dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
+ * TriAttention.decode_step over a paged spectral cache: what the reference does per sequence
+ * with SpectralKVCache.fetch_sequence (aither_kvcache/triattention/cache.py:163-198; block
+ * layout :9-15) followed by decode_step, for a whole batch and without the gather.
+ *   k/v_indices, k/v_coeffs [num_blocks][block_size][KVH][F] uint8, k/v_scales
+ *   [num_blocks][block_size][KVH] fp16, contiguous; block_tables [B][>= ceil(ctx/block_size)]
+ *   (row stride bt_stride elements; entries past the context are never dereferenced for
+ *   ctx > 0); context_lens [B], clamped to max_blocks_per_seq * block_size; key positions are
+ *   0..ctx-1; query_pos [B] or NULL (= ctx); out [B][QH][d] float32, zeros where ctx == 0.
+ * Workspace as for akv_tri_decode_step.  Built for d = 128, num_freqs = 12, at most 8 kv heads
+ * and 4-byte aligned arrays; anything else returns AKV_ERR_UNSUPPORTED (gather, then
+ * akv_tri_decode_step).
+ * ------------------------------------------------------------------------------- */
+int akv_tri_decode_paged(const void* query, int q_dtype,
+                         const uint8_t* k_indices, const uint8_t* k_coeffs, const void* k_scales,
+                         const uint8_t* v_indices, const uint8_t* v_coeffs, const void* v_scales,
+                         const float* theta,
+                         const void* query_pos, int qp_itype,
+                         const void* block_tables, int bt_itype, int64_t bt_stride,
+                         const void* context_lens, int cl_itype,
+                         float* out, int batch, int64_t num_blocks, int block_size,
+                         int64_t max_blocks_per_seq, int num_q_heads, int num_kv_heads,
+                         int d, int num_freqs,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
  * SpectralKVEncoder.encode, coeff_bits = 4 -- aither_kvcache/triattention/encoder.py:73-133
  * (the write side of TriAttention; TriAttention.encode_kv, attention.py:160-184, calls it for
  * keys and values): per vector the num_freqs RoPE pairs (dims 2i, 2i+1) of largest energy,

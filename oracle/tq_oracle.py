@@ -19,7 +19,9 @@ reference tree).  How each one is pinned:
       selection and scatter by a per-block loop in tests/test_oracle_pins.py),
       fwht, structured_hadamard, dimension_aware_codebook,
       hybrid_encode, hybrid_decode, rope_frequencies, spectral_encode,
-      tri_scores, tri_decode_step
+      tri_scores, tri_decode_step,
+      spectral_fetch_sequence / tri_decode_step_paged (indexing only, on top of the pinned
+      tri_decode_step: checked against a token-by-token loop in tests/test_oracle_pins.py)
   derived here (the reference has no such function; it always decompresses
   tq35 data before attending): hybrid_paged_attention is *defined* as
   hybrid_decode -> dense f32 softmax attention, i.e. the reference's
@@ -689,4 +691,34 @@ def tri_decode_step(query, k_enc, v_enc, theta, query_pos=None, key_positions=No
             wv1 = (w[b, qh][:, None] * v1[b, :, h]).reshape(-1)
             np.add.at(out[b, qh], 2 * ii, wv0)
             np.add.at(out[b, qh], 2 * ii + 1, wv1)
+    return out
+
+
+def spectral_fetch_sequence(cache_arrays, block_table, context_len, block_size):
+    """SpectralKVCache.fetch_sequence, triattention/cache.py:163-198: the first
+    ceil(context_len / block_size) entries of the block table select physical blocks, whose tokens
+    are laid end to end and cut at context_len.  cache_arrays: the six pool arrays
+    (k_indices, k_packed, k_scales, v_indices, v_packed, v_scales), each [num_blocks, block_size, ...].
+    Returns (k_enc, v_enc) triples with a leading axis of context_len."""
+    nb = -(-int(context_len) // block_size)
+    phys = np.asarray(block_table)[:nb].astype(np.int64)
+    got = [np.asarray(a)[phys].reshape((-1,) + np.asarray(a).shape[2:])[:context_len] for a in cache_arrays]
+    return tuple(got[:3]), tuple(got[3:])
+
+
+def tri_decode_step_paged(query, cache_arrays, block_tables, context_lens, block_size, theta, query_pos=None):
+    """A batch of sequences in one block pool: per sequence fetch_sequence then decode_step with the
+    default key positions 0..ctx-1 and query position ctx (scorer.py:142-146); an empty sequence
+    gives zeros (softmax over no tokens, nothing scattered).  Returns float32 [B, QH, D]."""
+    query = np.asarray(query)
+    B, QH, D = query.shape
+    out = np.zeros((B, QH, D), dtype=f32)
+    for b in range(B):
+        n = int(context_lens[b])
+        if n <= 0:
+            continue
+        k_enc, v_enc = spectral_fetch_sequence(cache_arrays, block_tables[b], n, block_size)
+        qp = None if query_pos is None else np.asarray(query_pos)[b:b + 1]
+        out[b] = tri_decode_step(query[b:b + 1], tuple(a[None] for a in k_enc), tuple(a[None] for a in v_enc),
+                                 theta, qp)[0]
     return out

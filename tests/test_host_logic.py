@@ -242,3 +242,46 @@ def test_primary_cache_layout_arithmetic():
     kh = reshape_primary(torch.zeros(2 * 16384, dtype=torch.uint8), 2, 16, 8, 128, fh)
     a, b = primary_views(kh, 128, fh)
     assert a.shape == (2, 16, 8, 64) and b.stride(2) == 64
+
+
+def test_spectral_kv_cache_bookkeeping():
+    """SpectralKVCache on the CPU: store / fetch round trips, copy, clear, statistics
+    (reference: tests/test_triattention.py:225-247, 460-473; triattention/cache.py)."""
+    from aitherkvcache_amd.triattention import SpectralKVCache, SpectralEncoding
+    from oracle import tq_oracle as O
+    cfg = TriAttentionConfig(num_kv_heads=2, num_query_heads=8)
+    cache = SpectralKVCache(cfg, max_blocks=6)
+    BS, KVH, F = cfg.block_size, 2, cfg.num_freqs
+    g = torch.Generator().manual_seed(5)
+
+    def enc(n):
+        return SpectralEncoding(torch.randint(0, 64, (n, KVH, F), dtype=torch.uint8, generator=g),
+                                torch.randint(0, 256, (n, KVH, F), dtype=torch.uint8, generator=g),
+                                torch.rand(n, KVH, generator=g).half())
+
+    S = 2 * BS + 5
+    k, v = enc(S), enc(S)
+    table = torch.tensor([4, 1, 3, 0])
+    cache.store_block(4, SpectralEncoding(*(x[:BS] for x in k)), SpectralEncoding(*(x[:BS] for x in v)))
+    cache.store_block(1, SpectralEncoding(*(x[BS:2 * BS] for x in k)), SpectralEncoding(*(x[BS:2 * BS] for x in v)))
+    for j in range(5):
+        tok = 2 * BS + j
+        cache.store_token(3, j, SpectralEncoding(*(x[tok] for x in k)), SpectralEncoding(*(x[tok] for x in v)))
+    k_out, v_out = cache.fetch_sequence(table, S)
+    for a, b in zip(tuple(k_out) + tuple(v_out), tuple(k) + tuple(v)):
+        assert torch.equal(a, b)
+    ko, vo = O.spectral_fetch_sequence([x.numpy() for x in cache._arrays()], table.numpy(), S, BS)
+    for a, b in zip(ko + vo, tuple(k) + tuple(v)):
+        assert np.array_equal(a, b.numpy())
+    stats = cache.memory_stats()
+    assert stats["used_blocks"] == 3 and stats["total_tokens"] == S
+    assert stats["bytes_allocated"] == 6 * BS * KVH * (F + F + 2) * 2 and cache.bytes_per_token == 52
+    cache.copy_block(3, 5)
+    assert torch.equal(cache.k_packed[5], cache.k_packed[3]) and cache.memory_stats()["total_tokens"] == S + 5
+    cache.clear_block(4)
+    assert int(cache.k_indices[4].sum()) == 0 and cache.memory_stats()["used_blocks"] == 3
+    other = SpectralKVCache(cfg, max_blocks=6)
+    other.store_sequence(table, k, v)
+    k2, v2 = other.fetch_sequence(table, S)
+    assert all(torch.equal(a, b) for a, b in zip(tuple(k2) + tuple(v2), tuple(k) + tuple(v)))
+    assert other.memory_stats()["total_tokens"] == S

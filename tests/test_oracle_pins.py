@@ -304,3 +304,20 @@ def test_tri_truncation_keeps_largest_pairs():
     for r in range(50):
         assert set(idx[r].tolist()) == set(np.argsort(-en[r])[:12].tolist())
     assert idx.shape[-1] + packed.shape[-1] + 2 == 26             # bytes per token
+
+
+def test_spectral_fetch_sequence_is_token_by_token_indexing():
+    """fetch_sequence (reference: triattention/cache.py:163-198) against a loop that looks every token up
+    by (block_table[t // block_size], t % block_size); permuted tables, a ragged last block, padding entries."""
+    rng = np.random.default_rng(11)
+    NB, BS, KVH, F = 9, 4, 2, 3
+    arrays = [rng.integers(0, 256, size=(NB, BS, KVH, F), dtype=np.uint8) for _ in range(2)]
+    arrays.append(rng.standard_normal((NB, BS, KVH)).astype(np.float16))
+    arrays += [rng.integers(0, 256, size=(NB, BS, KVH, F), dtype=np.uint8) for _ in range(2)]
+    arrays.append(rng.standard_normal((NB, BS, KVH)).astype(np.float16))
+    table = np.array([7, 2, 5, 0, 99, -1])          # the last two are padding: never dereferenced
+    for n in (1, 4, 5, 15, 16):
+        k_enc, v_enc = O.spectral_fetch_sequence(arrays, table, n, BS)
+        for j, got in enumerate(k_enc + v_enc):
+            want = np.stack([arrays[j][table[t // BS], t % BS] for t in range(n)])
+            assert got.shape == want.shape and np.array_equal(got, want)
