@@ -90,10 +90,13 @@ def timed(torch, fn, steps, warmup):
 
 
 def kernel_ms(torch, L, fn, steps):
-    """Mean duration of the dominant kernel over `steps` calls (HIP events on the launch stream)."""
+    """Mean duration of the dominant kernel over `steps` calls (HIP events on the launch stream).
+    The library keeps one pair of events, read back after every sample; the sampled call follows an
+    unsampled one directly, so that it runs on a busy device like the calls of the timed region."""
     L.akv_profile_enable(1)
     acc = 0.0
     for _ in range(steps):
+        fn()
         fn()
         acc += profile_ms(L)
     L.akv_profile_enable(0)

@@ -231,6 +231,53 @@ def test_config2_shape_properties(golden, dev):
     assert within_tol(o.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("bits", [3, 2])
+def test_config3_shape_properties(golden, dev, bits):
+    """The 3-bit and 2-bit benchmark shape (32Q/8KV, 64 sequences x 8192 tokens, block 16): too large
+    for the oracle at full size, so (a) with one value row everywhere the output must be that row
+    decoded, whatever the scores and wherever the workgroup cuts fall; (b) one whole sequence with
+    random values against the oracle."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(3)
+    S, CTX, KVH, QH = 64, 8192, 8, 32
+    nb_seq = CTX // 16
+    NB = S * nb_seq
+    P = tq._packed_dim
+    kp = torch.empty(NB, 16, KVH, P, dtype=torch.uint8, device=dev)
+    kn = torch.empty(NB, 16, KVH, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    CH = 2048
+    for b0 in range(0, NB, CH):
+        b1 = min(NB, b0 + CH)
+        x = torch.randn((b1 - b0) * 16 * KVH, 128, device=dev, generator=gen).half()
+        pk, nr = tq.encode(x)
+        kp[b0:b1] = pk.reshape(b1 - b0, 16, KVH, P)
+        kn[b0:b1] = nr.reshape(b1 - b0, 16, KVH)
+    v1 = kv_like(rng, (1, KVH, 128))
+    vp1, vn1 = tq.encode(t(v1, dev))
+    vp = vp1.reshape(1, 1, KVH, P).expand(NB, 16, KVH, P).contiguous()
+    vn = vn1.reshape(1, 1, KVH).expand(NB, 16, KVH).contiguous()
+    tables = rng.permutation(NB).reshape(S, nb_seq).astype(np.int32)
+    ctx = np.full(S, CTX, dtype=np.int64)
+    ctx[5], ctx[17] = CTX - 9, 1          # a ragged end and a one-token sequence
+    q = rng.standard_normal((S, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).float()
+    want = tq.decode(vp1, vn1).float().reshape(KVH, 1, 128).expand(KVH, 4, 128).reshape(1, QH, 128)
+    assert bool(torch.all(torch.abs(out - want) <= TOL + 2.0 ** -10 * want.abs()))
+    s = 5
+    vp_r, vn_r = kp.roll(3, 0), kn.roll(3, 0)
+    o = attn.forward(t(q[s:s + 1], dev), kp, kn, vp_r, vn_r, t(tables[s:s + 1], dev), t(ctx[s:s + 1], dev))
+    used = np.unique(tables[s])
+    remap = {b: i for i, b in enumerate(used)}
+    small_tab = np.array([[remap[b] for b in tables[s]]])
+    idx = t(used.astype(np.int64), dev)
+    ref = oracle_out(q[s:s + 1], kp[idx], kn[idx], vp_r[idx], vn_r[idx], small_tab, ctx[s:s + 1], golden, bits)
+    err = np.max(np.abs(o.cpu().numpy().astype(np.float64) - ref))
+    print(f"[attn config 3, {bits}-bit] one sequence max|diff|={err:.2e}")
+    assert within_tol(o.cpu().numpy(), ref)
+
+
 def test_decode_step_custom_op(golden, dev):
     """tq::decode_step: encode the step's token into the serving cache, attend, write output."""
     from aitherkvcache_amd.vllm import hooks

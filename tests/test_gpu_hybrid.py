@@ -122,6 +122,50 @@ def test_paged_attention_vs_oracle(golden, dev, qh, kvh):
     assert np.max(np.abs(o32.cpu().numpy() - ref32)) <= 2e-4
 
 
+def test_config3_shape_properties(golden, dev):
+    """tq35 at the benchmark shape (32Q/8KV, 64 sequences x 8192 tokens, block 16), too large for the
+    oracle: with one value row everywhere the output must be that row decoded, whatever the scores
+    and wherever the workgroup cuts fall; then one whole sequence with random values against the oracle."""
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform(num_kv_heads=8)
+    hp = params(golden)
+    rng = np.random.default_rng(33)
+    S, CTX, KVH, QH = 64, 8192, 8, 32
+    nb_seq = CTX // 16
+    NB = S * nb_seq
+    kc = torch.empty(NB, 16, KVH, 64, dtype=torch.uint8, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(9)
+    CH = 2048
+    for b0 in range(0, NB, CH):
+        b1 = min(NB, b0 + CH)
+        x = torch.randn((b1 - b0) * 16, KVH, 128, device=dev, generator=gen).half()
+        kc[b0:b1] = h.encode(x).reshape(b1 - b0, 16, KVH, 64)
+    v1 = kv_like(rng, (1, KVH, 128))
+    row = h.encode(t(v1, dev))                                   # [1, KVH, 64]
+    vc = row.reshape(1, 1, KVH, 64).expand(NB, 16, KVH, 64).contiguous()
+    tables = rng.permutation(NB).reshape(S, nb_seq).astype(np.int32)
+    ctx = np.full(S, CTX, dtype=np.int64)
+    ctx[5], ctx[17] = CTX - 9, 1
+    q = rng.standard_normal((S, QH, 128)).astype(np.float16)
+    scale = 1 / math.sqrt(128)
+    attn = akv.HybridPagedAttention(h, QH)
+    out = attn.forward(t(q, dev), kc, vc, t(tables, dev), t(ctx, dev), scale=scale).float()
+    want = h.decode(row).float().reshape(KVH, 1, 128).expand(KVH, 4, 128).reshape(1, QH, 128)
+    assert bool(torch.all(torch.abs(out - want) <= 2e-3 + 2.0 ** -10 * want.abs()))
+    s = 5
+    vc_r = kc.roll(3, 0)
+    o = attn.forward(t(q[s:s + 1], dev), kc, vc_r, t(tables[s:s + 1], dev), t(ctx[s:s + 1], dev), scale=scale)
+    used = np.unique(tables[s])
+    remap = {b: i for i, b in enumerate(used)}
+    small_tab = np.array([[remap[b] for b in tables[s]]])
+    idx = t(used.astype(np.int64), dev)
+    ref = O.hybrid_paged_attention(q[s:s + 1], kc[idx].cpu().numpy(), vc_r[idx].cpu().numpy(), small_tab,
+                                   ctx[s:s + 1], hp, scale, dtype=np.float64)
+    got = o.cpu().numpy().astype(np.float64)
+    print(f"[hybrid attn config 3] one sequence max|diff|={np.max(np.abs(got - ref)):.2e}")
+    assert np.all(np.abs(got - ref) <= 2e-3 + 2.0 ** -11 * np.abs(ref))
+
+
 def test_hybrid_decode_step_custom_op(golden, dev):
     from aitherkvcache_amd.vllm import hooks
     hooks.reset_state()
