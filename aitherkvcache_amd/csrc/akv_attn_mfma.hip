@@ -146,22 +146,26 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
   }
   const int s = blockIdx.x / KVH, h = blockIdx.x % KVH;
   const int gqa = QH / KVH;
+  // thread (dim, half): partial dot products over 64 of the 128 input coordinates for every query
+  // head of the group.  Its 64 matrix entries are requested first, together with the queries, so that
+  // the two round trips to memory overlap instead of following each other across the barrier.
+  const int dim = tid & 127, half = tid >> 7;
+  float pvr[64];
+#pragma unroll
+  for (int jj = 0; jj < 64; ++jj) pvr[jj] = PiT[(half * 64 + jj) * 128 + dim];
   for (int i = tid; i < 8 * 128; i += 256) {
     const int q = i >> 7, j = i & 127;
     q_lds[j][q] = q < gqa ? akv_elem<QDT>::load(query, s * qs_seq + (h * gqa + q) * qs_head + j) : 0.f;
   }
   __syncthreads();
   {
-    // thread (dim, half): partial dot products over 64 of the 128 input coordinates for every
-    // query head of the group; the 64 matrix loads of a thread are independent and unrolled
-    const int dim = tid & 127, half = tid >> 7;
     float part[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) part[q] = 0.f;
 #pragma unroll
     for (int jj = 0; jj < 64; ++jj) {
       const int j = half * 64 + jj;
-      const float pv = PiT[j * 128 + dim];
+      const float pv = pvr[jj];
       const float4 qa = *(const float4*)&q_lds[j][0];
       const float4 qc = *(const float4*)&q_lds[j][4];
       part[0] = fmaf(pv, qa.x, part[0]); part[1] = fmaf(pv, qa.y, part[1]);
