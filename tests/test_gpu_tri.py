@@ -42,7 +42,9 @@ def test_golden_decode_step(golden, dev):
 
 
 @pytest.mark.parametrize("B,S,QH,KVH,D,F,base", [(3, 1000, 32, 8, 128, 12, 1e6), (2, 333, 6, 2, 32, 4, 1e4),
-                                                 (1, 64, 4, 4, 64, 32, 1e4), (2, 5000, 8, 1, 128, 12, 1e6)])
+                                                 (1, 64, 4, 4, 64, 32, 1e4), (2, 5000, 8, 1, 128, 12, 1e6),
+                                                 (2, 700, 8, 2, 128, 20, 1e6), (1, 1500, 16, 16, 128, 12, 1e6),
+                                                 (2, 130, 12, 4, 128, 12, 1e4)])
 def test_vs_oracle_shapes(dev, B, S, QH, KVH, D, F, base):
     cfg = TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=4, num_kv_heads=KVH, num_query_heads=QH, rope_base=base)
     tri = TriAttention(cfg, device=str(dev))
