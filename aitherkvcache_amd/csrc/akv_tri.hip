@@ -347,11 +347,17 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 #define TRH_WAVE_BYTES (TRH_VT_BYTES + 4 * TRH_WT_PITCH)
 
 __device__ __forceinline__ float tri_row16_max(float v) {
-  // maximum over the lane's row of 16 by row rotations (data-parallel primitives, no LDS crossbar)
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128 /*row_ror:8*/, 0xf, 0xf, false)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124 /*row_ror:4*/, 0xf, 0xf, false)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122 /*row_ror:2*/, 0xf, 0xf, false)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121 /*row_ror:1*/, 0xf, 0xf, false)));
+  // maximum over the lane's row of 16 by row rotations folded into the maximum instruction itself
+  // (data-parallel primitives, no LDS crossbar; scores are never NaN-quieted on the way)
+  asm("s_nop 1\n\t"      // a lane-crossing read needs two idle cycles after the register was written
+      "v_max_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf"
+      : "+v"(v));
   return v;
 }
 __device__ __forceinline__ float tri_wave_max(float v) {
