@@ -379,6 +379,10 @@ static size_t tri_heads_lds_bytes(int kvh, int gqa_pass) {
 // table up to its own context length (SpectralKVCache.fetch_sequence,
 // aither_kvcache/triattention/cache.py:163-198, fused into the load; a chunk of 64 tokens is then
 // four runs of contiguous bytes instead of one); key positions are 0..ctx-1, query_pos defaults to ctx.
+typedef __attribute__((address_space(3))) const float tri_lds_cfloat;
+typedef float tri_f32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const tri_f32x2 tri_lds_cfloat2;
+
 template <int GQ, bool PAGED>
 __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -458,7 +462,7 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       else v = akv_elem<AKV_F32>::load(a.query, off);
       *(float*)((unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW + (q * 2 + (d & 1)) * 4) = v;
     }
-    const unsigned char* qh = (const unsigned char*)q_lds + (size_t)h * 64 * QROW;
+    const uint32_t q_base = 64 * sizeof(float) + (uint32_t)h * 64 * QROW;
     tri_float4 oacc[4];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
@@ -510,15 +514,17 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
         const uint32_t idx4 = (ki4[f >> 2] >> (8 * (f & 3))) & 255u;          // byte offset of theta[idx]
         const float k0 = fmaf((float)((chi[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
         const float k1 = fmaf((float)((clo[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
-        const float ph = __fmul_rn(delta, *(const float*)((const unsigned char*)theta + idx4));
+        // (the dynamic LDS of this kernel starts at LDS address 0 and theta is its first object: the
+        // byte offset is the address, no base to add)
+        const float ph = __fmul_rn(delta, *(tri_lds_cfloat*)(uintptr_t)idx4);
         float sn, cs;
         tri_sincos(ph, sn, cs);
         const float ka = k0 * cs - k1 * sn;
         const float kb = k1 * cs + k0 * sn;
-        const unsigned char* qrow = qh + idx4 * (QROW / 4);
+        const uint32_t qrow = idx4 * (QROW / 4) + q_base;      // LDS address of the pair's row of this head
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float2 qq = *(const float2*)(qrow + 8 * q);
+          const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
           sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
         }
       }
