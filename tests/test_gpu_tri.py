@@ -126,19 +126,20 @@ def test_spectral_encode_vs_oracle(dev, dtype, D, F):
     assert e0.indices.shape == (0, F)
 
 
-@pytest.mark.parametrize("KVH,QH,bt_dtype", [(8, 32, torch.int32), (2, 8, torch.int64), (4, 4, torch.int32)])
-def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype):
+@pytest.mark.parametrize("KVH,QH,bt_dtype,BS", [(8, 32, torch.int32, 16), (2, 8, torch.int64, 16), (4, 4, torch.int32, 16),
+                                                 (8, 32, torch.int64, 32), (1, 4, torch.int32, 8), (16, 16, torch.int32, 16)])
+def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
     """decode_step_paged over a block pool with permuted block tables, ragged context lengths (one
     empty, one ending inside a block, one filling its table) against the oracle's fetch + decode and
     against fetch_sequence + decode_step on the device."""
     from aitherkvcache_amd.triattention import SpectralKVCache
-    cfg = TriAttentionConfig(num_kv_heads=KVH, num_query_heads=QH)
+    cfg = TriAttentionConfig(num_kv_heads=KVH, num_query_heads=QH, block_size=BS)
     tri = TriAttention(cfg, device=str(dev))
     rng = np.random.default_rng(100 + KVH)
-    BS, D = cfg.block_size, 128
+    D = 128
     lens = [0, 1, 777, 2048, 1500]
-    B, max_bps = len(lens), 128
-    NB = 400
+    B, max_bps = len(lens), 2048 // BS
+    NB = 6400 // BS
     cache = SpectralKVCache(cfg, max_blocks=NB, device=str(dev))
     perm = rng.permutation(NB)
     tables = np.full((B, max_bps), -7, dtype=np.int64)        # padding entries are never dereferenced
