@@ -810,7 +810,13 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
                     "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads and 4-byte "
                     "aligned arrays");
   if (batch == 0) return AKV_OK;
-  AKV_REQUIRE(query && out && theta && block_tables && context_lens, "akv_tri_decode_paged: null pointer");
+  AKV_REQUIRE(out != nullptr, "akv_tri_decode_paged: null pointer");
+  if (max_blocks_per_seq == 0) {   // block tables without columns: every sequence is empty
+    tri_zero_kernel<<<64, 256, 0, stream>>>(out, (size_t)batch * num_q_heads * d);
+    AKV_LAUNCH_CHECK("tri_zero_kernel");
+    return AKV_OK;
+  }
+  AKV_REQUIRE(query && theta && block_tables && context_lens, "akv_tri_decode_paged: null pointer");
   AKV_REQUIRE(k_indices && k_coeffs && k_scales && v_indices && v_coeffs && v_scales,
               "akv_tri_decode_paged: null cache pointer");
   AKV_REQUIRE(workspace != nullptr, "akv_tri_decode_paged: null workspace");

@@ -174,3 +174,15 @@ def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
         one = tri.decode_step(t(q[b:b + 1], dev), SpectralEncoding(*(x[None] for x in k_enc)),
                               SpectralEncoding(*(x[None] for x in v_enc))).cpu().numpy()
         assert np.max(np.abs(one[0] - out[b])) <= 2e-6
+
+
+def test_paged_decode_without_table_columns(dev):
+    """A block table with no columns: every sequence is empty, the output is zero."""
+    from aitherkvcache_amd.triattention import SpectralKVCache
+    cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32)
+    tri = TriAttention(cfg, device=str(dev))
+    cache = SpectralKVCache(cfg, max_blocks=4, device=str(dev))
+    q = torch.randn(3, 32, 128, device=dev)
+    out = tri.decode_step_paged(q, cache, torch.zeros(3, 0, dtype=torch.int32, device=dev),
+                                torch.tensor([5, 0, 9], device=dev, dtype=torch.int32))
+    assert out.shape == (3, 32, 128) and not bool(out.any())
