@@ -47,7 +47,7 @@ class SpectralKVCache:
 
     @property
     def bytes_per_token(self) -> int:
-        """Bytes of one token's K and V over all kv heads' worth of one head (reference: cache.py:100-103)."""
+        """Bytes of one token's K row plus V row of one kv head (reference: cache.py:100-103)."""
         return self.config.bytes_per_kv_token * 2
 
     def store_token(self, block_idx: int, slot_idx: int, k_enc: SpectralEncoding, v_enc: SpectralEncoding) -> None:
