@@ -311,3 +311,72 @@ def test_decode_step_custom_op(golden, dev):
     assert within_tol(output[:2].cpu().numpy(), ref)
     # the new token really was written (its norm is in place), layer 0 untouched
     assert float(k_norms[1, tables[0, hist // BS], hist % BS, 0]) > 0 and torch.all(k_norms[0] == 0)
+
+
+def test_decode_step_replays_from_a_graph(golden, dev):
+    """The decode step (two encode-on-write launches and the attention launches) recorded into a HIP
+    graph: every replay, with eager work and synchronisations in between and fresh inputs copied into
+    the graph's static tensors, must equal the eager result for those inputs."""
+    from aitherkvcache_amd.vllm import hooks
+    hooks.reset_state()
+    assert hooks.register_custom_ops()
+    tq = hooks.init_quantizer(128, bits=4, device=str(dev))
+    tq.rotation = torch.from_numpy(golden["rotation_d128_seed42"]).to(dev)
+    rng = np.random.default_rng(56)
+    NB, BS, KVH, QH, L, S = 400, 16, 8, 32, 1, 4
+    hist = np.array([1500, 37, 640, 1023])
+    tables = rng.permutation(NB)[:S * 96].reshape(S, 96).astype(np.int32)
+
+    def fresh_cache():
+        kv = torch.zeros(NB, 2, BS, KVH, 68, dtype=torch.uint8, device=dev)
+        kn = torch.zeros(L, NB, BS, KVH, device=dev)
+        vn = torch.zeros_like(kn)
+        for s in range(S):
+            n = int(hist[s])
+            slots = t(np.array([tables[s, p // BS] * BS + p % BS for p in range(n)]), dev)
+            g = torch.Generator(device=dev).manual_seed(100 + s)
+            akv.fused_tq4_kv_update(torch.randn(n, KVH, 128, device=dev, generator=g).half(), slots, kv[:, 0], kn[0],
+                                    tq.rotation, tq.boundaries_inner)
+            akv.fused_tq4_kv_update(torch.randn(n, KVH, 128, device=dev, generator=g).half(), slots, kv[:, 1], vn[0],
+                                    tq.rotation, tq.boundaries_inner)
+        return kv, kn, vn
+
+    new_slots = t(np.array([tables[s, hist[s] // BS] * BS + hist[s] % BS for s in range(S)], dtype=np.int64), dev)
+    bt, sl = t(tables, dev), t((hist + 1).astype(np.int32), dev)
+    scale = 1 / math.sqrt(128)
+
+    def inputs(seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return tuple(torch.randn(S, n, 128, device=dev, generator=g).half() for n in (QH, KVH, KVH))
+
+    def run(q, k, v, kv, kn, vn, out):
+        return torch.ops.tq.decode_step(q, k, v, kv, out, kn, vn, new_slots, bt, sl, 0, QH, KVH, 128, scale, S)
+
+    # eager results for three different steps, each on a cache of its own
+    want = []
+    for seed in (1, 2, 3):
+        kv, kn, vn = fresh_cache()
+        out = torch.zeros(S, QH, 128, dtype=torch.float16, device=dev)
+        run(*inputs(seed), kv, kn, vn, out)
+        want.append((out.clone(), kv.clone(), kn.clone()))
+    # one graph over static tensors
+    kv, kn, vn = fresh_cache()
+    sq, sk, sv = (x.clone() for x in inputs(1))
+    sout = torch.zeros(S, QH, 128, dtype=torch.float16, device=dev)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run(sq, sk, sv, kv, kn, vn, sout)          # warm-up outside the capture (workspaces, tables)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(sq, sk, sv, kv, kn, vn, sout)
+    for rep in range(2):
+        for i, seed in enumerate((1, 2, 3)):
+            q, k, v = inputs(seed)
+            sq.copy_(q); sk.copy_(k); sv.copy_(v)
+            sout.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(sout, want[i][0]), (rep, seed)
+            assert torch.equal(kv, want[i][1]) and torch.equal(kn, want[i][2])
+            _ = (torch.randn(1 << 16, device=dev) * 2).sum().item()       # unrelated eager work between replays
