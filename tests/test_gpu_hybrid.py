@@ -193,3 +193,62 @@ def test_hybrid_decode_step_custom_op(golden, dev):
     ref = O.hybrid_paged_attention(q, kv_cache[:, 0].cpu().numpy(), kv_cache[:, 1].cpu().numpy(), tables,
                                    seq_lens, hp, scale, dtype=np.float64)
     assert np.max(np.abs(output.cpu().numpy().astype(np.float64) - ref)) <= 2e-3
+
+
+def test_hybrid_decode_step_replays_from_a_graph(golden, dev):
+    """tq::hybrid_decode_step recorded into a HIP graph: replays with new inputs in the static tensors,
+    eager work and synchronisations in between, equal the eager results bit for bit."""
+    from aitherkvcache_amd.vllm import hooks
+    hooks.reset_state()
+    hooks.register_custom_ops()
+    h = hooks.init_quantizer(128, mode="tq35", device=str(dev), num_kv_heads=8)
+    rng = np.random.default_rng(67)
+    NB, BS, KVH, QH, S = 200, 16, 8, 32, 3
+    hist = np.array([700, 15, 333])
+    tables = rng.permutation(NB)[:S * 48].reshape(S, 48).astype(np.int32)
+
+    def fresh_cache():
+        kv = torch.zeros(NB, 2, BS, KVH, 64, dtype=torch.uint8, device=dev)
+        for s in range(S):
+            n = int(hist[s])
+            slots = t(np.array([tables[s, p // BS] * BS + p % BS for p in range(n)]), dev)
+            g = torch.Generator(device=dev).manual_seed(300 + s)
+            akv.hybrid_encode_and_store(h, torch.randn(n, KVH, 128, device=dev, generator=g).half(), slots, kv[:, 0], BS)
+            akv.hybrid_encode_and_store(h, torch.randn(n, KVH, 128, device=dev, generator=g).half(), slots, kv[:, 1], BS)
+        return kv
+
+    new_slots = t(np.array([tables[s, hist[s] // BS] * BS + hist[s] % BS for s in range(S)], dtype=np.int64), dev)
+    bt, sl = t(tables, dev), t((hist + 1).astype(np.int32), dev)
+
+    def inputs(seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return tuple(torch.randn(S, n, 128, device=dev, generator=g).half() for n in (QH, KVH, KVH))
+
+    def run(q, k, v, kv, out):
+        return torch.ops.tq.hybrid_decode_step(q, k, v, kv, out, new_slots, bt, sl, 0, QH, KVH, 128, 0.09, S)
+
+    want = []
+    for seed in (1, 2):
+        kv = fresh_cache()
+        out = torch.zeros(S, QH, 128, dtype=torch.float16, device=dev)
+        run(*inputs(seed), kv, out)
+        want.append((out.clone(), kv.clone()))
+    kv = fresh_cache()
+    sq, sk, sv = (x.clone() for x in inputs(1))
+    sout = torch.zeros(S, QH, 128, dtype=torch.float16, device=dev)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run(sq, sk, sv, kv, sout)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(sq, sk, sv, kv, sout)
+    for rep in range(2):
+        for i, seed in enumerate((1, 2)):
+            q, k, v = inputs(seed)
+            sq.copy_(q); sk.copy_(k); sv.copy_(v)
+            sout.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(sout, want[i][0]) and torch.equal(kv, want[i][1]), (rep, seed)
+            _ = (torch.randn(1 << 16, device=dev) * 2).sum().item()
