@@ -4,7 +4,8 @@ from .kv_cache_dtype import resolve_kv_cache_dtype, KV_CACHE_DTYPES
 from .decompress import batch_decompress_active_blocks, decode_blocks
 from .hooks import register_custom_ops, init_quantizer, reset_state
 from .engine import tq_page_size_bytes, align_page_size, reshape_primary, primary_views
+from .cache import TQGPUCache
 
 __all__ = ["resolve_kv_cache_dtype", "KV_CACHE_DTYPES", "register_custom_ops", "init_quantizer",
            "reset_state", "batch_decompress_active_blocks", "decode_blocks", "tq_page_size_bytes",
-           "align_page_size", "reshape_primary", "primary_views"]
+           "align_page_size", "reshape_primary", "primary_views", "TQGPUCache"]

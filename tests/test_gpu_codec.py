@@ -349,3 +349,48 @@ def test_config0_round_trip_full_size(golden, dev):
     assert (p2 == packed).float().mean().item() > 0.97
     rep = tq.validate(num_vectors=20000)
     assert rep["mse_theory_lower"] <= rep["mse"] <= rep["mse_theory_upper"] and rep["hip_active"]
+
+
+def test_gpu_cache_encode_spill_warm(golden, dev):
+    """TQGPUCache (reference: vllm/cache.py:22-173): encode_and_store equals the fused update on the
+    layer's tensors, spilled blocks survive being overwritten on the device and come back bit for
+    bit, blocks that were never spilled are left alone by warm_blocks."""
+    from aitherkvcache_amd.vllm import TQGPUCache
+
+    def t(a, dev):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    cache = TQGPUCache(num_layers=3, max_blocks=24, block_size=16, num_kv_heads=4, head_dim=128, bits=4, device=str(dev))
+    cache.tq.rotation = torch.from_numpy(golden["rotation_d128_seed42"]).to(dev)
+    rng = np.random.default_rng(77)
+    T = 150
+    slots = rng.permutation(24 * 16)[:T].astype(np.int64)
+    slots[5] = -1                                             # a padding token
+    for layer in range(3):
+        key, val = kv_like(rng, (T, 4, 128)), kv_like(rng, (T, 4, 128))
+        cache.encode_and_store(layer, t(key, dev), t(val, dev), t(slots, dev))
+        kp = torch.zeros_like(cache.k_packed[layer]); kn = torch.zeros_like(cache.k_norms[layer])
+        akv.fused_tq4_kv_update(t(key, dev), t(slots, dev), kp, kn, cache.tq.rotation, cache.tq.boundaries_inner)
+        assert torch.equal(kp, cache.k_packed[layer]) and torch.equal(kn, cache.k_norms[layer])
+        assert int(cache.v_norms[layer].count_nonzero()) == (T - 1) * 4
+    snap = [x.clone() for x in (cache._k_packed, cache._k_norms, cache._v_packed, cache._v_norms)]
+    spill = torch.tensor([3, 17, 0, 9], device=dev)
+    cache.spill_blocks(spill)
+    assert cache.has_spilled(17) and not cache.has_spilled(4)
+    stats = cache.cold_tier_stats()
+    assert stats["cold_blocks"] == 4 and stats["cold_tokens"] == 64 and stats["max_blocks"] == 24
+    assert abs(stats["cold_mb"] - 4 * 2 * 16 * 4 * 68 * 3 / 2 ** 20) < 1e-9
+    for x in (cache._k_packed, cache._k_norms, cache._v_packed, cache._v_norms):
+        x[:, spill] = 0                                       # the device blocks are reused
+        x[:, 5] = 0                                           # so is one that was never spilled
+    cache.warm_blocks(torch.tensor([17, 5, 3, 0, 9]))
+    torch.cuda.synchronize()
+    for now, before in zip((cache._k_packed, cache._k_norms, cache._v_packed, cache._v_norms), snap):
+        keep = torch.ones(24, dtype=torch.bool, device=dev)
+        keep[5] = False
+        assert torch.equal(now[:, keep], before[:, keep])
+        assert not bool(now[:, 5].any())
+    cache.clear_spilled([3, 9])
+    assert not cache.has_spilled(3) and cache.has_spilled(0)
+    cache.spill_blocks(torch.empty(0, dtype=torch.long))
+    cache.warm_blocks(torch.empty(0, dtype=torch.long))
