@@ -629,6 +629,15 @@ __global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict
   __shared__ float w[TRI_MAX_SPLITS];
   __shared__ float red[2];
   const size_t pair = blockIdx.x;  // b * QH + qh
+  // the first partial sums of the thread's coordinate are requested before the weights exist: the
+  // two round trips to memory overlap (D <= 128 coordinates take one pass of the 128 threads)
+  constexpr int PRE = 16;
+  float pre[PRE];
+  {
+    const int i0 = min((int)threadIdx.x, D - 1);
+#pragma unroll
+    for (int s = 0; s < PRE; ++s) pre[s] = part_acc[(pair * nsplit + min(s, nsplit - 1)) * D + i0];
+  }
   if (threadIdx.x < 64) {
     float m = -INFINITY;
     for (int s = threadIdx.x; s < nsplit; s += 64) m = fmaxf(m, part_ml[(pair * nsplit + s) * 2]);
@@ -645,12 +654,19 @@ __global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict
   }
   __syncthreads();
   const float inv = red[0];
+  // (every range writes its partial sums, zeros when it holds no token: the loads need no guard and
+  // can all be in flight together)
   for (int i = threadIdx.x; i < D; i += 128) {
     float acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float ws = w[s];
-      if (ws != 0.f) acc = fmaf(ws, part_acc[(pair * nsplit + s) * D + i], acc);
+    const float* src = part_acc + pair * nsplit * D + i;
+    int s0 = 0;
+    if (i == (int)threadIdx.x) {          // first pass: the prefetched ranges
+#pragma unroll
+      for (int s = 0; s < PRE; ++s) acc = fmaf(s < nsplit ? w[s] : 0.f, pre[s], acc);
+      s0 = PRE;
     }
+#pragma unroll 16
+    for (int s = s0; s < nsplit; ++s) acc = fmaf(w[s], src[(size_t)s * D], acc);
     out[pair * D + i] = acc * inv;
   }
 }
