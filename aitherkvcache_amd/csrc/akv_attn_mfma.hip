@@ -710,8 +710,10 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   if (d != 128 || bits < 2 || bits > 4 || a.block_size != 16) return false;
   const int gqa = a.QH / a.KVH;
   if (gqa > 8) return false;
-  // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword
-  const uintptr_t kalign = bits == 4 ? 15 : bits == 3 ? 3 : 7, valign = bits == 2 ? 1 : 3;
+  // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword.  Multi-dword
+  // loads need dword alignment only, so the serving layout (rows of packed + 4 bytes: pitch 68 / 52 /
+  // 36) qualifies as well as dense rows.
+  const uintptr_t kalign = 3, valign = bits == 2 ? 1 : 3;
   if ((((uintptr_t)a.kp | (uintptr_t)a.kps_blk | (uintptr_t)a.kps_pos | (uintptr_t)a.kps_head) & kalign) != 0) return false;
   if ((((uintptr_t)a.vp | (uintptr_t)a.vps_blk | (uintptr_t)a.vps_pos | (uintptr_t)a.vps_head) & valign) != 0) return false;
   const int64_t strides[12] = {a.kps_blk, a.kps_pos, a.kps_head, a.kns_blk, a.kns_pos, a.kns_head,
