@@ -281,7 +281,7 @@ static bool dm_disabled() {
 int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int out_dtype, const void* rot_prep,
                         hipStream_t stream) {
   if (dm_disabled() || d != 128 || bits < 2 || bits > 4) return AKV_ERR_UNSUPPORTED;
-  const uintptr_t palign = bits == 4 ? 15 : bits == 3 ? 3 : 7;      // a lane reads 16 / 12 / 8 bytes of a row
+  const uintptr_t palign = 3;      // a lane reads 16 / 12 / 8 bytes of a row: multi-dword loads need dword alignment only
   if ((((uintptr_t)a.packed | (uintptr_t)a.ps0) & palign) || ((uintptr_t)a.out & 15)) return AKV_ERR_UNSUPPORTED;
   if (a.os0 & 7) return AKV_ERR_UNSUPPORTED;      // rows of the output are written 8 elements (16 or 32 bytes) per lane
   if (blocks && (((uintptr_t)a.ps1 | (uintptr_t)a.ps2) & palign || ((a.os1 | a.os2) & 7))) return AKV_ERR_UNSUPPORTED;

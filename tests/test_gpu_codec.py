@@ -274,7 +274,8 @@ def test_decode_other_output_dtypes_vs_oracle(golden, dev, bits, dtype):
 
 
 @pytest.mark.parametrize("bits,out_dtype,extra", [(4, torch.float16, 0), (4, torch.float16, 16), (4, torch.bfloat16, 0),
-                                                  (3, torch.float16, 0), (2, torch.float32, 4)])
+                                                  (3, torch.float16, 0), (2, torch.float32, 4),
+                                                  (4, torch.float16, 4), (3, torch.bfloat16, 4)])
 @pytest.mark.parametrize("itype", [torch.int32, torch.int64])
 def test_batch_decompress_active_blocks_vs_oracle(golden, dev, bits, out_dtype, extra, itype):
     from aitherkvcache_amd.vllm import batch_decompress_active_blocks
