@@ -1,4 +1,4 @@
-// MFMA paged decode attention for the 4-, 3- and 2-bit caches at head_dim 128, block_size 16.
+// MFMA paged decode attention for the 4-, 3- and 2-bit caches at head_dim 128, block_size 16 or 32.
 //
 // One workgroup = 16 wavefronts working on one range of (sequence, block) pairs for all kv
 // heads: wavefronts 0-7 are SCORE wavefronts (one per kv head), 8-15 VALUE wavefronts (same
@@ -337,6 +337,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   uint32_t T = 0;        // chunks of this head slot finished in earlier segments (same on both sides)
 
   const int G = gridDim.x;
+  // blocks of 16 tokens: a chunk (32 tokens, two 16-token tiles) is two blocks; blocks of 32: one
+  // block, its second tile 16 positions further in.  bs32 is the same in every wavefront.
+  const bool bs32 = a.block_size == 32;
+  const int bs = bs32 ? 32 : 16;
   const int total = a.prefix[a.S];
   const int per = (total + G - 1) / G;
   const int g0 = blockIdx.x * per;
@@ -349,11 +353,11 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
     const int sb0 = a.prefix[s], sb1 = a.prefix[s + 1];
     const int blk_lo = gcur - sb0;
     const int blk_hi = min(g1, sb1) - sb0;
-    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, 16, a.max_blocks_per_seq);
-    const int t_end = (int)min((int64_t)blk_hi * 16, ctx);
+    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
+    const int t_end = (int)min((int64_t)blk_hi * bs, ctx);
     gcur = sb0 + blk_hi;
     const int nblk = blk_hi - blk_lo;
-    const int nchunks = (nblk + 1) >> 1;
+    const int nchunks = bs32 ? nblk : (nblk + 1) >> 1;
 
     for (int hbase = 0; hbase < a.KVH; hbase += MF_HEADS) {
       const int h = hbase + hs;
@@ -365,21 +369,22 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       if (!active || nchunks <= 0) continue;
       const int hh = h;
 
-      // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment.
+      // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment
+      // (win_c0 + i for blocks of 32).
       // A window of 64 ids serves MF_WIN chunks plus the two-chunk lookahead of the prefetch.  Its
       // reload drains every outstanding load (once per MF_WIN chunks); the chunk loop itself issues
       // the same loads on every path, so its waits stay counted waits for the chunk that is due.
       int pbwin = 0, win_c0 = 0;
       auto load_window = [&](int c0) {
-        const int bi = min(blk_lo + 2 * c0 + lane, blk_hi - 1);
+        const int bi = min(blk_lo + (bs32 ? c0 : 2 * c0) + lane, blk_hi - 1);
         pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
         asm volatile("" : "+v"(pbwin));   // the window is complete here, not "maybe in flight" in the loop
         win_c0 = c0;
       };
       auto chunk_blocks = [&](int c_in, uint32_t& p0, uint32_t& p1) {
         const int c = min(c_in, nchunks - 1);      // lookahead past the end re-reads the last chunk
-        const int w0 = 2 * (c - win_c0);
-        const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
+        const int w0 = bs32 ? c - win_c0 : 2 * (c - win_c0);
+        const int w1 = (!bs32 && 2 * c + 1 < nblk) ? w0 + 1 : w0;
         p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
         p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
       };
@@ -405,8 +410,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const bool nrm_is_v = lane >= 32;
         const float* nrm_base = nrm_is_v ? a.vn : a.kn;
         const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vns_blk : a.kns_blk);
-        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hh * a.vns_head + (ntok & 15) * a.vns_pos
-                                                     : hh * a.kns_head + (ntok & 15) * a.kns_pos);
+        const int npos = bs32 ? ntok : (ntok & 15);        // position of token ntok inside its block
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hh * a.vns_head + npos * a.vns_pos
+                                                     : hh * a.kns_head + npos * a.kns_pos);
+        const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
         const uint32_t nw_addr = MF_TABB + (32u * hs + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = MF_TABB + (32u * hs + 10u) * 256u + 128u + (uint32_t)g * 16u;
         auto load_chunk = [&](mf_kraw& r, int c) {
@@ -414,7 +421,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const unsigned char* kr = a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + mf_here(koff);
+            const unsigned char* kr = a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + (j ? ktile1 : 0u) + mf_here(koff);
             if constexpr (BITS == 4) {
               r.k[j] = *(const uint4*)kr;
             } else if constexpr (BITS == 3) {
@@ -475,13 +482,13 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             }
           }
           if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
-            const int tok0 = (blk_lo + 2 * c) * 16;
+            const int tok0 = blk_lo * bs + 32 * c;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 const int tok = tok0 + 16 * j + 4 * g + i;
-                const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
+                const bool ok = (tok < t_end) && (j == 0 || bs32 || 2 * c + 1 < nblk);
                 if (!ok) sv[4 * j + i] = -INFINITY;
               }
           }
@@ -559,6 +566,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         // (taken from the aligned dword holding the first of them and, where they run over, from the
         // neighbour lane's dword), or one halfword
         const uint32_t voff = (uint32_t)(hh * a.vps_head + 4 * g * a.vps_pos + (BITS == 4 ? 4 * col : BITS == 3 ? ((3 * col) & ~3) : 2 * col));
+        const uint32_t vtile1 = bs32 ? 16u * (uint32_t)a.vps_pos : 0u;     // second tile inside the same block
         const uint32_t o3 = (uint32_t)(3 * col) & 3u;
         const uint32_t sel3 = 0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u);   // big-endian 24-bit word
         auto load_chunk = [&](mf_vraw& r, int c) {
@@ -566,7 +574,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const unsigned char* vb = a.vp + mf_umul(pb[j], (uint32_t)a.vps_blk);
+            const unsigned char* vb = a.vp + mf_umul(pb[j], (uint32_t)a.vps_blk) + (j ? vtile1 : 0u);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {    // the token step rides in the uniform base
               const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff);
@@ -707,7 +715,7 @@ size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
 
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   if (mfma_disabled()) return false;
-  if (d != 128 || bits < 2 || bits > 4 || a.block_size != 16) return false;
+  if (d != 128 || bits < 2 || bits > 4 || (a.block_size != 16 && a.block_size != 32)) return false;
   const int gqa = a.QH / a.KVH;
   if (gqa > 8) return false;
   // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword.  Multi-dword

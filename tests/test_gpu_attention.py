@@ -145,6 +145,70 @@ def test_other_block_sizes(golden, dev, block_size):
     assert within_tol(out.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_blocks_of_32_tokens(golden, dev, bits):
+    """Blocks of 32 tokens (one chunk of the matrix-core kernel = one block, its second 16-token tile
+    sixteen positions in): ragged batch against the oracle, then a batch large enough that every
+    workgroup runs through several windows of block ids, checked by the uniform-value property and,
+    for one sequence, against the oracle."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(320 + bits)
+    KVH, QH, BS = 8, 32, 32
+    NB = 200
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, bits, block_size=BS)
+    ctx = np.array([1, 31, 32, 33, 1000, 0, 2048, 777], dtype=np.int64)
+    tables = np.full((len(ctx), 64), -5, dtype=np.int64)
+    perm = rng.permutation(NB)
+    off = 0
+    for s_, c_ in enumerate(ctx):
+        nb = -(-int(c_) // BS)
+        tables[s_, :nb] = perm[off:off + nb]
+        off += nb
+    q = rng.standard_normal((len(ctx), QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), block_size=BS)
+    ref = oracle_out(q, kp, kn, vp, vn, np.maximum(tables, 0), ctx, golden, bits, block_size=BS)
+    assert within_tol(out.cpu().numpy(), ref) and not bool(out[5].any())
+    # large: 16 sequences x 32768 tokens
+    S, CTX = 16, 32768
+    nb_seq = CTX // BS
+    NBL = S * nb_seq
+    P = tq._packed_dim
+    kpl = torch.empty(NBL, BS, KVH, P, dtype=torch.uint8, device=dev)
+    knl = torch.empty(NBL, BS, KVH, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(11)
+    CH = 1024
+    for b0 in range(0, NBL, CH):
+        b1 = min(NBL, b0 + CH)
+        x = torch.randn((b1 - b0) * BS * KVH, 128, device=dev, generator=gen).half()
+        pk, nr = tq.encode(x)
+        kpl[b0:b1] = pk.reshape(b1 - b0, BS, KVH, P)
+        knl[b0:b1] = nr.reshape(b1 - b0, BS, KVH)
+    v1 = kv_like(rng, (1, KVH, 128))
+    vp1, vn1 = tq.encode(t(v1, dev))
+    vpl = vp1.reshape(1, 1, KVH, P).expand(NBL, BS, KVH, P).contiguous()
+    vnl = vn1.reshape(1, 1, KVH).expand(NBL, BS, KVH).contiguous()
+    tabl = rng.permutation(NBL).reshape(S, nb_seq).astype(np.int32)
+    ctxl = np.full(S, CTX, dtype=np.int64)
+    ctxl[3], ctxl[9] = CTX - 45, 3000
+    ql = rng.standard_normal((S, QH, 128)).astype(np.float16)
+    outl = attn.forward(t(ql, dev), kpl, knl, vpl, vnl, t(tabl, dev), t(ctxl, dev), block_size=BS).float()
+    want = tq.decode(vp1, vn1).float().reshape(KVH, 1, 128).expand(KVH, 4, 128).reshape(1, QH, 128)
+    assert bool(torch.all(torch.abs(outl - want) <= TOL + 2.0 ** -10 * want.abs()))
+    s_ = 9
+    vp_r, vn_r = kpl.roll(3, 0), knl.roll(3, 0)
+    o = attn.forward(t(ql[s_:s_ + 1], dev), kpl, knl, vp_r, vn_r, t(tabl[s_:s_ + 1], dev), t(ctxl[s_:s_ + 1], dev),
+                     block_size=BS)
+    nbu = -(-int(ctxl[s_]) // BS)
+    used = np.unique(tabl[s_, :nbu])
+    remap = {b: i for i, b in enumerate(used)}
+    small_tab = np.array([[remap[b] for b in tabl[s_, :nbu]]])
+    idx = t(used.astype(np.int64), dev)
+    ref1 = oracle_out(ql[s_:s_ + 1], kpl[idx], knl[idx], vp_r[idx], vn_r[idx], small_tab, ctxl[s_:s_ + 1], golden, bits,
+                      block_size=BS)
+    assert within_tol(o.cpu().numpy(), ref1)
+
+
 def test_long_context_split_invariants(golden, dev):
     """Sizes where a sequence is cut across many workgroups: results must not depend on where the
     cuts fall.  (a) against the float64 oracle; (b) the same sequence alone or inside a batch
