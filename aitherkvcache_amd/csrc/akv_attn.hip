@@ -380,6 +380,7 @@ extern "C" int akv_paged_attn(
   a.S = num_seqs; a.QH = num_q_heads; a.KVH = num_kv_heads; a.block_size = block_size;
   a.max_blocks_per_seq = max_blocks_per_seq; a.scale = scale;
   a.prefix = ws.prefix; a.qrot = ws.qrot; a.part_acc = ws.part_acc; a.part_ml = ws.part_ml;
+  a.hgroup = 1;
 
   int rc;
   int Gused = G;

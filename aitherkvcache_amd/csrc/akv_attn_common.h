@@ -31,6 +31,9 @@ struct akv_attn_args {
   const float* qrot;
   float* part_acc;
   float* part_ml;
+  // matrix-core kernel only: a kv head with more than eight query heads is presented as `hgroup`
+  // heads of QH / (KVH * hgroup) query heads each that read the same rows (KVH then counts those)
+  int hgroup;
 };
 
 static inline int akv_attn_grid() {

@@ -368,6 +368,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       // for ALL loads, prefetches included, wherever the loop first touches their registers.)
       if (!active || nchunks <= 0) continue;
       const int hh = h;
+      const int hd = a.hgroup > 1 ? h / a.hgroup : h;      // the head whose rows are read
 
       // physical block ids: lane i of pbwin holds the id of block (2 * win_c0 + i) of the segment
       // (win_c0 + i for blocks of 32).
@@ -402,7 +403,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           }
         }
         float m_run = -INFINITY, l_run = 0.f;
-        const uint32_t koff = (uint32_t)(hh * a.kps_head + col * a.kps_pos + (BITS == 4 ? 16 : BITS == 3 ? 12 : 8) * g);
+        const uint32_t koff = (uint32_t)(hd * a.kps_head + col * a.kps_pos + (BITS == 4 ? 16 : BITS == 3 ? 12 : 8) * g);
         // norms travel one per lane (lanes [0,32): K norm of token l, lanes [32,64): V norm of token
         // l - 32), prefetched with the codes, and are spread to the accumulator layout through the
         // spare halves of table B entries 16q + 10 (K) and 16q + 11 (V)
@@ -411,8 +412,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const float* nrm_base = nrm_is_v ? a.vn : a.kn;
         const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vns_blk : a.kns_blk);
         const int npos = bs32 ? ntok : (ntok & 15);        // position of token ntok inside its block
-        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hh * a.vns_head + npos * a.vns_pos
-                                                     : hh * a.kns_head + npos * a.kns_pos);
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vns_head + npos * a.vns_pos
+                                                     : hd * a.kns_head + npos * a.kns_pos);
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
         const uint32_t nw_addr = MF_TABB + (32u * hs + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = MF_TABB + (32u * hs + 10u) * 256u + 128u + (uint32_t)g * 16u;
@@ -565,7 +566,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         // token 4g of a tile; the eight codes of coordinates 8 col .. 8 col + 7: one dword, three bytes
         // (taken from the aligned dword holding the first of them and, where they run over, from the
         // neighbour lane's dword), or one halfword
-        const uint32_t voff = (uint32_t)(hh * a.vps_head + 4 * g * a.vps_pos + (BITS == 4 ? 4 * col : BITS == 3 ? ((3 * col) & ~3) : 2 * col));
+        const uint32_t voff = (uint32_t)(hd * a.vps_head + 4 * g * a.vps_pos + (BITS == 4 ? 4 * col : BITS == 3 ? ((3 * col) & ~3) : 2 * col));
         const uint32_t vtile1 = bs32 ? 16u * (uint32_t)a.vps_pos : 0u;     // second tile inside the same block
         const uint32_t o3 = (uint32_t)(3 * col) & 3u;
         const uint32_t sel3 = 0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u);   // big-endian 24-bit word
@@ -713,11 +714,17 @@ size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
   return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * KVH * 8 * 64 * 16);
 }
 
+// query heads per kv head -> number of groups of at most eight the kv head is presented as (0: none fits)
+static int akv_attn_mfma_head_groups(int gqa) {
+  for (int hg = (gqa + 7) / 8; hg <= gqa && hg <= 8; ++hg)
+    if (gqa % hg == 0) return hg;
+  return 0;
+}
+
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   if (mfma_disabled()) return false;
   if (d != 128 || bits < 2 || bits > 4 || (a.block_size != 16 && a.block_size != 32)) return false;
-  const int gqa = a.QH / a.KVH;
-  if (gqa > 8) return false;
+  if (akv_attn_mfma_head_groups(a.QH / a.KVH) == 0) return false;
   // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword.  Multi-dword
   // loads need dword alignment only, so the serving layout (rows of packed + 4 bytes: pitch 68 / 52 /
   // 36) qualifies as well as dense rows.
@@ -732,7 +739,10 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
 }
 
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                      const akv_attn_args& a, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
+                      const akv_attn_args& a_in, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
+  akv_attn_args a = a_in;
+  a.hgroup = akv_attn_mfma_head_groups(a.QH / a.KVH);
+  a.KVH *= a.hgroup;                        // from here on: groups of at most eight query heads
   akv_mfma_extra x;
   char* p = (char*)extra_ws;
   x.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
