@@ -117,6 +117,161 @@ __global__ __launch_bounds__(256) void hyb_encode_kernel(hyb_enc_args a) {
 }
 
 // ----------------------------------------------------------------------------------
+// encode, one LANE per vector (rows of 16-byte aligned input and output): the 64-point transforms run
+// in the lane's registers, so no lane ever talks to another -- 384 additions per transform where the
+// wavefront-per-vector form above spends six shuffles per coordinate for one vector at a time.  Every
+// operation, the order of the butterflies and the order of the sums are those of the kernel above
+// (and of the reference); only the division is a reciprocal with one correction step.
+// ----------------------------------------------------------------------------------
+__device__ __forceinline__ void hyb_fwht64_regs(float (&v)[64]) {
+#pragma unroll
+  for (int h = 1; h < 64; h <<= 1)
+#pragma unroll
+    for (int i = 0; i < 64; ++i)
+      if ((i & h) == 0) {
+        const float lo = v[i], hi = v[i + h];
+        v[i] = __fadd_rn(lo, hi);
+        v[i + h] = __fsub_rn(lo, hi);
+      }
+}
+// sum in the order of the wavefront reduction (partners 32, 16, ..., 1 apart)
+__device__ __forceinline__ float hyb_tree_sum64(float (&t)[64]) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1)
+#pragma unroll
+    for (int i = 0; i < m; ++i) t[i] = __fadd_rn(t[i], t[i + m]);
+  return t[0];
+}
+__device__ __forceinline__ void hyb_put_byte(uint32_t* words, int k, uint32_t byte) { words[k >> 2] |= byte << (8 * (k & 3)); }
+
+// one group of 64 coordinates of the lane's vector -> MB-bit codes, sign bits and the two norms as
+// dwords of the packed row (6 / 4 dwords of codes, 2 of signs, 1 of norms)
+template <int XDT, int MB>
+__device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off, const float* had,
+                                                       const float* qjl, const float* cen, const float* bnd,
+                                                       uint32_t* words) {
+  constexpr int CW = 64 * MB / 32;       // dwords of codes
+  float u[64], v[64];
+  if constexpr (XDT == AKV_F32) {
+    const float4* p = (const float4*)((const float*)x + off);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { const float4 q = p[i]; u[4 * i] = q.x; u[4 * i + 1] = q.y; u[4 * i + 2] = q.z; u[4 * i + 3] = q.w; }
+  } else {
+    const uint4* p = (const uint4*)((const unsigned short*)x + off);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint4 q = p[i];
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (XDT == AKV_F16) {
+          u[8 * i + 2 * j] = __half2float(__ushort_as_half((unsigned short)(w[j] & 0xffffu)));
+          u[8 * i + 2 * j + 1] = __half2float(__ushort_as_half((unsigned short)(w[j] >> 16)));
+        } else {
+          u[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+          u[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 64; ++j) v[j] = __fmul_rn(u[j], u[j]);
+  const float nrm = sqrtf(hyb_tree_sum64(v));
+  const float den = __fadd_rn(nrm, 1e-10f);
+  const float rcp = __frcp_rn(den);
+  const bool plain = !(den < INFINITY);
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    // x / den: reciprocal, then one correction step (the correctly rounded quotient but for rare ties)
+    const float q0 = __fmul_rn(u[j], rcp);
+    const float e = fmaf(-q0, den, u[j]);
+    // (an infinite or NaN norm: x * (1 / den) alone already is what the division gives)
+    const float q = plain ? q0 : fmaf(e, rcp, q0);
+    u[j] = q;
+    v[j] = __fmul_rn(q, had[j]);
+  }
+  hyb_fwht64_regs(v);
+#pragma unroll
+  for (int k = 0; k < CW + 3; ++k) words[k] = 0u;
+  // codes: MSB-first stream; the centroid of every code goes straight into the next transform
+  if constexpr (MB == 3) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      uint32_t g24 = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t c = akv_search<3>(__fmul_rn(v[8 * g + i], 0.125f), bnd);
+        g24 |= c << (21 - 3 * i);
+        v[8 * g + i] = cen[c];
+      }
+      hyb_put_byte(words, 3 * g, g24 >> 16);
+      hyb_put_byte(words, 3 * g + 1, (g24 >> 8) & 0xffu);
+      hyb_put_byte(words, 3 * g + 2, g24 & 0xffu);
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      uint32_t b = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t c = akv_search<2>(__fmul_rn(v[4 * k + i], 0.125f), bnd);
+        b |= c << (6 - 2 * i);
+        v[4 * k + i] = cen[c];
+      }
+      hyb_put_byte(words, k, b);
+    }
+  }
+  hyb_fwht64_regs(v);
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    const float mse_hat = __fmul_rn(__fmul_rn(v[j], had[j]), 0.125f);
+    u[j] = __fsub_rn(u[j], mse_hat);              // residual
+    v[j] = __fmul_rn(u[j], u[j]);
+  }
+  const float rn = sqrtf(hyb_tree_sum64(v));
+#pragma unroll
+  for (int j = 0; j < 64; ++j) v[j] = __fmul_rn(u[j], qjl[j]);
+  hyb_fwht64_regs(v);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    uint32_t b = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b |= (__fmul_rn(v[8 * k + i], 0.125f) >= 0.f ? 1u : 0u) << (7 - i);
+    hyb_put_byte(words + CW, k, b);
+  }
+  words[CW + 2] = (uint32_t)__half_as_ushort(__float2half_rn(nrm)) | ((uint32_t)__half_as_ushort(__float2half_rn(rn)) << 16);
+}
+
+template <int XDT, bool PAGED>
+__global__ __launch_bounds__(256) void hyb_encode_lane_kernel(hyb_enc_args a) {
+  __shared__ float tab[AKV_HYB_TABLE_FLOATS];
+  for (int i = threadIdx.x; i < AKV_HYB_TABLE_FLOATS; i += 256) tab[i] = a.table[i];
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= a.n) return;
+  uint8_t* dst;
+  int64_t off;
+  if (PAGED) {
+    const int64_t tok = n / a.heads, head = n - tok * a.heads;
+    off = tok * a.xs0 + head * a.xs1;
+    const int64_t slot = akv_load_index(a.slots, a.slot_itype, tok);
+    if (slot < 0) return;
+    const int64_t blk = slot / a.block_size, pos = slot - blk * a.block_size;
+    if (blk >= a.max_blocks) return;
+    dst = a.out + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+  } else {
+    off = n * a.xs0;
+    dst = a.out + n * a.ps0;
+  }
+  uint32_t row[16];
+  hyb_encode_group_lane<XDT, 3>(a.x, off, tab + HYB_HAD0, tab + HYB_QJL0, tab + HYB_CEN0, tab + HYB_BND0, row);
+  hyb_encode_group_lane<XDT, 2>(a.x, off + 64, tab + HYB_HAD1, tab + HYB_QJL1, tab + HYB_CEN1, tab + HYB_BND1, row + 9);
+  uint4* d4 = (uint4*)dst;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) d4[i] = make_uint4(row[4 * i], row[4 * i + 1], row[4 * i + 2], row[4 * i + 3]);
+}
+
+// ----------------------------------------------------------------------------------
 // decode: one wavefront per vector
 // ----------------------------------------------------------------------------------
 template <int MB>
@@ -393,8 +548,31 @@ static int hyb_grid(int64_t n) {
   return (int)(g < 1 ? 1 : (g > cap ? cap : g));
 }
 
+static bool hyb_lane_disabled() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("AKV_HYBRID_WAVE_ENCODE");
+    v = (e && e[0] == '1') ? 1 : 0;
+  }
+  return v == 1;
+}
+
 template <bool PAGED>
 static int hyb_launch_encode(int dt, const hyb_enc_args& a, hipStream_t stream) {
+  // 16-byte aligned input rows and packed rows: one lane per vector
+  const int64_t xal = dt == AKV_F32 ? 3 : 7;      // elements per 16 bytes, minus one
+  const bool lane_form = (((uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.ps0 | (uintptr_t)(PAGED ? a.ps1 | a.ps2 : 0)) & 15) == 0 &&
+                         ((a.xs0 | (PAGED ? a.xs1 : 0)) & xal) == 0 && !hyb_lane_disabled();
+  if (lane_form) {
+    const int lgrid = (int)((a.n + 255) / 256);
+    switch (dt) {
+      case AKV_F16: hyb_encode_lane_kernel<AKV_F16, PAGED><<<lgrid, 256, 0, stream>>>(a); break;
+      case AKV_BF16: hyb_encode_lane_kernel<AKV_BF16, PAGED><<<lgrid, 256, 0, stream>>>(a); break;
+      default: hyb_encode_lane_kernel<AKV_F32, PAGED><<<lgrid, 256, 0, stream>>>(a); break;
+    }
+    AKV_LAUNCH_CHECK("hyb_encode_lane_kernel");
+    return AKV_OK;
+  }
   const int grid = hyb_grid(a.n);
   switch (dt) {
     case AKV_F16: hyb_encode_kernel<AKV_F16, PAGED><<<grid, 256, 0, stream>>>(a); break;
