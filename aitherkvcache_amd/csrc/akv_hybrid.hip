@@ -24,6 +24,7 @@
 #define HYB_BND0 268
 #define HYB_BND1 275
 
+static bool hyb_lane_disabled();
 static const float kHybKappa = (float)(1.2533141373155001 / 64.0);  // sqrt(pi/2) / 64
 
 __device__ __forceinline__ float hyb_fwht64(float v, int lane) {
@@ -123,6 +124,13 @@ __global__ __launch_bounds__(256) void hyb_encode_kernel(hyb_enc_args a) {
 // operation, the order of the butterflies and the order of the sums are those of the kernel above
 // (and of the reference); only the division is a reciprocal with one correction step.
 // ----------------------------------------------------------------------------------
+// (The "_rn" arithmetic helpers of the HIP headers are plain operators, which the compiler may fuse
+// into multiply-adds; the reference rounds every operation.  Where a product that is not exact feeds
+// a sum, it passes through hyb_rounded(), an empty asm statement the optimiser cannot see through.)
+__device__ __forceinline__ float hyb_rounded(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
 __device__ __forceinline__ void hyb_fwht64_regs(float (&v)[64]) {
 #pragma unroll
   for (int h = 1; h < 64; h <<= 1)
@@ -175,7 +183,7 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
     }
   }
 #pragma unroll
-  for (int j = 0; j < 64; ++j) v[j] = __fmul_rn(u[j], u[j]);
+  for (int j = 0; j < 64; ++j) v[j] = hyb_rounded(__fmul_rn(u[j], u[j]));
   const float nrm = sqrtf(hyb_tree_sum64(v));
   const float den = __fadd_rn(nrm, 1e-10f);
   const float rcp = __frcp_rn(den);
@@ -226,7 +234,7 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
   for (int j = 0; j < 64; ++j) {
     const float mse_hat = __fmul_rn(__fmul_rn(v[j], had[j]), 0.125f);
     u[j] = __fsub_rn(u[j], mse_hat);              // residual
-    v[j] = __fmul_rn(u[j], u[j]);
+    v[j] = hyb_rounded(__fmul_rn(u[j], u[j]));
   }
   const float rn = sqrtf(hyb_tree_sum64(v));
 #pragma unroll
@@ -308,6 +316,50 @@ __global__ __launch_bounds__(256) void hyb_decode_kernel(const uint8_t* __restri
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
+}
+
+// decode, one lane per vector (16-byte aligned rows): the same operations as above, transforms in registers
+template <int MB>
+__device__ __forceinline__ void hyb_decode_group_lane(const uint32_t* words, const float* had, const float* qjl,
+                                                       const float* cen, float kappa, float* out) {
+  constexpr int CW = 64 * MB / 32;
+  auto byte_of = [&](int k) { return (words[k >> 2] >> (8 * (k & 3))) & 0xffu; };
+  float v[64], w[64];
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    v[j] = cen[akv_stream_code<MB>(j, byte_of)];
+    const uint32_t bit = (byte_of(4 * CW + (j >> 3)) >> (7 - (j & 7))) & 1u;
+    w[j] = bit ? kappa : -kappa;
+  }
+  hyb_fwht64_regs(v);
+  hyb_fwht64_regs(w);
+  const float n = hyb_half_bits_to_float(words[CW + 2]);
+  const float rn = hyb_half_bits_to_float(words[CW + 2] >> 16);
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    const float mse_hat = __fmul_rn(__fmul_rn(v[j], had[j]), 0.125f);
+    const float qjl_hat = __fmul_rn(__fmul_rn(w[j], qjl[j]), 0.125f);
+    v[j] = __fmul_rn(__fadd_rn(mse_hat, hyb_rounded(__fmul_rn(qjl_hat, rn))), n);
+  }
+  float4* o4 = (float4*)out;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o4[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+}
+
+__global__ __launch_bounds__(256) void hyb_decode_lane_kernel(const uint8_t* __restrict__ packed, int64_t ps,
+                                                              int64_t n_vec, const float* __restrict__ table,
+                                                              float kappa, float* __restrict__ out, int64_t os) {
+  __shared__ float tab[AKV_HYB_TABLE_FLOATS];
+  for (int i = threadIdx.x; i < AKV_HYB_TABLE_FLOATS; i += 256) tab[i] = table[i];
+  __syncthreads();
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= n_vec) return;
+  uint32_t row[16];
+  const uint4* p = (const uint4*)(packed + n * ps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { const uint4 q = p[i]; row[4 * i] = q.x; row[4 * i + 1] = q.y; row[4 * i + 2] = q.z; row[4 * i + 3] = q.w; }
+  hyb_decode_group_lane<3>(row, tab + HYB_HAD0, tab + HYB_QJL0, tab + HYB_CEN0, kappa, out + n * os);
+  hyb_decode_group_lane<2>(row + 9, tab + HYB_HAD1, tab + HYB_QJL1, tab + HYB_CEN1, kappa, out + n * os + 64);
 }
 
 // ----------------------------------------------------------------------------------
@@ -621,6 +673,13 @@ extern "C" int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_by
   if (n == 0) return AKV_OK;
   AKV_REQUIRE(packed && hyb_table && out, "akv_hybrid_decode: null pointer");
   AKV_REQUIRE(packed_stride_bytes >= 64 && out_stride >= 128, "akv_hybrid_decode: stride smaller than row");
+  if (!hyb_lane_disabled() && (((uintptr_t)packed | (uintptr_t)packed_stride_bytes | (uintptr_t)out) & 15) == 0 &&
+      (out_stride & 3) == 0) {
+    hyb_decode_lane_kernel<<<(int)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(packed, packed_stride_bytes, n,
+                                                                                  hyb_table, kHybKappa, out, out_stride);
+    AKV_LAUNCH_CHECK("hyb_decode_lane_kernel");
+    return AKV_OK;
+  }
   hyb_decode_kernel<<<hyb_grid(n), 256, 0, (hipStream_t)stream>>>(packed, packed_stride_bytes, n, hyb_table,
                                                                   kHybKappa, out, out_stride);
   AKV_LAUNCH_CHECK("hyb_decode_kernel");
