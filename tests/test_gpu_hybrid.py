@@ -252,3 +252,28 @@ def test_hybrid_decode_step_replays_from_a_graph(golden, dev):
             torch.cuda.synchronize()
             assert torch.equal(sout, want[i][0]) and torch.equal(kv, want[i][1]), (rep, seed)
             _ = (torch.randn(1 << 16, device=dev) * 2).sum().item()
+
+
+def test_both_codec_forms_agree(golden, dev):
+    """Rows that are 16-byte aligned take the lane-per-vector kernels, any others the
+    wavefront-per-vector kernels: same bytes from both on the same vectors (paged store into rows of
+    pitch 68, flat encode of an input whose rows start at odd element offsets), same decoded floats."""
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform(num_kv_heads=4)
+    rng = np.random.default_rng(71)
+    NB, BS, KVH = 6, 16, 4
+    x = t(kv_like(rng, (NB * BS, KVH, 128)), dev)
+    slots = torch.arange(NB * BS, device=dev)
+    aligned = torch.zeros(NB, BS, KVH, 64, dtype=torch.uint8, device=dev)
+    pitched = torch.zeros(NB, BS, KVH, 68, dtype=torch.uint8, device=dev)
+    akv.hybrid_encode_and_store(h, x, slots, aligned, BS)
+    akv.hybrid_encode_and_store(h, x, slots, pitched, BS)
+    assert torch.equal(aligned, pitched[..., :64]) and not bool(pitched[..., 64:].any())
+    flat = h.encode(x.reshape(-1, 128))
+    assert torch.equal(flat.reshape(NB, BS, KVH, 64), aligned)
+    shifted = torch.zeros(NB * BS * KVH, 131, dtype=x.dtype, device=dev)
+    shifted[:, 3:] = x.reshape(-1, 128)
+    assert torch.equal(h.encode(shifted[:, 3:]), flat)
+    d_a = h.decode(aligned.reshape(-1, 64))
+    d_p = h.decode(pitched.reshape(-1, 68)[:, :64])
+    assert torch.equal(d_a, d_p)
