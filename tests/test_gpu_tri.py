@@ -186,3 +186,41 @@ def test_paged_decode_without_table_columns(dev):
     out = tri.decode_step_paged(q, cache, torch.zeros(3, 0, dtype=torch.int32, device=dev),
                                 torch.tensor([5, 0, 9], device=dev, dtype=torch.int32))
     assert out.shape == (3, 32, 128) and not bool(out.any())
+
+
+@pytest.mark.parametrize("S", [1, 63, 64, 65, 200])
+@pytest.mark.parametrize("qdtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_short_sequences_zero_and_large_values(dev, S, qdtype):
+    """Sequences around one chunk of 64 tokens; value rows that are all zero (their stored scale is 0)
+    and value rows a thousand times larger than the rest; float16 / bfloat16 queries."""
+    cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(S)
+    B, KVH, QH, D = 2, 8, 32, 128
+    keys = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    vals[:, ::3] = 0
+    vals[:, 1::7] *= 1000
+    k_enc, v_enc = tri.encode_kv(t(keys, dev), t(vals, dev))
+    assert float(v_enc.scales[0, 0, 0]) == 0.0
+    q = torch.from_numpy(rng.standard_normal((B, QH, D)).astype(np.float32)).to(dev).to(qdtype)
+    out = tri.decode_step(q, k_enc, v_enc).cpu().numpy()
+    ref = O.tri_decode_step(q.float().cpu().numpy(), tuple(x.cpu().numpy() for x in k_enc),
+                            tuple(x.cpu().numpy() for x in v_enc), tri._theta.cpu().numpy())
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert np.max(np.abs(out - ref)) <= TOL * scale
+
+
+def test_empty_batch_and_empty_sequence(dev):
+    cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32)
+    tri = TriAttention(cfg, device=str(dev))
+
+    def enc(b, s):
+        return SpectralEncoding(torch.zeros(b, s, 8, 12, dtype=torch.uint8, device=dev),
+                                torch.zeros(b, s, 8, 12, dtype=torch.uint8, device=dev),
+                                torch.zeros(b, s, 8, dtype=torch.float16, device=dev))
+
+    out = tri.decode_step(torch.randn(3, 32, 128, device=dev), enc(3, 0), enc(3, 0))
+    assert out.shape == (3, 32, 128) and not bool(out.any())
+    out0 = tri.decode_step(torch.randn(0, 32, 128, device=dev), enc(0, 5), enc(0, 5))
+    assert out0.shape == (0, 32, 128)
