@@ -768,3 +768,618 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   AKV_LAUNCH_CHECK("akv_attn_mfma_kernel");
   return AKV_OK;
 }
+
+// ==================================================================================
+// tq35 rows on the same machinery
+// ==================================================================================
+// A tq35 row is four parts per token: A0 (64 codes of 3 bits), B0 (64 sign bits), A1 (64 codes of
+// 2 bits), B1 (64 sign bits), plus two fp16 factors per group inside the row.  Spread to one code
+// per nibble they are 256 "virtual coordinates" over ONE table of sixteen levels -- 0..7 the 3-bit
+// codebook, 8..11 the 2-bit codebook, 12 / 13 the signs -1 / +1 -- so the byte-pair tables and
+// both products of the kernel above serve unchanged:
+//
+//   scores   four accumulators per 16-token tile, one per part (lane group g supplies nibble dwords
+//            2g and 2g+1 of the part, four MFMAs per part), combined per token as
+//            n0 (A0 + r0 B0) + n1 (A1 + r1 B1); the query operand holds the four transformed copies of
+//            the query (aither_kvcache/hybrid_quantizer.py:600-640) in the coordinate order the
+//            spreading leaves.
+//   values   an M-tile mixes two parts so that a lane owns a dword-aligned piece of the row.  Pass C:
+//            rows 0-7 the eight 3-byte groups of A0, rows 8-15 the eight halfwords of A1; pass S: rows
+//            0-7 the sign bytes of B0, rows 8-15 those of B1.  The weight operand of a pass carries both
+//            of its parts' weights (p n0 and p n1, or p n0 r0 and p n1 r1): columns 4t + q hold the fp16
+//            part of set t for query head q of the group of four, columns 8 + 4t + q the remainder, and
+//            a lane keeps the results whose rows belong to its column's set.  The V table holds
+//            fp16(alpha c) with one alpha per codebook and the signs as exactly -1 / +1; 1 / alpha and
+//            kappa = sqrt(pi/2)/64 are applied to the finished sums (on the score side kappa rides in
+//            the query copies).
+//
+// One workgroup = 8 wavefronts: 4 score + 4 value (two passes of 8 accumulator tiles need twice the
+// registers of the uniform formats), four groups of four query heads at a time.
+#include "akv_hybrid_layout.h"
+
+#define HM_HEADS 4
+#define HM_THREADS 512
+#define HM_NORMX ((uint32_t)MF_LDS_BYTES)    // float32 factors of a chunk: [parity][head slot][K | V][tile][field][16 tokens]
+#define HM_WBUF2 (HM_NORMX + 2u * HM_HEADS * 1024u)   // weight operand of the second value pass
+#define HM_LDS_BYTES (MF_LDS_BYTES + 4 * HM_HEADS * 1024)
+#define HM_BITS_TAG 35
+
+// level v of the merged table; the sign levels carry `sign_mag`
+__device__ __forceinline__ float hm_level(const float* __restrict__ table, int v, float sign_mag) {
+  return v < 12 ? table[HYB_CEN0 + v] : v == 12 ? -sign_mag : v == 13 ? sign_mag : 0.f;
+}
+
+// coordinate (0..63 inside its part) of nibble (byte b, lo = low nibble) of nibble dword D of part X
+// (0 = A0, 1 = B0, 2 = A1, 3 = B1)
+__host__ __device__ constexpr int hm_coord(int X, int D, int b, int lo) {
+  if (X == 0) return 8 * D + mf_kcoord<3>(0, b, lo);
+  if (X == 2) return 8 * D + (b == 0 ? 2 : b == 1 ? 0 : b == 2 ? 6 : 4) + lo;   // mf_spread2: bytes (c2,c3) (c0,c1) (c6,c7) (c4,c5)
+  return 8 * D + 6 - 2 * b + lo;                                                  // hm_spread1: nibble i <- bit i <- coordinate 7 - i
+}
+
+// eight sign bits (coordinate k at bit 7 - k) -> nibbles 12 | bit, nibble i <- bit i
+__device__ __forceinline__ uint32_t hm_spread1(uint32_t b) {
+  uint32_t t = (b | (b << 12)) & 0x000F000Fu;
+  t = (t | (t << 6)) & 0x03030303u;
+  return ((t | (t << 3)) & 0x11111111u) | 0xCCCCCCCCu;
+}
+
+template <int QDT>
+__global__ __launch_bounds__(256) void akv_hyb_mfma_prologue_kernel(
+    const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ table,
+    float kappa, float qscale, int S, int QH, int KVH, const void* context_lens, int cl_itype,
+    int block_size, int64_t max_blocks_per_seq, int32_t* prefix, uint4* __restrict__ qop,
+    uint32_t* __restrict__ lut) {
+  __shared__ float qv[4][4][64];     // [query head of the group][part][coordinate]
+  __shared__ int32_t scratch[257];
+  __shared__ float best_err[256];
+  __shared__ float best_alpha[256];
+  const int tid = threadIdx.x;
+  const int nq = S * KVH;
+  if ((int)blockIdx.x == nq) {
+    akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
+    return;
+  }
+  if ((int)blockIdx.x == nq + 1) {
+    // tables of the merged sixteen levels, rebuilt only when the codebooks in the table change
+    __shared__ int stale;
+    __shared__ float alphas[2];
+    if (tid == 0) stale = (lut[MF_W_MARK] != MF_MARK + (uint32_t)HM_BITS_TAG) ? 1 : 0;
+    __syncthreads();
+    if (tid < 12 && __float_as_uint(table[HYB_CEN0 + tid]) != lut[MF_W_TAG + tid]) stale = 1;
+    __syncthreads();
+    if (!stale) return;
+    // V table: fp16(alpha0 c) for the 3-bit codebook, fp16(alpha1 c) for the 2-bit codebook, each alpha in
+    // [1,2) minimising the largest relative rounding error of its levels; the signs are exactly -1 / +1
+    // (kappa and 1 / alpha are applied to the sums at the end)
+    float c[12];
+    for (int v = 0; v < 12; ++v) c[v] = table[HYB_CEN0 + v];
+    for (int set = 0; set < 2; ++set) {
+      const int v0 = set ? 8 : 0, v1 = set ? 12 : 8;
+      float berr = 1e30f, balpha = 1.f;
+      for (int k = 0; k < MF_ALPHA_CANDIDATES / 256; ++k) {
+        const float al = 1.f + (float)(tid * (MF_ALPHA_CANDIDATES / 256) + k) / (float)MF_ALPHA_CANDIDATES;
+        float worst = 0.f;
+        for (int v = v0; v < v1; ++v) {
+          const float x = al * c[v];
+          const float r = __half2float(__float2half_rn(x));
+          const float e = x != 0.f ? fabsf(r - x) / fabsf(x) : 0.f;
+          worst = fmaxf(worst, e);
+        }
+        if (worst < berr) { berr = worst; balpha = al; }
+      }
+      __syncthreads();
+      best_err[tid] = berr;
+      best_alpha[tid] = balpha;
+      __syncthreads();
+      if (tid == 0) {
+        for (int t = 1; t < 256; ++t)
+          if (best_err[t] < best_err[0]) { best_err[0] = best_err[t]; best_alpha[0] = best_alpha[t]; }
+        lut[MF_W_ALPHA + set] = __float_as_uint(best_alpha[0]);
+        alphas[set] = best_alpha[0];
+      }
+    }
+    __syncthreads();
+    auto vlevel = [&](int v) { return v < 8 ? alphas[0] * c[v] : v < 12 ? alphas[1] * c[v] : v == 12 ? -1.f : v == 13 ? 1.f : 0.f; };
+    const float c0 = hm_level(table, tid >> 4, 1.f), c1 = hm_level(table, tid & 15, 1.f);
+    const __half k0 = __float2half_rn(c0), k1 = __float2half_rn(c1);
+    lut[MF_W_KHI + tid] = (unsigned)__half_as_ushort(k0) | ((unsigned)__half_as_ushort(k1) << 16);
+    const __half l0 = __float2half_rn(c0 - __half2float(k0)), l1 = __float2half_rn(c1 - __half2float(k1));
+    lut[MF_W_KLO + tid] = (unsigned)__half_as_ushort(l0) | ((unsigned)__half_as_ushort(l1) << 16);
+    const __half v0 = __float2half_rn(vlevel(tid >> 4)), v1 = __float2half_rn(vlevel(tid & 15));
+    lut[MF_W_VHI + tid] = (unsigned)__half_as_ushort(v0) | ((unsigned)__half_as_ushort(v1) << 16);
+    if (tid < 12) lut[MF_W_TAG + tid] = __float_as_uint(table[HYB_CEN0 + tid]);
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) lut[MF_W_MARK] = MF_MARK + (uint32_t)HM_BITS_TAG;
+    return;
+  }
+  const int s = blockIdx.x / KVH, hv = blockIdx.x % KVH;
+  const int lane = tid & 63, w = tid >> 6;
+  {
+    const int64_t off = s * qs_seq + (int64_t)(hv * 4 + w) * qs_head;
+    const float q0 = akv_elem<QDT>::load(query, off + lane);
+    const float q1 = akv_elem<QDT>::load(query, off + 64 + lane);
+    qv[w][0][lane] = hyb_fwht64(q0 * table[HYB_HAD0 + lane], lane) * 0.125f * qscale;
+    qv[w][1][lane] = hyb_fwht64(q0 * table[HYB_QJL0 + lane], lane) * 0.125f * kappa * qscale;
+    qv[w][2][lane] = hyb_fwht64(q1 * table[HYB_HAD1 + lane], lane) * 0.125f * qscale;
+    qv[w][3][lane] = hyb_fwht64(q1 * table[HYB_QJL1 + lane], lane) * 0.125f * kappa * qscale;
+  }
+  __syncthreads();
+  // operand layout: [k-step n = 4 X + n4][lane (col, g)][e]: nibble dword 2g + n4/2 of part X, byte
+  // 2(n4 % 2) + e/4, nibble e % 2 (0 = high); elements 2,3 and 6,7 repeat 0,1 and 4,5 (they face the lo
+  // halves of the K table entries); columns [0,4) the fp16 rounding of the query copy, [8,12) its remainder
+  for (int n = w; n < 16; n += 4) {
+    const int X = n >> 2, n4 = n & 3;
+    const int col = lane & 15, g = lane >> 4;
+    unsigned short hbits[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int D = 2 * g + (n4 >> 1), b = 2 * (n4 & 1) + (e >> 2), lo = e & 1;
+      const int coord = hm_coord(X, D, b, lo);
+      float v = 0.f;
+      if (col < 4) {
+        v = __half2float(__float2half_rn(qv[col][X][coord]));
+      } else if (col >= 8 && col < 12) {
+        const float full = qv[col - 8][X][coord];
+        v = full - __half2float(__float2half_rn(full));
+      }
+      hbits[e] = __half_as_ushort(__float2half_rn(v));
+    }
+    uint4 o;
+    o.x = hbits[0] | (hbits[1] << 16); o.y = hbits[2] | (hbits[3] << 16);
+    o.z = hbits[4] | (hbits[5] << 16); o.w = hbits[6] | (hbits[7] << 16);
+    qop[((size_t)(s * KVH + hv) * 16 + n) * 64 + lane] = o;
+  }
+}
+
+struct hm_kraw {        // score wavefront, one 32-token chunk: the lane's pieces of token l%16 of both tiles
+  mf_u32x2 a0[2];       // 8 bytes holding 3-byte groups 2g, 2g+1 of A0
+  uint32_t b0[2];       // dword holding sign bytes 2g, 2g+1 of B0
+  uint32_t a1[2];       // halfwords 2g, 2g+1 of A1
+  uint32_t b1[2];
+  uint32_t n0, n1;      // lane < 32: the two factor dwords of token l's K row, else of token (l - 32)'s V row
+};
+struct hm_vraw {        // value wavefront: tokens 4g + i of both tiles
+  uint32_t c[8];        // pass C dword (A0 group col / A1 halfword col - 8)
+  uint32_t s[8];        // pass S dword (sign byte)
+};
+
+template <int ROLE>
+__device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const int hs) {
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15, g = lane >> 4;
+  const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * 4u;
+  const uint32_t lane4k = (uint32_t)(lane & 31) * 8u;
+  // exchange buffers as in the kernel above: weights (16 B per reader lane L) at entry 32 hs + L/8,
+  // rescale factors (4 B per lane) at entries 32 hs + 8, 9, flags at entry 32 hs + 12
+  auto pbx = [&](uint32_t L) { return MF_TABB + (32u * hs + (L >> 3)) * 256u + 128u + (L & 7u) * 16u; };
+  auto wsx = [&](uint32_t L) { return HM_WBUF2 + (uint32_t)hs * 1024u + L * 16u; };   // pass S weights: [parity][head slot][lane]
+  auto rsx = [&](uint32_t L) { return MF_TABB + (32u * hs + 8u + (L >> 5)) * 256u + 128u + (L & 31u) * 4u; };
+  const uint32_t fl_addr = MF_TABB + (32u * hs + 12u) * 256u + 128u;
+  uint32_t T = 0;
+
+  const int G = gridDim.x;
+  const int total = a.prefix[a.S];
+  const int per = (total + G - 1) / G;
+  const int g0 = blockIdx.x * per;
+  const int g1 = min(total, g0 + per);
+
+  int gcur = g0;
+  while (gcur < g1) {
+    const int s = akv_find_seq(a.prefix, a.S, gcur);
+    const int sb0 = a.prefix[s], sb1 = a.prefix[s + 1];
+    const int blk_lo = gcur - sb0;
+    const int blk_hi = min(g1, sb1) - sb0;
+    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, 16, a.max_blocks_per_seq);
+    const int t_end = (int)min((int64_t)blk_hi * 16, ctx);
+    gcur = sb0 + blk_hi;
+    const int nblk = blk_hi - blk_lo;
+    const int nchunks = (nblk + 1) >> 1;
+
+    for (int hbase = 0; hbase < a.KVH; hbase += HM_HEADS) {
+      const int h = hbase + hs;
+      if (h >= a.KVH || nchunks <= 0) continue;
+      const int hd = h / a.hgroup;      // the kv head whose rows are read
+
+      int pbwin = 0, win_c0 = 0;
+      auto load_window = [&](int c0) {
+        const int bi = min(blk_lo + 2 * c0 + lane, blk_hi - 1);
+        pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
+        asm volatile("" : "+v"(pbwin));
+        win_c0 = c0;
+      };
+      auto chunk_blocks = [&](int c_in, uint32_t& p0, uint32_t& p1) {
+        const int c = min(c_in, nchunks - 1);
+        const int w0 = 2 * (c - win_c0);
+        const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
+        p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
+        p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
+      };
+      load_window(0);
+
+      if constexpr (ROLE == 0) {
+        // =========================== score wavefront ===========================
+        half8 qb[16];
+        {
+          const uint4* qp = a.qop + ((size_t)(s * a.KVH + h) * 16) * 64 + lane;
+#pragma unroll
+          for (int st = 0; st < 16; ++st) {
+            const uint4 u = qp[st * 64];
+            qb[st] = mf_pack(u.x, u.y, u.z, u.w);
+          }
+        }
+        float m_run = -INFINITY, l_run = 0.f;
+        const uint32_t krow = (uint32_t)(hd * a.kps_head + col * a.kps_pos);
+        const uint32_t offA0 = krow + (g == 0 ? 0u : g == 1 ? 4u : g == 2 ? 12u : 16u);
+        const uint32_t offB0 = krow + 24u + 4u * (uint32_t)(g >> 1);
+        const uint32_t offA1 = krow + 36u + 4u * (uint32_t)g;
+        const uint32_t offB1 = krow + 52u + 4u * (uint32_t)(g >> 1);
+        const uint32_t selA = (g & 1) ? 0x0c020304u : 0x0c000102u;    // big-endian 24-bit words of the two groups
+        const uint32_t selB = (g & 1) ? 0x0c050607u : 0x0c030405u;
+        const uint32_t hsh = 16u * (uint32_t)(g & 1);
+        const int ntok = lane & 31;
+        const bool nrm_is_v = lane >= 32;
+        const uint8_t* nrm_base = nrm_is_v ? a.vc : a.kc;
+        const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vps_blk : a.kps_blk);
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vps_head + (ntok & 15) * a.vps_pos
+                                                     : hd * a.kps_head + (ntok & 15) * a.kps_pos);
+        // factor exchange: writer lane (kind = l/32, tile = (l/16)%2, token l%16) field f; reader lane (col, g)
+        // takes tokens 4g..4g+3 of a (kind, tile, field) with one 16-byte read
+        const uint32_t nw_addr = HM_NORMX + (uint32_t)hs * 1024u + (uint32_t)(lane >> 4) * 256u + (uint32_t)(lane & 15) * 4u;
+        const uint32_t nr_addr = HM_NORMX + (uint32_t)hs * 1024u + (uint32_t)g * 16u;
+        auto load_chunk = [&](hm_kraw& r, int c) {
+          uint32_t pb[2];
+          chunk_blocks(c, pb[0], pb[1]);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const unsigned char* kb = a.kc + mf_umul(pb[j], (uint32_t)a.kps_blk);
+            r.a0[j] = *(const mf_u32x2*)(kb + mf_here(offA0));
+            r.b0[j] = *(const uint32_t*)(kb + mf_here(offB0));
+            r.a1[j] = *(const uint32_t*)(kb + mf_here(offA1));
+            r.b1[j] = *(const uint32_t*)(kb + mf_here(offB1));
+          }
+          const unsigned char* nb = nrm_base + mf_umul(ntok >= 16 ? pb[1] : pb[0], nrm_blk) + mf_here(nrm_off);
+          r.n0 = *(const uint32_t*)(nb + 32);
+          r.n1 = *(const uint32_t*)(nb + 60);
+        };
+        auto half_lo = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); };
+        auto half_hi = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); };
+        auto produce = [&](hm_kraw& r, int c, const uint32_t par) {
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + 4096u * par) = __float_as_uint(half_lo(r.n0));
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + 4096u * par + 64u) = __float_as_uint(half_hi(r.n0));
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + 4096u * par + 128u) = __float_as_uint(half_lo(r.n1));
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + 4096u * par + 192u) = __float_as_uint(half_hi(r.n1));
+          // nibble dwords: step n = 8 j + 2 X + Dl
+          uint32_t kw[16];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            kw[8 * j + 0] = mf_spread3(__builtin_amdgcn_perm(r.a0[j].y, r.a0[j].x, selA));
+            kw[8 * j + 1] = mf_spread3(__builtin_amdgcn_perm(r.a0[j].y, r.a0[j].x, selB));
+            const uint32_t s0 = r.b0[j] >> hsh;
+            kw[8 * j + 2] = hm_spread1(s0 & 0xffu);
+            kw[8 * j + 3] = hm_spread1((s0 >> 8) & 0xffu);
+            kw[8 * j + 4] = mf_spread2(r.a1[j] & 0xffffu) | 0x88888888u;
+            kw[8 * j + 5] = mf_spread2(r.a1[j] >> 16) | 0x88888888u;
+            const uint32_t s1 = r.b1[j] >> hsh;
+            kw[8 * j + 6] = hm_spread1(s1 & 0xffu);
+            kw[8 * j + 7] = hm_spread1((s1 >> 8) & 0xffu);
+          }
+          mf_u32x2 w[3][4];
+          float4v acc[2][4];
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int X = 0; X < 4; ++X) acc[j][X] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) w[n][b] = mf_lut2(lane4k, kw[n], MF_SEL(b));
+#pragma unroll
+          for (int n = 0; n < 16; ++n) {
+            if (n + 2 < 16) {
+#pragma unroll
+              for (int b = 0; b < 4; ++b) w[(n + 2) % 3][b] = mf_lut2(lane4k, kw[n + 2], MF_SEL(b));
+            }
+            const int j = n >> 3, X = (n >> 1) & 3, st = 2 * (n & 7);
+            acc[j][X] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                mf_pack(w[n % 3][0].x, w[n % 3][0].y, w[n % 3][1].x, w[n % 3][1].y), qb[st], acc[j][X], 0, 0, 0);
+            acc[j][X] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                mf_pack(w[n % 3][2].x, w[n % 3][2].y, w[n % 3][3].x, w[n % 3][3].y), qb[st + 1], acc[j][X], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          load_chunk(r, c + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          float sv[8];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            union { mf_u32x4 u; float f[4]; } kn0, kr0, kn1, kr1;
+            const uint32_t base = nr_addr + 4096u * par + 256u * j;
+            kn0.u = *(mf_lds_u128*)(uintptr_t)(base);
+            kr0.u = *(mf_lds_u128*)(uintptr_t)(base + 64u);
+            kn1.u = *(mf_lds_u128*)(uintptr_t)(base + 128u);
+            kr1.u = *(mf_lds_u128*)(uintptr_t)(base + 192u);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float t0 = fmaf(kr0.f[i], acc[j][1][i], acc[j][0][i]);
+              const float t1 = fmaf(kr1.f[i], acc[j][3][i], acc[j][2][i]);
+              const float raw = fmaf(kn1.f[i], t1, kn0.f[i] * t0);
+              sv[4 * j + i] = raw + mf_from_hi_cols(raw);
+            }
+          }
+          // value-side factors of the lane's eight tokens
+          float vn0[8], vr0[8], vn1[8], vr1[8];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            union { mf_u32x4 u; float f[4]; } t0, t1, t2, t3;
+            const uint32_t base = nr_addr + 4096u * par + 512u + 256u * j;
+            t0.u = *(mf_lds_u128*)(uintptr_t)(base);
+            t1.u = *(mf_lds_u128*)(uintptr_t)(base + 64u);
+            t2.u = *(mf_lds_u128*)(uintptr_t)(base + 128u);
+            t3.u = *(mf_lds_u128*)(uintptr_t)(base + 192u);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { vn0[4 * j + i] = t0.f[i]; vr0[4 * j + i] = t1.f[i]; vn1[4 * j + i] = t2.f[i]; vr1[4 * j + i] = t3.f[i]; }
+          }
+          if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens (whose rows may hold anything)
+            const int tok0 = blk_lo * 16 + 32 * c;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const int tok = tok0 + 16 * j + 4 * g + i;
+                const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
+                if (!ok) { sv[4 * j + i] = -INFINITY; vn0[4 * j + i] = 0.f; vr0[4 * j + i] = 0.f; vn1[4 * j + i] = 0.f; vr1[4 * j + i] = 0.f; }
+              }
+          }
+          float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+          mx = mf_rows_max(mx);
+          const float m_new = fmaxf(m_run, mx);
+          const float resc = __builtin_amdgcn_exp2f(m_run - m_new);
+          m_run = m_new;
+          float psum = 0.f;
+          float pw[4][8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);
+            psum += p;
+            pw[0][i] = p * vn0[i];
+            pw[1][i] = pw[0][i] * vr0[i];
+            pw[2][i] = p * vn1[i];
+            pw[3][i] = pw[2][i] * vr1[i];
+          }
+          l_run = l_run * resc + psum;
+          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T);
+          if (col < 4) {
+            // weight operand of pass P (0 = C: sets A0, A1; 1 = S: sets B0, B1): column 4 t + col holds the
+            // fp16 part of set t of query head col, column 8 + 4 t + col its remainder; column k of the
+            // tile is read by lane 16 g + k
+#pragma unroll
+            for (int X = 0; X < 4; ++X) {
+              union { mf_u32x4 u; uint32_t w[4]; } hi, lo;
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[X][2 * q], pw[X][2 * q + 1]);
+                auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[X][2 * q] - (float)h2[0], pw[X][2 * q + 1] - (float)h2[1]);
+                union { decltype(h2) h; uint32_t u; } hb, lb;
+                hb.h = h2;
+                lb.h = l2;
+                hi.w[q] = hb.u;
+                lo.w[q] = lb.u;
+              }
+              const uint32_t L = (uint32_t)(16 * g + 4 * (X >> 1) + col);
+              const uint32_t base = ((X & 1) ? wsx(L) + 4096u * par : pbx(L) + MF_XBUF * par);
+              const uint32_t base8 = ((X & 1) ? wsx(L + 8u) + 4096u * par : pbx(L + 8u) + MF_XBUF * par);
+              *(mf_lds_u128*)(uintptr_t)base = hi.u;
+              *(mf_lds_u128*)(uintptr_t)base8 = lo.u;
+            }
+          }
+          *(mf_lds_u32*)(uintptr_t)(rsx((uint32_t)lane) + MF_XBUF * par) = __float_as_uint(resc);
+          mf_publish(fl_addr, T + (uint32_t)c + 1u);
+        };
+
+        hm_kraw ra, rb;
+        __builtin_amdgcn_sched_barrier(0);
+        load_chunk(ra, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_chunk(rb, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        int c = 0;
+        for (; c + 1 < nchunks; c += 2) {
+          if (c - win_c0 >= MF_WIN) load_window(c);
+          produce(ra, c, 0);
+          produce(rb, c + 1, 1);
+        }
+        if (c < nchunks) produce(ra, c, 0);
+        __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
+        T += (uint32_t)nchunks;
+        float lsum = l_run;
+        lsum = mf_rows_sum(lsum);
+        if (col < 4 && g == 0) {
+          const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * 4 + col);
+          a.part_ml[slot * 2] = m_run * 0.6931471805599453f;
+          a.part_ml[slot * 2 + 1] = lsum;
+        }
+      } else {
+        // =========================== value wavefront ===========================
+        float4v oC[8], oS[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { oC[j] = (float4v){0.f, 0.f, 0.f, 0.f}; oS[j] = (float4v){0.f, 0.f, 0.f, 0.f}; }
+        const int m = col;
+        const bool is3 = m < 8;
+        const uint32_t vrow = (uint32_t)(hd * a.vps_head + 4 * g * a.vps_pos);
+        const uint32_t offC = vrow + (is3 ? 4u * (uint32_t)((3 * m) >> 2) : 36u + 4u * (uint32_t)((m - 8) >> 1));
+        const uint32_t offS = vrow + (is3 ? 24u + 4u * (uint32_t)(m >> 2) : 52u + 4u * (uint32_t)((m - 8) >> 2));
+        const uint32_t o3 = (uint32_t)(3 * m) & 3u;
+        const uint32_t sel3 = 0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u);
+        const uint32_t sh2 = 16u * (uint32_t)(m & 1), shS = 8u * (uint32_t)(m & 3);
+        auto load_chunk = [&](hm_vraw& r, int c) {
+          uint32_t pb[2];
+          chunk_blocks(c, pb[0], pb[1]);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const unsigned char* vb = a.vc + mf_umul(pb[j], (uint32_t)a.vps_blk);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos);
+              r.c[4 * j + i] = *(const uint32_t*)(vr + mf_here(offC));
+              r.s[4 * j + i] = *(const uint32_t*)(vr + mf_here(offS));
+            }
+          }
+        };
+        auto step = [&](hm_vraw& r, int c, const uint32_t par) {
+          uint32_t xc[8], xs[8];
+#pragma unroll
+          for (int t = 0; t < 8; ++t) {
+            const uint32_t wa = r.c[t];
+            const uint32_t na = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wa, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
+            const uint32_t x3 = mf_spread3(__builtin_amdgcn_perm(na, wa, sel3));
+            const uint32_t x2 = mf_spread2((wa >> sh2) & 0xffffu) | 0x88888888u;
+            xc[t] = is3 ? x3 : x2;
+            xs[t] = hm_spread1((r.s[t] >> shS) & 0xffu);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          load_chunk(r, c + 1);
+          __builtin_amdgcn_sched_barrier(0);
+          uint32_t ce[4], co[4], se[4], so[4];
+#pragma unroll
+          for (int p = 0; p < 4; ++p) {
+            ce[p] = (xc[2 * p] & 0xF0F0F0F0u) | ((xc[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
+            co[p] = ((xc[2 * p] << 4) & 0xF0F0F0F0u) | (xc[2 * p + 1] & 0x0F0F0F0Fu);
+            se[p] = (xs[2 * p] & 0xF0F0F0F0u) | ((xs[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
+            so[p] = ((xs[2 * p] << 4) & 0xF0F0F0F0u) | (xs[2 * p + 1] & 0x0F0F0F0Fu);
+          }
+          uint32_t wv[8][4];
+#pragma unroll
+          for (int n = 0; n < 8; ++n)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? co[p] : ce[p], MF_SEL(n >> 1));
+          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
+          union { half8 h; mf_u32x4 u; } cv, cs;
+          cv.u = *(mf_lds_u128*)(uintptr_t)(pbx((uint32_t)lane) + MF_XBUF * par);
+          cs.u = *(mf_lds_u128*)(uintptr_t)(wsx((uint32_t)lane) + 4096u * par);
+          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rsx((uint32_t)(16 * g + (col & 3))) + MF_XBUF * par));
+          mf_publish(fl_addr + 4u, T + (uint32_t)c + 1u);
+          if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) { oC[j][i] *= resc; oS[j][i] *= resc; }
+          }
+#pragma unroll
+          for (int n = 0; n < 8; ++n)
+            oC[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cv.h, oC[n], 0, 0, 0);
+#pragma unroll
+          for (int n = 0; n < 8; ++n)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? so[p] : se[p], MF_SEL(n >> 1));
+#pragma unroll
+          for (int n = 0; n < 8; ++n)
+            oS[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cs.h, oS[n], 0, 0, 0);
+        };
+        hm_vraw ra;
+        load_chunk(ra, 0);
+        for (int c = 0; c < nchunks; ++c) {
+          if (c - win_c0 >= MF_WIN) load_window(c);
+          step(ra, c, (uint32_t)(c & 1));
+        }
+        __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
+        T += (uint32_t)nchunks;
+        // columns k and k + 8 carry the two fp16 terms of one weight; lane (column 4 t + q, g) then holds
+        // rows 4g + i of every tile for set t of query head q, and rows [0,8) belong to set 0 (A0 in pass
+        // C, B0 in pass S), rows [8,16) to set 1 (A1, B1)
+        const int t = col >> 2, q = col & 3;
+        const float inv_alpha = 1.f / __uint_as_float(a.lut[MF_W_ALPHA + (t & 1)]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            oC[j][i] = (oC[j][i] + mf_from_hi_cols(oC[j][i])) * inv_alpha;
+            oS[j][i] = (oS[j][i] + mf_from_hi_cols(oS[j][i])) * a.kappa;
+          }
+        if (col < 8 && (g >= 2) == (t == 1)) {
+          const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * 4 + q);
+          float* dst = a.part_acc + slot * 256 + 128 * t + 32 * (g & 1);      // parts A_t | B_t, rows 4 (g & 1) + i
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float v[8], u[8];
+            if (t == 0) {
+#pragma unroll
+              for (int n = 0; n < 8; ++n) v[hm_coord(0, 0, n >> 1, n & 1)] = oC[n][i];
+            } else {
+#pragma unroll
+              for (int n = 0; n < 8; ++n) v[hm_coord(2, 0, n >> 1, n & 1)] = oC[n][i];
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) u[hm_coord(1, 0, n >> 1, n & 1)] = oS[n][i];
+            *(float4*)(dst + 8 * i) = make_float4(v[0], v[1], v[2], v[3]);
+            *(float4*)(dst + 8 * i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+            *(float4*)(dst + 64 + 8 * i) = make_float4(u[0], u[1], u[2], u[3]);
+            *(float4*)(dst + 64 + 8 * i + 4) = make_float4(u[4], u[5], u[6], u[7]);
+          }
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(HM_THREADS) void akv_hyb_mfma_kernel(akv_hyb_mfma_args a) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  {
+    // thread (entry e, half hf) writes 16 of the entry's 32 copies
+    const int e = threadIdx.x >> 1, hf = threadIdx.x & 1;
+    const uint32_t khi = a.lut[MF_W_KHI + e], klo = a.lut[MF_W_KLO + e], vhi = a.lut[MF_W_VHI + e];
+    uint4* ka = (uint4*)(lds_raw + e * 256 + hf * 128);
+    uint4* va = (uint4*)(lds_raw + MF_TABB + e * 256 + hf * 64);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ka[i] = make_uint4(khi, klo, khi, klo);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) va[i] = make_uint4(vhi, vhi, vhi, vhi);
+  }
+  if (threadIdx.x < HM_HEADS) *(uint2*)(lds_raw + MF_TABB + (32u * threadIdx.x + 12u) * 256u + 128u) = make_uint2(0u, 0u);
+  __syncthreads();
+  if ((wave >> 2) == 0) hm_role_main<0>(a, wave & 3);
+  else hm_role_main<1>(a, wave & 3);
+}
+
+size_t akv_hyb_mfma_extra_bytes(int S, int QH) {
+  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * ((QH + 3) / 4) * 16 * 64 * 16);
+}
+
+// rows are dword-aligned (the caller checks); groups of four query heads; blocks of 16 tokens
+bool akv_hyb_mfma_applicable(int QH, int KVH, int block_size, const int64_t* strides6) {
+  if (mfma_disabled()) return false;
+  const int gqa = QH / KVH;
+  if (gqa % 4 != 0 || block_size != 16) return false;
+  for (int i = 0; i < 6; ++i)
+    if (strides6[i] < 0 || strides6[i] >= ((int64_t)1 << 27)) return false;
+  return true;
+}
+
+int akv_hyb_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* table, float kappa,
+                     float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, void* extra_ws, int grid,
+                     hipStream_t stream) {
+  a.hgroup = (a.QH / a.KVH) / 4;
+  a.KVH *= a.hgroup;
+  char* p = (char*)extra_ws;
+  a.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
+  a.qop = (const uint4*)p;
+  a.prefix = prefix;
+  const float qscale = scale * 1.4426950408889634f;
+  a.kappa = kappa;
+  const int pgrid = a.S * a.KVH + 2;
+#define HM_PRO(DT) akv_hyb_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, table, kappa, qscale, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, block_size, a.max_blocks_per_seq, prefix, (uint4*)a.qop, (uint32_t*)a.lut)
+  if (q_dtype == AKV_F16) HM_PRO(AKV_F16); else if (q_dtype == AKV_BF16) HM_PRO(AKV_BF16); else HM_PRO(AKV_F32);
+#undef HM_PRO
+  AKV_LAUNCH_CHECK("akv_hyb_mfma_prologue_kernel");
+  static bool configured = false;
+  if (!configured) {
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_hyb_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HM_LDS_BYTES));
+    configured = true;
+  }
+  akv_profile_mark_begin(stream);
+  akv_hyb_mfma_kernel<<<grid, HM_THREADS, HM_LDS_BYTES, stream>>>(a);
+  akv_profile_mark_end(stream);
+  AKV_LAUNCH_CHECK("akv_hyb_mfma_kernel");
+  return AKV_OK;
+}

@@ -14,27 +14,10 @@
 // the codes and sign bits directly with four transformed copies of the query, and the value
 // sum is accumulated in the four transformed domains and inverted once at the end.
 #include "akv_attn_common.h"
-
-#define HYB_HAD0 0
-#define HYB_HAD1 64
-#define HYB_QJL0 128
-#define HYB_QJL1 192
-#define HYB_CEN0 256
-#define HYB_CEN1 264
-#define HYB_BND0 268
-#define HYB_BND1 275
+#include "akv_hybrid_layout.h"
 
 static bool hyb_lane_disabled();
 static const float kHybKappa = (float)(1.2533141373155001 / 64.0);  // sqrt(pi/2) / 64
-
-__device__ __forceinline__ float hyb_fwht64(float v, int lane) {
-#pragma unroll
-  for (int h = 1; h < 64; h <<= 1) {
-    const float o = __shfl_xor(v, h, AKV_WAVE);
-    v = (lane & h) ? __fsub_rn(o, v) : __fadd_rn(v, o);
-  }
-  return v;
-}
 
 __device__ __forceinline__ float hyb_half_bits_to_float(uint32_t b) {
   return __half2float(__ushort_as_half((unsigned short)(b & 0xffffu)));
@@ -688,7 +671,8 @@ extern "C" int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_by
 
 extern "C" size_t akv_hybrid_paged_attn_workspace_bytes(int num_seqs, int num_q_heads) {
   if (num_seqs < 0 || num_q_heads <= 0) return 0;
-  return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, 256, akv_attn_grid()).bytes;
+  return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, 256, akv_attn_grid()).bytes +
+         akv_hyb_mfma_extra_bytes(num_seqs, num_q_heads);
 }
 
 template <int GQ>
@@ -729,8 +713,29 @@ extern "C" int akv_hybrid_paged_attn(
   const int G = akv_attn_grid();
   AKV_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 255) == 0, "akv_hybrid_paged_attn: workspace null or not 256-byte aligned");
   akv_attn_ws ws = akv_attn_ws_layout(workspace, num_seqs, num_q_heads, 256, G);
-  if (workspace_bytes < ws.bytes)
-    return akv_fail(AKV_ERR_WORKSPACE, "akv_hybrid_paged_attn: workspace %zu < %zu bytes", workspace_bytes, ws.bytes);
+  const size_t need = ws.bytes + akv_hyb_mfma_extra_bytes(num_seqs, num_q_heads);
+  if (workspace_bytes < need)
+    return akv_fail(AKV_ERR_WORKSPACE, "akv_hybrid_paged_attn: workspace %zu < %zu bytes", workspace_bytes, need);
+
+  // groups of four query heads over blocks of 16 tokens: the matrix-core kernel
+  const int64_t strides6[6] = {kps_blk, kps_pos, kps_head, vps_blk, vps_pos, vps_head};
+  const int rgrid = num_seqs * num_q_heads;
+  int Gused = G;
+  if (max_blocks_per_seq > 0 && akv_hyb_mfma_applicable(num_q_heads, num_kv_heads, block_size, strides6)) {
+    akv_hyb_mfma_args m;
+    m.kc = k_cache; m.kps_blk = kps_blk; m.kps_pos = kps_pos; m.kps_head = kps_head;
+    m.vc = v_cache; m.vps_blk = vps_blk; m.vps_pos = vps_pos; m.vps_head = vps_head;
+    m.block_tables = block_tables; m.bt_itype = bt_itype; m.bt_stride = bt_stride;
+    m.context_lens = context_lens; m.cl_itype = cl_itype;
+    m.S = num_seqs; m.QH = num_q_heads; m.KVH = num_kv_heads; m.hgroup = 1;
+    m.max_blocks_per_seq = max_blocks_per_seq;
+    m.prefix = ws.prefix; m.lut = nullptr; m.qop = nullptr;
+    m.part_acc = ws.part_acc; m.part_ml = ws.part_ml;
+    Gused = G / AKV_ATTN_WG_PER_CU;      // one workgroup per CU (its tables fill most of the LDS)
+    const int rc = akv_hyb_mfma_run(query, q_dtype, qs_seq, qs_head, hyb_table, kHybKappa, scale, m, block_size,
+                                    ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
+    if (rc) return rc;
+  } else {
 
   const int nblocks_q = (num_seqs * num_q_heads + 3) / 4;
 #define HYB_PRO(DT) hyb_attn_prologue_kernel<DT><<<nblocks_q + 1, 256, 0, stream>>>(query, qs_seq, qs_head, hyb_table, kHybKappa, num_seqs, num_q_heads, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot, nblocks_q)
@@ -749,11 +754,11 @@ extern "C" int akv_hybrid_paged_attn(
   const int gqa = num_q_heads / num_kv_heads;
   int rc = (gqa % 4 == 0) ? hyb_launch_attn<4>(a, G, stream) : hyb_launch_attn<1>(a, G, stream);
   if (rc) return rc;
-  const int rgrid = num_seqs * num_q_heads;
+  }
   switch (out_dtype) {
-    case AKV_F16: hyb_attn_reduce_kernel<AKV_F16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, G, out, os_seq, os_head); break;
-    case AKV_BF16: hyb_attn_reduce_kernel<AKV_BF16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, G, out, os_seq, os_head); break;
-    default: hyb_attn_reduce_kernel<AKV_F32><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, G, out, os_seq, os_head); break;
+    case AKV_F16: hyb_attn_reduce_kernel<AKV_F16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
+    case AKV_BF16: hyb_attn_reduce_kernel<AKV_BF16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
+    default: hyb_attn_reduce_kernel<AKV_F32><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
   }
   AKV_LAUNCH_CHECK("hyb_attn_reduce_kernel");
   return AKV_OK;
