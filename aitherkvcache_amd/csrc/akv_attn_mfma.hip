@@ -817,6 +817,13 @@ __host__ __device__ constexpr int hm_coord(int X, int D, int b, int lo) {
   return 8 * D + 6 - 2 * b + lo;                                                  // hm_spread1: nibble i <- bit i <- coordinate 7 - i
 }
 
+// value side, 2-bit lanes: code of M-tile n (byte n/2; odd n = low nibble) among the lane's eight; the
+// nibbles are [c3 c1 c7 c5 c2 c0 c6 c4] from bit 0 up
+__host__ __device__ constexpr int hm_vcoord2(int n) {
+  constexpr int nib[8] = {3, 1, 7, 5, 2, 0, 6, 4};
+  return nib[2 * (n >> 1) + ((n & 1) ? 0 : 1)];
+}
+
 // eight sign bits (coordinate k at bit 7 - k) -> nibbles 12 | bit, nibble i <- bit i
 __device__ __forceinline__ uint32_t hm_spread1(uint32_t b) {
   uint32_t t = (b | (b << 12)) & 0x000F000Fu;
@@ -1209,9 +1216,20 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
         const uint32_t vrow = (uint32_t)(hd * a.vps_head + 4 * g * a.vps_pos);
         const uint32_t offC = vrow + (is3 ? 4u * (uint32_t)((3 * m) >> 2) : 36u + 4u * (uint32_t)((m - 8) >> 1));
         const uint32_t offS = vrow + (is3 ? 24u + 4u * (uint32_t)(m >> 2) : 52u + 4u * (uint32_t)((m - 8) >> 2));
+        // pass C pieces as one word: lanes [0,8) the big-endian 24-bit word of 3-byte group m (from the
+        // aligned dword holding its first byte and, where it runs over, the neighbour lane's dword), lanes
+        // [8,16) halfword m - 8 of A1
         const uint32_t o3 = (uint32_t)(3 * m) & 3u;
-        const uint32_t sel3 = 0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u);
-        const uint32_t sh2 = 16u * (uint32_t)(m & 1), shS = 8u * (uint32_t)(m & 3);
+        const uint32_t selC = is3 ? (0x0c000000u | (o3 << 16) | ((o3 + 1u) << 8) | (o3 + 2u))
+                                  : ((m & 1) ? 0x0c0c0302u : 0x0c0c0100u);
+        // ... spread to one code per nibble by five (shift, mask) terms whose constants differ by lane class:
+        // mf_spread3 for the 3-bit lanes; for the 2-bit lanes (shift 0, mask 0x3333) and (shift 14, mask
+        // 0x33330000) do the whole job (nibbles [c3 c1 c7 c5 c2 c0 c6 c4] from bit 0 up) and the levels
+        // 8..11 of the merged table are selected by the constant 8 in every nibble
+        const uint32_t cm0 = is3 ? 0x7007u : 0x3333u, corc = is3 ? 0u : 0x88888888u;
+        const uint32_t cs1 = is3 ? 1u : 14u, cm1 = is3 ? 0x70070u : 0x33330000u;
+        const uint32_t cm2 = is3 ? 0x700700u : 0u, cm3 = is3 ? 0x07000000u : 0u, cm4 = is3 ? 0x70000000u : 0u;
+        const uint32_t shS = 8u * (uint32_t)(m & 3);
         auto load_chunk = [&](hm_vraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
@@ -1226,33 +1244,45 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             }
           }
         };
-        auto step = [&](hm_vraw& r, int c, const uint32_t par) {
+        struct hm_vx { uint32_t ce[4], co[4], se[4], so[4]; };   // token pairs: bytes of (high | low) nibbles
+        auto transcode = [&](const hm_vraw& r, hm_vx& x) {
           uint32_t xc[8], xs[8];
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             const uint32_t wa = r.c[t];
             const uint32_t na = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wa, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
-            const uint32_t x3 = mf_spread3(__builtin_amdgcn_perm(na, wa, sel3));
-            const uint32_t x2 = mf_spread2((wa >> sh2) & 0xffffu) | 0x88888888u;
-            xc[t] = is3 ? x3 : x2;
+            const uint32_t w = __builtin_amdgcn_perm(na, wa, selC);
+            uint32_t v = (w & cm0) | corc;
+            v = ((w << cs1) & cm1) | v;
+            v = ((w << 2) & cm2) | v;
+            v = ((w << 15) & cm3) | v;
+            v = ((w << 7) & cm4) | v;
+            xc[t] = v;
             xs[t] = hm_spread1((r.s[t] >> shS) & 0xffu);
           }
+#pragma unroll
+          for (int p = 0; p < 4; ++p) {
+            x.ce[p] = (xc[2 * p] & 0xF0F0F0F0u) | ((xc[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
+            x.co[p] = ((xc[2 * p] << 4) & 0xF0F0F0F0u) | (xc[2 * p + 1] & 0x0F0F0F0Fu);
+            x.se[p] = (xs[2 * p] & 0xF0F0F0F0u) | ((xs[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
+            x.so[p] = ((xs[2 * p] << 4) & 0xF0F0F0F0u) | (xs[2 * p + 1] & 0x0F0F0F0Fu);
+          }
+        };
+        hm_vraw r;
+        load_chunk(r, 0);
+        for (int c = 0; c < nchunks; ++c) {
+          const uint32_t par = (uint32_t)(c & 1);
+          if (c - win_c0 >= MF_WIN) load_window(c);
+          hm_vx x;
+          transcode(r, x);
           __builtin_amdgcn_sched_barrier(0);
           load_chunk(r, c + 1);
           __builtin_amdgcn_sched_barrier(0);
-          uint32_t ce[4], co[4], se[4], so[4];
-#pragma unroll
-          for (int p = 0; p < 4; ++p) {
-            ce[p] = (xc[2 * p] & 0xF0F0F0F0u) | ((xc[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
-            co[p] = ((xc[2 * p] << 4) & 0xF0F0F0F0u) | (xc[2 * p + 1] & 0x0F0F0F0Fu);
-            se[p] = (xs[2 * p] & 0xF0F0F0F0u) | ((xs[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
-            so[p] = ((xs[2 * p] << 4) & 0xF0F0F0F0u) | (xs[2 * p + 1] & 0x0F0F0F0Fu);
-          }
           uint32_t wv[8][4];
 #pragma unroll
           for (int n = 0; n < 8; ++n)
 #pragma unroll
-            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? co[p] : ce[p], MF_SEL(n >> 1));
+            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? x.co[p] : x.ce[p], MF_SEL(n >> 1));
           mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
           union { half8 h; mf_u32x4 u; } cv, cs;
           cv.u = *(mf_lds_u128*)(uintptr_t)(pbx((uint32_t)lane) + MF_XBUF * par);
@@ -1271,16 +1301,10 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
 #pragma unroll
           for (int n = 0; n < 8; ++n)
 #pragma unroll
-            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? so[p] : se[p], MF_SEL(n >> 1));
+            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? x.so[p] : x.se[p], MF_SEL(n >> 1));
 #pragma unroll
           for (int n = 0; n < 8; ++n)
             oS[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cs.h, oS[n], 0, 0, 0);
-        };
-        hm_vraw ra;
-        load_chunk(ra, 0);
-        for (int c = 0; c < nchunks; ++c) {
-          if (c - win_c0 >= MF_WIN) load_window(c);
-          step(ra, c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         T += (uint32_t)nchunks;
@@ -1307,7 +1331,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
               for (int n = 0; n < 8; ++n) v[hm_coord(0, 0, n >> 1, n & 1)] = oC[n][i];
             } else {
 #pragma unroll
-              for (int n = 0; n < 8; ++n) v[hm_coord(2, 0, n >> 1, n & 1)] = oC[n][i];
+              for (int n = 0; n < 8; ++n) v[hm_vcoord2(n)] = oC[n][i];
             }
 #pragma unroll
             for (int n = 0; n < 8; ++n) u[hm_coord(1, 0, n >> 1, n & 1)] = oS[n][i];
