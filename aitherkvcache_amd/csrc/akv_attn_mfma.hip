@@ -966,6 +966,9 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
   const uint32_t fl_addr = MF_TABB + (32u * hs + 12u) * 256u + 128u;
   uint32_t T = 0;
 
+  // blocks of 16 tokens: a chunk is two blocks; blocks of 32: one block, its second tile 16 positions further in
+  const bool bs32 = a.block_size == 32;
+  const int bs = bs32 ? 32 : 16;
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
   const int per = (total + G - 1) / G;
@@ -978,11 +981,11 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
     const int sb0 = a.prefix[s], sb1 = a.prefix[s + 1];
     const int blk_lo = gcur - sb0;
     const int blk_hi = min(g1, sb1) - sb0;
-    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, 16, a.max_blocks_per_seq);
-    const int t_end = (int)min((int64_t)blk_hi * 16, ctx);
+    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
+    const int t_end = (int)min((int64_t)blk_hi * bs, ctx);
     gcur = sb0 + blk_hi;
     const int nblk = blk_hi - blk_lo;
-    const int nchunks = (nblk + 1) >> 1;
+    const int nchunks = bs32 ? nblk : (nblk + 1) >> 1;
 
     for (int hbase = 0; hbase < a.KVH; hbase += HM_HEADS) {
       const int h = hbase + hs;
@@ -991,15 +994,15 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
 
       int pbwin = 0, win_c0 = 0;
       auto load_window = [&](int c0) {
-        const int bi = min(blk_lo + 2 * c0 + lane, blk_hi - 1);
+        const int bi = min(blk_lo + (bs32 ? c0 : 2 * c0) + lane, blk_hi - 1);
         pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
         asm volatile("" : "+v"(pbwin));
         win_c0 = c0;
       };
       auto chunk_blocks = [&](int c_in, uint32_t& p0, uint32_t& p1) {
         const int c = min(c_in, nchunks - 1);
-        const int w0 = 2 * (c - win_c0);
-        const int w1 = (2 * c + 1 < nblk) ? w0 + 1 : w0;
+        const int w0 = bs32 ? c - win_c0 : 2 * (c - win_c0);
+        const int w1 = (!bs32 && 2 * c + 1 < nblk) ? w0 + 1 : w0;
         p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
         p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
       };
@@ -1029,8 +1032,10 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
         const bool nrm_is_v = lane >= 32;
         const uint8_t* nrm_base = nrm_is_v ? a.vc : a.kc;
         const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vps_blk : a.kps_blk);
-        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vps_head + (ntok & 15) * a.vps_pos
-                                                     : hd * a.kps_head + (ntok & 15) * a.kps_pos);
+        const int npos = bs32 ? ntok : (ntok & 15);          // position of token ntok inside its block
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vps_head + npos * a.vps_pos
+                                                     : hd * a.kps_head + npos * a.kps_pos);
+        const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;
         // factor exchange: writer lane (kind = l/32, tile = (l/16)%2, token l%16) field f; reader lane (col, g)
         // takes tokens 4g..4g+3 of a (kind, tile, field) with one 16-byte read
         const uint32_t nw_addr = HM_NORMX + (uint32_t)hs * 1024u + (uint32_t)(lane >> 4) * 256u + (uint32_t)(lane & 15) * 4u;
@@ -1040,7 +1045,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const unsigned char* kb = a.kc + mf_umul(pb[j], (uint32_t)a.kps_blk);
+            const unsigned char* kb = a.kc + mf_umul(pb[j], (uint32_t)a.kps_blk) + (j ? ktile1 : 0u);
             r.a0[j] = *(const mf_u32x2*)(kb + mf_here(offA0));
             r.b0[j] = *(const uint32_t*)(kb + mf_here(offB0));
             r.a1[j] = *(const uint32_t*)(kb + mf_here(offA1));
@@ -1128,13 +1133,13 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             for (int i = 0; i < 4; ++i) { vn0[4 * j + i] = t0.f[i]; vr0[4 * j + i] = t1.f[i]; vn1[4 * j + i] = t2.f[i]; vr1[4 * j + i] = t3.f[i]; }
           }
           if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens (whose rows may hold anything)
-            const int tok0 = blk_lo * 16 + 32 * c;
+            const int tok0 = blk_lo * bs + 32 * c;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 const int tok = tok0 + 16 * j + 4 * g + i;
-                const bool ok = (tok < t_end) && (j == 0 || 2 * c + 1 < nblk);
+                const bool ok = (tok < t_end) && (j == 0 || bs32 || 2 * c + 1 < nblk);
                 if (!ok) { sv[4 * j + i] = -INFINITY; vn0[4 * j + i] = 0.f; vr0[4 * j + i] = 0.f; vn1[4 * j + i] = 0.f; vr1[4 * j + i] = 0.f; }
               }
           }
@@ -1230,12 +1235,13 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
         const uint32_t cs1 = is3 ? 1u : 14u, cm1 = is3 ? 0x70070u : 0x33330000u;
         const uint32_t cm2 = is3 ? 0x700700u : 0u, cm3 = is3 ? 0x07000000u : 0u, cm4 = is3 ? 0x70000000u : 0u;
         const uint32_t shS = 8u * (uint32_t)(m & 3);
+        const uint32_t vtile1 = bs32 ? 16u * (uint32_t)a.vps_pos : 0u;
         auto load_chunk = [&](hm_vraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const unsigned char* vb = a.vc + mf_umul(pb[j], (uint32_t)a.vps_blk);
+            const unsigned char* vb = a.vc + mf_umul(pb[j], (uint32_t)a.vps_blk) + (j ? vtile1 : 0u);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos);
@@ -1370,11 +1376,11 @@ size_t akv_hyb_mfma_extra_bytes(int S, int QH) {
   return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * ((QH + 3) / 4) * 16 * 64 * 16);
 }
 
-// rows are dword-aligned (the caller checks); groups of four query heads; blocks of 16 tokens
+// rows are dword-aligned (the caller checks); groups of four query heads; blocks of 16 or 32 tokens
 bool akv_hyb_mfma_applicable(int QH, int KVH, int block_size, const int64_t* strides6) {
   if (mfma_disabled()) return false;
   const int gqa = QH / KVH;
-  if (gqa % 4 != 0 || block_size != 16) return false;
+  if (gqa % 4 != 0 || (block_size != 16 && block_size != 32)) return false;
   for (int i = 0; i < 6; ++i)
     if (strides6[i] < 0 || strides6[i] >= ((int64_t)1 << 27)) return false;
   return true;
@@ -1383,6 +1389,7 @@ bool akv_hyb_mfma_applicable(int QH, int KVH, int block_size, const int64_t* str
 int akv_hyb_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* table, float kappa,
                      float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, void* extra_ws, int grid,
                      hipStream_t stream) {
+  a.block_size = block_size;
   a.hgroup = (a.QH / a.KVH) / 4;
   a.KVH *= a.hgroup;
   char* p = (char*)extra_ws;

@@ -717,7 +717,7 @@ extern "C" int akv_hybrid_paged_attn(
   if (workspace_bytes < need)
     return akv_fail(AKV_ERR_WORKSPACE, "akv_hybrid_paged_attn: workspace %zu < %zu bytes", workspace_bytes, need);
 
-  // groups of four query heads over blocks of 16 tokens: the matrix-core kernel
+  // groups of four query heads over blocks of 16 or 32 tokens: the matrix-core kernel
   const int64_t strides6[6] = {kps_blk, kps_pos, kps_head, vps_blk, vps_pos, vps_head};
   const int rgrid = num_seqs * num_q_heads;
   int Gused = G;
@@ -727,7 +727,7 @@ extern "C" int akv_hybrid_paged_attn(
     m.vc = v_cache; m.vps_blk = vps_blk; m.vps_pos = vps_pos; m.vps_head = vps_head;
     m.block_tables = block_tables; m.bt_itype = bt_itype; m.bt_stride = bt_stride;
     m.context_lens = context_lens; m.cl_itype = cl_itype;
-    m.S = num_seqs; m.QH = num_q_heads; m.KVH = num_kv_heads; m.hgroup = 1;
+    m.S = num_seqs; m.QH = num_q_heads; m.KVH = num_kv_heads; m.hgroup = 1; m.block_size = block_size;
     m.max_blocks_per_seq = max_blocks_per_seq;
     m.prefix = ws.prefix; m.lut = nullptr; m.qop = nullptr;
     m.part_acc = ws.part_acc; m.part_ml = ws.part_ml;

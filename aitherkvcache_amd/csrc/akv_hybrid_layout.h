@@ -36,7 +36,7 @@ struct akv_hyb_mfma_args {
   const uint8_t* vc; int64_t vps_blk, vps_pos, vps_head;
   const void* block_tables; int bt_itype; int64_t bt_stride;
   const void* context_lens; int cl_itype;
-  int S, QH, KVH, hgroup;      // KVH counts groups of four query heads; hgroup of them share a kv head's rows
+  int S, QH, KVH, hgroup, block_size;      // KVH counts groups of four query heads; hgroup of them share a kv head's rows
   int64_t max_blocks_per_seq;
   const int32_t* prefix;
   const uint32_t* lut;         // table block, MF_W_*

@@ -122,7 +122,8 @@ def test_paged_attention_vs_oracle(golden, dev, qh, kvh):
     assert np.max(np.abs(o32.cpu().numpy() - ref32)) <= 2e-4
 
 
-@pytest.mark.parametrize("qh,kvh,bs", [(32, 8, 16), (16, 2, 16), (12, 1, 16), (20, 1, 16), (8, 2, 32), (4, 4, 16)])
+@pytest.mark.parametrize("qh,kvh,bs", [(32, 8, 16), (16, 2, 16), (12, 1, 16), (20, 1, 16), (8, 2, 32), (32, 8, 32), (4, 4, 16),
+                                       (6, 2, 32), (8, 2, 8)])
 def test_paged_attention_ragged_batch_with_stale_rows(golden, dev, qh, kvh, bs):
     """Forty sequences of 0..900 tokens over a shuffled pool (so that workgroup cuts fall inside
     sequences, chunks end on odd block counts and contexts end inside blocks), groups of 4, 8, 12 and
