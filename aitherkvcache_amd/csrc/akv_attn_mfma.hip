@@ -789,9 +789,9 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
 //            of its parts' weights (p n0 and p n1, or p n0 r0 and p n1 r1): columns 4t + q hold the fp16
 //            part of set t for query head q of the group of four, columns 8 + 4t + q the remainder, and
 //            a lane keeps the results whose rows belong to its column's set.  The V table holds
-//            fp16(alpha c) with one alpha per codebook and the signs as exactly -1 / +1; 1 / alpha and
-//            kappa = sqrt(pi/2)/64 are applied to the finished sums (on the score side kappa rides in
-//            the query copies).
+//            fp16(alpha c) with one alpha per codebook; pass S builds its operand straight from the sign
+//            bits (fp16 -1 and +1 differ in one bit), no table; 1 / alpha and kappa = sqrt(pi/2)/64 are
+//            applied to the finished sums (on the score side kappa rides in the query copies).
 //
 // One workgroup = 8 wavefronts: 4 score + 4 value (two passes of 8 accumulator tiles need twice the
 // registers of the uniform formats), four groups of four query heads at a time.
@@ -1234,7 +1234,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
         const uint32_t cm0 = is3 ? 0x7007u : 0x3333u, corc = is3 ? 0u : 0x88888888u;
         const uint32_t cs1 = is3 ? 1u : 14u, cm1 = is3 ? 0x70070u : 0x33330000u;
         const uint32_t cm2 = is3 ? 0x700700u : 0u, cm3 = is3 ? 0x07000000u : 0u, cm4 = is3 ? 0x70000000u : 0u;
-        const uint32_t shS = 8u * (uint32_t)(m & 3);
+        const uint32_t selS = 0x0c000c00u | ((4u + (uint32_t)(m & 3)) << 16) | (uint32_t)(m & 3);
         const uint32_t vtile1 = bs32 ? 16u * (uint32_t)a.vps_pos : 0u;
         auto load_chunk = [&](hm_vraw& r, int c) {
           uint32_t pb[2];
@@ -1250,9 +1250,9 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             }
           }
         };
-        struct hm_vx { uint32_t ce[4], co[4], se[4], so[4]; };   // token pairs: bytes of (high | low) nibbles
+        struct hm_vx { uint32_t ce[4], co[4], sg[4]; };   // token pairs: bytes of (high | low) nibbles; sign bytes
         auto transcode = [&](const hm_vraw& r, hm_vx& x) {
-          uint32_t xc[8], xs[8];
+          uint32_t xc[8];
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             const uint32_t wa = r.c[t];
@@ -1264,14 +1264,13 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             v = ((w << 15) & cm3) | v;
             v = ((w << 7) & cm4) | v;
             xc[t] = v;
-            xs[t] = hm_spread1((r.s[t] >> shS) & 0xffu);
           }
 #pragma unroll
           for (int p = 0; p < 4; ++p) {
             x.ce[p] = (xc[2 * p] & 0xF0F0F0F0u) | ((xc[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
             x.co[p] = ((xc[2 * p] << 4) & 0xF0F0F0F0u) | (xc[2 * p + 1] & 0x0F0F0F0Fu);
-            x.se[p] = (xs[2 * p] & 0xF0F0F0F0u) | ((xs[2 * p + 1] >> 4) & 0x0F0F0F0Fu);
-            x.so[p] = ((xs[2 * p] << 4) & 0xF0F0F0F0u) | (xs[2 * p + 1] & 0x0F0F0F0Fu);
+            // the lane's sign byte of token 2p in bits [0,8), of token 2p + 1 in bits [16,24)
+            x.sg[p] = __builtin_amdgcn_perm(r.s[2 * p + 1], r.s[2 * p], selS);
           }
         };
         hm_vraw r;
@@ -1304,13 +1303,15 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
 #pragma unroll
           for (int n = 0; n < 8; ++n)
             oC[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cv.h, oC[n], 0, 0, 0);
+          // pass S needs no table: fp16 -1 and +1 differ in the sign bit only, so the operand of tile n
+          // (coordinate n of the byte = bit 7 - n) is that bit moved to bits 15 / 31 over the pattern of 1.0
+          // (a set bit reads as -1 here; the sign is turned back with kappa at the end)
 #pragma unroll
-          for (int n = 0; n < 8; ++n)
+          for (int n = 0; n < 8; ++n) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? x.so[p] : x.se[p], MF_SEL(n >> 1));
-#pragma unroll
-          for (int n = 0; n < 8; ++n)
+            for (int p = 0; p < 4; ++p) wv[n][p] = ((x.sg[p] << (8 + n)) & 0x80008000u) | 0x3C003C00u;
             oS[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cs.h, oS[n], 0, 0, 0);
+          }
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         T += (uint32_t)nchunks;
@@ -1324,7 +1325,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             oC[j][i] = (oC[j][i] + mf_from_hi_cols(oC[j][i])) * inv_alpha;
-            oS[j][i] = (oS[j][i] + mf_from_hi_cols(oS[j][i])) * a.kappa;
+            oS[j][i] = (oS[j][i] + mf_from_hi_cols(oS[j][i])) * -a.kappa;
           }
         if (col < 8 && (g >= 2) == (t == 1)) {
           const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * 4 + q);
@@ -1340,7 +1341,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
               for (int n = 0; n < 8; ++n) v[hm_vcoord2(n)] = oC[n][i];
             }
 #pragma unroll
-            for (int n = 0; n < 8; ++n) u[hm_coord(1, 0, n >> 1, n & 1)] = oS[n][i];
+            for (int n = 0; n < 8; ++n) u[n] = oS[n][i];
             *(float4*)(dst + 8 * i) = make_float4(v[0], v[1], v[2], v[3]);
             *(float4*)(dst + 8 * i + 4) = make_float4(v[4], v[5], v[6], v[7]);
             *(float4*)(dst + 64 + 8 * i) = make_float4(u[0], u[1], u[2], u[3]);
