@@ -50,6 +50,14 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
   const int s = blockIdx.x / groups, hg = blockIdx.x % groups;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int h = hg * 4 + wave;
+  // head_dim 128: the first half of this thread's column of Pi is requested before anything else, its
+  // round trip overlaps those of the partials
+  constexpr int PIPF = D == 128 ? 64 : 1;
+  float pvr[PIPF];
+  if constexpr (D == 128) {
+#pragma unroll
+    for (int k = 0; k < PIPF; ++k) pvr[k] = Pi[(size_t)k * D + (threadIdx.x & 127)];
+  }
   const int b0 = prefix[s], b1 = prefix[s + 1];
   if (b1 <= b0) {
     if (h < QH) {
@@ -62,28 +70,67 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     const int total = prefix[S];
     const int per = (total + G - 1) / G;
     const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
-    // pass 1 (lanes over slots, all loads in flight together): global max and sum
-    float M = -INFINITY;
-    for (int w = w_lo + lane; w <= w_hi; w += 64) M = fmaxf(M, part_ml[((size_t)(w + s) * QH + h) * 2]);
-    M = akv_wave_max(M);
-    float l = 0.f;
+    // the first RED_PF partial accumulators are requested before anything is known about their
+    // weights, so that their round trip overlaps the one of the (max, sum) pairs
+    constexpr int RED_PF = 16;
+    float pre[RED_PF][DPL];
+#pragma unroll
+    for (int u = 0; u < RED_PF; ++u) {
+      const size_t slot = (size_t)(min(w_lo + u, w_hi) + s) * QH + h;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) pre[u][i] = part_acc[slot * D + lane * DPL + i];
+    }
+    // lanes over slots: global max and sum; with at most 64 slots (the usual case) lane u keeps the
+    // weight of slot w_lo + u and the second pass takes it from there
+    const bool few = w_hi - w_lo < 64;
+    float M = -INFINITY, ms0 = -INFINITY, ls0 = 0.f;
     for (int w = w_lo + lane; w <= w_hi; w += 64) {
+      const size_t slot = (size_t)(w + s) * QH + h;
+      const float2 ml = *(const float2*)(part_ml + slot * 2);
+      if (w < w_lo + 64) { ms0 = ml.x; ls0 = ml.y; }
+      M = fmaxf(M, ml.x);
+    }
+    M = akv_wave_max(M);
+    const float wgt0 = ms0 > -INFINITY ? __expf(ms0 - M) : 0.f;
+    float l = wgt0 * ls0;
+    for (int w = w_lo + 64 + lane; w <= w_hi; w += 64) {
       const size_t slot = (size_t)(w + s) * QH + h;
       const float ms = part_ml[slot * 2];
       if (ms > -INFINITY) l += __expf(ms - M) * part_ml[slot * 2 + 1];
     }
     l = akv_wave_sum(l);
-    // pass 2: weighted sum of the partial accumulators (independent loads, unrolled)
     float acc[DPL];
 #pragma unroll
     for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
-#pragma unroll 8
-    for (int w = w_lo; w <= w_hi; ++w) {
-      const size_t slot = (size_t)(w + s) * QH + h;
-      const float ms = part_ml[slot * 2];
-      const float wgt = ms > -INFINITY ? __expf(ms - M) : 0.f;
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) acc[i] = fmaf(wgt, part_acc[slot * D + lane * DPL + i], acc[i]);
+    for (int u = 0; u < RED_PF; ++u) {
+      const float wu = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wgt0), u));
+      const float wgt = (w_lo + u <= w_hi) ? wu : 0.f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) acc[i] = fmaf(wgt, pre[u][i], acc[i]);
+    }
+    if (few) {
+      // batches of eight independent loads (a batch past the end repeats the last slot with weight 0)
+      for (int w0 = w_lo + RED_PF; w0 <= w_hi; w0 += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int w = min(w0 + u, w_hi);
+          const size_t slot = (size_t)(w + s) * QH + h;
+          const float wl = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wgt0), w - w_lo));
+          const float wgt = (w0 + u <= w_hi) ? wl : 0.f;
+#pragma unroll
+          for (int i = 0; i < DPL; ++i) acc[i] = fmaf(wgt, part_acc[slot * D + lane * DPL + i], acc[i]);
+        }
+      }
+    } else {
+#pragma unroll 8
+      for (int w = w_lo + RED_PF; w <= w_hi; ++w) {
+        const size_t slot = (size_t)(w + s) * QH + h;
+        const float ms = part_ml[slot * 2];
+        const float wgt = ms > -INFINITY ? __expf(ms - M) : 0.f;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) acc[i] = fmaf(wgt, part_acc[slot * D + lane * DPL + i], acc[i]);
+      }
     }
     const float inv = l > 0.f ? 1.f / l : 1.f;
 #pragma unroll
@@ -103,8 +150,15 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     for (int q = 0; q < 2; ++q)
 #pragma unroll
       for (int i = 0; i < JP; ++i) o[q][i] = 0.f;
+    if constexpr (D == 128) {
+#pragma unroll
+      for (int k = 0; k < PIPF; ++k) {
+        o[0][0] = fmaf(a_lds[2 * pr][k], pvr[k], o[0][0]);
+        o[1][0] = fmaf(a_lds[2 * pr + 1][k], pvr[k], o[1][0]);
+      }
+    }
 #pragma unroll 64
-    for (int k = 0; k < D; ++k) {
+    for (int k = (D == 128 ? PIPF : 0); k < D; ++k) {
       const float a0v = a_lds[2 * pr][k], a1v = a_lds[2 * pr + 1][k];
 #pragma unroll
       for (int i = 0; i < JP; ++i) {
