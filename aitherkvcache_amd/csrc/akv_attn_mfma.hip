@@ -1250,6 +1250,11 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             }
           }
         };
+        // both constants of (x & mask) | pattern live in registers: as literals they would split the
+        // operation in two
+        uint32_t sgn_mask = 0x80008000u, one_pair = 0x3C003C00u;
+        asm volatile("" : "+v"(sgn_mask));
+        asm volatile("" : "+s"(one_pair));
         struct hm_vx { uint32_t ce[4], co[4], sg[4]; };   // token pairs: bytes of (high | low) nibbles; sign bytes
         auto transcode = [&](const hm_vraw& r, hm_vx& x) {
           uint32_t xc[8];
@@ -1309,7 +1314,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
 #pragma unroll
           for (int n = 0; n < 8; ++n) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) wv[n][p] = ((x.sg[p] << (8 + n)) & 0x80008000u) | 0x3C003C00u;
+            for (int p = 0; p < 4; ++p) wv[n][p] = ((x.sg[p] << (8 + n)) & sgn_mask) | one_pair;
             oS[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mf_pack(wv[n][0], wv[n][1], wv[n][2], wv[n][3]), cs.h, oS[n], 0, 0, 0);
           }
         }
