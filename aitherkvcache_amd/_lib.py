@@ -49,8 +49,10 @@ SIGNATURES = {
                             _p, _i, _i64, _p, _i,
                             _p, _p, _i,
                             _p, _i, _i64, _i64,
-                            _i, _i, _i, _i, _i, _i64, _f,
+                            _i, _i, _i, _i, _i, _i64, _i64, _f,
                             _p, _sz, _p]),
+    "akv_paged_attn_status": (_i, [_p, C.POINTER(C.c_int), _p]),
+    "akv_debug_set_handoff_spin_limit": (_i, [_i]),
     "akv_hybrid_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
                                      _p, _i64, _i64, _i64, _i, _i64, _p]),
@@ -60,7 +62,7 @@ SIGNATURES = {
                                    _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,
                                    _p, _i, _i64, _p, _i, _p,
                                    _p, _i, _i64, _i64,
-                                   _i, _i, _i, _i, _i64, _f,
+                                   _i, _i, _i, _i, _i64, _i64, _f,
                                    _p, _sz, _p]),
     "akv_block_rep_update": (_i, [_p, _i, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "akv_block_rep_finalize": (_i, [_p, _i, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
@@ -148,6 +150,15 @@ def require_gpu(*tensors: torch.Tensor) -> torch.device:
 
 def stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def attn_status(workspace: Optional[torch.Tensor]) -> int:
+    """Status word of the most recent attention call on `workspace` (0 = clean)."""
+    if workspace is None:
+        return 0
+    flags = C.c_int(0)
+    check(lib().akv_paged_attn_status(workspace.data_ptr(), C.byref(flags), stream_ptr(workspace.device)))
+    return flags.value
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:

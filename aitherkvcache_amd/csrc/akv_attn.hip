@@ -15,11 +15,12 @@ template <int QDT>
 __global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
     int S, int QH, int D, const void* context_lens, int cl_itype, int block_size,
-    int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qrot) {
+    int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qrot, uint32_t* __restrict__ status) {
   __shared__ float q_lds[256];
   __shared__ int32_t scratch[257];
   const int b = blockIdx.x;
   if (b == S * QH) {
+    if (threadIdx.x == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
@@ -43,7 +44,7 @@ template <int D, int ODT>
 __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
     const float* __restrict__ part_ml, const float* __restrict__ Pi, int S, int QH, int G,
-    void* __restrict__ out, int64_t os_seq, int64_t os_head) {
+    void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status) {
   constexpr int DPL = D / 64;
   __shared__ float a_lds[4][D];
   const int groups = (QH + 3) / 4;
@@ -59,10 +60,12 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     for (int k = 0; k < PIPF; ++k) pvr[k] = Pi[(size_t)k * D + (threadIdx.x & 127)];
   }
   const int b0 = prefix[s], b1 = prefix[s + 1];
+  // a main kernel whose bounded wait gave up has produced garbage: say so in every output
+  const float poison = status[0] != 0u ? __uint_as_float(0x7fc00000u) : 0.f;
   if (b1 <= b0) {
     if (h < QH) {
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, s * os_seq + h * os_head + lane * DPL + i, 0.f);
+      for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, s * os_seq + h * os_head + lane * DPL + i, poison);
     }
     return;
   }
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
       if (hq < QH) {
 #pragma unroll
         for (int i = 0; i < JP; ++i)
-          akv_elem<ODT>::store(out, s * os_seq + hq * os_head + jt * JP + i, o[q][i]);
+          akv_elem<ODT>::store(out, s * os_seq + hq * os_head + jt * JP + i, o[q][i] + poison);
       }
     }
   }
@@ -251,7 +254,7 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
           const int t = c0 + lane;
           const bool valid = t < t1;
           const int tc = valid ? t : t1 - 1;
-          const int64_t phys = akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs);
+          const int64_t phys = akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs), a.num_blocks);
           const int pos = tc % bs;
           // ---- scores: lanes <-> tokens; 32 coordinates (= BITS dwords of codes) per step
           const uint32_t* kr = (const uint32_t*)(a.kp + phys * a.kps_blk + pos * a.kps_pos + h * a.kps_head);
@@ -339,13 +342,23 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
 size_t akv_attn_mfma_extra_bytes(int S, int KVH);
 bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits);
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                      const akv_attn_args& a, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream);
+                      const akv_attn_args& a, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream);
 
 extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
   if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
   // the number of kv heads is not known here; it is at most the number of query heads
   return akv_attn_ws_layout(nullptr, num_seqs, num_q_heads, d, akv_attn_grid()).bytes +
          akv_attn_mfma_extra_bytes(num_seqs, num_q_heads);
+}
+
+extern "C" int akv_paged_attn_status(const void* workspace, int* flags, void* stream_) {
+  AKV_REQUIRE(workspace != nullptr && flags != nullptr, "akv_paged_attn_status: null pointer");
+  hipStream_t stream = (hipStream_t)stream_;
+  uint32_t word = 0;
+  AKV_HIP(hipMemcpyAsync(&word, (const char*)workspace + AKV_WS_LUT_BYTES, sizeof(word), hipMemcpyDeviceToHost, stream));
+  AKV_HIP(hipStreamSynchronize(stream));
+  *flags = (int)word;
+  return AKV_OK;
 }
 
 template <int D, int BITS, int GQ>
@@ -371,18 +384,18 @@ static int akv_launch_attn_general(const akv_attn_args& a, int grid, hipStream_t
 
 template <int D>
 static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, int G, void* out,
-                             int64_t os_seq, int64_t os_head, hipStream_t stream) {
+                             int64_t os_seq, int64_t os_head, const uint32_t* status, hipStream_t stream) {
   const int grid = a.S * ((a.QH + 3) / 4);
   switch (odt) {
-    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
-    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
-    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head); break;
+    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
   }
   AKV_LAUNCH_CHECK("akv_attn_reduce_kernel");
   return AKV_OK;
 }
 
-extern "C" int akv_paged_attn(
+static int akv_paged_attn_impl(
     const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
     const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
     const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
@@ -393,10 +406,11 @@ extern "C" int akv_paged_attn(
     const void* rot_prep, const float* centroids, int bits,
     void* out, int out_dtype, int64_t os_seq, int64_t os_head,
     int num_seqs, int num_q_heads, int num_kv_heads, int d,
-    int block_size, int64_t max_blocks_per_seq, float scale,
+    int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
     void* workspace, size_t workspace_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   AKV_REQUIRE(num_seqs >= 0 && num_q_heads > 0 && num_kv_heads > 0, "akv_paged_attn: bad head/seq counts");
+  AKV_REQUIRE(num_blocks > 0 || max_blocks_per_seq == 0, "akv_paged_attn: num_blocks=%lld with a non-empty block table", (long long)num_blocks);
   AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_paged_attn: num_q_heads %% num_kv_heads != 0");
   AKV_REQUIRE(akv_valid_dtype(q_dtype) && akv_valid_dtype(out_dtype), "akv_paged_attn: bad dtype");
   AKV_REQUIRE(akv_valid_itype(bt_itype) && akv_valid_itype(cl_itype), "akv_paged_attn: bad index type");
@@ -432,7 +446,7 @@ extern "C" int akv_paged_attn(
   a.context_lens = context_lens; a.cl_itype = cl_itype;
   a.centroids = centroids;
   a.S = num_seqs; a.QH = num_q_heads; a.KVH = num_kv_heads; a.block_size = block_size;
-  a.max_blocks_per_seq = max_blocks_per_seq; a.scale = scale;
+  a.max_blocks_per_seq = max_blocks_per_seq; a.num_blocks = num_blocks; a.scale = scale;
   a.prefix = ws.prefix; a.qrot = ws.qrot; a.part_acc = ws.part_acc; a.part_ml = ws.part_ml;
   a.hgroup = 1;
 
@@ -440,10 +454,10 @@ extern "C" int akv_paged_attn(
   int Gused = G;
   if (akv_attn_mfma_applicable(a, d, bits)) {
     Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
-    rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
+    rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
   } else {
     const int pgrid = num_seqs * num_q_heads + 1;
-#define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot)
+#define AKV_PRO(DT) akv_attn_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, num_seqs, num_q_heads, d, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot, ws.status)
     if (q_dtype == AKV_F16) AKV_PRO(AKV_F16); else if (q_dtype == AKV_BF16) AKV_PRO(AKV_BF16); else AKV_PRO(AKV_F32);
 #undef AKV_PRO
     AKV_LAUNCH_CHECK("akv_attn_prologue_kernel");
@@ -455,7 +469,28 @@ extern "C" int akv_paged_attn(
 #undef AKV_CASE
   }
   if (rc) return rc;
-  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
-  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
-  return akv_launch_reduce<256>(out_dtype, a, Pi, Gused, out, os_seq, os_head, stream);
+  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
+  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
+  return akv_launch_reduce<256>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
+}
+
+extern "C" int akv_paged_attn(
+    const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+    const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+    const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
+    const uint8_t* v_packed, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+    const float* v_norms, int64_t vns_blk, int64_t vns_pos, int64_t vns_head,
+    const void* block_tables, int bt_itype, int64_t bt_stride,
+    const void* context_lens, int cl_itype,
+    const void* rot_prep, const float* centroids, int bits,
+    void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+    int num_seqs, int num_q_heads, int num_kv_heads, int d,
+    int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
+    void* workspace, size_t workspace_bytes, void* stream) {
+  return akv_paged_attn_impl(query, q_dtype, qs_seq, qs_head, k_packed, kps_blk, kps_pos, kps_head,
+                             k_norms, kns_blk, kns_pos, kns_head, v_packed, vps_blk, vps_pos, vps_head,
+                             v_norms, vns_blk, vns_pos, vns_head, block_tables, bt_itype, bt_stride,
+                             context_lens, cl_itype, rot_prep, centroids, bits, out, out_dtype, os_seq, os_head,
+                             num_seqs, num_q_heads, num_kv_heads, d, block_size, num_blocks, max_blocks_per_seq,
+                             scale, workspace, workspace_bytes, stream);
 }

@@ -26,6 +26,7 @@ struct akv_attn_args {
   const float* centroids;
   int S, QH, KVH, block_size;
   int64_t max_blocks_per_seq;
+  int64_t num_blocks;      // physical blocks in the cache; table entries are clamped into [0, num_blocks)
   float scale;
   const int32_t* prefix;
   const float* qrot;
@@ -44,8 +45,19 @@ static inline int akv_attn_grid() {
 static inline size_t akv_align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // Workspace carve-up.  acc_floats = floats of accumulator per query head
-// (head_dim for the uniform codec, 256 for tq35).
+// (head_dim for the uniform codec, 256 for tq35).  The workspace starts with a header whose place
+// does not depend on the batch: the cached lookup tables of the matrix-core kernels (their
+// validity tag would otherwise outlive a call at another batch size that overwrote the words it
+// vouches for) and the status words of the most recent call.
+#define AKV_WS_LUT_BYTES 4096
+#define AKV_WS_STATUS_BYTES 256
+#define AKV_WS_HEADER_BYTES (AKV_WS_LUT_BYTES + AKV_WS_STATUS_BYTES)
+// status word 0: nonzero when a bounded wait inside the main kernel of the most recent call gave up
+// (cleared by the prologue, set with a plain vector store, turned into NaN outputs by the reduce)
+#define AKV_STATUS_HANDOFF_TIMEOUT 1u
 struct akv_attn_ws {
+  uint32_t* lut;     // AKV_WS_LUT_BYTES of cached tables (matrix-core kernels)
+  uint32_t* status;  // AKV_WS_STATUS_BYTES
   int32_t* prefix;   // [S + 1] exclusive prefix of blocks per sequence; prefix[S] = total
   float* qrot;       // [S][QH][acc_floats] transformed queries
   float* part_acc;   // [G + S][QH][acc_floats]
@@ -55,7 +67,9 @@ struct akv_attn_ws {
 
 static inline akv_attn_ws akv_attn_ws_layout(void* base, int S, int QH, int acc_floats, int G) {
   akv_attn_ws w;
-  size_t off = 0;
+  w.lut = (uint32_t*)base;
+  w.status = (uint32_t*)((char*)base + AKV_WS_LUT_BYTES);
+  size_t off = AKV_WS_HEADER_BYTES;
   w.prefix = (int32_t*)((char*)base + off);
   off += akv_align256((size_t)(S + 1) * 4);
   w.qrot = (float*)((char*)base + off);
@@ -76,6 +90,12 @@ __device__ __forceinline__ int akv_seq_blocks(const void* context_lens, int cl_i
   int64_t nb = (ctx + block_size - 1) / block_size;
   if (nb > max_blocks_per_seq) nb = max_blocks_per_seq;
   return (int)nb;
+}
+
+// physical block id of a table entry, clamped into the cache (a corrupt entry then reads a wrong
+// block instead of memory outside the cache)
+__device__ __forceinline__ int64_t akv_clamp_block(int64_t id, int64_t num_blocks) {
+  return id < 0 ? 0 : (id >= num_blocks ? num_blocks - 1 : id);
 }
 
 __device__ __forceinline__ int64_t akv_seq_tokens(const void* context_lens, int cl_itype, int s,

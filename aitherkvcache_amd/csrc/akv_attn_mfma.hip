@@ -69,10 +69,13 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 #define MF_W_ALPHA 785
 #define MF_W_WORDS 1024
 #define MF_MARK 0x7452u
+static_assert(MF_W_WORDS * 4 <= AKV_WS_LUT_BYTES, "table block must fit the workspace header");
 
 struct akv_mfma_extra {
-  const uint32_t* lut;   // table block, MF_W_* (workspace)
+  const uint32_t* lut;   // table block, MF_W_* (workspace header)
   const uint4* qop;      // [S][KVH][8 k-steps][64 lanes] half8 as uint4 (workspace)
+  uint32_t* status;      // status words of the call (workspace header)
+  int spin_limit;        // polls a hand-off wait makes before it gives up
 };
 
 // ----------------------------------------------------------------------------------
@@ -83,7 +86,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
-    uint4* __restrict__ qop, uint32_t* __restrict__ lut, float qscale, int bits) {
+    uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits) {
   __shared__ __align__(16) float q_lds[128][8];   // [input coordinate][query head of the group], zero-padded
   __shared__ float qr_lds[8][128];
   __shared__ int32_t scratch[257];
@@ -92,6 +95,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
   const int tid = threadIdx.x;
   const int nq = S * KVH;
   if ((int)blockIdx.x == nq) {
+    if (tid == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
@@ -287,16 +291,19 @@ __device__ __forceinline__ float mf_rows_sum(float v) {
 // `ready` (chunks whose weights are written) and `done` (chunks whose weights have been read), both
 // counted from the start of the kernel.  LDS operations of a wavefront are executed in order, so a
 // counter written after the data is seen after the data.  Waiting polls the counter with a short
-// sleep; the wait is bounded (a logic error shows up as a wrong result in the tests, never as a
-// wavefront that does not finish).
+// sleep; the wait is bounded, so every wavefront finishes whatever happens.  A wait that gives up
+// leaves a mark in the status word of the call (an ordinary vector store): the kernel goes on with
+// whatever the buffer holds, the reduce kernel turns every output of the call into NaN, and the host
+// can read the word back (akv_paged_attn_status).
 #define MF_SPIN_LIMIT (1 << 16)
-__device__ __forceinline__ void mf_wait_ge(uint32_t addr, uint32_t need) {
-  for (int spin = 0; spin < MF_SPIN_LIMIT; ++spin) {
+__device__ __forceinline__ void mf_wait_ge(uint32_t addr, uint32_t need, uint32_t* status, int limit) {
+  for (int spin = 0; spin < limit; ++spin) {
     uint32_t v;
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
     if ((int32_t)((uint32_t)__builtin_amdgcn_readfirstlane((int)v) - need) >= 0) return;
     __builtin_amdgcn_s_sleep(2);
   }
+  if ((threadIdx.x & 63) == 0) *(volatile uint32_t*)status = AKV_STATUS_HANDOFF_TIMEOUT;
 }
 __device__ __forceinline__ void mf_publish(uint32_t addr, uint32_t value) {
   asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(value) : "memory");
@@ -378,7 +385,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       int pbwin = 0, win_c0 = 0;
       auto load_window = [&](int c0) {
         const int bi = min(blk_lo + (bs32 ? c0 : 2 * c0) + lane, blk_hi - 1);
-        pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
+        pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi), a.num_blocks);
         asm volatile("" : "+v"(pbwin));   // the window is complete here, not "maybe in flight" in the loop
         win_c0 = c0;
       };
@@ -528,7 +535,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           const float resc_left = mf_from_lo_cols(resc);
           const float resc_out = col < 8 ? resc : resc_left;
           // the buffer was last read for chunk c - 2 (or, for the first two chunks, in the previous segment)
-          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T);
+          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T, x.status, x.spin_limit);
           *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + MF_XBUF * par) = __float_as_uint(resc_out);
           mf_publish(fl_addr, T + (uint32_t)c + 1u);
@@ -642,7 +649,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 
         auto step = [&](mf_vraw& r, int c, const uint32_t par) {
           regroup(r, c);
-          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
+          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u, x.status, x.spin_limit);
           consume(c, par);
         };
         mf_vraw ra;
@@ -711,7 +718,15 @@ static bool mfma_disabled() {
 
 // extra workspace the MFMA path needs beyond akv_attn_ws (appended after it)
 size_t akv_attn_mfma_extra_bytes(int S, int KVH) {
-  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * KVH * 8 * 64 * 16);
+  return akv_align256((size_t)S * KVH * 8 * 64 * 16);
+}
+
+// polls a hand-off wait makes before it gives up (akv_debug_set_handoff_spin_limit)
+static int g_spin_limit = MF_SPIN_LIMIT;
+int akv_attn_spin_limit() { return g_spin_limit; }
+extern "C" int akv_debug_set_handoff_spin_limit(int polls) {
+  g_spin_limit = polls < 0 ? MF_SPIN_LIMIT : polls;
+  return AKV_OK;
 }
 
 // query heads per kv head -> number of groups of at most eight the kv head is presented as (0: none fits)
@@ -725,6 +740,7 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
   if (mfma_disabled()) return false;
   if (d != 128 || bits < 2 || bits > 4 || (a.block_size != 16 && a.block_size != 32)) return false;
   if (akv_attn_mfma_head_groups(a.QH / a.KVH) == 0) return false;
+  if (a.num_blocks >= ((int64_t)1 << 31)) return false;                       // block ids travel as 32-bit lanes
   // K rows are read 16 / 12 / 8 bytes per lane, V rows by dword / dword / halfword.  Multi-dword
   // loads need dword alignment only, so the serving layout (rows of packed + 4 bytes: pitch 68 / 52 /
   // 36) qualifies as well as dense rows.
@@ -735,21 +751,27 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits) {
                                a.vps_blk, a.vps_pos, a.vps_head, a.vns_blk, a.vns_pos, a.vns_head};
   for (int i = 0; i < 12; ++i)
     if (strides[i] < 0 || strides[i] >= ((int64_t)1 << 27)) return false;   // 32-bit in-block offsets
+  // the largest in-block offset a lane forms (head, then position of the second tile, then the row) fits 32 bits
+  const int64_t kmax = (int64_t)a.KVH * a.kps_head + 32 * a.kps_pos + 64, vmax = (int64_t)a.KVH * a.vps_head + 32 * a.vps_pos + 64;
+  const int64_t nmax = (int64_t)a.KVH * (a.kns_head > a.vns_head ? a.kns_head : a.vns_head) + 32 * (a.kns_pos > a.vns_pos ? a.kns_pos : a.vns_pos);
+  if (kmax >= ((int64_t)1 << 32) || vmax >= ((int64_t)1 << 32) || nmax >= ((int64_t)1 << 32)) return false;
   return true;
 }
 
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                      const akv_attn_args& a_in, int bits, int32_t* prefix, void* extra_ws, int grid, hipStream_t stream) {
+                      const akv_attn_args& a_in, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream) {
   akv_attn_args a = a_in;
   a.hgroup = akv_attn_mfma_head_groups(a.QH / a.KVH);
   a.KVH *= a.hgroup;                        // from here on: groups of at most eight query heads
+  int32_t* prefix = ws.prefix;
   akv_mfma_extra x;
-  char* p = (char*)extra_ws;
-  x.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
-  x.qop = (const uint4*)p;
+  x.lut = ws.lut;
+  x.qop = (const uint4*)extra_ws;
+  x.status = ws.status;
+  x.spin_limit = g_spin_limit;
   const float qscale = a.scale * 1.4426950408889634f;   // scores come out in the log2 domain
   const int pgrid = a.S * a.KVH + 2;
-#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, qscale, bits)
+#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, x.status, qscale, bits)
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
@@ -836,7 +858,7 @@ __global__ __launch_bounds__(256) void akv_hyb_mfma_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ table,
     float kappa, float qscale, int S, int QH, int KVH, const void* context_lens, int cl_itype,
     int block_size, int64_t max_blocks_per_seq, int32_t* prefix, uint4* __restrict__ qop,
-    uint32_t* __restrict__ lut) {
+    uint32_t* __restrict__ lut, uint32_t* __restrict__ status) {
   __shared__ float qv[4][4][64];     // [query head of the group][part][coordinate]
   __shared__ int32_t scratch[257];
   __shared__ float best_err[256];
@@ -844,6 +866,7 @@ __global__ __launch_bounds__(256) void akv_hyb_mfma_prologue_kernel(
   const int tid = threadIdx.x;
   const int nq = S * KVH;
   if ((int)blockIdx.x == nq) {
+    if (tid == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
@@ -995,7 +1018,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
       int pbwin = 0, win_c0 = 0;
       auto load_window = [&](int c0) {
         const int bi = min(blk_lo + (bs32 ? c0 : 2 * c0) + lane, blk_hi - 1);
-        pbwin = (int)akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi);
+        pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi), a.num_blocks);
         asm volatile("" : "+v"(pbwin));
         win_c0 = c0;
       };
@@ -1160,7 +1183,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
             pw[3][i] = pw[2][i] * vr1[i];
           }
           l_run = l_run * resc + psum;
-          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T);
+          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T, a.status, a.spin_limit);
           if (col < 4) {
             // weight operand of pass P (0 = C: sets A0, A1; 1 = S: sets B0, B1): column 4 t + col holds the
             // fp16 part of set t of query head col, column 8 + 4 t + col its remainder; column k of the
@@ -1293,7 +1316,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
           for (int n = 0; n < 8; ++n)
 #pragma unroll
             for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? x.co[p] : x.ce[p], MF_SEL(n >> 1));
-          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u);
+          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u, a.status, a.spin_limit);
           union { half8 h; mf_u32x4 u; } cv, cs;
           cv.u = *(mf_lds_u128*)(uintptr_t)(pbx((uint32_t)lane) + MF_XBUF * par);
           cs.u = *(mf_lds_u128*)(uintptr_t)(wsx((uint32_t)lane) + 4096u * par);
@@ -1379,7 +1402,7 @@ __global__ __launch_bounds__(HM_THREADS) void akv_hyb_mfma_kernel(akv_hyb_mfma_a
 }
 
 size_t akv_hyb_mfma_extra_bytes(int S, int QH) {
-  return akv_align256(MF_W_WORDS * 4) + akv_align256((size_t)S * ((QH + 3) / 4) * 16 * 64 * 16);
+  return akv_align256((size_t)S * ((QH + 3) / 4) * 16 * 64 * 16);
 }
 
 // rows are dword-aligned (the caller checks); groups of four query heads; blocks of 16 or 32 tokens
@@ -1393,19 +1416,19 @@ bool akv_hyb_mfma_applicable(int QH, int KVH, int block_size, const int64_t* str
 }
 
 int akv_hyb_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* table, float kappa,
-                     float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, void* extra_ws, int grid,
-                     hipStream_t stream) {
+                     float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, uint32_t* lut, void* extra_ws,
+                     int grid, hipStream_t stream) {
   a.block_size = block_size;
   a.hgroup = (a.QH / a.KVH) / 4;
   a.KVH *= a.hgroup;
-  char* p = (char*)extra_ws;
-  a.lut = (const uint32_t*)p; p += akv_align256(MF_W_WORDS * 4);
-  a.qop = (const uint4*)p;
+  a.lut = lut;
+  a.qop = (const uint4*)extra_ws;
   a.prefix = prefix;
+  a.spin_limit = g_spin_limit;
   const float qscale = scale * 1.4426950408889634f;
   a.kappa = kappa;
   const int pgrid = a.S * a.KVH + 2;
-#define HM_PRO(DT) akv_hyb_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, table, kappa, qscale, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, block_size, a.max_blocks_per_seq, prefix, (uint4*)a.qop, (uint32_t*)a.lut)
+#define HM_PRO(DT) akv_hyb_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, table, kappa, qscale, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, block_size, a.max_blocks_per_seq, prefix, (uint4*)a.qop, (uint32_t*)a.lut, a.status)
   if (q_dtype == AKV_F16) HM_PRO(AKV_F16); else if (q_dtype == AKV_BF16) HM_PRO(AKV_BF16); else HM_PRO(AKV_F32);
 #undef HM_PRO
   AKV_LAUNCH_CHECK("akv_hyb_mfma_prologue_kernel");

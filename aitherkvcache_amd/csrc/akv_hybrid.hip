@@ -356,6 +356,7 @@ struct hyb_attn_args {
   const float* table;
   int S, QH, KVH, block_size;
   int64_t max_blocks_per_seq;
+  int64_t num_blocks;  // physical blocks in the cache; table entries are clamped into [0, num_blocks)
   float scale, kappa;
   const int32_t* prefix;
   const float* qt;     // [S][QH][256]: Fwd_had(q0) | kappa Fwd_qjl(q0) | Fwd_had(q1) | kappa Fwd_qjl(q1)
@@ -368,9 +369,11 @@ template <int QDT>
 __global__ __launch_bounds__(256) void hyb_attn_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ table,
     float kappa, int S, int QH, const void* context_lens, int cl_itype, int block_size,
-    int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qt, int nblocks_q) {
+    int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qt, int nblocks_q,
+    uint32_t* __restrict__ status) {
   __shared__ int32_t scratch[257];
   if ((int)blockIdx.x == nblocks_q) {
+    if (threadIdx.x == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
@@ -450,7 +453,7 @@ __global__ __launch_bounds__(512) void hyb_attn_kernel(hyb_attn_args a) {
           const int t = c0 + lane;
           const bool valid = t < t1;
           const int tc = valid ? t : t1 - 1;
-          const int64_t phys = akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs);
+          const int64_t phys = akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs), a.num_blocks);
           const int pos = tc % bs;
           uint32_t row[16];
           {
@@ -543,14 +546,16 @@ template <int ODT>
 __global__ __launch_bounds__(64) void hyb_attn_reduce_kernel(
     const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
     const float* __restrict__ part_ml, const float* __restrict__ table, int S, int QH, int G,
-    void* __restrict__ out, int64_t os_seq, int64_t os_head) {
+    void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status) {
   const int s = blockIdx.x / QH, h = blockIdx.x % QH;
   const int lane = threadIdx.x;
   const int b0 = prefix[s], b1 = prefix[s + 1];
   const int64_t obase = s * os_seq + h * os_head;
+  // a main kernel whose bounded wait gave up has produced garbage: say so in every output
+  const float poison = status[0] != 0u ? __uint_as_float(0x7fc00000u) : 0.f;
   if (b1 <= b0) {
-    akv_elem<ODT>::store(out, obase + lane, 0.f);
-    akv_elem<ODT>::store(out, obase + 64 + lane, 0.f);
+    akv_elem<ODT>::store(out, obase + lane, poison);
+    akv_elem<ODT>::store(out, obase + 64 + lane, poison);
     return;
   }
   const int total = prefix[S];
@@ -569,8 +574,8 @@ __global__ __launch_bounds__(64) void hyb_attn_reduce_kernel(
                     hyb_fwht64(acc[1] * inv, lane) * table[HYB_QJL0 + lane]) * 0.125f;
   const float o1 = (hyb_fwht64(acc[2] * inv, lane) * table[HYB_HAD1 + lane] +
                     hyb_fwht64(acc[3] * inv, lane) * table[HYB_QJL1 + lane]) * 0.125f;
-  akv_elem<ODT>::store(out, obase + lane, o0);
-  akv_elem<ODT>::store(out, obase + 64 + lane, o1);
+  akv_elem<ODT>::store(out, obase + lane, o0 + poison);
+  akv_elem<ODT>::store(out, obase + 64 + lane, o1 + poison);
 }
 
 // ----------------------------------------------------------------------------------
@@ -696,10 +701,12 @@ extern "C" int akv_hybrid_paged_attn(
     const void* context_lens, int cl_itype, const float* hyb_table,
     void* out, int out_dtype, int64_t os_seq, int64_t os_head,
     int num_seqs, int num_q_heads, int num_kv_heads,
-    int block_size, int64_t max_blocks_per_seq, float scale,
+    int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
     void* workspace, size_t workspace_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   AKV_REQUIRE(num_seqs >= 0 && num_q_heads > 0 && num_kv_heads > 0, "akv_hybrid_paged_attn: bad head/seq counts");
+  AKV_REQUIRE((num_blocks > 0 && num_blocks < ((int64_t)1 << 31)) || max_blocks_per_seq == 0,
+              "akv_hybrid_paged_attn: num_blocks=%lld with a non-empty block table", (long long)num_blocks);
   AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_hybrid_paged_attn: num_q_heads %% num_kv_heads != 0");
   AKV_REQUIRE(akv_valid_dtype(q_dtype) && akv_valid_dtype(out_dtype), "akv_hybrid_paged_attn: bad dtype");
   AKV_REQUIRE(akv_valid_itype(bt_itype) && akv_valid_itype(cl_itype), "akv_hybrid_paged_attn: bad index type");
@@ -728,17 +735,17 @@ extern "C" int akv_hybrid_paged_attn(
     m.block_tables = block_tables; m.bt_itype = bt_itype; m.bt_stride = bt_stride;
     m.context_lens = context_lens; m.cl_itype = cl_itype;
     m.S = num_seqs; m.QH = num_q_heads; m.KVH = num_kv_heads; m.hgroup = 1; m.block_size = block_size;
-    m.max_blocks_per_seq = max_blocks_per_seq;
-    m.prefix = ws.prefix; m.lut = nullptr; m.qop = nullptr;
+    m.max_blocks_per_seq = max_blocks_per_seq; m.num_blocks = num_blocks;
+    m.prefix = ws.prefix; m.lut = nullptr; m.qop = nullptr; m.status = ws.status; m.spin_limit = 0;
     m.part_acc = ws.part_acc; m.part_ml = ws.part_ml;
     Gused = G / AKV_ATTN_WG_PER_CU;      // one workgroup per CU (its tables fill most of the LDS)
     const int rc = akv_hyb_mfma_run(query, q_dtype, qs_seq, qs_head, hyb_table, kHybKappa, scale, m, block_size,
-                                    ws.prefix, (char*)workspace + ws.bytes, Gused, stream);
+                                    ws.prefix, ws.lut, (char*)workspace + ws.bytes, Gused, stream);
     if (rc) return rc;
   } else {
 
   const int nblocks_q = (num_seqs * num_q_heads + 3) / 4;
-#define HYB_PRO(DT) hyb_attn_prologue_kernel<DT><<<nblocks_q + 1, 256, 0, stream>>>(query, qs_seq, qs_head, hyb_table, kHybKappa, num_seqs, num_q_heads, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot, nblocks_q)
+#define HYB_PRO(DT) hyb_attn_prologue_kernel<DT><<<nblocks_q + 1, 256, 0, stream>>>(query, qs_seq, qs_head, hyb_table, kHybKappa, num_seqs, num_q_heads, context_lens, cl_itype, block_size, max_blocks_per_seq, ws.prefix, ws.qrot, nblocks_q, ws.status)
   if (q_dtype == AKV_F16) HYB_PRO(AKV_F16); else if (q_dtype == AKV_BF16) HYB_PRO(AKV_BF16); else HYB_PRO(AKV_F32);
 #undef HYB_PRO
   AKV_LAUNCH_CHECK("hyb_attn_prologue_kernel");
@@ -749,16 +756,16 @@ extern "C" int akv_hybrid_paged_attn(
   a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
   a.context_lens = context_lens; a.cl_itype = cl_itype; a.table = hyb_table;
   a.S = num_seqs; a.QH = num_q_heads; a.KVH = num_kv_heads; a.block_size = block_size;
-  a.max_blocks_per_seq = max_blocks_per_seq; a.scale = scale; a.kappa = kHybKappa;
+  a.max_blocks_per_seq = max_blocks_per_seq; a.num_blocks = num_blocks; a.scale = scale; a.kappa = kHybKappa;
   a.prefix = ws.prefix; a.qt = ws.qrot; a.part_acc = ws.part_acc; a.part_ml = ws.part_ml;
   const int gqa = num_q_heads / num_kv_heads;
   int rc = (gqa % 4 == 0) ? hyb_launch_attn<4>(a, G, stream) : hyb_launch_attn<1>(a, G, stream);
   if (rc) return rc;
   }
   switch (out_dtype) {
-    case AKV_F16: hyb_attn_reduce_kernel<AKV_F16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
-    case AKV_BF16: hyb_attn_reduce_kernel<AKV_BF16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
-    default: hyb_attn_reduce_kernel<AKV_F32><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head); break;
+    case AKV_F16: hyb_attn_reduce_kernel<AKV_F16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head, ws.status); break;
+    case AKV_BF16: hyb_attn_reduce_kernel<AKV_BF16><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head, ws.status); break;
+    default: hyb_attn_reduce_kernel<AKV_F32><<<rgrid, 64, 0, stream>>>(ws.prefix, ws.part_acc, ws.part_ml, hyb_table, num_seqs, num_q_heads, Gused, out, os_seq, os_head, ws.status); break;
   }
   AKV_LAUNCH_CHECK("hyb_attn_reduce_kernel");
   return AKV_OK;

@@ -38,7 +38,10 @@ struct akv_hyb_mfma_args {
   const void* context_lens; int cl_itype;
   int S, QH, KVH, hgroup, block_size;      // KVH counts groups of four query heads; hgroup of them share a kv head's rows
   int64_t max_blocks_per_seq;
+  int64_t num_blocks;          // physical blocks in the cache; table entries are clamped into [0, num_blocks)
   const int32_t* prefix;
+  uint32_t* status;            // status words of the call (workspace header)
+  int spin_limit;              // polls a hand-off wait makes before it gives up
   const uint32_t* lut;         // table block, MF_W_*
   const uint4* qop;            // [S][KVH][16 k-steps][64 lanes] half8
   float* part_acc;             // [G + S][QH][256]: A0 | B0 | A1 | B1, natural coordinate order
@@ -49,5 +52,5 @@ struct akv_hyb_mfma_args {
 size_t akv_hyb_mfma_extra_bytes(int S, int QH);
 bool akv_hyb_mfma_applicable(int QH, int KVH, int block_size, const int64_t* strides6);
 int akv_hyb_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* table, float kappa,
-                     float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, void* extra_ws, int grid,
-                     hipStream_t stream);
+                     float scale, akv_hyb_mfma_args a, int block_size, int32_t* prefix, uint32_t* lut, void* extra_ws,
+                     int grid, hipStream_t stream);

@@ -60,6 +60,9 @@ class TQPagedAttention:
         block_tables [num_seqs, max_blocks_per_seq] int32/int64, context_lens [num_seqs]."""
         if num_kv_heads is None:
             num_kv_heads = k_packed.shape[2]
+        tq = self._tq
+        if tq.rotation is not self.rotation:     # the quantizer's matrix was reassigned: follow it
+            self.rotation = tq.rotation
         if self._block_selector is not None:
             # as in the reference (:659-668): even / odd coordinates of the rotated query score the blocks,
             # the kernel then walks the filtered table
@@ -87,10 +90,8 @@ class TQPagedAttention:
         v_norms = v_norms if v_norms.dtype == torch.float32 else v_norms.float()
         bt = block_tables if block_tables.stride(-1) == 1 else block_tables.contiguous()
         cl = context_lens if context_lens.is_contiguous() else context_lens.contiguous()
+        num_blocks = min(k_packed.shape[0], k_norms.shape[0], v_packed.shape[0], v_norms.shape[0])
         ws = self._get_workspace(num_seqs, dev)
-        tq = self._tq
-        if tq.rotation is not self.rotation:
-            self.rotation = tq.rotation
         _lib.check(_lib.lib().akv_paged_attn(
             q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
             k_packed.data_ptr(), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2),
@@ -100,6 +101,11 @@ class TQPagedAttention:
             bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
             tq.prepared_rotation().ptr, self.centroids.data_ptr(), self.bits,
             out.data_ptr(), _lib.dtype_code(out), out.stride(0), out.stride(1),
-            num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, bt.shape[1], self.scale,
+            num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, bt.shape[1], self.scale,
             ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev)))
         return out if out.dtype == query.dtype else out.to(query.dtype)
+
+    def last_call_status(self) -> int:
+        """0 when the most recent forward() ran clean; bit 0 set when a bounded hand-off wait inside
+        its main kernel gave up (the outputs of that call are NaN).  Synchronises the stream."""
+        return _lib.attn_status(self._workspace)

@@ -89,6 +89,12 @@ class HybridPagedAttention:
             bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
             table.data_ptr(),
             out.data_ptr(), _lib.dtype_code(out), out.stride(0), out.stride(1),
-            num_seqs, num_q_heads, num_kv_heads, block_size, bt.shape[1], float(scale),
+            num_seqs, num_q_heads, num_kv_heads, block_size, min(k_cache.shape[0], v_cache.shape[0]),
+            bt.shape[1], float(scale),
             ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev)))
         return out if out.dtype == query.dtype else out.to(query.dtype)
+
+    def last_call_status(self) -> int:
+        """0 when the most recent forward() ran clean; bit 0 set when a bounded hand-off wait inside
+        its main kernel gave up (the outputs of that call are NaN).  Synchronises the stream."""
+        return _lib.attn_status(self._workspace)

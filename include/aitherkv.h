@@ -149,8 +149,13 @@ int akv_decode_blocks(const uint8_t* packed, int64_t ps_blk, int64_t ps_pos, int
  *   context_lens [num_seqs]; 0 gives a zero output row
  *   out          [num_seqs][num_q_heads][d] in out_dtype, strides os_seq / os_head
  * kv head of query head h is h / (num_q_heads / num_kv_heads).
+ * `num_blocks` is the number of physical blocks behind k/v_packed and k/v_norms: table
+ * entries inside a context are clamped into [0, num_blocks), so a corrupt entry reads a wrong
+ * block of the cache, never memory outside it.
  * `workspace` (device, >= akv_paged_attn_workspace_bytes(...), 256-byte aligned) holds the
- * rotated queries and the split partials; the caller allocates it once.
+ * rotated queries and the split partials; the caller allocates it once.  One workspace may
+ * serve calls of any batch size up to the one it was sized for; calls that share a workspace
+ * must not overlap in time.
  * ------------------------------------------------------------------------------- */
 size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d);
 int akv_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
@@ -163,8 +168,19 @@ int akv_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_he
                    const void* rot_prep, const float* centroids, int bits,
                    void* out, int out_dtype, int64_t os_seq, int64_t os_head,
                    int num_seqs, int num_q_heads, int num_kv_heads, int d,
-                   int block_size, int64_t max_blocks_per_seq, float scale,
+                   int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Status of the most recent akv_paged_attn / akv_hybrid_paged_attn call that used `workspace`
+ * (no counterpart in the reference).  Inside the main kernel pairs of wavefronts hand chunks to
+ * each other through counters with BOUNDED waits, so that a kernel always finishes; a wait
+ * that gives up marks the call, whose outputs are then all NaN.  This waits for `stream` and
+ * copies the mark to *flags (host pointer): 0 = clean, bit 0 = a hand-off wait gave up.
+ * akv_debug_set_handoff_spin_limit changes the number of polls such a wait makes (negative =
+ * the default, 65536); it exists so that a test can exercise the failure path from the host
+ * (0 polls: every wait gives up at once, every kernel still runs to its end). */
+int akv_paged_attn_status(const void* workspace, int* flags, void* stream);
+int akv_debug_set_handoff_spin_limit(int polls);
 
 /* ---------------------------------------------------------------------------------
  * HybridTurboQuant, mode tq35 with calibrate_uniform() groups (dims 0..63 at 3-bit MSE,
@@ -193,7 +209,8 @@ int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_bytes, int64_
 /* Decode attention over a tq35 paged cache.  The reference has no fused kernel for this: its
  * tq::hybrid_decode_step (aither_kvcache/vllm/hooks.py:240-345) decompresses every addressed
  * block and runs dense attention; this computes the same softmax(q K^T * scale) V directly on
- * the packed rows (float32 accumulation).  `scale` is explicit, as at hooks.py:341. */
+ * the packed rows (float32 accumulation).  `scale` is explicit, as at hooks.py:341.
+ * num_blocks, workspace sharing and akv_paged_attn_status as for akv_paged_attn. */
 size_t akv_hybrid_paged_attn_workspace_bytes(int num_seqs, int num_q_heads);
 int akv_hybrid_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
                           const uint8_t* k_cache, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
@@ -202,7 +219,7 @@ int akv_hybrid_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_
                           const void* context_lens, int cl_itype, const float* hyb_table,
                           void* out, int out_dtype, int64_t os_seq, int64_t os_head,
                           int num_seqs, int num_q_heads, int num_kv_heads,
-                          int block_size, int64_t max_blocks_per_seq, float scale,
+                          int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------

@@ -445,3 +445,70 @@ def test_decode_step_replays_from_a_graph(golden, dev):
             assert torch.equal(sout, want[i][0]), (rep, seed)
             assert torch.equal(kv, want[i][1]) and torch.equal(kn, want[i][2])
             _ = (torch.randn(1 << 16, device=dev) * 2).sum().item()       # unrelated eager work between replays
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+def test_one_object_across_batch_sizes(golden, dev, bits):
+    """One TQPagedAttention (one workspace) serves calls at batch sizes 6, 2, 6, 4, 8, 4, as a server
+    that records one graph per batch size does: the cached lookup tables sit at a place in the
+    workspace that no batch size moves, so a call at another batch size cannot overwrite them
+    behind their validity tag.  Every call is checked against the oracle."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(900 + bits)
+    NB, KVH, QH = 64, 8, 32
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, bits)
+    attn = akv.TQPagedAttention(tq, num_query_heads=QH)
+    for S in (6, 2, 6, 4, 8, 4):
+        ctx = rng.integers(1, 200, size=S).astype(np.int64)
+        width = 16
+        tables = np.stack([rng.permutation(NB)[:width] for _ in range(S)]).astype(np.int64)
+        q = rng.standard_normal((S, QH, 128)).astype(np.float16)
+        out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), block_size=16, num_kv_heads=KVH)
+        ref = oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, bits)
+        assert within_tol(out.cpu().numpy(), ref), f"batch size {S}"
+        assert attn.last_call_status() == 0
+
+
+def test_corrupt_table_entry_stays_inside_the_cache(golden, dev):
+    """Table entries inside a context are clamped into [0, num_blocks): a negative or huge entry
+    reads a wrong block of the cache, never memory outside it.  The result equals the oracle's on
+    the clamped table."""
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(77)
+    NB, KVH, QH = 32, 8, 32
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, 4)
+    ctx = np.array([100, 64], dtype=np.int64)
+    tables = np.stack([rng.permutation(NB)[:8] for _ in range(2)]).astype(np.int64)
+    tables[0, 2] = -5
+    tables[1, 1] = 10 ** 9
+    q = rng.standard_normal((2, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, num_query_heads=QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), block_size=16, num_kv_heads=KVH)
+    ref = oracle_out(q, kp, kn, vp, vn, np.clip(tables, 0, NB - 1), ctx, golden, 4)
+    assert within_tol(out.cpu().numpy(), ref)
+
+
+def test_handoff_timeout_is_reported(golden, dev):
+    """The failure path of the bounded hand-off waits, driven from the host: with a limit of zero
+    polls every wait gives up at once (all kernels still run to their end), the call's outputs are
+    NaN and the status query says so; with the default limit restored the next call is clean."""
+    from aitherkvcache_amd import _lib
+    tq = make_tq(golden, dev, 4)
+    rng = np.random.default_rng(78)
+    NB, KVH, QH = 32, 8, 32
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, 4)
+    ctx = np.array([300, 64], dtype=np.int64)
+    tables = np.stack([rng.permutation(NB)[:20] for _ in range(2)]).astype(np.int64)
+    q = rng.standard_normal((2, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, num_query_heads=QH)
+    args = (t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev))
+    try:
+        _lib.check(_lib.lib().akv_debug_set_handoff_spin_limit(0))
+        bad = attn.forward(*args, block_size=16, num_kv_heads=KVH)
+        assert attn.last_call_status() & 1
+        assert bool(torch.isnan(bad).all())
+    finally:
+        _lib.check(_lib.lib().akv_debug_set_handoff_spin_limit(-1))
+    good = attn.forward(*args, block_size=16, num_kv_heads=KVH)
+    assert attn.last_call_status() == 0
+    assert within_tol(good.cpu().numpy(), oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, 4))

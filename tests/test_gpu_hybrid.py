@@ -324,3 +324,25 @@ def test_both_codec_forms_agree(golden, dev):
     d_a = h.decode(aligned.reshape(-1, 64))
     d_p = h.decode(pitched.reshape(-1, 68)[:, :64])
     assert torch.equal(d_a, d_p)
+
+
+def test_one_object_across_batch_sizes(golden, dev):
+    """One HybridPagedAttention (one workspace) at batch sizes 6, 2, 6, 4, 8, 4: the cached tables keep
+    their place in the workspace whatever the batch size.  Every call against the oracle."""
+    kvh, qh, NB = 8, 32, 64
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform(num_kv_heads=kvh)
+    hp = params(golden)
+    rng = np.random.default_rng(4242)
+    kc, vc, _, _ = build_cache(rng, h, dev, NB, kvh)
+    attn = akv.HybridPagedAttention(h, qh)
+    scale = 1 / math.sqrt(128)
+    for S in (6, 2, 6, 4, 8, 4):
+        ctx = rng.integers(1, 200, size=S).astype(np.int64)
+        tables = np.stack([rng.permutation(NB)[:16] for _ in range(S)]).astype(np.int64)
+        q = rng.standard_normal((S, qh, 128)).astype(np.float32)
+        out = attn.forward(t(q, dev), kc, vc, t(tables, dev), t(ctx, dev), scale=scale)
+        ref = O.hybrid_paged_attention(q, kc.cpu().numpy(), vc.cpu().numpy(), tables, ctx, hp, scale, dtype=np.float64)
+        err = np.max(np.abs(out.cpu().numpy().astype(np.float64) - ref))
+        assert err <= 3e-4, f"batch size {S}: {err:.2e}"
+        assert attn.last_call_status() == 0
