@@ -51,6 +51,15 @@ SIGNATURES = {
                             _p, _i, _i64, _i64,
                             _i, _i, _i, _i, _i, _i64, _i64, _f,
                             _p, _sz, _p]),
+    "akv_paged_attn_static_scratch_bytes": (_sz, []),
+    "akv_paged_attn_static": (_i, [_p, _i, _i64, _i64,
+                                   _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,
+                                   _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,
+                                   _p, _i, _i64, _p, _i,
+                                   _p, _p, _i,
+                                   _p, _i, _i64, _i64,
+                                   _i, _i, _i, _i, _i, _i64, _i64, _f,
+                                   _p]),
     "akv_paged_attn_status": (_i, [_p, C.POINTER(C.c_int), _p]),
     "akv_debug_set_handoff_spin_limit": (_i, [_i]),
     "akv_hybrid_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),

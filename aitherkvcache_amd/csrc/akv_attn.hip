@@ -494,3 +494,59 @@ extern "C" int akv_paged_attn(
                              num_seqs, num_q_heads, num_kv_heads, d, block_size, num_blocks, max_blocks_per_seq,
                              scale, workspace, workspace_bytes, stream);
 }
+
+// ----------------------------------------------------------------------------------
+// The same call for callers that cannot bring a workspace of their own and cannot allocate one
+// (code under HIP-graph capture, serving loops and harnesses that forbid allocation): the rotated
+// queries, the split partials and the cached tables live in a fixed array inside the library's
+// device image.  The array's name is a host-side stand-in, not a device address: its address on a
+// device is asked for once per device (hipGetSymbolAddress, with that device current) and only that
+// pointer is ever handed to kernels.  Every call on a GPU shares that GPU's array: the kernels
+// rewrite every word they read (the prologue clears the status word, rebuilds the prefix and the
+// query operands; the table block is validated by its tag), and calls that overlap on one GPU race.
+// ----------------------------------------------------------------------------------
+#define AKV_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+#define AKV_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char akv_attn_scratch[AKV_STATIC_SCRATCH_BYTES];
+static void* g_attn_scratch_ptr[AKV_STATIC_MAX_DEVICES];
+
+extern "C" size_t akv_paged_attn_static_scratch_bytes(void) { return AKV_STATIC_SCRATCH_BYTES; }
+
+extern "C" int akv_paged_attn_static(
+    const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+    const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+    const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
+    const uint8_t* v_packed, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+    const float* v_norms, int64_t vns_blk, int64_t vns_pos, int64_t vns_head,
+    const void* block_tables, int bt_itype, int64_t bt_stride,
+    const void* context_lens, int cl_itype,
+    const void* rot_prep, const float* centroids, int bits,
+    void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+    int num_seqs, int num_q_heads, int num_kv_heads, int d,
+    int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale, void* stream) {
+  AKV_REQUIRE(num_seqs >= 0 && num_q_heads > 0 && d > 0, "akv_paged_attn_static: bad head/seq counts");
+  const size_t need = akv_paged_attn_workspace_bytes(num_seqs, num_q_heads, d);
+  if (need > AKV_STATIC_SCRATCH_BYTES)
+    return akv_fail(AKV_ERR_WORKSPACE,
+                    "akv_paged_attn_static: %d sequences x %d query heads need %zu bytes of scratch, the built-in "
+                    "array holds %zu; use akv_paged_attn with a workspace of your own",
+                    num_seqs, num_q_heads, need, (size_t)AKV_STATIC_SCRATCH_BYTES);
+  int dev = -1;
+  AKV_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= AKV_STATIC_MAX_DEVICES)
+    return akv_fail(AKV_ERR_UNSUPPORTED, "akv_paged_attn_static: device index %d beyond %d", dev, AKV_STATIC_MAX_DEVICES);
+  void* ptr = __atomic_load_n(&g_attn_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (ptr == nullptr) {
+    // first call on this device (two threads racing here both obtain the same address)
+    AKV_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(akv_attn_scratch)));
+    if (ptr == nullptr || ((uintptr_t)ptr & 255) != 0)
+      return akv_fail(AKV_ERR_HIP, "akv_paged_attn_static: built-in scratch array has no usable device address");
+    __atomic_store_n(&g_attn_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+  }
+  return akv_paged_attn_impl(query, q_dtype, qs_seq, qs_head, k_packed, kps_blk, kps_pos, kps_head,
+                             k_norms, kns_blk, kns_pos, kns_head, v_packed, vps_blk, vps_pos, vps_head,
+                             v_norms, vns_blk, vns_pos, vns_head, block_tables, bt_itype, bt_stride,
+                             context_lens, cl_itype, rot_prep, centroids, bits, out, out_dtype, os_seq, os_head,
+                             num_seqs, num_q_heads, num_kv_heads, d, block_size, num_blocks, max_blocks_per_seq,
+                             scale, ptr, AKV_STATIC_SCRATCH_BYTES, stream);
+}

@@ -51,8 +51,20 @@ class TQPagedAttention:
             self._workspace = ws
         return ws
 
+    def forward_no_alloc(self, query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
+                         out: torch.Tensor, block_size: int = 16, num_kv_heads: Optional[int] = None) -> torch.Tensor:
+        """forward() for callers that may not allocate (under graph capture, in a loop that forbids
+        it): the result goes into `out` (same shape as `query`, float16 / bfloat16 / float32) and the
+        library works in a fixed scratch array of its own instead of a workspace tensor.  Inputs must
+        already be in the form the kernels take (float query with contiguous rows, float32 norms,
+        contiguous table rows); batches too large for the built-in array raise.  No block selector."""
+        if self._block_selector is not None:
+            raise ValueError("forward_no_alloc does not run the block selector (it allocates)")
+        return self.forward(query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
+                            block_size, num_kv_heads, _static_out=out)
+
     def forward(self, query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
-                block_size: int = 16, num_kv_heads: Optional[int] = None) -> torch.Tensor:
+                block_size: int = 16, num_kv_heads: Optional[int] = None, _static_out=None) -> torch.Tensor:
         """query [num_seqs, num_query_heads, head_dim] -> same shape and dtype.
 
         k/v_packed [num_blocks, block_size, num_kv_heads, >= packed_dim] uint8 (may be strided
@@ -80,9 +92,14 @@ class TQPagedAttention:
             q = q.float()
         if q.stride(-1) != 1:
             q = q.contiguous()
-        out = torch.empty((num_seqs, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+        if _static_out is not None:
+            out = _static_out
+            if out.shape != query.shape or out.stride(-1) != 1 or not out.is_cuda:
+                raise ValueError("out must be a device tensor of the query's shape with contiguous rows")
+        else:
+            out = torch.empty((num_seqs, num_q_heads, head_dim), dtype=q.dtype, device=dev)
         if num_seqs == 0:
-            return out.to(query.dtype)
+            return out if _static_out is not None else out.to(query.dtype)
         for name, t in (("k_packed", k_packed), ("v_packed", v_packed)):
             if t.dtype != torch.uint8 or t.stride(-1) != 1 or t.shape[-1] < self.packed_dim:
                 raise ValueError(f"{name} must be uint8 with contiguous rows of >= {self.packed_dim} bytes")
@@ -91,6 +108,22 @@ class TQPagedAttention:
         bt = block_tables if block_tables.stride(-1) == 1 else block_tables.contiguous()
         cl = context_lens if context_lens.is_contiguous() else context_lens.contiguous()
         num_blocks = min(k_packed.shape[0], k_norms.shape[0], v_packed.shape[0], v_norms.shape[0])
+        if _static_out is not None:
+            if (q is not query or k_norms.dtype != torch.float32 or v_norms.dtype != torch.float32
+                    or bt is not block_tables or cl is not context_lens):
+                raise ValueError("forward_no_alloc needs inputs that take no conversion")
+            _lib.check(_lib.lib().akv_paged_attn_static(
+                q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
+                k_packed.data_ptr(), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2),
+                k_norms.data_ptr(), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2),
+                v_packed.data_ptr(), v_packed.stride(0), v_packed.stride(1), v_packed.stride(2),
+                v_norms.data_ptr(), v_norms.stride(0), v_norms.stride(1), v_norms.stride(2),
+                bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
+                self._tq.prepared_rotation().ptr, self.centroids.data_ptr(), self.bits,
+                out.data_ptr(), _lib.dtype_code(out), out.stride(0), out.stride(1),
+                num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, bt.shape[1], self.scale,
+                _lib.stream_ptr(dev)))
+            return out
         ws = self._get_workspace(num_seqs, dev)
         _lib.check(_lib.lib().akv_paged_attn(
             q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),

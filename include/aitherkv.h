@@ -171,6 +171,30 @@ int akv_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_he
                    int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* akv_paged_attn without a workspace argument.  No counterpart in the reference: it is for callers
+ * that cannot allocate and cannot bring a workspace -- code under HIP-graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The rotated queries, split partials and cached tables
+ * live in one fixed array of akv_paged_attn_static_scratch_bytes() (32 MiB) inside the library's
+ * device image, held by every GPU the library runs on until the process ends.  The call allocates
+ * and frees nothing.  A batch whose akv_paged_attn_workspace_bytes(...) exceeds the array is
+ * refused with AKV_ERR_WORKSPACE (at 32 query heads and head_dim 128: up to 64 sequences).  All
+ * calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
+ * two threads) race; calls on one stream, or otherwise ordered, are fine, whatever their sizes.
+ * Results are those of akv_paged_attn bit for bit. */
+size_t akv_paged_attn_static_scratch_bytes(void);
+int akv_paged_attn_static(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+                          const uint8_t* k_packed, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+                          const float* k_norms, int64_t kns_blk, int64_t kns_pos, int64_t kns_head,
+                          const uint8_t* v_packed, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+                          const float* v_norms, int64_t vns_blk, int64_t vns_pos, int64_t vns_head,
+                          const void* block_tables, int bt_itype, int64_t bt_stride,
+                          const void* context_lens, int cl_itype,
+                          const void* rot_prep, const float* centroids, int bits,
+                          void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+                          int num_seqs, int num_q_heads, int num_kv_heads, int d,
+                          int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
+                          void* stream);
+
 /* Status of the most recent akv_paged_attn / akv_hybrid_paged_attn call that used `workspace`
  * (no counterpart in the reference).  Inside the main kernel pairs of wavefronts hand chunks to
  * each other through counters with BOUNDED waits, so that a kernel always finishes; a wait
