@@ -344,6 +344,12 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits);
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
                       const akv_attn_args& a, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream);
 
+// streaming kernel for the dense 4-bit layout (akv_attn_stream.hip)
+size_t akv_attn_stream_extra_bytes(int S);
+bool akv_attn_stream_applicable(const akv_attn_args& a, int d, int bits);
+int akv_attn_stream_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
+                        const akv_attn_args& a, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream);
+
 extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
   if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
   // the number of kv heads is not known here; it is at most the number of query heads
@@ -452,7 +458,10 @@ static int akv_paged_attn_impl(
 
   int rc;
   int Gused = G;
-  if (akv_attn_mfma_applicable(a, d, bits)) {
+  if (akv_attn_stream_applicable(a, d, bits)) {
+    Gused = G / AKV_ATTN_WG_PER_CU;   // one 16-wavefront workgroup per CU (its rings and table fill the LDS)
+    rc = akv_attn_stream_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
+  } else if (akv_attn_mfma_applicable(a, d, bits)) {
     Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
     rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
   } else {
