@@ -58,6 +58,7 @@ static inline size_t akv_align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct akv_attn_ws {
   uint32_t* lut;     // AKV_WS_LUT_BYTES of cached tables (matrix-core kernels)
   uint32_t* status;  // AKV_WS_STATUS_BYTES
+  int32_t* wgdesc;   // [G][8] start record of every workgroup of the streaming kernel (written by its prologue)
   int32_t* prefix;   // [S + 1] exclusive prefix of blocks per sequence; prefix[S] = total
   float* qrot;       // [S][QH][acc_floats] transformed queries
   float* part_acc;   // [G + S][QH][acc_floats]
@@ -70,6 +71,8 @@ static inline akv_attn_ws akv_attn_ws_layout(void* base, int S, int QH, int acc_
   w.lut = (uint32_t*)base;
   w.status = (uint32_t*)((char*)base + AKV_WS_LUT_BYTES);
   size_t off = AKV_WS_HEADER_BYTES;
+  w.wgdesc = (int32_t*)((char*)base + off);
+  off += akv_align256((size_t)G * 8 * 4);
   w.prefix = (int32_t*)((char*)base + off);
   off += akv_align256((size_t)(S + 1) * 4);
   w.qrot = (float*)((char*)base + off);

@@ -205,6 +205,13 @@ int akv_paged_attn_static(const void* query, int q_dtype, int64_t qs_seq, int64_
  * (0 polls: every wait gives up at once, every kernel still runs to its end). */
 int akv_paged_attn_status(const void* workspace, int* flags, void* stream);
 int akv_debug_set_handoff_spin_limit(int polls);
+/* Two matrix-core kernels can serve a dense 4-bit cache of eight kv heads ([blocks][block_size][8][64]
+ * codes, [blocks][block_size][8] norms, 16-byte aligned, at most 8 query heads per kv head): the general one,
+ * which loads rows into registers, and a streaming one, which fetches whole 8 KB tiles straight into LDS
+ * (HBM traffic exactly the algorithmic bytes).  Sustained, both take the same time; in short bursts the
+ * general one is faster and is the default.  akv_debug_set_attn_stream(1) (or AKV_ATTN_STREAM=1 in the
+ * environment) selects the streaming one where it applies; results are the same to rounding. */
+int akv_debug_set_attn_stream(int on);
 
 /* ---------------------------------------------------------------------------------
  * HybridTurboQuant, mode tq35 with calibrate_uniform() groups (dims 0..63 at 3-bit MSE,

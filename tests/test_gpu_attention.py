@@ -14,6 +14,17 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-3
 
 
+@pytest.fixture(autouse=True, params=["general", "streaming"])
+def attention_kernel(request):
+    """Every test of this file runs twice: with the general matrix-core kernel (the default) and with
+    the streaming kernel selected for the layouts it serves (dense 4-bit cache of eight kv heads;
+    elsewhere the choice changes nothing)."""
+    from aitherkvcache_amd import _lib
+    _lib.check(_lib.lib().akv_debug_set_attn_stream(1 if request.param == "streaming" else 0))
+    yield request.param
+    _lib.check(_lib.lib().akv_debug_set_attn_stream(0))
+
+
 def within_tol(got, ref64):
     """|got - ref| <= 2e-3, plus the rounding of the fp16 output itself (half an fp16 ulp =
     2**-11 relative) where |ref| is large enough for that to matter (|out| >= 4)."""
@@ -488,14 +499,17 @@ def test_corrupt_table_entry_stays_inside_the_cache(golden, dev):
     assert within_tol(out.cpu().numpy(), ref)
 
 
-def test_handoff_timeout_is_reported(golden, dev):
+@pytest.mark.parametrize("kvh,qh", [(8, 32), (2, 8)])
+def test_handoff_timeout_is_reported(golden, dev, kvh, qh):
     """The failure path of the bounded hand-off waits, driven from the host: with a limit of zero
     polls every wait gives up at once (all kernels still run to their end), the call's outputs are
-    NaN and the status query says so; with the default limit restored the next call is clean."""
+    NaN and the status query says so; with the default limit restored the next call is clean.
+    Both matrix-core kernels: the streaming one (dense layout, eight kv heads) and the one that
+    serves the other layouts."""
     from aitherkvcache_amd import _lib
     tq = make_tq(golden, dev, 4)
     rng = np.random.default_rng(78)
-    NB, KVH, QH = 32, 8, 32
+    NB, KVH, QH = 32, kvh, qh
     kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, 4)
     ctx = np.array([300, 64], dtype=np.int64)
     tables = np.stack([rng.permutation(NB)[:20] for _ in range(2)]).astype(np.int64)

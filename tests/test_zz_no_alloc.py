@@ -14,8 +14,16 @@ from tests.test_gpu_attention import build_cache, make_tq, oracle_out, t, within
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("bits", [4, 3])
-def test_static_scratch_entry_matches_workspace_entry(golden, dev, bits):
+@pytest.mark.parametrize("bits,streaming", [(4, 0), (3, 0), (4, 1)])
+def test_static_scratch_entry_matches_workspace_entry(golden, dev, bits, streaming):
+    _lib.check(_lib.lib().akv_debug_set_attn_stream(streaming))
+    try:
+        _static_vs_workspace(golden, dev, bits)
+    finally:
+        _lib.check(_lib.lib().akv_debug_set_attn_stream(0))
+
+
+def _static_vs_workspace(golden, dev, bits):
     tq = make_tq(golden, dev, bits)
     rng = np.random.default_rng(5000 + bits)
     NB, KVH, QH = 160, 8, 32
