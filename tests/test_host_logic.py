@@ -285,3 +285,27 @@ def test_spectral_kv_cache_bookkeeping():
     k2, v2 = other.fetch_sequence(table, S)
     assert all(torch.equal(a, b) for a, b in zip(tuple(k2) + tuple(v2), tuple(k) + tuple(v)))
     assert other.memory_stats()["total_tokens"] == S
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_packing_helpers_match_the_pinned_layouts(bits):
+    """pack_* / unpack_* of the public packing module against the oracle's restatement (itself pinned
+    exhaustively over all bytes / all 2^24 three-bit words): random indices in several shapes, the
+    round trip, and the reference's divisibility asserts."""
+    import torch
+    from aitherkvcache_amd import packing as P
+    from oracle import tq_oracle as O
+    rng = np.random.default_rng(bits)
+    pack = {2: P.pack_2bit, 3: P.pack_3bit, 4: P.pack_4bit}[bits]
+    unpack = {2: P.unpack_2bit, 3: P.unpack_3bit, 4: P.unpack_4bit}[bits]
+    opack = {2: O.pack_2bit, 3: O.pack_3bit, 4: O.pack_4bit}[bits]
+    for shape in ((128,), (5, 64), (2, 3, 128), (0, 128), (7, 8)):
+        idx = rng.integers(0, 1 << bits, size=shape).astype(np.uint8)
+        got = pack(torch.from_numpy(idx))
+        assert got.dtype == torch.uint8 and got.shape[-1] == P.packed_size(shape[-1], bits)
+        assert np.array_equal(got.numpy(), opack(idx))
+        back = unpack(got, shape[-1])
+        assert back.dtype == torch.uint8 and np.array_equal(back.numpy(), idx)
+        assert np.array_equal(pack(torch.from_numpy(idx.astype(np.int64))).numpy(), got.numpy())   # any integer dtype
+    with pytest.raises(AssertionError):
+        pack(torch.zeros(1, {2: 6, 3: 12, 4: 7}[bits], dtype=torch.uint8))
