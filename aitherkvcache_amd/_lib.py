@@ -32,6 +32,7 @@ SIGNATURES = {
     "akv_device_cu_count": (_i, [C.POINTER(C.c_int)]),
     "akv_profile_enable": (_i, [_i]),
     "akv_profile_last_ms": (_i, [C.POINTER(C.c_float)]),
+    "akv_profile_mean_ms": (_i, [C.POINTER(C.c_float), C.POINTER(C.c_int)]),
     "akv_rotation_prepared_bytes": (_sz, [_i]),
     "akv_rotation_prepare": (_i, [_p, _i, _p, _sz, _p]),
     "akv_quantize_pack": (_i, [_p, _i64, _i, _i64, _p, _i, _p, _i64, _p]),

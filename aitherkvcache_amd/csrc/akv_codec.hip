@@ -24,32 +24,63 @@ int akv_cached_cu_count() {
   return cached;
 }
 
+// Ring of event pairs: nothing is read back between launches, so sampled calls run back to back
+// like unsampled ones.  Once the ring is full, later pairs overwrite the oldest.
+static constexpr int kProfRing = 64;
 static bool g_profile_on = false;
-static hipEvent_t g_ev_begin = nullptr, g_ev_end = nullptr;
-static bool g_ev_recorded = false;
+static hipEvent_t g_ev_begin[kProfRing], g_ev_end[kProfRing];
+static bool g_ev_created = false;
+static long g_ev_count = 0;       // pairs recorded since akv_profile_enable(1)
+static bool g_ev_open = false;    // a begin without its end
 
 void akv_profile_mark_begin(hipStream_t s) {
-  if (g_profile_on) (void)hipEventRecord(g_ev_begin, s);
+  if (!g_profile_on) return;
+  (void)hipEventRecord(g_ev_begin[g_ev_count % kProfRing], s);
+  g_ev_open = true;
 }
 void akv_profile_mark_end(hipStream_t s) {
-  if (g_profile_on) { (void)hipEventRecord(g_ev_end, s); g_ev_recorded = true; }
+  if (!g_profile_on || !g_ev_open) return;
+  (void)hipEventRecord(g_ev_end[g_ev_count % kProfRing], s);
+  g_ev_open = false;
+  ++g_ev_count;
 }
 
 extern "C" int akv_profile_enable(int on) {
-  if (on && !g_ev_begin) {
-    AKV_HIP(hipEventCreate(&g_ev_begin));
-    AKV_HIP(hipEventCreate(&g_ev_end));
+  if (on && !g_ev_created) {
+    for (int i = 0; i < kProfRing; ++i) {
+      AKV_HIP(hipEventCreate(&g_ev_begin[i]));
+      AKV_HIP(hipEventCreate(&g_ev_end[i]));
+    }
+    g_ev_created = true;
   }
   g_profile_on = on != 0;
-  g_ev_recorded = false;
+  if (on) { g_ev_count = 0; g_ev_open = false; }
   return AKV_OK;
 }
 
 extern "C" int akv_profile_last_ms(float* ms) {
   AKV_REQUIRE(ms != nullptr, "akv_profile_last_ms: null output");
-  if (!g_ev_recorded) return akv_fail(AKV_ERR_INVALID, "akv_profile_last_ms: nothing recorded");
-  AKV_HIP(hipEventSynchronize(g_ev_end));
-  AKV_HIP(hipEventElapsedTime(ms, g_ev_begin, g_ev_end));
+  if (g_ev_count == 0) return akv_fail(AKV_ERR_INVALID, "akv_profile_last_ms: nothing recorded");
+  const int i = (int)((g_ev_count - 1) % kProfRing);
+  AKV_HIP(hipEventSynchronize(g_ev_end[i]));
+  AKV_HIP(hipEventElapsedTime(ms, g_ev_begin[i], g_ev_end[i]));
+  return AKV_OK;
+}
+
+extern "C" int akv_profile_mean_ms(float* ms, int* samples) {
+  AKV_REQUIRE(ms != nullptr, "akv_profile_mean_ms: null output");
+  if (g_ev_count == 0) return akv_fail(AKV_ERR_INVALID, "akv_profile_mean_ms: nothing recorded");
+  const int n = (int)(g_ev_count < kProfRing ? g_ev_count : kProfRing);
+  AKV_HIP(hipEventSynchronize(g_ev_end[(g_ev_count - 1) % kProfRing]));
+  double acc = 0.0;
+  for (int k = 0; k < n; ++k) {
+    const int i = (int)((g_ev_count - 1 - k) % kProfRing);
+    float t = 0.f;
+    AKV_HIP(hipEventElapsedTime(&t, g_ev_begin[i], g_ev_end[i]));
+    acc += t;
+  }
+  *ms = (float)(acc / n);
+  if (samples) *samples = n;
   return AKV_OK;
 }
 

@@ -54,11 +54,16 @@ int akv_device_cu_count(int* cu_count);
  * Measurement hook (no counterpart in the reference).  While enabled, every entry point
  * brackets its dominant kernel (the main decode-attention kernel, the encode kernel, the
  * TriAttention scoring kernel) with a pair of HIP events recorded on the launch stream.
- * akv_profile_last_ms waits for the pair of the most recent call and returns its elapsed
- * time in milliseconds.  Meant for benchmarks; leave it off in serving code.
+ * The pairs go into a ring of 64, and nothing is read back between calls, so sampled calls
+ * run back to back.  akv_profile_last_ms waits for the pair of the most recent call and
+ * returns its elapsed time in milliseconds; akv_profile_mean_ms waits for the most recent
+ * pair and returns the mean over the (at most 64) latest pairs recorded since the hook was
+ * switched on, with their number in *samples (may be NULL).  Meant for benchmarks; leave
+ * it off in serving code.
  * ------------------------------------------------------------------------------- */
 int akv_profile_enable(int on);
 int akv_profile_last_ms(float* ms);
+int akv_profile_mean_ms(float* ms, int* samples);
 
 /* ---------------------------------------------------------------------------------
  * Rotation matrix, prepared once per quantizer.
