@@ -6,40 +6,14 @@ import torch
 import aitherkvcache_amd as akv
 from aitherkvcache_amd import triton_ops
 from oracle import tq_oracle as O
-from tests.util import kv_like, code_mismatch_report
+from tests.util import kv_like, code_mismatch_report, check_codes, MAX_ULPS
 
 pytestmark = pytest.mark.gpu
-
-MAX_ULPS = 16       # a code may differ from the float32 oracle only if the float64 rotated value
-                    # lies within this many float32 ulps of a decision boundary
-
 
 def make_tq(golden, dev, bits, d=128):
     tq = akv.TurboQuant(head_dim=d, bits=bits, device=str(dev))
     tq.rotation = torch.from_numpy(golden[f"rotation_d{d}_seed42"]).to(dev)   # the reference's matrix
     return tq
-
-
-def check_codes(packed, norms, x, R, bits, ref_packed=None, ref_norms=None, d=128):
-    """Bit-exact codes modulo the boundary-ulp rule; norms to 1e-6 relative."""
-    _, b, _ = O.get_codebook(d, bits)
-    if ref_packed is None:
-        ref_packed, ref_norms = O.encode(x, R, b, bits)
-    ca = O._UNPACK[bits](packed.reshape(-1, packed.shape[-1]), d)
-    cb = O._UNPACK[bits](ref_packed.reshape(-1, ref_packed.shape[-1]), d)
-    y64 = O.rotate_unit_f64(np.asarray(x).reshape(-1, d), R)
-    n, max_ulps, hist = code_mismatch_report(ca, cb, y64, b, O)
-    total = ca.size
-    print(f"[codes] bits={bits} mismatching={n}/{total} max_ulps={max_ulps:.2f} hist={hist}")
-    assert max_ulps <= MAX_ULPS, hist
-    assert hist.get("max_code_step", 1) == 1
-    assert n <= max(3, total * 2e-5), (n, total)
-    nr = np.asarray(ref_norms).reshape(-1).astype(np.float64)
-    ng = np.asarray(norms).reshape(-1).astype(np.float64)
-    nz = nr > 0
-    assert np.max(np.abs(ng[nz] - nr[nz]) / nr[nz]) < 1e-6
-    assert np.all(ng[~nz] == 0)
-    return n
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
@@ -228,11 +202,17 @@ def test_fused_encode_and_store(golden, dev):
     v = torch.randn(5, 2, 128, device=dev, dtype=torch.float16)
     slots = torch.tensor([3, 17, 40, 63, 64], device=dev)      # 64 -> block 4 >= max_blocks: skipped
     akv.fused_encode_and_store(c, 1, k, v, slots)
-    kp, kn = c.tq.encode(k[:4])
-    vp, vn = c.tq.encode(v[:4])
-    b, p = (slots[:4] // 16).cpu(), (slots[:4] % 16).cpu()
-    assert torch.equal(c.k_packed[1][b, p].cpu(), kp.cpu()) and torch.equal(c.v_packed[1][b, p].cpu(), vp.cpu())
-    assert torch.equal(c.k_norms[1][b, p].cpu(), kn.cpu()) and torch.equal(c.v_norms[1][b, p].cpu(), vn.cpu())
+    R = golden["rotation_d128_seed42"]
+    _, bnd, _ = O.get_codebook(128, 4)
+    for x, packed, norms in ((k, c.k_packed, c.k_norms), (v, c.v_packed, c.v_norms)):
+        ref_p = np.zeros((4, 16, 2, 64), np.uint8)
+        ref_n = np.zeros((4, 16, 2), np.float32)
+        O.kv_update(x.cpu().numpy(), slots.cpu().numpy(), ref_p, ref_n, R, bnd, block_size=16, max_blocks=4, bits=4)
+        written = ref_n > 0
+        assert np.array_equal(norms[1].cpu().numpy() > 0, written)            # the same slots, nothing else
+        check_codes(packed[1].cpu().numpy()[written], norms[1].cpu().numpy()[written],
+                    x[:4].cpu().numpy().reshape(-1, 128), R, 4, ref_p[written], ref_n[written])
+        assert np.all(packed[1].cpu().numpy()[~written] == 0)
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 

@@ -309,3 +309,45 @@ def test_packing_helpers_match_the_pinned_layouts(bits):
         assert np.array_equal(pack(torch.from_numpy(idx.astype(np.int64))).numpy(), got.numpy())   # any integer dtype
     with pytest.raises(AssertionError):
         pack(torch.zeros(1, {2: 6, 3: 12, 4: 7}[bits], dtype=torch.uint8))
+
+
+def test_backend_module_needs_no_vllm_and_no_gpu():
+    """Importing the backend module and making its classes imports no vLLM; the class answers vLLM's
+    questions (reference: vllm/backend.py:264-311) and the plugin entry point reports that there is
+    nothing to register with (vllm/plugin.py:18-53)."""
+    import sys
+    from aitherkvcache_amd.vllm import backend, plugin
+    bk = backend.TurboQuantBackend
+    assert not any(m == "vllm" or m.startswith("vllm.") for m in sys.modules)
+    assert bk.get_name() == "CUSTOM" and bk.accept_output_buffer is True
+    assert bk.forward_includes_kv_cache_update is False
+    assert bk.get_kv_cache_shape(9, 16, 8, 128) == (9, 2, 16, 8, 128)
+    assert bk.get_kv_cache_shape(9, 16, 8, 128, "fp8") == (9, 2, 16, 8, 128)
+    assert bk.get_kv_cache_shape(9, 16, 8, 128, "tq-t4nc") == (9, 2, 16, 8, 68)
+    assert bk.get_kv_cache_shape(9, 16, 8, 128, "tq-t3nc") == (9, 2, 16, 8, 52)
+    assert bk.get_kv_cache_shape(9, 16, 8, 128, "tq-t2nc") == (9, 2, 16, 8, 36)
+    assert bk.get_kv_cache_shape(9, 16, 8, 128, "tq35") == (9, 2, 16, 8, 64)
+    assert bk.get_supported_head_sizes() == [64, 96, 128, 256, 512]
+    assert {"auto", "bfloat16", "fp8", "tq-t4nc", "tq-t3nc", "tq-t2nc", "tq35"} <= set(bk.supported_kv_cache_dtypes)
+    impl = bk.get_impl_cls()
+    assert impl is backend.TurboQuantImpl and callable(impl.do_kv_cache_update) and callable(impl.forward)
+    assert backend.register_turboquant_backend() is False and plugin.register() is False
+    with pytest.raises(AttributeError):
+        backend.NoSuchName
+
+
+def test_backend_format_selection_from_environment(monkeypatch):
+    from aitherkvcache_amd.vllm import backend
+    for mode, bits_env, want in (("", None, ("uniform", 4)), ("", "3", ("uniform", 3)), ("tq35", None, ("hybrid", None)),
+                                 ("tq35-primary", None, ("hybrid", None)), ("tq-t2nc-primary", "4", ("uniform", 2))):
+        monkeypatch.setenv("AITHER_TQ_MODE", mode)
+        if bits_env is None:
+            monkeypatch.delenv("AITHER_TQ_BITS", raising=False)
+        else:
+            monkeypatch.setenv("AITHER_TQ_BITS", bits_env)
+        fmt = backend.format_from_env()
+        assert (fmt.kind, fmt.bits) == want
+        assert backend.primary_from_env() == mode.endswith("-primary")
+    monkeypatch.setenv("AITHER_TQ_MODE", "")
+    monkeypatch.setenv("AITHER_TQ_PRIMARY", "1")
+    assert backend.primary_from_env()
