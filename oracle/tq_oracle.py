@@ -551,6 +551,67 @@ def hybrid_encode(x, hp: HybridParams):
     return out.reshape(x.shape[:-1] + (64,))
 
 
+def _hadamard_matrix64():
+    h = np.array([[1.0]])
+    while h.shape[0] < 64:
+        h = np.block([[h, h], [h, -h]])
+    return h
+
+
+def hybrid_encode_margins(x, packed, hp: HybridParams):
+    """Float64 account of every bit of `packed` (rows produced by ANY float32 implementation of
+    hybrid_encode for the vectors `x`): how far the quantity behind each code, each sign bit and
+    each stored norm lies from the value at which that bit would flip.  A float32 implementation
+    may differ from another one (summation order of the norm and of the butterflies) only where
+    these margins are a few float32 ulps; anywhere else a difference is a defect.
+
+    For both groups g, with the codes and signs READ FROM `packed` (so that a code which
+    legitimately flipped does not make the signs that follow from it look wrong):
+      code_ulps[g]  [n,64]  |rot64 - boundary| for the farthest boundary the stored code would have
+                            to cross to reach the float64 code, in float32 ulps of the larger of that
+                            boundary and the row's largest |rot64| (0 where the codes agree)
+      sign_ulps[g]  [n,64]  |proj64| in float32 ulps of the row's largest |proj64| where the stored
+                            sign differs from sign(proj64), else 0
+      norm_steps[g], rnorm_steps[g]  [n]  stored fp16 norm / residual norm minus the fp16 rounding
+                            of the float64 value, in fp16 steps (bit patterns)
+    Same operations as _hybrid_encode_group (hybrid_quantizer.py:706-779) carried in float64."""
+    x = np.asarray(x).reshape(-1, 128).astype(f32).astype(np.float64)
+    packed = np.asarray(packed, dtype=np.uint8).reshape(-1, 64)
+    H = _hadamard_matrix64() / 8.0
+    out = {"code_ulps": [], "sign_ulps": [], "norm_steps": [], "rnorm_steps": []}
+    for g, (lo, off) in enumerate(((0, 0), (64, 36))):
+        xg = x[:, lo:lo + 64]
+        pg = packed[:, off:off + hp.group_bytes[g]]
+        mb = hp.mse_bytes[g]
+        n64 = np.sqrt(np.sum(xg * xg, axis=-1))
+        # the reference divides by the float32 norm + 1e-10 (float32 arithmetic)
+        unit = xg / (n64.astype(f32) + f32(1e-10)).astype(np.float64)[:, None]
+        had = hp.had[g].astype(np.float64)
+        rot = (unit * had) @ H
+        b = hp.boundaries[g].astype(np.float64)
+        idx64 = np.clip(np.searchsorted(b, rot, side="left"), 0, (1 << hp.mse_bits[g]) - 1)
+        idx = unpack_multibit(pg[:, :mb], 64, hp.mse_bits[g]).astype(np.int64)
+        # boundaries between the stored code and the float64 code: the farthest one decides
+        far = np.where(idx > idx64, b[np.clip(idx - 1, 0, len(b) - 1)], b[np.clip(idx, 0, len(b) - 1)])
+        # the rounding error of a butterfly sum is absolute, of the size of the terms summed: a result
+        # that cancels to (nearly) zero is no more accurate than the row's large outputs
+        floor = np.max(np.abs(rot), axis=-1, keepdims=True)
+        ulp = np.spacing(np.maximum(np.maximum(np.maximum(np.abs(far), np.abs(rot)), floor), 1e-30).astype(f32)).astype(np.float64)
+        out["code_ulps"].append(np.where(idx != idx64, np.abs(rot - far) / ulp, 0.0))
+        mse_hat = (hp.centroids[g].astype(np.float64)[idx] @ H) * had
+        res = unit - mse_hat
+        rn64 = np.sqrt(np.sum(res * res, axis=-1))
+        proj = (res * hp.qjl[g].astype(np.float64)) @ H
+        sgn = unpack_multibit(pg[:, mb:mb + 8], 64, 1).astype(bool)
+        row_ulp = np.spacing(np.maximum(np.max(np.abs(proj), axis=-1), 1e-30).astype(f32)).astype(np.float64)
+        out["sign_ulps"].append(np.where(sgn != (proj >= 0), np.abs(proj) / row_ulp[:, None], 0.0))
+        for key, val, at in (("norm_steps", n64, mb + 8), ("rnorm_steps", rn64, mb + 10)):
+            stored = np.ascontiguousarray(pg[:, at:at + 2]).view(np.uint16).reshape(-1).astype(np.int64)
+            want = val.astype(np.float16).view(np.uint16).astype(np.int64)
+            out[key].append(stored - want)
+    return out
+
+
 def _hybrid_decode_group(pg, hp: HybridParams, g):
     """_decode_single_group, hybrid_quantizer.py:876-933."""
     mb = hp.mse_bytes[g]

@@ -216,6 +216,46 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+def test_config1_literal_shape_steps_vs_oracle(golden, dev):
+    """The serving write at its benchmark shape: 8 kv heads, a cache of 8,192 blocks of 16, steps of 256
+    tokens (K and V) whose slots are consecutive runs of ONE random permutation of all 131,072 slots, so
+    no step overwrites another.  After four steps the whole cache equals what the oracle's kv_update
+    wrote: the same slots and nothing else, codes under the boundary-ulp rule, norms to 1e-6."""
+    NB, BS, H, T, STEPS = 8192, 16, 8, 256, 4
+
+    class Cache:
+        pass
+    c = Cache()
+    c.tq = make_tq(golden, dev, 4)
+    c.block_size, c.max_blocks = BS, NB
+    c.k_packed = torch.zeros(1, NB, BS, H, 64, dtype=torch.uint8, device=dev)
+    c.v_packed = torch.zeros_like(c.k_packed)
+    c.k_norms = torch.zeros(1, NB, BS, H, device=dev)
+    c.v_norms = torch.zeros_like(c.k_norms)
+    rng = np.random.default_rng(1)
+    perm = rng.permutation(NB * BS)
+    R = golden["rotation_d128_seed42"]
+    _, bnd, _ = O.get_codebook(128, 4)
+    ref = {n: (np.zeros((NB, BS, H, 64), np.uint8), np.zeros((NB, BS, H), np.float32)) for n in "kv"}
+    rows = {"k": [], "v": []}
+    for step in range(STEPS):
+        slots = perm[step * T:(step + 1) * T].astype(np.int64)
+        k, v = kv_like(rng, (T, H, 128)), kv_like(rng, (T, H, 128))
+        akv.fused_encode_and_store(c, 0, torch.from_numpy(k).to(dev), torch.from_numpy(v).to(dev),
+                                   torch.from_numpy(slots).to(dev))
+        for n, x in (("k", k), ("v", v)):
+            O.kv_update(x, slots, ref[n][0], ref[n][1], R, bnd, block_size=BS, bits=4)
+            rows[n].append((slots, x))
+    for n, packed, norms in (("k", c.k_packed, c.k_norms), ("v", c.v_packed, c.v_norms)):
+        got_p, got_n = packed[0].cpu().numpy(), norms[0].cpu().numpy()
+        written = ref[n][1] > 0
+        assert int(written.sum()) == STEPS * T * H and np.array_equal(got_n > 0, written)
+        assert not got_p[~written].any()
+        slots = np.concatenate([s for s, _ in rows[n]])
+        x = np.concatenate([x for _, x in rows[n]])[np.argsort(slots)]             # rows in slot order, like the cache
+        check_codes(got_p[written], got_n[written], x.reshape(-1, 128), R, 4, ref[n][0][written], ref[n][1][written])
+
+
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("n", [1, 33, 4097])
 def test_decode_random_codes_vs_oracle(golden, dev, bits, n):

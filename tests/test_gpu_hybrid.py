@@ -7,7 +7,7 @@ import torch
 
 import aitherkvcache_amd as akv
 from oracle import tq_oracle as O
-from tests.util import kv_like
+from tests.util import kv_like, MAX_ULPS
 
 pytestmark = pytest.mark.gpu
 
@@ -70,9 +70,20 @@ def test_encode_vs_oracle_bulk(golden, dev, dtype):
     packed = h.encode(x).cpu().numpy()
     ref = O.hybrid_encode(x.float().cpu().numpy(), hp)
     st = compare_rows(packed, ref)
-    print("[hybrid bulk]", dtype, st)
-    assert st["rows_differing"] <= 0.01 * st["rows"]
-    assert st["code_bytes"] + st["sign_bytes"] <= 0.002 * st["rows"]
+    # every bit that differs from a float64 evaluation must sit within MAX_ULPS float32 ulps of its flip
+    # point (codes: rotated value against the boundary; signs: projection against zero, with the row's own
+    # codes); stored norms at most one fp16 step from the rounded float64 norm
+    m = O.hybrid_encode_margins(x.float().cpu().numpy(), packed, hp)
+    worst = {k: max(float(np.abs(v[g]).max()) for g in (0, 1)) for k, v in m.items()}
+    flips = {k: sum(int((v[g] != 0).sum()) for g in (0, 1)) for k, v in m.items()}
+    print("[hybrid bulk]", dtype, st, "worst", worst, "flips", flips)
+    assert worst["code_ulps"] <= MAX_ULPS and worst["sign_ulps"] <= MAX_ULPS
+    assert worst["norm_steps"] <= 1 and worst["rnorm_steps"] <= 1
+    # observed: at most 8 of 20,000 rows differ from the float32 oracle (norms one fp16 step apart, and with
+    # bfloat16 input three codes whose rotated value cancels to zero, the middle boundary, with the sign bits
+    # that follow from them); the gates are five times that
+    assert st["rows_differing"] <= 40
+    assert st["code_bytes"] + st["sign_bytes"] <= 50
     # decode is exact integer/butterfly work
     dec = h.decode(t(ref, dev)).cpu().numpy()
     assert np.array_equal(dec, O.hybrid_decode(ref, hp))

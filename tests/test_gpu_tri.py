@@ -71,6 +71,40 @@ def test_vs_oracle_shapes(dev, B, S, QH, KVH, D, F, base):
     assert np.max(np.abs(out_d - ref_d)) <= TOL
 
 
+def test_config4_literal_shape(dev):
+    """The benchmark shape itself: batch 8 x 32,768 tokens, 32 query / 8 kv heads, d = 128, F = 12 int4,
+    keys with a power-law pair spectrum (seed 4).  One batch element against the oracle (its encoder and
+    its decode_step), and for the whole batch: every element computed alone equals its row of the batched
+    call, and elements given the same cache rows and query produce the same output."""
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=8, num_query_heads=32, rope_base=1e6)
+    tri = TriAttention(cfg, device=str(dev))
+    B, S = 8, 32768
+    g = torch.Generator(device=dev).manual_seed(4)
+    std = (torch.arange(64, device=dev) + 1.0) ** -0.75
+    keys = (torch.randn(B, S, 8, 64, 2, device=dev, generator=g) * std[:, None]).reshape(B, S, 8, 128).half()
+    vals = torch.randn(B, S, 8, 128, device=dev, generator=g).half()
+    keys[7], vals[7] = keys[2], vals[2]                      # element 7 repeats element 2
+    q = torch.randn(B, 32, 128, device=dev, generator=g)
+    q[7] = q[2]
+    k_enc, v_enc = tri.encode_kv(keys, vals)
+    out = tri.decode_step(q, k_enc, v_enc)
+    assert out.shape == (B, 32, 128) and torch.isfinite(out).all()
+    assert torch.equal(out[7], out[2])
+    for b in (0, 5):
+        one = tri.decode_step(q[b:b + 1], SpectralEncoding(*(x[b:b + 1] for x in k_enc)),
+                              SpectralEncoding(*(x[b:b + 1] for x in v_enc)))
+        assert torch.max(torch.abs(one[0] - out[b])).item() <= TOL      # the split count may differ
+    b = 3
+    ke = O.spectral_encode(keys[b:b + 1].cpu().numpy(), 12)
+    ve = O.spectral_encode(vals[b:b + 1].cpu().numpy(), 12)
+    for got, want in zip(tuple(k_enc) + tuple(v_enc), ke + ve):
+        assert np.array_equal(got[b:b + 1].cpu().numpy(), want)
+    ref = O.tri_decode_step(q[b:b + 1].cpu().numpy(), ke, ve, tri._theta.cpu().numpy())
+    err = np.max(np.abs(out[b:b + 1].cpu().numpy() - ref))
+    print(f"[tri config 4] element {b}: max|diff|={err:.2e} max|out|={np.abs(ref).max():.3f}")
+    assert err <= TOL
+
+
 def test_uniform_values_property(dev):
     """Every token holds the same value row -> the output is that row, whatever the scores
     (softmax weights sum to one across all splits)."""

@@ -321,3 +321,30 @@ def test_spectral_fetch_sequence_is_token_by_token_indexing():
         for j, got in enumerate(k_enc + v_enc):
             want = np.stack([arrays[j][table[t // BS], t % BS] for t in range(n)])
             assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def test_hybrid_margins_accept_the_oracle_and_catch_defects(golden):
+    """hybrid_encode_margins (float64) against the float32 oracle: no code or sign of the oracle's own
+    rows, nor of the reference's golden rows, is more than a rounding away from the float64 answer, and
+    a flipped code bit or sign bit shows up as a margin of millions of ulps."""
+    books = tuple((golden[f"hyb_centroids_64_{k}"], golden[f"hyb_boundaries_64_{k}"]) for k in (3, 2))
+    hp = O.HybridParams(golden["hyb_g0_had_signs"], golden["hyb_g1_had_signs"],
+                        golden["hyb_g0_qjl_signs"], golden["hyb_g1_qjl_signs"], codebooks=books)
+    m = O.hybrid_encode_margins(golden["hyb_x"], golden["hyb_packed"], hp)
+    assert all(float(np.abs(v[g]).max()) == 0 for v in m.values() for g in (0, 1))
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal((3000, 128)) * rng.lognormal(0, 0.5, (3000, 1))).astype(np.float32)
+    p = O.hybrid_encode(x, hp)
+    m = O.hybrid_encode_margins(x, p, hp)
+    for g in (0, 1):
+        assert m["code_ulps"][g].max() <= 4 and m["sign_ulps"][g].max() <= 4
+        assert np.abs(m["norm_steps"][g]).max() <= 1 and np.abs(m["rnorm_steps"][g]).max() <= 1
+    bad = p.copy()
+    bad[7, 3] ^= 0x10          # a group-0 code bit
+    bad[9, 25] ^= 0x01         # a group-0 sign bit
+    bad[11, 40] ^= 0x40        # a group-1 code bit
+    bad[13, 61] ^= 0x04        # group-1 norm, fp16 high byte
+    m = O.hybrid_encode_margins(x, bad, hp)
+    assert m["code_ulps"][0][7].max() > 1e3 and m["sign_ulps"][0][9].max() > 1e3
+    assert m["code_ulps"][1][11].max() > 1e3 and abs(int(m["norm_steps"][1][13])) > 100
+    assert m["code_ulps"][0][8].max() == 0 and m["sign_ulps"][1][9].max() == 0
