@@ -40,6 +40,8 @@ SIGNATURES = {
     "akv_encode": (_i, [_p, _i, _i64, _i, _i64, _p, _p, _i, _p, _i64, _p, _p]),
     "akv_encode_paged": (_i, [_p, _i, _i64, _i, _i, _i64, _i64, _p, _i, _p, _p, _i,
                               _p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i, _i64, _p]),
+    "akv_encode_paged_kv": (_i, [_p, _p, _i, _i64, _i, _i, _i64, _i64, _p, _i, _p, _p, _i,
+                                 _p, _p, _i64, _i64, _i64, _p, _p, _i64, _i64, _i64, _i, _i64, _p]),
     "akv_decode": (_i, [_p, _i64, _p, _i64, _i, _p, _p, _i, _p, _i, _i64, _p]),
     "akv_decode_blocks": (_i, [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _p, _i, _i64, _i64,
                                _i, _i, _i, _p, _p, _i, _p, _i, _i64, _i64, _i64, _p]),

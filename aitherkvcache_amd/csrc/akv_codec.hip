@@ -532,6 +532,40 @@ extern "C" int akv_encode(const void* x, int x_dtype, int64_t n, int d, int64_t 
   return akv_encode_dispatch<false>(d, bits, x_dtype, a, stream);
 }
 
+extern "C" int akv_encode_paged_kv(const void* k, const void* v, int x_dtype, int64_t num_tokens,
+                                   int num_kv_heads, int d, int64_t xs_token, int64_t xs_head,
+                                   const void* slot_mapping, int slot_itype, const void* rot_prep,
+                                   const float* boundaries, int bits, uint8_t* k_packed, uint8_t* v_packed,
+                                   int64_t ps_blk, int64_t ps_pos, int64_t ps_head, float* k_norms,
+                                   float* v_norms, int64_t ns_blk, int64_t ns_pos, int64_t ns_head,
+                                   int block_size, int64_t max_blocks, void* stream) {
+  AKV_REQUIRE(num_tokens >= 0 && num_kv_heads > 0, "akv_encode_paged_kv: bad sizes");
+  AKV_REQUIRE(akv_valid_dtype(x_dtype) && akv_valid_itype(slot_itype), "akv_encode_paged_kv: bad dtype");
+  AKV_REQUIRE(block_size > 0 && max_blocks >= 0, "akv_encode_paged_kv: bad block_size/max_blocks");
+  int rc = akv_check_codec_args("akv_encode_paged_kv", d, bits);
+  if (rc) return rc;
+  if (num_tokens == 0 || max_blocks == 0) return AKV_OK;
+  AKV_REQUIRE(k && v && slot_mapping && rot_prep && boundaries && k_packed && v_packed && k_norms && v_norms,
+              "akv_encode_paged_kv: null pointer");
+  akv_gen_args a = {};
+  a.x = k; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
+  a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
+  a.mat = (const float*)rot_prep + (size_t)d * d;
+  a.table = boundaries;
+  a.packed = k_packed; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
+  a.norms = k_norms; a.ns0 = ns_blk; a.ns1 = ns_pos; a.ns2 = ns_head;
+  a.x2 = v; a.packed2 = v_packed; a.norms2 = v_norms;
+  rc = akv_encode_mfma_try(a, true, x_dtype, d, bits, rot_prep, (hipStream_t)stream);
+  if (rc != AKV_ERR_UNSUPPORTED) return rc;
+  // layouts the matrix-core kernel does not take: one launch per tensor
+  akv_gen_args b = a;
+  a.x2 = nullptr; a.packed2 = nullptr; a.norms2 = nullptr;
+  b.x = v; b.packed = v_packed; b.norms = v_norms; b.x2 = nullptr; b.packed2 = nullptr; b.norms2 = nullptr;
+  rc = akv_encode_dispatch<true>(d, bits, x_dtype, a, stream);
+  if (rc) return rc;
+  return akv_encode_dispatch<true>(d, bits, x_dtype, b, stream);
+}
+
 extern "C" int akv_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads,
                                 int d, int64_t xs_token, int64_t xs_head, const void* slot_mapping,
                                 int slot_itype, const void* rot_prep, const float* boundaries,

@@ -80,6 +80,11 @@ struct akv_gen_args {
   int64_t ps0, ps1, ps2; // flat: ps0 = row stride (bytes); paged: blk, pos, head strides (bytes)
   float* norms;
   int64_t ns0, ns1, ns2;
+  // paged encode of a second tensor in the same launch (K and V of one step): same shapes, strides and
+  // slots as x / packed / norms; vectors n .. 2n - 1 of the launch.  Null when there is none.
+  const void* x2;
+  uint8_t* packed2;
+  float* norms2;
   // decode output
   void* out;
   int64_t os0, os1, os2;  // flat: os0 = row stride; block-wise decode: blk, pos, head strides (elements)

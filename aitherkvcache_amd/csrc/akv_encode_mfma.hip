@@ -171,12 +171,13 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   const float* bnd = (const float*)(lds + EM_BND_OFF);
 
   unsigned char* wl = lds + EM_WAVE_OFF + wave * EM_WAVE_BYTES;
-  int64_t* src_off = (int64_t*)wl;                    // element offset of the vector in x, or -1
-  int64_t* dst_p = (int64_t*)(wl + EM_ROWS * 8);      // byte offset of the packed row, or -1
-  int64_t* dst_n = (int64_t*)(wl + EM_ROWS * 16);     // element offset of the norm
+  int64_t* src_off = (int64_t*)wl;                    // address of the vector, or 0
+  int64_t* dst_p = (int64_t*)(wl + EM_ROWS * 8);      // address of the packed row, or 0
+  int64_t* dst_n = (int64_t*)(wl + EM_ROWS * 16);     // address of the norm
   float* rinv = (float*)(wl + EM_ROWS * 24);          // 1/(|x| + 1e-10), scaled back by 1/EM_PSCALE; NaN rows flagged
 
-  const int64_t steps = (a.n + EM_ROWS - 1) / EM_ROWS;
+  const int64_t n_total = (PAGED && a.x2) ? 2 * a.n : a.n;      // a second tensor rides along (K and V of a step)
+  const int64_t steps = (n_total + EM_ROWS - 1) / EM_ROWS;
   const int64_t stride = (int64_t)gridDim.x * EM_WAVES;
 
   // A operands of one step straight from memory (zeros past the end): lane l resolves the source
@@ -203,22 +204,25 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       }
       return;
     }
-    const int64_t n = step * EM_ROWS + lane;
-    int64_t so = -1;
-    if (step < steps && n < a.n && lane < EM_ROWS) {
+    int64_t n = step * EM_ROWS + lane;
+    int64_t so = 0;      // byte address of the vector, 0 = none
+    if (step < steps && n < n_total && lane < EM_ROWS) {
+      const bool second = PAGED && n >= a.n;
+      if (second) n -= a.n;
+      const char* xb = (const char*)(second ? a.x2 : a.x);
       if (PAGED) {
         const int64_t tok = n / a.heads, head = n - tok * a.heads;
-        so = tok * a.xs0 + head * a.xs1;
+        so = (int64_t)(uintptr_t)(xb + 2 * (tok * a.xs0 + head * a.xs1));
       } else {
-        so = n * a.xs0;
+        so = (int64_t)(uintptr_t)(xb + 2 * n * a.xs0);
       }
     }
     if (lane < EM_ROWS) src_off[lane] = so;
 #pragma unroll
     for (int mt = 0; mt < EM_MT; ++mt) {
       const int64_t ro = src_off[16 * mt + (lane & 15)];
-      if (ro >= 0) {
-        const uint4* p = (const uint4*)((const __half*)a.x + ro + 32 * g);
+      if (ro != 0) {
+        const uint4* p = (const uint4*)(uintptr_t)(ro + 64 * g);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
           union { uint4 u; em_half8 h; } cv;
@@ -239,22 +243,26 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     const int64_t base = step * EM_ROWS;
     // ---- lane l resolves the destination of vector base + l
     if constexpr (!DIRECT) {
-      const int64_t n = base + lane;
-      int64_t dp = -1, dn = 0;
-      if (n < a.n && lane < EM_ROWS) {
+      int64_t n = base + lane;
+      int64_t dp = 0, dn = 0;      // byte addresses of the packed row and of the norm, 0 = skip
+      if (n < n_total && lane < EM_ROWS) {
+        const bool second = PAGED && n >= a.n;
+        if (second) n -= a.n;
+        uint8_t* pb = second ? a.packed2 : a.packed;
+        float* nb = second ? a.norms2 : a.norms;
         if (PAGED) {
           const int64_t tok = n / a.heads, head = n - tok * a.heads;
           const int64_t slot = akv_load_index(a.slots, a.slot_itype, tok);
           if (slot >= 0) {
             const int64_t blk = slot / a.block_size, pos = slot - blk * a.block_size;
             if (blk < a.max_blocks) {
-              dp = blk * a.ps0 + pos * a.ps1 + head * a.ps2;
-              dn = blk * a.ns0 + pos * a.ns1 + head * a.ns2;
+              dp = (int64_t)(uintptr_t)(pb + blk * a.ps0 + pos * a.ps1 + head * a.ps2);
+              dn = (int64_t)(uintptr_t)(nb + blk * a.ns0 + pos * a.ns1 + head * a.ns2);
             }
           }
         } else {
-          dp = n * a.ps0;
-          dn = n;
+          dp = (int64_t)(uintptr_t)(pb + n * a.ps0);
+          dn = (int64_t)(uintptr_t)(nb + n);
         }
       }
       if (lane < EM_ROWS) {
@@ -364,7 +372,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         if constexpr (DIRECT) {
           if ((uint32_t)base + lane < (uint32_t)a.n) a.norms[(uint32_t)base + lane] = nrm;
         } else {
-          if (dst_p[lane] >= 0) a.norms[dst_n[lane]] = nrm;
+          if (dst_p[lane] != 0) *(float*)(uintptr_t)dst_n[lane] = nrm;
         }
       }
     }
@@ -400,12 +408,13 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         }
       }
     };
-    auto search_tile = [&](int nt, const em_float4 (&acc)[EM_MT]) {
-      // output coordinate 8 col + nt of rows 4g + i; position of code nt inside the lane's packed
-      // group of eight codes
-      const int sh = BITS == 4 ? 8 * (nt >> 1) + ((nt & 1) ? 0 : 4)
-                   : BITS == 3 ? 21 - 3 * nt
-                               : 8 * (nt >> 2) + 6 - 2 * (nt & 3);
+    // A lane's packed group is built by shift-and-add, one instruction per code: the N-tiles are visited
+    // in the order in which their codes enter the group from the top (4-bit: 6 7 4 5 2 3 0 1 -- a dword
+    // is four little-endian bytes of two nibbles; 3-bit: 0 .. 7; 2-bit: 4 5 6 7 0 1 2 3).
+    auto tile_at = [&](int k) -> int {
+      return BITS == 4 ? 6 - (k & ~1) + (k & 1) : BITS == 3 ? k : ((k + 4) & 7);
+    };
+    auto search_tile = [&](const em_float4 (&acc)[EM_MT]) {
       float y[EM_MT][4];
 #pragma unroll
       for (int mt = 0; mt < EM_MT; ++mt)
@@ -423,7 +432,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t code = e[mt][i].x + ((__uint_as_float(e[mt][i].y) < y[mt][i]) ? 1u : 0u);
-            packed[mt][i] |= code << sh;
+            packed[mt][i] = (packed[mt][i] << BITS) + code;
           }
       } else {
 #pragma unroll
@@ -433,18 +442,18 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
             uint32_t code = 0;
 #pragma unroll 1
             for (int k = 0; k < NB; ++k) code += (bnd[k] < y[mt][i]) ? 1u : 0u;
-            packed[mt][i] |= code << sh;
+            packed[mt][i] = (packed[mt][i] << BITS) + code;
           }
       }
     };
     em_float4 accA[EM_MT], accB[EM_MT];
-    mfma_tile(0, accA);
+    mfma_tile(tile_at(0), accA);
 #pragma unroll 1
-    for (int nt = 0; nt < 6; nt += 2) {
-      mfma_tile(nt + 1, accB);
-      search_tile(nt, accA);
-      mfma_tile(nt + 2, accA);
-      search_tile(nt + 1, accB);
+    for (int k = 0; k < 6; k += 2) {
+      mfma_tile(tile_at(k + 1), accB);
+      search_tile(accA);
+      mfma_tile(tile_at(k + 2), accA);
+      search_tile(accB);
       // issue order of the pass: one MFMA, then the vector and LDS work that fits in its shadow
 #pragma unroll
       for (int q = 0; q < 16 * EM_MT; ++q) {
@@ -453,15 +462,15 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
       }
     }
-    mfma_tile(7, accB);
-    search_tile(6, accA);
+    mfma_tile(tile_at(7), accB);
+    search_tile(accA);
 #pragma unroll
     for (int q = 0; q < 8 * EM_MT; ++q) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    search_tile(7, accB);
+    search_tile(accB);
     // ---- store: lane (col, g) writes group col of rows 4g + i
 #pragma unroll
     for (int mt = 0; mt < EM_MT; ++mt)
@@ -475,8 +484,8 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           prow = a.packed + n * (uint32_t)a.ps0;
         } else {
           const int64_t dp = dst_p[row];
-          if (dp < 0) continue;
-          prow = a.packed + dp;
+          if (dp == 0) continue;
+          prow = (uint8_t*)(uintptr_t)dp;
         }
         uint32_t v = packed[mt][i];
         if (!(rv[mt][i] == rv[mt][i])) v = 0xffffffffu;     // NaN vector: last level everywhere
@@ -513,11 +522,12 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
                         const void* rot_prep, hipStream_t stream) {
   if (em_disabled() || d != 128 || (x_dtype != AKV_F16 && x_dtype != AKV_BF16)) return AKV_ERR_UNSUPPORTED;
   // 16-byte loads of the input rows; aligned stores of the packed groups
-  if (((uintptr_t)a.x & 15) || (a.xs0 & 7) || (paged && (a.xs1 & 7))) return AKV_ERR_UNSUPPORTED;
+  if (((uintptr_t)a.x & 15) || ((uintptr_t)a.x2 & 15) || (a.xs0 & 7) || (paged && (a.xs1 & 7))) return AKV_ERR_UNSUPPORTED;
   const int64_t amask = bits == 4 ? 3 : bits == 2 ? 1 : 0;
-  if (((uintptr_t)a.packed | (uintptr_t)a.ps0 | (uintptr_t)a.ps1 | (uintptr_t)a.ps2) & amask) return AKV_ERR_UNSUPPORTED;
+  if (((uintptr_t)a.packed | (uintptr_t)a.packed2 | (uintptr_t)a.ps0 | (uintptr_t)a.ps1 | (uintptr_t)a.ps2) & amask) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const float*)rot_prep + (size_t)2 * d * d);
-  const int64_t steps = (a.n + EM_ROWS - 1) / EM_ROWS;
+  const int64_t n_total = (paged && a.x2) ? 2 * a.n : a.n;
+  const int64_t steps = (n_total + EM_ROWS - 1) / EM_ROWS;
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());

@@ -69,13 +69,52 @@ def fused_tq4_kv_update(x, slot_mapping, out_packed, out_norms, rotation, bounda
                     block_size=block_size, max_blocks=max_blocks)
 
 
+def fused_kv_update_pair(key, value, slot_mapping, k_packed, k_norms, v_packed, v_norms, rotation,
+                         boundaries, bits, block_size=16, max_blocks=0, prepared=None) -> None:
+    """K and V of one step ([num_tokens, num_kv_heads, head_dim] each) into their caches with ONE
+    kernel launch when the two tensors and the two caches have the same dtype, shapes and strides
+    (key / value of a layer and the halves of a serving cache tensor do); two launches otherwise.
+    Results equal two fused_kv_update calls."""
+    same = (key.shape == value.shape and key.dtype == value.dtype and key.stride() == value.stride()
+            and key.stride(-1) == 1 and key.dtype in (torch.float16, torch.bfloat16, torch.float32)
+            and k_packed.shape == v_packed.shape and k_packed.stride() == v_packed.stride()
+            and k_norms.shape == v_norms.shape and k_norms.stride() == v_norms.stride())
+    if not same:
+        for x, packed, norms in ((key, k_packed, k_norms), (value, v_packed, v_norms)):
+            fused_kv_update(x, slot_mapping, packed, norms, rotation, boundaries, bits,
+                            block_size=block_size, max_blocks=max_blocks, prepared=prepared)
+        return
+    if max_blocks == 0:
+        max_blocks = k_packed.shape[0]
+    num_tokens, num_kv_heads, head_dim = key.shape
+    if num_tokens == 0:
+        return
+    if head_dim <= 0 or (head_dim & (head_dim - 1)) != 0:
+        raise ValueError(f"head_dim must be a power of 2, got {head_dim}")
+    dev = _lib.require_gpu(key, value, slot_mapping, k_packed, v_packed, k_norms, v_norms, rotation, boundaries)
+    if k_packed.dtype != torch.uint8 or v_packed.dtype != torch.uint8 \
+            or k_norms.dtype != torch.float32 or v_norms.dtype != torch.float32:
+        raise ValueError("packed caches must be uint8 and norms float32")
+    if k_packed.shape[-1] < packed_size(head_dim, bits) or k_packed.stride(-1) != 1:
+        raise ValueError("packed rows are too short or not contiguous in the last dim")
+    slots = slot_mapping if slot_mapping.is_contiguous() else slot_mapping.contiguous()
+    prep = prepared if prepared is not None else prepared_rotation_for(rotation)
+    bnd = boundaries if (boundaries.dtype == torch.float32 and boundaries.is_contiguous()) \
+        else boundaries.float().contiguous()
+    _lib.check(_lib.lib().akv_encode_paged_kv(
+        key.data_ptr(), value.data_ptr(), _lib.dtype_code(key), num_tokens, num_kv_heads, head_dim,
+        key.stride(0), key.stride(1), slots.data_ptr(), _lib.itype_code(slots), prep.ptr, bnd.data_ptr(), bits,
+        k_packed.data_ptr(), v_packed.data_ptr(), k_packed.stride(0), k_packed.stride(1), k_packed.stride(2),
+        k_norms.data_ptr(), v_norms.data_ptr(), k_norms.stride(0), k_norms.stride(1), k_norms.stride(2),
+        block_size, max_blocks, _lib.stream_ptr(dev)))
+
+
 def fused_encode_and_store(tq_cache, layer_idx: int, key, value, slot_mapping) -> None:
-    """K then V for one layer into a cache object with attributes tq, k_packed, k_norms,
+    """K and V for one layer into a cache object with attributes tq, k_packed, k_norms,
     v_packed, v_norms, block_size, max_blocks (reference: fused_kv_update.py:412-468)."""
     tq = tq_cache.tq
     prep = tq.prepared_rotation() if hasattr(tq, "prepared_rotation") else None
-    for x, packed, norms in ((key, tq_cache.k_packed, tq_cache.k_norms),
-                             (value, tq_cache.v_packed, tq_cache.v_norms)):
-        fused_kv_update(x, slot_mapping, packed[layer_idx], norms[layer_idx], tq.rotation,
-                        tq.boundaries_inner, tq.bits, block_size=tq_cache.block_size,
-                        max_blocks=tq_cache.max_blocks, prepared=prep)
+    fused_kv_update_pair(key, value, slot_mapping, tq_cache.k_packed[layer_idx], tq_cache.k_norms[layer_idx],
+                         tq_cache.v_packed[layer_idx], tq_cache.v_norms[layer_idx], tq.rotation,
+                         tq.boundaries_inner, tq.bits, block_size=tq_cache.block_size,
+                         max_blocks=tq_cache.max_blocks, prepared=prep)

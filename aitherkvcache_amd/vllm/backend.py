@@ -185,7 +185,7 @@ def _make_impl_class():
         base = _StandaloneImplBase
 
     from ..fused_attention import TQPagedAttention
-    from ..fused_kv_update import fused_encode_and_store, fused_kv_update
+    from ..fused_kv_update import fused_encode_and_store, fused_kv_update_pair
     from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store
     from . import hooks
     from .cache import TQGPUCache
@@ -303,9 +303,9 @@ def _make_impl_class():
             self._ensure_norms(kv_cache)
             li = self._tq_layer_idx
             prep = tq.prepared_rotation()
-            for x, rows, norms in ((key, k_rows, cls._primary_k_norms[li]), (value, v_rows, cls._primary_v_norms[li])):
-                fused_kv_update(x, slot_mapping, rows, norms, tq.rotation, tq.boundaries_inner, tq.bits,
-                                block_size=block_size, prepared=prep)
+            fused_kv_update_pair(key, value, slot_mapping, k_rows, cls._primary_k_norms[li], v_rows,
+                                 cls._primary_v_norms[li], tq.rotation, tq.boundaries_inner, tq.bits,
+                                 block_size=block_size, prepared=prep)
 
         # ---- attention --------------------------------------------------------------------
         def forward(self, layer, query, key, value, kv_cache, attn_metadata, output=None,

@@ -2,7 +2,7 @@
 reference's aither_kvcache/vllm/hooks.py:129-213 (tq::decode_step) and :240-363
 (tq::hybrid_decode_step): encode the step's new K/V tokens into the paged cache, then attend.
 
-Each op is two C-ABI calls for the write (K, V) and one for the attention; nothing in the body
+Each op is one C-ABI call for the write (K and V in one launch) and one for the attention; nothing in the body
 synchronises with the host or allocates after the first call for a given batch shape, so the
 ops can be recorded into a HIP graph after a warm-up call.
 
@@ -17,7 +17,7 @@ from typing import Dict, Optional
 import torch
 
 from ..fused_attention import TQPagedAttention
-from ..fused_kv_update import fused_kv_update
+from ..fused_kv_update import fused_kv_update_pair
 from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store
 from ..hybrid_quantizer import HybridTurboQuant
 from ..quantizer import TurboQuant
@@ -60,10 +60,9 @@ def decode_step(query, key, value, kv_cache, output, k_norms, v_norms, slot_mapp
     block_size = key_cache.shape[1]
     n = key.shape[0]
     prep = tq.prepared_rotation()
-    fused_kv_update(key, slot_mapping[:n], key_cache, k_norms[layer_idx], tq.rotation,
-                    tq.boundaries_inner, tq.bits, block_size=block_size, prepared=prep)
-    fused_kv_update(value, slot_mapping[:n], value_cache, v_norms[layer_idx], tq.rotation,
-                    tq.boundaries_inner, tq.bits, block_size=block_size, prepared=prep)
+    fused_kv_update_pair(key, value, slot_mapping[:n], key_cache, k_norms[layer_idx], value_cache,
+                         v_norms[layer_idx], tq.rotation, tq.boundaries_inner, tq.bits,
+                         block_size=block_size, prepared=prep)
     attn = _tq_fused_attn.get((layer_idx, head_size))
     if attn is None:
         attn = TQPagedAttention(tq, num_heads)

@@ -115,6 +115,23 @@ int akv_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_
                      int block_size, int64_t max_blocks, void* stream);
 
 /* ---------------------------------------------------------------------------------
+ * K and V of one serving step in ONE launch -- what fused_encode_and_store does with two
+ * calls, aither_kvcache/fused_kv_update.py:412-468.  k and v are [num_tokens][num_kv_heads][d]
+ * with the same strides and dtype; the two caches and the two norm tensors share their
+ * strides as well (the K and V halves of one serving cache tensor do); one slot_mapping.
+ * Same results as two akv_encode_paged calls.
+ * ------------------------------------------------------------------------------- */
+int akv_encode_paged_kv(const void* k, const void* v, int x_dtype, int64_t num_tokens,
+                        int num_kv_heads, int d, int64_t xs_token, int64_t xs_head,
+                        const void* slot_mapping, int slot_itype,
+                        const void* rot_prep, const float* boundaries, int bits,
+                        uint8_t* k_packed, uint8_t* v_packed,
+                        int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                        float* k_norms, float* v_norms,
+                        int64_t ns_blk, int64_t ns_pos, int64_t ns_head,
+                        int block_size, int64_t max_blocks, void* stream);
+
+/* ---------------------------------------------------------------------------------
  * TurboQuant.decode -- aither_kvcache/quantizer.py:168-197:
  * out[i] = (centroids[codes_i] @ Pi) * norms[i], cast to out_dtype.
  * ------------------------------------------------------------------------------- */

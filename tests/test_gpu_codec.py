@@ -216,6 +216,33 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tokens", [1, 37, 256])
+def test_k_and_v_in_one_launch_equal_two_launches(golden, dev, bits, dtype, tokens):
+    """fused_kv_update_pair against two fused_kv_update calls (those are checked against the oracle
+    above): byte-identical caches and norms.  Token counts that leave the K / V seam inside a step of the
+    kernel, padding slots, slots beyond max_blocks, and the K / V halves of one serving cache tensor
+    (rows 4 bytes longer than the codes).  float32 input takes two launches inside the pair call."""
+    tq = make_tq(golden, dev, bits)
+    H, NB, BS, P = 8, 40, 16, tq._packed_dim
+    g = torch.Generator(device=dev).manual_seed(1000 * bits + tokens)
+    k = (torch.randn(tokens, H, 128, device=dev, generator=g) * 3).to(dtype)
+    v = torch.randn(tokens, H, 128, device=dev, generator=g).to(dtype)
+    slots = torch.randperm(NB * BS + 64, device=dev, generator=g)[:tokens] - 32        # some negative, some too large
+    kv_a = torch.zeros(NB, 2, BS, H, P + 4, dtype=torch.uint8, device=dev)
+    kv_b = torch.zeros_like(kv_a)
+    norms_a = torch.zeros(2, NB, BS, H, device=dev)
+    norms_b = torch.zeros_like(norms_a)
+    akv.fused_kv_update_pair(k, v, slots, kv_a[:, 0], norms_a[0], kv_a[:, 1], norms_a[1], tq.rotation,
+                             tq.boundaries_inner, bits, block_size=BS, max_blocks=NB - 1)
+    akv.fused_kv_update(k, slots, kv_b[:, 0], norms_b[0], tq.rotation, tq.boundaries_inner, bits, BS, NB - 1)
+    akv.fused_kv_update(v, slots, kv_b[:, 1], norms_b[1], tq.rotation, tq.boundaries_inner, bits, BS, NB - 1)
+    assert torch.equal(kv_a, kv_b) and torch.equal(norms_a, norms_b)
+    ok = (slots >= 0) & (slots < (NB - 1) * BS)
+    assert int((norms_a[0] > 0).sum()) == int(ok.sum()) * H and torch.all(kv_a[..., P:] == 0)
+
+
 def test_config1_literal_shape_steps_vs_oracle(golden, dev):
     """The serving write at its benchmark shape: 8 kv heads, a cache of 8,192 blocks of 16, steps of 256
     tokens (K and V) whose slots are consecutive runs of ONE random permutation of all 131,072 slots, so
