@@ -330,6 +330,12 @@ template <int ROLE, int BITS>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
+  // One workgroup barrier per chunk keeps the wavefronts of the eight heads on the same tokens.  The code
+  // rows of neighbouring heads share 64-byte memory sectors when a row is narrower than a sector (48 bytes
+  // at 3 bits): left to drift a few chunks apart, the heads fetch 40 % of those sectors from memory twice;
+  // in step they fetch 4 % more than the algorithmic bytes.  At 4 bits the barrier is worth 2 % of the
+  // kernel time, at 2 bits (short chunks, the barrier's own cost dominates) it costs 20 % and stays out.
+  constexpr bool SYNC = BITS != 2;
   const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * 4u;   // V lookups: first halves of table B entries
   const uint32_t lane4k = (uint32_t)(lane & 31) * 8u;             // K lookups: table A
   // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
@@ -373,7 +379,12 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       // here leaves ONE path into the chunk loops: were the first loads conditional, the compiler would
       // have to assume that the loads issued before them are the newest outstanding ones and would wait
       // for ALL loads, prefetches included, wherever the loop first touches their registers.)
-      if (!active || nchunks <= 0) continue;
+      if (nchunks <= 0) continue;
+      if (!active) {
+        if constexpr (SYNC)
+          for (int i = 0; i <= nchunks; ++i) mf_barrier();     // the workgroup's barriers are counted by all
+        continue;
+      }
       const int hh = h;
       const int hd = a.hgroup > 1 ? h / a.hgroup : h;      // the head whose rows are read
 
@@ -552,10 +563,16 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         int c = 0;
         for (; c + 1 < nchunks; c += 2) {
           if (c - win_c0 >= MF_WIN) load_window(c);
+          if constexpr (SYNC) mf_barrier();
           produce(ra, c, 0);
+          if constexpr (SYNC) mf_barrier();
           produce(rb, c + 1, 1);
         }
-        if (c < nchunks) produce(ra, c, 0);      // odd tail, already in ra
+        if (c < nchunks) {
+          if constexpr (SYNC) mf_barrier();
+          produce(ra, c, 0);      // odd tail, already in ra
+        }
+        if constexpr (SYNC) mf_barrier();
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
         T += (uint32_t)nchunks;
         float lsum = l_run;
@@ -654,8 +671,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
         mf_vraw ra;
         load_chunk(ra, 0);
+        if constexpr (SYNC) mf_barrier();
         for (int c = 0; c < nchunks; ++c) {
           if (c - win_c0 >= MF_WIN) load_window(c);
+          if constexpr (SYNC) mf_barrier();
           step(ra, c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
