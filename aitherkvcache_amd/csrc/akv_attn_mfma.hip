@@ -287,7 +287,8 @@ __device__ __forceinline__ float mf_rows_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// Pairwise hand-off between the score and the value wavefront of a head slot: two counters in LDS,
+// Pairwise hand-off between the score and the value wavefront of a head slot (tq35 kernel; the kernel
+// for the uniform formats orders its chunks with workgroup barriers instead): two counters in LDS,
 // `ready` (chunks whose weights are written) and `done` (chunks whose weights have been read), both
 // counted from the start of the kernel.  LDS operations of a wavefront are executed in order, so a
 // counter written after the data is seen after the data.  Waiting polls the counter with a short
@@ -330,12 +331,15 @@ template <int ROLE, int BITS>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
-  // One workgroup barrier per chunk keeps the wavefronts of the eight heads on the same tokens.  The code
-  // rows of neighbouring heads share 64-byte memory sectors when a row is narrower than a sector (48 bytes
-  // at 3 bits): left to drift a few chunks apart, the heads fetch 40 % of those sectors from memory twice;
-  // in step they fetch 4 % more than the algorithmic bytes.  At 4 bits the barrier is worth 2 % of the
-  // kernel time, at 2 bits (short chunks, the barrier's own cost dominates) it costs 20 % and stays out.
-  constexpr bool SYNC = BITS != 2;
+  // One workgroup barrier per chunk orders everything: in interval k the score wavefronts produce the
+  // weights of chunk k into exchange buffer k % 2 while the value wavefronts, one interval behind, consume
+  // chunk k - 1 from the other buffer.  The barrier also keeps the wavefronts of the eight heads on the
+  // same tokens: the code rows of neighbouring heads share 64-byte memory sectors when a row is narrower
+  // than a sector (48 bytes at 3 bits), and heads left to drift a few chunks apart fetch 40 % of those
+  // sectors from memory twice; in step the kernel fetches 4 % more than the algorithmic bytes.  (Per-head
+  // flag hand-offs through LDS instead of the barrier, polled by the waiting side, were 5 % slower at
+  // 4 bits: every poll is an LDS round trip on the critical path of its wavefront.)
+  constexpr bool SYNC = true;
   const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * 4u;   // V lookups: first halves of table B entries
   const uint32_t lane4k = (uint32_t)(lane & 31) * 8u;             // K lookups: table A
   // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
@@ -346,8 +350,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   const uint32_t pb_addr = MF_TABB + (32u * hs + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
   const uint32_t rs_addr = MF_TABB + (32u * hs + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
 
-  const uint32_t fl_addr = MF_TABB + (32u * hs + 12u) * 256u + 128u;   // ready at +0, done at +4
-  uint32_t T = 0;        // chunks of this head slot finished in earlier segments (same on both sides)
 
   const int G = gridDim.x;
   // blocks of 16 tokens: a chunk (32 tokens, two 16-token tiles) is two blocks; blocks of 32: one
@@ -545,11 +547,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           l_run = l_run * resc + psum;
           const float resc_left = mf_from_lo_cols(resc);
           const float resc_out = col < 8 ? resc : resc_left;
-          // the buffer was last read for chunk c - 2 (or, for the first two chunks, in the previous segment)
-          mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T, x.status, x.spin_limit);
+          // the buffer was last read for chunk c - 2, two barriers ago
           *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + MF_XBUF * par) = __float_as_uint(resc_out);
-          mf_publish(fl_addr, T + (uint32_t)c + 1u);
         };
 
         mf_kraw ra, rb;
@@ -574,7 +574,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         }
         if constexpr (SYNC) mf_barrier();
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
-        T += (uint32_t)nchunks;
         float lsum = l_run;
         lsum = mf_rows_sum(lsum);
         if (active && col < gqa && g == 0) {
@@ -649,7 +648,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           union { half8 h; mf_u32x4 u; } cv;
           cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par);
           const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + MF_XBUF * par));
-          mf_publish(fl_addr + 4u, T + (uint32_t)c + 1u);     // queued behind the two reads
           if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -666,7 +664,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 
         auto step = [&](mf_vraw& r, int c, const uint32_t par) {
           regroup(r, c);
-          mf_wait_ge(fl_addr, T + (uint32_t)c + 1u, x.status, x.spin_limit);
           consume(c, par);
         };
         mf_vraw ra;
@@ -678,7 +675,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           step(ra, c, (uint32_t)(c & 1));
         }
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
-        T += (uint32_t)nchunks;
         // columns [0,8) + [8,16); lane (col < gqa, g) holds coordinates 32g + 8i + (coordinate of M-tile j)
         const float inv_alpha = 1.f / __uint_as_float(x.lut[MF_W_ALPHA]);
 #pragma unroll

@@ -357,3 +357,31 @@ def test_one_object_across_batch_sizes(golden, dev):
         err = np.max(np.abs(out.cpu().numpy().astype(np.float64) - ref))
         assert err <= 3e-4, f"batch size {S}: {err:.2e}"
         assert attn.last_call_status() == 0
+
+
+def test_handoff_timeout_is_reported(golden, dev):
+    """The tq35 kernel hands chunks from its score to its value wavefronts through polled counters with a
+    bounded wait.  With a limit of zero polls every wait gives up at once (the kernels still run to their
+    end): outputs are NaN and the status query says so; with the default limit the next call is clean."""
+    from aitherkvcache_amd import _lib
+    h = akv.HybridTurboQuant(device=str(dev))
+    h.calibrate_uniform(num_kv_heads=8)
+    hp = params(golden)
+    rng = np.random.default_rng(91)
+    NB = 40
+    kc, vc, _, _ = build_cache(rng, h, dev, NB, 8)
+    ctx = np.array([300, 64], dtype=np.int64)
+    tables = np.stack([rng.permutation(NB)[:20] for _ in range(2)]).astype(np.int64)
+    q = rng.standard_normal((2, 32, 128)).astype(np.float16)
+    attn = akv.HybridPagedAttention(h, 32)
+    args = (t(q, dev), kc, vc, t(tables, dev), t(ctx, dev))
+    try:
+        _lib.check(_lib.lib().akv_debug_set_handoff_spin_limit(0))
+        bad = attn.forward(*args, scale=0.09)
+        assert attn.last_call_status() & 1 and bool(torch.isnan(bad).all())
+    finally:
+        _lib.check(_lib.lib().akv_debug_set_handoff_spin_limit(-1))
+    good = attn.forward(*args, scale=0.09)
+    assert attn.last_call_status() == 0
+    ref = O.hybrid_paged_attention(q, kc.cpu().numpy(), vc.cpu().numpy(), tables, ctx, hp, 0.09, dtype=np.float64)
+    assert np.max(np.abs(good.cpu().numpy().astype(np.float64) - ref)) <= 2e-3
