@@ -797,11 +797,9 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
     AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
     configured = true;
   }
-  akv_profile_mark_begin(stream);
-  if (bits == 4) akv_attn_mfma_kernel<4><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
-  else if (bits == 3) akv_attn_mfma_kernel<3><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
-  else akv_attn_mfma_kernel<2><<<grid, MF_THREADS, MF_LDS_BYTES, stream>>>(a, x);
-  akv_profile_mark_end(stream);
+  if (bits == 4) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<4>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
+  else if (bits == 3) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<3>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
+  else AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<2>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
   AKV_LAUNCH_CHECK("akv_attn_mfma_kernel");
   return AKV_OK;
 }
@@ -1452,9 +1450,7 @@ int akv_hyb_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_
     AKV_HIP(hipFuncSetAttribute((const void*)akv_hyb_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HM_LDS_BYTES));
     configured = true;
   }
-  akv_profile_mark_begin(stream);
-  akv_hyb_mfma_kernel<<<grid, HM_THREADS, HM_LDS_BYTES, stream>>>(a);
-  akv_profile_mark_end(stream);
+  AKV_LAUNCH_TIMED(akv_hyb_mfma_kernel, grid, HM_THREADS, HM_LDS_BYTES, stream, a);
   AKV_LAUNCH_CHECK("akv_hyb_mfma_kernel");
   return AKV_OK;
 }

@@ -876,9 +876,8 @@ int akv_attn_stream_run(const void* query, int q_dtype, int64_t qs_seq, int64_t 
     AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS_BYTES));
     configured = true;
   }
-  akv_profile_mark_begin(stream);
-  akv_attn_stream_kernel<<<grid, SK_THREADS, SK_LDS_BYTES, stream>>>(a, x, ws.prefix, a.block_tables, a.context_lens, ws.wgdesc);
-  akv_profile_mark_end(stream);
+  AKV_LAUNCH_TIMED(akv_attn_stream_kernel, grid, SK_THREADS, SK_LDS_BYTES, stream, a, x, ws.prefix, a.block_tables,
+                   a.context_lens, ws.wgdesc);
   AKV_LAUNCH_CHECK("akv_attn_stream_kernel");
   return AKV_OK;
 }

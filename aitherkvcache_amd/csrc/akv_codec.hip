@@ -45,6 +45,20 @@ void akv_profile_mark_end(hipStream_t s) {
   ++g_ev_count;
 }
 
+bool akv_profile_take(hipEvent_t* begin, hipEvent_t* end) {
+  if (!g_profile_on) return false;
+  *begin = g_ev_begin[g_ev_count % kProfRing];
+  *end = g_ev_end[g_ev_count % kProfRing];
+  g_ev_open = false;
+  ++g_ev_count;
+  return true;
+}
+
+__global__ void akv_stamp_kernel() {}
+void akv_profile_stamp(hipStream_t s, hipEvent_t begin) {
+  hipExtLaunchKernelGGL(akv_stamp_kernel, dim3(1), dim3(1), 0, s, nullptr, begin, 0);
+}
+
 extern "C" int akv_profile_enable(int on) {
   if (on && !g_ev_created) {
     for (int i = 0; i < kProfRing; ++i) {

@@ -296,8 +296,7 @@ int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int
                                   hipFuncAttributeMaxDynamicSharedMemorySize, DM_LDS_BYTES));                \
       configured = true;                                                                                     \
     }                                                                                                        \
-    akv_profile_mark_begin(stream);                                                                          \
-    akv_decode_mfma_kernel<BL, BB, OD><<<grid, DM_THREADS, DM_LDS_BYTES, stream>>>(a, bop);                  \
+    AKV_LAUNCH_TIMED((akv_decode_mfma_kernel<BL, BB, OD>), grid, DM_THREADS, DM_LDS_BYTES, stream, a, bop);  \
   } while (0)
 #define DM_GO_DT(BL, BB)                                                                                       \
   do {                                                                                                       \
@@ -309,7 +308,6 @@ int akv_decode_mfma_try(const akv_gen_args& a, bool blocks, int d, int bits, int
   else { if (bits == 4) DM_GO_DT(false, 4); else if (bits == 3) DM_GO_DT(false, 3); else DM_GO_DT(false, 2); }
 #undef DM_GO_DT
 #undef DM_GO
-  akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_decode_mfma_kernel");
   return AKV_OK;
 }

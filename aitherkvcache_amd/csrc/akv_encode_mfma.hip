@@ -539,9 +539,7 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
                                   hipFuncAttributeMaxDynamicSharedMemorySize, EM_LDS_BYTES));        \
       configured = true;                                                                             \
     }                                                                                                \
-    akv_profile_mark_begin(stream);                                                                  \
-    akv_encode_mfma_kernel<BB, PG, DT, DR><<<grid, EM_THREADS, EM_LDS_BYTES, stream>>>(a, bop);      \
-    akv_profile_mark_end(stream);                                                                    \
+    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, DR>), grid, EM_THREADS, EM_LDS_BYTES, stream, a, bop); \
   } while (0)
 #define EM_LAUNCH_DT(BB, PG, DR) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16, DR); else EM_LAUNCH(BB, PG, AKV_BF16, DR); } while (0)
   // flat rows whose byte offsets stay below 2^31 take the variant with 32-bit lane offsets

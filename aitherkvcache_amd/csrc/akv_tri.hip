@@ -760,10 +760,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
         configured = lds;
       }
       dim3 hgrid(a.nsplit, batch);
-      akv_profile_mark_begin(stream);
-      if (gq == 4) tri_decode_heads_kernel<4, false><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
-      else tri_decode_heads_kernel<1, false><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
-      akv_profile_mark_end(stream);
+      if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, false>), hgrid, num_kv_heads * 64, lds, stream, a);
+      else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, false>), hgrid, num_kv_heads * 64, lds, stream, a);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
       AKV_LAUNCH_CHECK("tri_reduce_kernel");
@@ -866,10 +864,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
     configured = lds;
   }
   dim3 hgrid(a.nsplit, batch);
-  akv_profile_mark_begin(stream);
-  if (gq == 4) tri_decode_heads_kernel<4, true><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
-  else tri_decode_heads_kernel<1, true><<<hgrid, num_kv_heads * 64, lds, stream>>>(a);
-  akv_profile_mark_end(stream);
+  if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, true>), hgrid, num_kv_heads * 64, lds, stream, a);
+  else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, true>), hgrid, num_kv_heads * 64, lds, stream, a);
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");

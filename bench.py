@@ -59,6 +59,8 @@ def parse():
     ap.add_argument("--workload", default="decode4",
                     choices=["decode4", "decode3", "decode2", "tq35", "tri", "encode"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the encode size sweep (a profiler run then sees the encode kernel at 2**20 vectors only)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (a dispatch of known traffic, to scale "
@@ -126,7 +128,7 @@ def kernel_ms(torch, L, fn, steps):
 
 
 # ---------------------------------------------------------------------------------------------
-def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds):
+def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds, sweep=True):
     tq = akv.TurboQuant(head_dim=128, bits=4, device=str(dev))
     gen = torch.Generator(device=dev).manual_seed(1)
     res = {}
@@ -177,7 +179,8 @@ def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds):
     res["decode_mvec_s"] = n / dms / 1e3
     res["decode_gbs"] = n * 324 / dms / 1e6
     del coded, xs
-    res["sweep"], res["vectors_at_60pct_hbm"] = encode_sweep(torch, akv, L, tq, dev, gen)
+    if sweep:
+        res["sweep"], res["vectors_at_60pct_hbm"] = encode_sweep(torch, akv, L, tq, dev, gen)
     if cpu:
         from oracle import tq_oracle as O
         R = tq.rotation.cpu().numpy()
@@ -336,7 +339,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    enc, tq4 = bench_encode(torch, akv, L, dev, args.steps, args.warmup, cpu, args.cpu_seconds)
+    enc, tq4 = bench_encode(torch, akv, L, dev, args.steps, args.warmup, cpu, args.cpu_seconds, sweep=not args.no_sweep)
     out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "data": "synthetic", "unit": "GB/s"}
     cpu_obj = None

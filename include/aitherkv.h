@@ -52,8 +52,10 @@ int akv_device_cu_count(int* cu_count);
 
 /* ---------------------------------------------------------------------------------
  * Measurement hook (no counterpart in the reference).  While enabled, every entry point
- * brackets its dominant kernel (the main decode-attention kernel, the encode kernel, the
- * TriAttention scoring kernel) with a pair of HIP events recorded on the launch stream.
+ * times its dominant kernel (the main decode-attention kernel, the encode kernel, the
+ * TriAttention scoring kernel) with a pair of HIP events on the launch stream: the matrix-core
+ * kernels are launched with the pair attached to the dispatch (its own start and end time
+ * stamps, as a kernel trace reports them), the others are bracketed by two recorded events.
  * The pairs go into a ring of 64, and nothing is read back between calls, so sampled calls
  * run back to back.  akv_profile_last_ms waits for the pair of the most recent call and
  * returns its elapsed time in milliseconds; akv_profile_mean_ms waits for the most recent
