@@ -81,12 +81,12 @@ SIGNATURES = {
     "akv_block_rep_finalize": (_i, [_p, _i, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "akv_block_scores": (_i, [_p, _p, _p, _p, _p, _i, _i64, _p, _i, _i, _i, _i, _i, _i64, _i, _i64, _p, _p]),
     "akv_block_select": (_i, [_p, _p, _i, _i64, _p, _i, _i, _i64, _i, _i, _i, _i, _p, _p, _p]),
-    "akv_tri_encode": (_i, [_p, _i, _i64, _i, _i64, _i, _p, _p, _p, _p]),
+    "akv_tri_encode": (_i, [_p, _i, _i64, _i, _i64, _i, _i, _p, _p, _p, _p]),
     "akv_tri_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "akv_tri_decode_step": (_i, [_p, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i,
-                                 _p, _i, _i64, _i, _i, _i, _i, _p, _sz, _p]),
+                                 _p, _i, _i64, _i, _i, _i, _i, _i, _i, _p, _sz, _p]),
     "akv_tri_decode_paged": (_i, [_p, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i64, _p, _i,
-                                  _p, _i, _i64, _i, _i64, _i, _i, _i, _i, _p, _sz, _p]),
+                                  _p, _i, _i64, _i, _i64, _i, _i, _i, _i, _i, _p, _sz, _p]),
 }
 
 _lib: Optional[C.CDLL] = None

@@ -1,5 +1,8 @@
 // TriAttention decode_step (aither_kvcache/triattention/attention.py:186-280 with
-// TrigSeriesScorer.score, scorer.py:115-208), int4 coefficients.
+// TrigSeriesScorer.score, scorer.py:115-208).  Coefficients: int4 nibble pairs (the reference's default and the
+// only width its paged cache stores), or -- in the general kernel only -- uint8 pairs / float16 pairs
+// (scorer.py:84-113).  Post-RoPE scoring (scorer.py:200-202) is the same series at a position difference
+// of zero: cos 0 = 1 and sin 0 = 0 exactly, which leaves sum_f c_f.
 //
 // Per (batch, kv head) the S cached tokens are cut into NSPLIT contiguous ranges, one
 // wavefront each.  Lanes <-> tokens: a lane unpacks its token's F retained pairs, forms
@@ -43,6 +46,8 @@ struct tri_args {
   const void* qpos; int qp_itype;
   const void* kpos; int kp_itype;
   int B; int64_t S; int QH, KVH, D, F;
+  int cbits;       // coefficient width: 4 (a byte per pair), 8 (two bytes per pair), 16 (two float16 per pair, scales unused)
+  int post_rope;   // keys were stored after RoPE: plain sparse dot product, positions unused
   int nsplit;
   // paged cache (arrays are [num_blocks][block_size][KVH][...]; S = max_blocks_per_seq * block_size)
   const void* block_tables; int bt_itype; int64_t bt_stride;
@@ -71,13 +76,16 @@ __device__ __forceinline__ void tri_sincos(float x, float& sn, float& cs) {
   cs = __builtin_amdgcn_cosf(f);
 }
 
-template <int GQ, bool F12, bool DENSE>
+// WIDE: the coefficient width is a.cbits (4, 8 or 16) instead of 4; only without F12
+template <int GQ, bool F12, bool DENSE, bool WIDE>
 __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
+  static_assert(!(F12 && WIDE), "rows of three dwords are the 4-bit layout");
   extern __shared__ __align__(16) unsigned char lds_raw[];
+  constexpr int DQN = WIDE ? 256 : 16;
   float* theta = (float*)lds_raw;                         // [D/2]
   float* q_lds = theta + a.D / 2;                         // [GQ][D]   (per workgroup pass)
-  float* dq = q_lds + GQ * a.D;                           // [16]: code / 7.5 - 1 with the reference's roundings
-  float* acc_base = dq + 16;                              // [TRI_WAVES][GQ][D]
+  float* dq = q_lds + GQ * a.D;                           // [DQN]: code / half - 1 with the reference's roundings
+  float* acc_base = dq + DQN;                             // [TRI_WAVES][GQ][D]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* acc = acc_base + (size_t)wave * GQ * a.D;
   // DENSE (head_dim 128): instead of bins updated by LDS atomics (which serialise when many tokens
@@ -103,7 +111,10 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
   const float inv_sqrt_d = 1.0f / sqrtf((float)D);
 
   for (int i = threadIdx.x; i < D / 2; i += 256) theta[i] = a.theta[i];
-  if (threadIdx.x < 16) dq[threadIdx.x] = __fsub_rn(__fdiv_rn((float)threadIdx.x, 7.5f), 1.0f);
+  const int cb = WIDE ? a.cbits : 4;
+  if ((int)threadIdx.x < DQN) dq[threadIdx.x] = __fsub_rn(__fdiv_rn((float)threadIdx.x, cb == 8 ? 127.5f : 7.5f), 1.0f);
+  // DENSE: the value tile holds 2 code - (15 | 255) or the float16 values themselves
+  const float vfac = cb == 4 ? 1.f / (15.f * TRI_WSCALE) : cb == 8 ? 1.f / (255.f * TRI_WSCALE) : 1.f / TRI_WSCALE;
 
   const int64_t per = (a.S + a.nsplit - 1) / a.nsplit;
   const int64_t s0 = min(a.S, (int64_t)split * per);
@@ -150,8 +161,11 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       const int64_t pe = a.kpos ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
       r.kp_lo = *(const uint32_t*)(kp_base + pe);
       r.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
-      r.ksc = ((const unsigned short*)a.k_sc)[row];
-      r.vsc = ((const unsigned short*)a.v_sc)[row];
+      r.ksc = r.vsc = 0x3c00;                       // float16 pairs carry no scale: 1.0
+      if (!WIDE || cb != 16) {
+        r.ksc = ((const unsigned short*)a.k_sc)[row];
+        r.vsc = ((const unsigned short*)a.v_sc)[row];
+      }
       if (F12) {
         const uint32_t* p0 = (const uint32_t*)(a.k_idx + row * 12);
         const uint32_t* p1 = (const uint32_t*)(a.k_cf + row * 12);
@@ -172,7 +186,7 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
       fetch(nxt, c0 + 64);
       const float kp = !a.kpos ? (float)tc
                        : kp_wide ? (float)(int64_t)(((uint64_t)cur.kp_hi << 32) | cur.kp_lo) : (float)(int32_t)cur.kp_lo;
-      const float delta = __fsub_rn(kp, qp);
+      const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
       const float ksc = __half2float(__ushort_as_half(cur.ksc));
       float sc[GQ];
 #pragma unroll
@@ -180,8 +194,17 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 #pragma unroll FU
       for (int f = 0; f < (F12 ? 12 : F); ++f) {
         const uint32_t idx = F12 ? (cur.ki[f >> 2] >> (8 * (f & 3))) & 255u : a.k_idx[row * F + f];
-        const uint32_t cf = F12 ? (cur.kc[f >> 2] >> (8 * (f & 3))) & 255u : a.k_cf[row * F + f];
-        const float k0 = __fmul_rn(dq[cf >> 4], ksc), k1 = __fmul_rn(dq[cf & 15u], ksc);
+        float k0, k1;
+        if (!WIDE || cb == 4) {
+          const uint32_t cf = F12 ? (cur.kc[f >> 2] >> (8 * (f & 3))) & 255u : a.k_cf[row * F + f];
+          k0 = __fmul_rn(dq[cf >> 4], ksc); k1 = __fmul_rn(dq[cf & 15u], ksc);
+        } else if (cb == 8) {
+          const uint8_t* pc = a.k_cf + (row * F + f) * 2;
+          k0 = __fmul_rn(dq[pc[0]], ksc); k1 = __fmul_rn(dq[pc[1]], ksc);
+        } else {
+          const __half* pc = (const __half*)a.k_cf + (row * F + f) * 2;
+          k0 = __half2float(pc[0]); k1 = __half2float(pc[1]);
+        }
         const float ph = __fmul_rn(delta, theta[idx]);
         float sn, cs;
         tri_sincos(ph, sn, cs);
@@ -235,11 +258,19 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 #pragma unroll FU
           for (int f = 0; f < (F12 ? 12 : F); ++f) {
             const uint32_t idx = F12 ? (cur.vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
-            const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
-            // (2a - 15, 2b - 15) as a float16 pair: 0x6400 + n is float16(1024 + n), minus 1039 is exact
             union { uint32_t u; tri_half2 h; } cv;
-            cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
-            cv.h = cv.h - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+            if (!WIDE || cb == 4) {
+              const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+              // (2a - 15, 2b - 15) as a float16 pair: 0x6400 + n is float16(1024 + n), minus 1039 is exact
+              cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+              cv.h = cv.h - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+            } else if (cb == 8) {
+              const uint8_t* pc = a.v_cf + (row * F + f) * 2;   // (2a - 255, 2b - 255): integers below 2^11, exact
+              cv.h = (tri_half2){(_Float16)(float)(2 * (int)pc[0] - 255), (_Float16)(float)(2 * (int)pc[1] - 255)};
+            } else {
+              const uint16_t* pc = (const uint16_t*)a.v_cf + (row * F + f) * 2;
+              cv.u = (uint32_t)pc[0] | ((uint32_t)pc[1] << 16);
+            }
             *(uint32_t*)(vt + (idx & 63u) * TRI_VT_PITCH + 4 * lane) = cv.u;
           }
         }
@@ -285,8 +316,17 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 #pragma unroll FU
         for (int f = 0; f < (F12 ? 12 : F); ++f) {
           const uint32_t idx = F12 ? (cur.vi[f >> 2] >> (8 * (f & 3))) & 255u : a.v_idx[row * F + f];
-          const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
-          const float v0 = __fmul_rn(dq[cf >> 4], vs), v1 = __fmul_rn(dq[cf & 15u], vs);
+          float v0, v1;
+          if (!WIDE || cb == 4) {
+            const uint32_t cf = F12 ? (cur.vc[f >> 2] >> (8 * (f & 3))) & 255u : a.v_cf[row * F + f];
+            v0 = __fmul_rn(dq[cf >> 4], vs); v1 = __fmul_rn(dq[cf & 15u], vs);
+          } else if (cb == 8) {
+            const uint8_t* pc = a.v_cf + (row * F + f) * 2;
+            v0 = __fmul_rn(dq[pc[0]], vs); v1 = __fmul_rn(dq[pc[1]], vs);
+          } else {
+            const __half* pc = (const __half*)a.v_cf + (row * F + f) * 2;
+            v0 = __half2float(pc[0]); v1 = __half2float(pc[1]);
+          }
 #pragma unroll
           for (int q = 0; q < GQ; ++q) {
             atomicAdd(&acc[q * D + 2 * idx], p[q] * v0);
@@ -314,7 +354,7 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
               const float hi = oacc[mt][i];
               const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
               if (col_n < 8 && col_q == q)
-                a.part_acc[slot * D + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
+                a.part_acc[slot * D + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * vfac;
             }
         } else {
           for (int i = lane; i < D; i += 64) a.part_acc[slot * D + i] = acc[q * D + i];
@@ -492,7 +532,7 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       const bool valid = t < s1;
       const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
                        : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
-      const float delta = __fsub_rn(kp, qp);
+      const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
       const float kscale = ksc * (inv_sqrt_d / 15.f);
       float sc[GQ];
 #pragma unroll
@@ -693,18 +733,20 @@ extern "C" size_t akv_tri_decode_workspace_bytes(int batch, int num_q_heads, int
 }
 
 extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t* k_indices,
-                                   const uint8_t* k_coeffs, const void* k_scales,
-                                   const uint8_t* v_indices, const uint8_t* v_coeffs,
+                                   const void* k_coeffs, const void* k_scales,
+                                   const uint8_t* v_indices, const void* v_coeffs,
                                    const void* v_scales, const float* theta, const void* query_pos,
                                    int qp_itype, const void* key_positions, int kp_itype, float* out,
                                    int batch, int64_t seq_len, int num_q_heads, int num_kv_heads,
-                                   int d, int num_freqs, void* workspace, size_t workspace_bytes,
-                                   void* stream_) {
+                                   int d, int num_freqs, int coeff_bits, int pre_rope, void* workspace,
+                                   size_t workspace_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   AKV_REQUIRE(batch >= 0 && seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0, "akv_tri_decode_step: bad sizes");
   AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_tri_decode_step: num_q_heads %% num_kv_heads != 0");
   AKV_REQUIRE(d > 0 && d % 2 == 0 && d <= 512, "akv_tri_decode_step: head_dim=%d must be even and <= 512", d);
   AKV_REQUIRE(num_freqs > 0 && num_freqs <= d / 2, "akv_tri_decode_step: num_freqs=%d out of range", num_freqs);
+  AKV_REQUIRE(coeff_bits == 4 || coeff_bits == 8 || coeff_bits == 16,
+              "akv_tri_decode_step: coeff_bits=%d, must be 4, 8 or 16", coeff_bits);
   AKV_REQUIRE(akv_valid_dtype(q_dtype), "akv_tri_decode_step: bad dtype");
   AKV_REQUIRE(!query_pos || akv_valid_itype(qp_itype), "akv_tri_decode_step: bad query_pos type");
   AKV_REQUIRE(!key_positions || akv_valid_itype(kp_itype), "akv_tri_decode_step: bad key_positions type");
@@ -715,18 +757,21 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
     AKV_LAUNCH_CHECK("tri_zero_kernel");
     return AKV_OK;
   }
-  AKV_REQUIRE(k_indices && k_coeffs && k_scales && v_indices && v_coeffs && v_scales,
-              "akv_tri_decode_step: null cache pointer");
+  AKV_REQUIRE(k_indices && k_coeffs && v_indices && v_coeffs, "akv_tri_decode_step: null cache pointer");
+  AKV_REQUIRE(coeff_bits == 16 || (k_scales && v_scales), "akv_tri_decode_step: null scales");
+  AKV_REQUIRE(coeff_bits != 16 || ((((uintptr_t)k_coeffs | (uintptr_t)v_coeffs) & 1) == 0),
+              "akv_tri_decode_step: float16 coefficients must be 2-byte aligned");
   AKV_REQUIRE(workspace != nullptr, "akv_tri_decode_step: null workspace");
   if (workspace_bytes < akv_tri_decode_workspace_bytes(batch, num_q_heads, d))
     return akv_fail(AKV_ERR_WORKSPACE, "akv_tri_decode_step: workspace %zu < %zu bytes", workspace_bytes,
                     akv_tri_decode_workspace_bytes(batch, num_q_heads, d));
   tri_args a;
   a.query = query; a.q_dtype = q_dtype;
-  a.k_idx = k_indices; a.k_cf = k_coeffs; a.k_sc = (const __half*)k_scales;
-  a.v_idx = v_indices; a.v_cf = v_coeffs; a.v_sc = (const __half*)v_scales;
+  a.k_idx = k_indices; a.k_cf = (const uint8_t*)k_coeffs; a.k_sc = (const __half*)k_scales;
+  a.v_idx = v_indices; a.v_cf = (const uint8_t*)v_coeffs; a.v_sc = (const __half*)v_scales;
   a.theta = theta; a.qpos = query_pos; a.qp_itype = qp_itype; a.kpos = key_positions; a.kp_itype = kp_itype;
   a.B = batch; a.S = seq_len; a.QH = num_q_heads; a.KVH = num_kv_heads; a.D = d; a.F = num_freqs;
+  a.cbits = coeff_bits; a.post_rope = pre_rope ? 0 : 1;
   a.nsplit = tri_pick_splits(batch, num_kv_heads, seq_len);
   a.block_tables = nullptr; a.bt_itype = AKV_I32; a.bt_stride = 0; a.context_lens = nullptr; a.cl_itype = AKV_I32;
   a.block_size = 0; a.num_blocks = 0;
@@ -735,7 +780,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
   const int gqa = num_q_heads / num_kv_heads;
   // rows of 12 bytes can be read as dwords when the arrays are 4-byte aligned
-  const bool f12 = num_freqs == 12 &&
+  const bool wide = coeff_bits != 4;
+  const bool f12 = !wide && num_freqs == 12 &&
                    ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
   const bool dense = d == 128;
   if (dense && f12 && num_kv_heads <= 8) {
@@ -773,21 +819,26 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
 #define TRI_LAUNCH(GQV)                                                                                   \
   do {                                                                                                    \
     const size_t per_wave = dense ? (size_t)(TRI_DENSE_WAVE_BYTES / 4) : (size_t)GQV * d;                 \
-    const size_t lds = ((size_t)d / 2 + (size_t)GQV * d + 16 + TRI_WAVES * per_wave) * sizeof(float);     \
+    const size_t lds = ((size_t)d / 2 + (size_t)GQV * d + (wide ? 256 : 16) + TRI_WAVES * per_wave) * sizeof(float); \
     if (dense) {   /* more than 64 KB of dynamic LDS has to be allowed once per kernel */               \
       static bool configured = false;                                                                     \
       if (!configured) {                                                                                  \
-        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, true, true>,                      \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
-        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, false, true>,                     \
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
+        const int most = (int)(lds + 240 * sizeof(float));                                                \
+        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, true, true, false>,               \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, most));                   \
+        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, false, true, false>,              \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, most));                   \
+        AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_kernel<GQV, false, true, true>,               \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, most));                   \
         configured = true;                                                                                \
       }                                                                                                   \
     }                                                                                                     \
-    if (dense && f12) tri_decode_kernel<GQV, true, true><<<grid, 256, lds, stream>>>(a);                  \
-    else if (dense) tri_decode_kernel<GQV, false, true><<<grid, 256, lds, stream>>>(a);                   \
-    else if (f12) tri_decode_kernel<GQV, true, false><<<grid, 256, lds, stream>>>(a);                     \
-    else tri_decode_kernel<GQV, false, false><<<grid, 256, lds, stream>>>(a);                             \
+    if (dense && wide) tri_decode_kernel<GQV, false, true, true><<<grid, 256, lds, stream>>>(a);          \
+    else if (wide) tri_decode_kernel<GQV, false, false, true><<<grid, 256, lds, stream>>>(a);             \
+    else if (dense && f12) tri_decode_kernel<GQV, true, true, false><<<grid, 256, lds, stream>>>(a);      \
+    else if (dense) tri_decode_kernel<GQV, false, true, false><<<grid, 256, lds, stream>>>(a);            \
+    else if (f12) tri_decode_kernel<GQV, true, false, false><<<grid, 256, lds, stream>>>(a);              \
+    else tri_decode_kernel<GQV, false, false, false><<<grid, 256, lds, stream>>>(a);                      \
   } while (0)
   if (gqa % 4 == 0) TRI_LAUNCH(4); else TRI_LAUNCH(1);
 #undef TRI_LAUNCH
@@ -806,8 +857,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
                                     int64_t bt_stride, const void* context_lens, int cl_itype,
                                     float* out, int batch, int64_t num_blocks, int block_size,
                                     int64_t max_blocks_per_seq, int num_q_heads, int num_kv_heads,
-                                    int d, int num_freqs, void* workspace, size_t workspace_bytes,
-                                    void* stream_) {
+                                    int d, int num_freqs, int pre_rope, void* workspace,
+                                    size_t workspace_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   AKV_REQUIRE(batch >= 0 && num_blocks > 0 && block_size > 0 && max_blocks_per_seq >= 0 && num_q_heads > 0 &&
               num_kv_heads > 0, "akv_tri_decode_paged: bad sizes");
@@ -843,6 +894,7 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   a.v_idx = v_indices; a.v_cf = v_coeffs; a.v_sc = (const __half*)v_scales;
   a.theta = theta; a.qpos = query_pos; a.qp_itype = qp_itype; a.kpos = nullptr; a.kp_itype = AKV_I32;
   a.B = batch; a.S = max_blocks_per_seq * block_size; a.QH = num_q_heads; a.KVH = num_kv_heads; a.D = d; a.F = num_freqs;
+  a.cbits = 4; a.post_rope = pre_rope ? 0 : 1;
   a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
   a.context_lens = context_lens; a.cl_itype = cl_itype; a.block_size = block_size; a.num_blocks = num_blocks;
   int cus = akv_cached_cu_count();
@@ -873,7 +925,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
 }
 
 // ----------------------------------------------------------------------------------
-// SpectralKVEncoder.encode, int4 coefficients (aither_kvcache/triattention/encoder.py:73-133):
+// SpectralKVEncoder.encode (aither_kvcache/triattention/encoder.py:73-149), coefficient widths 4 (a byte per
+// pair, :118-133), 8 (two bytes per pair, :135-147) and 16 (the pair as two float16, scale 1, :107-115):
 // one wavefront per vector, lane = RoPE pair.  A pair's rank is the number of pairs with larger
 // energy (equal energies: lower index first; a NaN energy ranks above everything, as in
 // torch.topk); pairs of rank < F are kept, their position in the ascending index order is the
@@ -882,7 +935,7 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
 // ----------------------------------------------------------------------------------
 template <int XDT>
 __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict__ x, int64_t n, int d, int64_t xs,
-                                                         int F, uint8_t* __restrict__ indices,
+                                                         int F, int cbits, uint8_t* __restrict__ indices,
                                                          uint8_t* __restrict__ coeffs, __half* __restrict__ scales) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int P = d >> 1;
@@ -922,37 +975,50 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
       m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
     }
     const float scale = (m != m) ? m : fmaxf(m, 1e-8f);
-    if (keep) {
-      const float c0 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x0, scale), 1.0f), 7.5f));
-      const float c1 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x1, scale), 1.0f), 7.5f));
-      // clamp(0, 15) then the cast to uint8; a NaN becomes 0 as in torch's float -> uint8 conversion on the CPU
-      const uint32_t q0 = c0 != c0 ? 0u : (uint32_t)fminf(fmaxf(c0, 0.f), 15.f);
-      const uint32_t q1 = c1 != c1 ? 0u : (uint32_t)fminf(fmaxf(c1, 0.f), 15.f);
+    if (keep && cbits == 16) {
       indices[v * F + pos] = (uint8_t)lane;
-      coeffs[v * F + pos] = (uint8_t)((q0 << 4) | q1);
+      ((__half*)coeffs)[(v * F + pos) * 2] = __float2half_rn(x0);
+      ((__half*)coeffs)[(v * F + pos) * 2 + 1] = __float2half_rn(x1);
+    } else if (keep) {
+      const float half_code = cbits == 8 ? 127.5f : 7.5f, top = cbits == 8 ? 255.f : 15.f;
+      const float c0 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x0, scale), 1.0f), half_code));
+      const float c1 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x1, scale), 1.0f), half_code));
+      // clamp(0, top) then the cast to uint8; a NaN becomes 0 as in torch's float -> uint8 conversion on the CPU
+      const uint32_t q0 = c0 != c0 ? 0u : (uint32_t)fminf(fmaxf(c0, 0.f), top);
+      const uint32_t q1 = c1 != c1 ? 0u : (uint32_t)fminf(fmaxf(c1, 0.f), top);
+      indices[v * F + pos] = (uint8_t)lane;
+      if (cbits == 8) {
+        coeffs[(v * F + pos) * 2] = (uint8_t)q0;
+        coeffs[(v * F + pos) * 2 + 1] = (uint8_t)q1;
+      } else {
+        coeffs[v * F + pos] = (uint8_t)((q0 << 4) | q1);
+      }
     }
-    if (lane == 0) scales[v] = __float2half_rn(scale);
+    if (lane == 0) scales[v] = cbits == 16 ? __float2half_rn(1.0f) : __float2half_rn(scale);
   }
 }
 
 extern "C" int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
-                              uint8_t* indices, uint8_t* coeffs, void* scales, void* stream_) {
+                              int coeff_bits, uint8_t* indices, void* coeffs, void* scales, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   AKV_REQUIRE(n >= 0, "akv_tri_encode: n=%lld", (long long)n);
   AKV_REQUIRE(akv_valid_dtype(x_dtype), "akv_tri_encode: bad dtype");
   AKV_REQUIRE(d > 0 && d % 2 == 0, "akv_tri_encode: head_dim=%d must be even", d);
   AKV_REQUIRE(num_freqs > 0 && num_freqs <= d / 2, "akv_tri_encode: num_freqs=%d out of range", num_freqs);
+  AKV_REQUIRE(coeff_bits == 4 || coeff_bits == 8 || coeff_bits == 16, "akv_tri_encode: coeff_bits=%d, must be 4, 8 or 16",
+              coeff_bits);
   if (d > 128) return akv_fail(AKV_ERR_UNSUPPORTED, "akv_tri_encode: head_dim=%d above 128 (one lane per pair)", d);
   if (n == 0) return AKV_OK;
   AKV_REQUIRE(x && indices && coeffs && scales, "akv_tri_encode: null pointer");
   AKV_REQUIRE(x_stride >= d, "akv_tri_encode: stride smaller than row");
+  AKV_REQUIRE(coeff_bits != 16 || ((uintptr_t)coeffs & 1) == 0, "akv_tri_encode: float16 coefficients must be 2-byte aligned");
   const int64_t want = (n + 3) / 4;
   const int cap = akv_cached_cu_count() * 32;
   const int grid = (int)(want < cap ? want : cap);
   switch (x_dtype) {
-    case AKV_F16: tri_encode_kernel<AKV_F16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
-    case AKV_BF16: tri_encode_kernel<AKV_BF16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
-    default: tri_encode_kernel<AKV_F32><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, indices, coeffs, (__half*)scales); break;
+    case AKV_F16: tri_encode_kernel<AKV_F16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
+    case AKV_BF16: tri_encode_kernel<AKV_BF16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
+    default: tri_encode_kernel<AKV_F32><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
   }
   AKV_LAUNCH_CHECK("tri_encode_kernel");
   return AKV_OK;

@@ -2,7 +2,8 @@
 with TrigSeriesScorer.score, scorer.py:115-208).
 
 score(q, k_t) = (1/sqrt d) sum_f [ c_f cos(delta theta_f) + s_f sin(delta theta_f) ] over the
-token's retained RoPE pairs, softmax over the cached tokens, and a weighted scatter-add of the
+token's retained RoPE pairs (config.pre_rope; otherwise the keys were stored after RoPE and the score is
+(1/sqrt d) sum_f c_f, scorer.py:200-202), coefficients of 4, 8 or 16 bits (scorer.py:84-113), softmax over the cached tokens, and a weighted scatter-add of the
 value coefficients -- one HIP kernel over the spectral cache plus a merge kernel, instead of the
 reference's chain of [B, QH, S, F] float32 temporaries.
 """
@@ -13,7 +14,7 @@ import torch
 
 from .. import _lib
 from .config import TriAttentionConfig
-from .encoder import SpectralEncoding, SpectralKVEncoder
+from .encoder import SpectralEncoding, SpectralKVEncoder, packed_shape
 from .spectral import rope_frequencies
 
 
@@ -45,8 +46,6 @@ class TriAttention:
                     key_positions: Optional[torch.Tensor] = None) -> torch.Tensor:
         """query [B, QH, D]; encodings with indices/packed [B, S, KVH, F], scales [B, S, KVH];
         query_pos [B] (default S), key_positions [B, S] (default 0..S-1) -> float32 [B, QH, D]."""
-        if not self.config.pre_rope:
-            raise NotImplementedError("post-RoPE scoring is not built")
         dev = _lib.require_gpu(query, k_enc.indices, k_enc.packed, k_enc.scales,
                                v_enc.indices, v_enc.packed, v_enc.scales, query_pos, key_positions)
         if self._theta.device != dev:
@@ -60,12 +59,21 @@ class TriAttention:
         q = query if query.dtype in (torch.float16, torch.bfloat16, torch.float32) else query.float()
         q = q.contiguous()
 
+        cbits = self.config.coeff_bits
+        cshape, cdtype = packed_shape([B, S, KVH], F, cbits)
+
         def u8(t):
             if t.dtype != torch.uint8:
-                raise ValueError("indices / packed must be uint8 (int4 coefficients)")
+                raise ValueError("indices must be uint8")
             return t.contiguous()
 
-        ki, kc, vi, vc = u8(k_enc.indices), u8(k_enc.packed), u8(v_enc.indices), u8(v_enc.packed)
+        def coeffs(t):
+            if t.dtype != cdtype or list(t.shape) != cshape:
+                raise ValueError(f"packed coefficients must be {cdtype} {cshape} at coeff_bits={cbits}, "
+                                 f"got {t.dtype} {list(t.shape)}")
+            return t.contiguous()
+
+        ki, kc, vi, vc = u8(k_enc.indices), coeffs(k_enc.packed), u8(v_enc.indices), coeffs(v_enc.packed)
         ks = k_enc.scales.to(torch.float16).contiguous()
         vs = v_enc.scales.to(torch.float16).contiguous()
 
@@ -88,7 +96,7 @@ class TriAttention:
             vi.data_ptr(), vc.data_ptr(), vs.data_ptr(), self._theta.data_ptr(),
             _lib.ptr(qp), _lib.itype_code(qp) if qp is not None else 0,
             _lib.ptr(kp), _lib.itype_code(kp) if kp is not None else 0,
-            out.data_ptr(), B, S, QH, KVH, D, F,
+            out.data_ptr(), B, S, QH, KVH, D, F, cbits, 1 if self.config.pre_rope else 0,
             self._workspace.data_ptr(), self._workspace.numel(), _lib.stream_ptr(dev)))
         return out
 
@@ -99,8 +107,6 @@ class TriAttention:
         with cache.fetch_sequence, cache.py:163-198, followed by decode_step).  query [B, QH, D];
         block_tables [B, max_blocks_per_seq] int32/int64; context_lens [B]; key positions are
         0..ctx-1 and query_pos defaults to ctx -> float32 [B, QH, D] (zeros where ctx == 0)."""
-        if not self.config.pre_rope:
-            raise NotImplementedError("post-RoPE scoring is not built")
         dev = _lib.require_gpu(query, cache.k_indices, cache.k_packed, cache.k_scales, cache.v_indices,
                                cache.v_packed, cache.v_scales, block_tables, context_lens, query_pos)
         if self._theta.device != dev:
@@ -136,7 +142,7 @@ class TriAttention:
             cache.v_scales.data_ptr(), self._theta.data_ptr(),
             _lib.ptr(qp), _lib.itype_code(qp) if qp is not None else 0,
             bt.data_ptr(), _lib.itype_code(bt), bt.stride(0), cl.data_ptr(), _lib.itype_code(cl),
-            out.data_ptr(), B, NB, BS, bt.shape[1], QH, KVH, D, F,
+            out.data_ptr(), B, NB, BS, bt.shape[1], QH, KVH, D, F, 1 if self.config.pre_rope else 0,
             self._workspace.data_ptr(), self._workspace.numel(), _lib.stream_ptr(dev))
         if rc == _lib.AKV_ERR_UNSUPPORTED:
             # shapes the paged kernel does not take: gather each sequence and use the dense-layout kernels

@@ -1,8 +1,9 @@
 """Spectral KV encoding (write side of TriAttention).
 
 Keeps the F RoPE pairs (dims 2i, 2i+1) of largest energy per token, ascending by index, and
-quantises their 2F values to 4 bits against the token's max-abs scale (reference:
-aither_kvcache/triattention/encoder.py:73-133).  On an MI355X tensor with head_dim <= 128 this is one
+quantises their 2F values against the token's max-abs scale to 4 bits (a byte per pair) or 8 bits (two
+bytes per pair), or keeps them as float16 (coeff_bits 16) (reference:
+aither_kvcache/triattention/encoder.py:73-149).  On an MI355X tensor with head_dim <= 128 this is one
 HIP kernel (akv_tri_encode); host tensors and wider heads take the same steps as torch ops.
 """
 from typing import NamedTuple, Optional
@@ -15,14 +16,41 @@ from .config import TriAttentionConfig
 
 class SpectralEncoding(NamedTuple):
     indices: torch.Tensor   # [..., F] uint8   retained pair indices, ascending
-    packed: torch.Tensor    # [..., F] uint8   code(even) << 4 | code(odd)
-    scales: torch.Tensor    # [...]    float16 max |coefficient| of the token
+    packed: torch.Tensor    # coeff_bits 4: [..., F] uint8, code(even) << 4 | code(odd); 8: [..., 2F] uint8,
+                            # code(even), code(odd) per pair; 16: [..., F, 2] float16, the components
+    scales: torch.Tensor    # [...]    float16 max |coefficient| of the token (ones for coeff_bits 16)
+
+
+def packed_shape(batch, num_freqs: int, coeff_bits: int):
+    """Shape and dtype of SpectralEncoding.packed for a batch shape (encoder.py:107-147 of the reference)."""
+    batch = list(batch)
+    if coeff_bits == 4:
+        return batch + [num_freqs], torch.uint8
+    if coeff_bits == 8:
+        return batch + [2 * num_freqs], torch.uint8
+    if coeff_bits == 16:
+        return batch + [num_freqs, 2], torch.float16
+    raise ValueError(f"Unsupported coeff_bits: {coeff_bits}")
+
+
+def unpack_coefficients(packed: torch.Tensor, scales: torch.Tensor, coeff_bits: int):
+    """(even, odd) float32 components [..., F] of an encoding, with the reference's arithmetic
+    (scorer.py:84-113): (code / half - 1) * scale for 4 and 8 bits, the float16 values for 16."""
+    if coeff_bits == 16:
+        return packed[..., 0].float(), packed[..., 1].float()
+    s = scales.float().unsqueeze(-1)
+    if coeff_bits == 4:
+        return ((packed >> 4).float() / 7.5 - 1.0) * s, ((packed & 0x0F).float() / 7.5 - 1.0) * s
+    if coeff_bits == 8:
+        raw = packed.float().reshape(*packed.shape[:-1], packed.shape[-1] // 2, 2)
+        return (raw[..., 0] / 127.5 - 1.0) * s, (raw[..., 1] / 127.5 - 1.0) * s
+    raise ValueError(f"Unsupported coeff_bits: {coeff_bits}")
 
 
 class SpectralKVEncoder:
     def __init__(self, config: TriAttentionConfig):
-        if config.coeff_bits != 4:
-            raise NotImplementedError("only int4 coefficients (coeff_bits=4) are built")
+        if config.coeff_bits not in (4, 8, 16):
+            raise ValueError(f"Unsupported coeff_bits: {config.coeff_bits}")
         self.config = config
         self.head_dim = config.head_dim
         self.num_pairs = config.num_pairs
@@ -38,26 +66,29 @@ class SpectralKVEncoder:
                 xf = xf.contiguous()
             n = xf.shape[0]
             idx = torch.empty(n, F, dtype=torch.uint8, device=x.device)
-            cf = torch.empty(n, F, dtype=torch.uint8, device=x.device)
+            cshape, cdtype = packed_shape([n], F, self.coeff_bits)
+            cf = torch.empty(cshape, dtype=cdtype, device=x.device)
             sc = torch.empty(n, dtype=torch.float16, device=x.device)
             _lib.check(_lib.lib().akv_tri_encode(
                 xf.data_ptr(), _lib.dtype_code(xf), n, self.head_dim, xf.stride(0) if n else self.head_dim, F,
-                idx.data_ptr(), cf.data_ptr(), sc.data_ptr(), _lib.stream_ptr(x.device)))
-            return SpectralEncoding(idx.reshape(batch + [F]), cf.reshape(batch + [F]), sc.reshape(batch))
+                self.coeff_bits, idx.data_ptr(), cf.data_ptr(), sc.data_ptr(), _lib.stream_ptr(x.device)))
+            return SpectralEncoding(idx.reshape(batch + [F]), cf.reshape(batch + cshape[1:]), sc.reshape(batch))
         pairs = x.reshape(*x.shape[:-1], self.num_pairs, 2).float()
         energy = pairs.pow(2).sum(-1)
         keep = energy.topk(F, dim=-1).indices.sort(dim=-1).values
         vals = torch.gather(pairs, -2, keep.unsqueeze(-1).expand(*keep.shape, 2))
+        if self.coeff_bits == 16:
+            return SpectralEncoding(keep.to(torch.uint8), vals.to(torch.float16),
+                                    torch.ones(x.shape[:-1], dtype=torch.float16, device=x.device))
         scales = vals.abs().flatten(-2).amax(-1).clamp(min=1e-8)
-        codes = ((vals / scales[..., None, None] + 1) * 7.5).round().clamp(0, 15).to(torch.uint8)
-        return SpectralEncoding(keep.to(torch.uint8), (codes[..., 0] << 4) | codes[..., 1],
-                                scales.to(torch.float16))
+        half, top = (7.5, 15) if self.coeff_bits == 4 else (127.5, 255)
+        codes = ((vals / scales[..., None, None] + 1) * half).round().clamp(0, top).to(torch.uint8)
+        packed = (codes[..., 0] << 4) | codes[..., 1] if self.coeff_bits == 4 else codes.flatten(-2)
+        return SpectralEncoding(keep.to(torch.uint8), packed, scales.to(torch.float16))
 
     def decode(self, enc: SpectralEncoding) -> torch.Tensor:
         """Dense [..., head_dim] float32 reconstruction (zeros at the discarded pairs)."""
-        s = enc.scales.float().unsqueeze(-1)
-        v0 = ((enc.packed >> 4).float() / 7.5 - 1.0) * s
-        v1 = ((enc.packed & 0x0F).float() / 7.5 - 1.0) * s
+        v0, v1 = unpack_coefficients(enc.packed, enc.scales, self.coeff_bits)
         idx = enc.indices.long()
         out = torch.zeros(*idx.shape[:-1], self.head_dim, dtype=torch.float32, device=idx.device)
         out.scatter_(-1, idx * 2, v0)

@@ -279,21 +279,27 @@ int akv_hybrid_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_
 
 /* ---------------------------------------------------------------------------------
  * TriAttention.decode_step -- aither_kvcache/triattention/attention.py:186-280 with
- * TrigSeriesScorer.score (scorer.py:115-208), int4 coefficients:
- *   k/v_indices [B][S][KVH][F] uint8, k/v_coeffs [B][S][KVH][F] uint8 (hi nibble = even
- *   component), k/v_scales [B][S][KVH] fp16, all contiguous; theta [d/2] float32
+ * TrigSeriesScorer.score (scorer.py:115-208):
+ *   k/v_indices [B][S][KVH][F] uint8; k/v_coeffs by coeff_bits (scorer.py:84-113):
+ *     4   [B][S][KVH][F] uint8, hi nibble = even component, value = (code / 7.5 - 1) * scale
+ *     8   [B][S][KVH][2F] uint8, even then odd component of each pair, (code / 127.5 - 1) * scale
+ *     16  [B][S][KVH][F][2] fp16, the components themselves; k/v_scales are not read (may be NULL)
+ *   k/v_scales [B][S][KVH] fp16, all contiguous; theta [d/2] float32
  *   (spectral.py:34-51); query [B][QH][d] (contiguous); query_pos [B] or NULL (= S);
  *   key_positions [B][S] or NULL (= 0..S-1); out [B][QH][d] float32.
+ *   pre_rope != 0: the trigonometric series over key position - query position (scorer.py:180-199);
+ *   pre_rope == 0: keys were stored after RoPE, the score is the plain sparse dot product
+ *   (scorer.py:200-202) and the positions are not used.
  * ------------------------------------------------------------------------------- */
 size_t akv_tri_decode_workspace_bytes(int batch, int num_q_heads, int d);
 int akv_tri_decode_step(const void* query, int q_dtype,
-                        const uint8_t* k_indices, const uint8_t* k_coeffs, const void* k_scales,
-                        const uint8_t* v_indices, const uint8_t* v_coeffs, const void* v_scales,
+                        const uint8_t* k_indices, const void* k_coeffs, const void* k_scales,
+                        const uint8_t* v_indices, const void* v_coeffs, const void* v_scales,
                         const float* theta,
                         const void* query_pos, int qp_itype,
                         const void* key_positions, int kp_itype,
                         float* out, int batch, int64_t seq_len, int num_q_heads, int num_kv_heads,
-                        int d, int num_freqs,
+                        int d, int num_freqs, int coeff_bits, int pre_rope,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
@@ -305,6 +311,8 @@ int akv_tri_decode_step(const void* query, int q_dtype,
  *   (row stride bt_stride elements; entries past the context are never dereferenced for
  *   ctx > 0); context_lens [B], clamped to max_blocks_per_seq * block_size; key positions are
  *   0..ctx-1; query_pos [B] or NULL (= ctx); out [B][QH][d] float32, zeros where ctx == 0.
+ *   Coefficients are int4 (the only width the reference's cache stores, cache.py:66-85); pre_rope as for
+ *   akv_tri_decode_step.
  * Workspace as for akv_tri_decode_step.  Built for d = 128, num_freqs = 12, at most 8 kv heads
  * and 4-byte aligned arrays; anything else returns AKV_ERR_UNSUPPORTED (gather, then
  * akv_tri_decode_step).
@@ -318,21 +326,25 @@ int akv_tri_decode_paged(const void* query, int q_dtype,
                          const void* context_lens, int cl_itype,
                          float* out, int batch, int64_t num_blocks, int block_size,
                          int64_t max_blocks_per_seq, int num_q_heads, int num_kv_heads,
-                         int d, int num_freqs,
+                         int d, int num_freqs, int pre_rope,
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
- * SpectralKVEncoder.encode, coeff_bits = 4 -- aither_kvcache/triattention/encoder.py:73-133
+ * SpectralKVEncoder.encode -- aither_kvcache/triattention/encoder.py:73-149
  * (the write side of TriAttention; TriAttention.encode_kv, attention.py:160-184, calls it for
  * keys and values): per vector the num_freqs RoPE pairs (dims 2i, 2i+1) of largest energy,
- * indices ascending; scale = max |kept coefficient| clamped at 1e-8; code =
- * clamp(round((v / scale + 1) * 7.5), 0, 15); byte = code(even) << 4 | code(odd).
- *   x [n][d] (row stride x_stride elements); indices, coeffs [n][num_freqs] uint8; scales [n] fp16.
+ * indices ascending; scale = max |kept coefficient| clamped at 1e-8; then by coeff_bits
+ *   4   code = clamp(round((v / scale + 1) * 7.5), 0, 15); byte = code(even) << 4 | code(odd);
+ *       coeffs [n][num_freqs] uint8                                                    (:118-133)
+ *   8   code = clamp(round((v / scale + 1) * 127.5), 0, 255); coeffs [n][2 num_freqs] uint8, even then
+ *       odd component of each pair                                                     (:135-147)
+ *   16  coeffs [n][num_freqs][2] fp16 = the components rounded to fp16; scales = 1     (:107-115)
+ *   x [n][d] (row stride x_stride elements); indices [n][num_freqs] uint8; scales [n] fp16.
  * Pairs of exactly equal energy are kept lowest index first (torch.topk leaves that open).
  * head_dim above 128 returns AKV_ERR_UNSUPPORTED.
  * ------------------------------------------------------------------------------- */
 int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
-                   uint8_t* indices, uint8_t* coeffs, void* scales, void* stream);
+                   int coeff_bits, uint8_t* indices, void* coeffs, void* scales, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * Block selection for sparse decode attention -- aither_kvcache/block_selector.py.

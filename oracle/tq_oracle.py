@@ -19,7 +19,8 @@ reference tree).  How each one is pinned:
       selection and scatter by a per-block loop in tests/test_oracle_pins.py),
       fwht, structured_hadamard, dimension_aware_codebook,
       hybrid_encode, hybrid_decode, rope_frequencies, spectral_encode,
-      tri_scores, tri_decode_step,
+      tri_scores, tri_decode_step (coefficient widths 8 / 16 and post-RoPE scoring by
+      tests/golden/golden_tri_widths.npz, also written by the reference itself),
       spectral_fetch_sequence / tri_decode_step_paged (indexing only, on top of the pinned
       tri_decode_step: checked against a token-by-token loop in tests/test_oracle_pins.py)
   derived here (the reference has no such function; it always decompresses
@@ -676,10 +677,13 @@ def rope_frequencies(head_dim, base=1_000_000.0):
     return np.power(f32(base), (f32(-2.0) * i) / f32(head_dim)).astype(f32)
 
 
-def spectral_encode(x, num_freqs=12):
-    """SpectralKVEncoder.encode for coeff_bits=4, encoder.py:73-133: top-F pairs by energy,
-    indices ascending, per-token max-abs scale (clamped at 1e-8), codes =
-    clamp(round((v/scale + 1) * 7.5), 0, 15), byte = code_even << 4 | code_odd, scale -> fp16."""
+def spectral_encode(x, num_freqs=12, coeff_bits=4):
+    """SpectralKVEncoder.encode, encoder.py:73-149: top-F pairs by energy, indices ascending; then by width
+      4   per-token max-abs scale (clamped at 1e-8), codes = clamp(round((v/scale + 1) * 7.5), 0, 15),
+          byte = code_even << 4 | code_odd, scale -> fp16                                 (:118-133)
+      8   the same with half-code 127.5 and range 0..255, the two codes of a pair in consecutive bytes:
+          packed [..., 2F] uint8                                                          (:135-147)
+      16  the pairs themselves rounded to fp16: packed [..., F, 2] float16, scales = 1    (:107-115)"""
     x = np.asarray(x)
     D = x.shape[-1]
     pairs = x.astype(f32).reshape(x.shape[:-1] + (D // 2, 2))
@@ -687,23 +691,43 @@ def spectral_encode(x, num_freqs=12):
     order = np.argsort(-en, axis=-1, kind="stable")[..., :num_freqs]
     top = np.sort(order, axis=-1)
     tp = np.take_along_axis(pairs, top[..., None], axis=-2)
+    if coeff_bits == 16:
+        return top.astype(np.uint8), tp.astype(np.float16), np.ones(x.shape[:-1], dtype=np.float16)
+    if coeff_bits not in (4, 8):
+        raise ValueError(f"Unsupported coeff_bits: {coeff_bits}")
+    half, top_code = (f32(7.5), 15) if coeff_bits == 4 else (f32(127.5), 255)
     scales = np.maximum(np.abs(tp).reshape(tp.shape[:-2] + (-1,)).max(axis=-1), f32(1e-8))
     nrm = tp / scales[..., None, None]
-    q = np.clip(np.round((nrm + f32(1)) * f32(7.5)), 0, 15).astype(np.uint8)
-    packed = ((q[..., 0] << 4) | q[..., 1]).astype(np.uint8)
+    q = np.clip(np.round((nrm + f32(1)) * half), 0, top_code).astype(np.uint8)
+    if coeff_bits == 4:
+        packed = ((q[..., 0] << 4) | q[..., 1]).astype(np.uint8)
+    else:
+        packed = q.reshape(q.shape[:-2] + (2 * num_freqs,))
     return top.astype(np.uint8), packed, scales.astype(np.float16)
 
 
-def unpack_coefficients(packed, scales):
-    """TrigSeriesScorer._unpack_coefficients (4-bit), scorer.py:84-104."""
+def unpack_coefficients(packed, scales, coeff_bits=4):
+    """TrigSeriesScorer._unpack_coefficients, scorer.py:84-113: (code / half - 1) * scale in float32 for
+    4 bits (nibbles, half 7.5) and 8 bits (byte pairs, half 127.5); the fp16 pairs as they are for 16."""
+    packed = np.asarray(packed)
+    if coeff_bits == 16:
+        return packed[..., 0].astype(f32), packed[..., 1].astype(f32)
     s = np.asarray(scales).astype(f32)[..., None]
-    v0 = (np.asarray(packed) >> 4).astype(f32)
-    v1 = (np.asarray(packed) & 0x0F).astype(f32)
-    return ((v0 / f32(7.5) - f32(1.0)) * s).astype(f32), ((v1 / f32(7.5) - f32(1.0)) * s).astype(f32)
+    if coeff_bits == 4:
+        v0, v1, half = (packed >> 4).astype(f32), (packed & 0x0F).astype(f32), f32(7.5)
+    elif coeff_bits == 8:
+        raw = packed.astype(f32).reshape(packed.shape[:-1] + (packed.shape[-1] // 2, 2))
+        v0, v1, half = raw[..., 0], raw[..., 1], f32(127.5)
+    else:
+        raise ValueError(f"Unsupported coeff_bits: {coeff_bits}")
+    return ((v0 / half - f32(1.0)) * s).astype(f32), ((v1 / half - f32(1.0)) * s).astype(f32)
 
 
-def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_positions=None):
-    """TrigSeriesScorer.score (pre-RoPE), scorer.py:115-208 -> [B, QH, S] float32 logits."""
+def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_positions=None, coeff_bits=4,
+               pre_rope=True):
+    """TrigSeriesScorer.score, scorer.py:115-208 -> [B, QH, S] float32 logits.  pre_rope: the trigonometric
+    series over the position difference (:180-199); otherwise the plain sparse dot product sum_f c_f
+    (:200-202), positions unused."""
     query = np.asarray(query)
     B, QH, D = query.shape
     S, KVH = k_idx.shape[1], k_idx.shape[2]
@@ -712,7 +736,7 @@ def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_posi
         key_positions = np.broadcast_to(np.arange(S)[None], (B, S))
     if query_pos is None:
         query_pos = np.full((B,), S)
-    k0, k1 = unpack_coefficients(k_packed, k_scales)              # [B,S,KVH,F]
+    k0, k1 = unpack_coefficients(k_packed, k_scales, coeff_bits)  # [B,S,KVH,F]
     hmap = np.arange(QH) // gqa
     idx = k_idx.astype(np.int64)[:, :, hmap].transpose(0, 2, 1, 3)  # [B,QH,S,F]
     k0 = k0[:, :, hmap].transpose(0, 2, 1, 3)
@@ -721,28 +745,32 @@ def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_posi
     qe = np.take_along_axis(np.broadcast_to(qf[..., 0::2][:, :, None], (B, QH, S, D // 2)), idx, -1)
     qo = np.take_along_axis(np.broadcast_to(qf[..., 1::2][:, :, None], (B, QH, S, D // 2)), idx, -1)
     c = qe * k0 + qo * k1
-    s = qo * k0 - qe * k1
-    delta = (np.asarray(key_positions).astype(f32).reshape(B, 1, S, 1)
-             - np.asarray(query_pos).astype(f32).reshape(B, 1, 1, 1))
-    ph = (delta * np.asarray(theta, dtype=f32)[idx]).astype(f32)
-    raw = np.sum(c * np.cos(ph) + s * np.sin(ph), axis=-1, dtype=f32)
+    if pre_rope:
+        s = qo * k0 - qe * k1
+        delta = (np.asarray(key_positions).astype(f32).reshape(B, 1, S, 1)
+                 - np.asarray(query_pos).astype(f32).reshape(B, 1, 1, 1))
+        ph = (delta * np.asarray(theta, dtype=f32)[idx]).astype(f32)
+        raw = np.sum(c * np.cos(ph) + s * np.sin(ph), axis=-1, dtype=f32)
+    else:
+        raw = np.sum(c, axis=-1, dtype=f32)
     return (raw * f32(1.0 / math.sqrt(D))).astype(f32)
 
 
-def tri_decode_step(query, k_enc, v_enc, theta, query_pos=None, key_positions=None):
+def tri_decode_step(query, k_enc, v_enc, theta, query_pos=None, key_positions=None, coeff_bits=4,
+                    pre_rope=True):
     """TriAttention.decode_step, attention.py:186-280: scores -> softmax over S -> weighted
     scatter-add of the value coefficients into even/odd bins -> interleave.  k_enc / v_enc are
     (indices, packed, scales) triples.  Returns float32 [B, QH, D]."""
     query = np.asarray(query)
     B, QH, D = query.shape
-    sc = tri_scores(query, *k_enc, theta, query_pos, key_positions)
+    sc = tri_scores(query, *k_enc, theta, query_pos, key_positions, coeff_bits, pre_rope)
     sc = sc - sc.max(axis=-1, keepdims=True)
     w = np.exp(sc)
     w = (w / w.sum(axis=-1, keepdims=True, dtype=f32)).astype(f32)
     v_idx, v_packed, v_scales = v_enc
     KVH = v_idx.shape[2]
     gqa = QH // KVH
-    v0, v1 = unpack_coefficients(v_packed, v_scales)               # [B,S,KVH,F]
+    v0, v1 = unpack_coefficients(v_packed, v_scales, coeff_bits)   # [B,S,KVH,F]
     out = np.zeros((B, QH, D), dtype=f32)
     for b in range(B):
         for qh in range(QH):
@@ -767,7 +795,8 @@ def spectral_fetch_sequence(cache_arrays, block_table, context_len, block_size):
     return tuple(got[:3]), tuple(got[3:])
 
 
-def tri_decode_step_paged(query, cache_arrays, block_tables, context_lens, block_size, theta, query_pos=None):
+def tri_decode_step_paged(query, cache_arrays, block_tables, context_lens, block_size, theta, query_pos=None,
+                          coeff_bits=4, pre_rope=True):
     """A batch of sequences in one block pool: per sequence fetch_sequence then decode_step with the
     default key positions 0..ctx-1 and query position ctx (scorer.py:142-146); an empty sequence
     gives zeros (softmax over no tokens, nothing scattered).  Returns float32 [B, QH, D]."""
@@ -781,5 +810,5 @@ def tri_decode_step_paged(query, cache_arrays, block_tables, context_lens, block
         k_enc, v_enc = spectral_fetch_sequence(cache_arrays, block_tables[b], n, block_size)
         qp = None if query_pos is None else np.asarray(query_pos)[b:b + 1]
         out[b] = tri_decode_step(query[b:b + 1], tuple(a[None] for a in k_enc), tuple(a[None] for a in v_enc),
-                                 theta, qp)[0]
+                                 theta, qp, None, coeff_bits, pre_rope)[0]
     return out

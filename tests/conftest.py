@@ -20,6 +20,13 @@ def golden():
 
 
 @pytest.fixture(scope="session")
+def tri_widths():
+    """TriAttention at coefficient widths 8 / 16 and post-RoPE scoring, produced by the reference itself
+    (tests/golden/make_golden_tri_widths.py)."""
+    return np.load(os.path.join(ROOT, "tests", "golden", "golden_tri_widths.npz"))
+
+
+@pytest.fixture(scope="session")
 def dev():
     import torch
     if not torch.cuda.is_available():

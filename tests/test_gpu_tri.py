@@ -258,3 +258,156 @@ def test_empty_batch_and_empty_sequence(dev):
     assert out.shape == (3, 32, 128) and not bool(out.any())
     out0 = tri.decode_step(torch.randn(0, 32, 128, device=dev), enc(0, 5), enc(0, 5))
     assert out0.shape == (0, 32, 128)
+
+
+# ---- coefficient widths 8 / 16 and post-RoPE scoring -------------------------------------------------
+WIDTH_MODES = [(8, True), (16, True), (4, False), (8, False), (16, False)]
+
+
+def _wenc(g, bits, nm, dev):
+    return SpectralEncoding(*(t(g[f"enc_b{bits}_{nm}_{part}"], dev) for part in ("indices", "packed", "scales")))
+
+
+@pytest.mark.parametrize("bits,pre", WIDTH_MODES)
+def test_widths_and_post_rope_golden(golden, tri_widths, dev, bits, pre):
+    """The reference's own encodings and outputs at coeff_bits 8 / 16 and with pre_rope=False: the
+    write-side kernel reproduces the encodings bit for bit, decode_step the outputs to TOL."""
+    g = tri_widths
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=bits, num_kv_heads=2, num_query_heads=8,
+                             rope_base=1_000_000.0, pre_rope=pre)
+    tri = TriAttention(cfg, device=str(dev))
+    k_enc, v_enc = tri.encode_kv(t(g["keys"], dev), t(g["vals"], dev))
+    for nm, e in (("k", k_enc), ("v", v_enc)):
+        for part, got in zip(("indices", "packed", "scales"), e):
+            want = g[f"enc_b{bits}_{nm}_{part}"]
+            assert got.cpu().numpy().dtype == want.dtype and got.shape == want.shape
+            assert np.array_equal(got.cpu().numpy().view(np.uint8), want.view(np.uint8)), (nm, part)
+    tag = f"b{bits}_{'pre' if pre else 'post'}"
+    ke, ve = _wenc(g, bits, "k", dev), _wenc(g, bits, "v", dev)
+    out = tri.decode_step(t(g["q"], dev), ke, ve, t(g["qpos"], dev), t(g["kpos"], dev)).cpu().numpy()
+    e1 = np.max(np.abs(out - g[f"out_{tag}"]))
+    out_d = tri.decode_step(t(g["q"], dev), ke, ve).cpu().numpy()
+    e2 = np.max(np.abs(out_d - g[f"out_default_pos_{tag}"]))
+    print(f"[tri widths golden] {tag}: explicit-pos {e1:.2e}, default-pos {e2:.2e}")
+    assert e1 <= TOL and e2 <= TOL
+
+
+@pytest.mark.parametrize("bits,pre", WIDTH_MODES)
+@pytest.mark.parametrize("B,S,QH,KVH,D,F,base", [(2, 1000, 32, 8, 128, 12, 1e6), (2, 333, 6, 2, 32, 4, 1e4),
+                                                 (1, 64, 4, 4, 64, 32, 1e4), (2, 700, 8, 2, 128, 20, 1e6),
+                                                 (1, 3000, 16, 16, 128, 12, 1e6)])
+def test_widths_and_post_rope_vs_oracle(dev, bits, pre, B, S, QH, KVH, D, F, base):
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=bits, num_kv_heads=KVH, num_query_heads=QH,
+                             rope_base=base, pre_rope=pre)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(S + bits)
+    pair_std = (np.arange(D // 2) + 1.0) ** -0.75
+    keys = (rng.standard_normal((B, S, KVH, D // 2, 2)) * pair_std[:, None]).reshape(B, S, KVH, D).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    k_enc, v_enc = tri.encode_kv(t(keys, dev), t(vals, dev))
+    ke, ve = O.spectral_encode(keys, F, bits), O.spectral_encode(vals, F, bits)
+    for got, want in zip(tuple(k_enc) + tuple(v_enc), ke + ve):
+        assert got.shape == want.shape and np.array_equal(got.cpu().numpy().view(np.uint8), want.view(np.uint8))
+    q = rng.standard_normal((B, QH, D)).astype(np.float32)
+    qpos = rng.integers(S, 40000, size=B)
+    kpos = np.sort(rng.integers(0, 32768, size=(B, S)), axis=-1)
+    theta = tri._theta.cpu().numpy()
+    out = tri.decode_step(t(q, dev), k_enc, v_enc, t(qpos, dev), t(kpos, dev)).cpu().numpy()
+    ref = O.tri_decode_step(q, ke, ve, theta, qpos, kpos, bits, pre)
+    err = np.max(np.abs(out - ref))
+    print(f"[tri widths] bits={bits} pre={pre} B={B} S={S} D={D} F={F} max|diff|={err:.2e} max|out|={np.abs(ref).max():.3f}")
+    assert err <= TOL
+    out_d = tri.decode_step(t(q, dev), k_enc, v_enc).cpu().numpy()
+    ref_d = O.tri_decode_step(q, ke, ve, theta, None, None, bits, pre)
+    assert np.max(np.abs(out_d - ref_d)) <= TOL
+    if not pre:                      # positions play no part
+        assert np.array_equal(out, out_d)
+
+
+@pytest.mark.parametrize("bits", [8, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_spectral_encode_widths_vs_oracle(dev, bits, dtype):
+    D, F = 128, 12
+    rng = np.random.default_rng(bits)
+    n = 5000
+    x = (rng.standard_normal((n, D)) * rng.lognormal(0, 1.0, (n, 1))).astype(np.float32)
+    x[7] = 0.0
+    x[8, 2:] = 0.0
+    x[9] *= 1e-6
+    xt = torch.from_numpy(x).to(dev).to(dtype)
+    tri = TriAttention(TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=bits, num_kv_heads=1, num_query_heads=1),
+                       device=str(dev))
+    e = tri.encoder.encode(xt)
+    ri, rp, rs = O.spectral_encode(xt.float().cpu().numpy(), F, bits)
+    assert np.array_equal(e.indices.cpu().numpy(), ri)
+    assert e.packed.shape == rp.shape and np.array_equal(e.packed.cpu().numpy().view(np.uint8), rp.view(np.uint8))
+    assert np.array_equal(e.scales.cpu().numpy(), rs)
+    # the host path (torch ops) of the encoder and the dense reconstruction agree with the kernel's encoding
+    # (rows without pairs of equal energy: torch.topk leaves the order among ties open)
+    eh = tri.encoder.encode(xt[10:].cpu())
+    assert torch.equal(eh.indices, e.indices[10:].cpu()) and torch.equal(eh.packed, e.packed[10:].cpu())
+    assert torch.equal(eh.scales, e.scales[10:].cpu())
+    dec = tri.encoder.decode(e).cpu().numpy()
+    v0, v1 = O.unpack_coefficients(rp, rs, bits)
+    want = np.zeros((n, D), np.float32)
+    np.put_along_axis(want, 2 * ri.astype(np.int64), v0, -1)
+    np.put_along_axis(want, 2 * ri.astype(np.int64) + 1, v1, -1)
+    # torch's device division may differ in the last place of code / half (values near 1): an absolute
+    # 2^-22 of the row's scale
+    assert np.all(np.abs(dec - want) <= 2.5e-7 * rs.astype(np.float32)[:, None])
+    e0 = tri.encoder.encode(xt[:0])
+    assert e0.indices.shape == (0, F) and e0.packed.shape[0] == 0
+
+
+def test_paged_decode_post_rope_vs_oracle(dev):
+    """The paged kernel with pre_rope=False: block pool of int4 rows, ragged contexts, against the oracle's
+    fetch_sequence + decode_step per sequence."""
+    from aitherkvcache_amd.triattention import SpectralKVCache
+    KVH, QH, BS = 8, 32, 16
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, num_kv_heads=KVH, num_query_heads=QH, block_size=BS,
+                             pre_rope=False)
+    tri = TriAttention(cfg, device=str(dev))
+    cache = SpectralKVCache(cfg, max_blocks=64, device=str(dev))
+    rng = np.random.default_rng(77)
+    ctx = np.array([200, 0, 33, 512], dtype=np.int64)
+    B, MB = len(ctx), 32
+    perm = rng.permutation(64)
+    bt = np.zeros((B, MB), dtype=np.int32)
+    used = 0
+    for b in range(B):
+        nb = -(-int(ctx[b]) // BS)
+        bt[b, :nb] = perm[used:used + nb]          # 13 + 0 + 3 + 32 blocks of the 64
+        used += nb
+    keys = rng.standard_normal((64 * BS, KVH, 128)).astype(np.float16)
+    vals = rng.standard_normal((64 * BS, KVH, 128)).astype(np.float16)
+    ke = tri.encoder.encode(t(keys, dev))
+    ve = tri.encoder.encode(t(vals, dev))
+    for dst, src in zip(cache._arrays(), tuple(ke) + tuple(ve)):
+        dst.copy_(src.reshape(dst.shape))
+    q = rng.standard_normal((B, QH, 128)).astype(np.float32)
+    out = tri.decode_step_paged(t(q, dev), cache, t(bt, dev), t(ctx, dev)).cpu().numpy()
+    arrays = tuple(a.cpu().numpy() for a in cache._arrays())
+    ref = O.tri_decode_step_paged(q, arrays, bt, ctx, BS, tri._theta.cpu().numpy(), None, 4, False)
+    err = np.max(np.abs(out - ref))
+    print(f"[tri paged post-rope] max|diff|={err:.2e}")
+    assert err <= TOL and np.all(out[1] == 0)
+    # and it differs from the pre-RoPE result (the flag is not ignored)
+    tri_pre = TriAttention(TriAttentionConfig(head_dim=128, num_freqs=12, num_kv_heads=KVH, num_query_heads=QH,
+                                              block_size=BS), device=str(dev))
+    out_pre = tri_pre.decode_step_paged(t(q, dev), cache, t(bt, dev), t(ctx, dev)).cpu().numpy()
+    assert np.max(np.abs(out_pre - out)) > 1e-3
+
+
+def test_width_argument_checks(dev):
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=8, num_kv_heads=2, num_query_heads=8)
+    tri = TriAttention(cfg, device=str(dev))
+    x = torch.randn(1, 10, 2, 128, device=dev).half()
+    k_enc, v_enc = tri.encode_kv(x, x)
+    assert k_enc.packed.shape == (1, 10, 2, 24)
+    tri4 = TriAttention(TriAttentionConfig(head_dim=128, num_freqs=12, num_kv_heads=2, num_query_heads=8), device=str(dev))
+    with pytest.raises(ValueError):          # 8-bit rows handed to a 4-bit configuration
+        tri4.decode_step(torch.randn(1, 8, 128, device=dev), k_enc, v_enc)
+    from aitherkvcache_amd import _lib
+    L = _lib.lib()
+    rc = L.akv_tri_encode(x.data_ptr(), _lib.dtype_code(x), 20, 128, 128, 12, 5, x.data_ptr(), x.data_ptr(), x.data_ptr(), None)
+    assert rc == _lib.AKV_ERR_INVALID

@@ -131,6 +131,29 @@ def test_tri_matches_reference(golden):
     assert np.max(np.abs(o2 - golden["tri_out_explicit_pos"])) < 1e-6
 
 
+@pytest.mark.parametrize("bits,pre", [(8, True), (16, True), (4, False), (8, False), (16, False)])
+def test_tri_coefficient_widths_and_post_rope_match_reference(golden, tri_widths, bits, pre):
+    """Encodings bit for bit; scores and outputs to a few float32 ulps of their sums (numpy's and torch's
+    cos / sin / exp and summation order differ in the last place)."""
+    g, th = tri_widths, golden["theta_d128_base1e6"]
+    tag = f"b{bits}_{'pre' if pre else 'post'}"
+    for nm, src in (("k", g["keys"]), ("v", g["vals"])):
+        i, p, s = O.spectral_encode(src, 12, bits)
+        assert np.array_equal(i, g[f"enc_b{bits}_{nm}_indices"])
+        assert p.dtype == g[f"enc_b{bits}_{nm}_packed"].dtype and np.array_equal(p, g[f"enc_b{bits}_{nm}_packed"])
+        assert np.array_equal(s, g[f"enc_b{bits}_{nm}_scales"])
+    ke = tuple(g[f"enc_b{bits}_k_{n}"] for n in ("indices", "packed", "scales"))
+    ve = tuple(g[f"enc_b{bits}_v_{n}"] for n in ("indices", "packed", "scales"))
+    sc = O.tri_scores(g["q"], *ke, th, g["qpos"], g["kpos"], bits, pre)
+    assert np.max(np.abs(sc - g[f"scores_{tag}"])) < 2e-6
+    o = O.tri_decode_step(g["q"], ke, ve, th, g["qpos"], g["kpos"], bits, pre)
+    assert np.max(np.abs(o - g[f"out_{tag}"])) < 1e-6
+    o = O.tri_decode_step(g["q"], ke, ve, th, None, None, bits, pre)
+    assert np.max(np.abs(o - g[f"out_default_pos_{tag}"])) < 1e-6
+    if not pre:      # positions play no part in the plain dot product
+        assert np.array_equal(g[f"out_{tag}"], g[f"out_default_pos_{tag}"])
+
+
 # ---- block selector (vectors written by tests/golden/make_golden_block_selector.py) -------------
 @pytest.fixture(scope="module")
 def bsel():
