@@ -410,11 +410,6 @@ __device__ __forceinline__ float tri_wave_max(float v) {
   return fmaxf(__uint_as_float(y[0]), __uint_as_float(y[1]));
 }
 
-static size_t tri_heads_lds_bytes(int kvh, int gqa_pass) {
-  return 64 * sizeof(float) + (size_t)kvh * 64 * (gqa_pass * 8 + TRH_Q_PAD) + 64 +
-         4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRH_WAVE_BYTES;
-}
-
 // PAGED: the arrays are a block pool, batch element b reads its tokens through row b of the block
 // table up to its own context length (SpectralKVCache.fetch_sequence,
 // aither_kvcache/triattention/cache.py:163-198, fused into the load; a chunk of 64 tokens is then
@@ -423,8 +418,23 @@ typedef __attribute__((address_space(3))) const float tri_lds_cfloat;
 typedef float tri_f32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) const tri_f32x2 tri_lds_cfloat2;
 
+// Two wavefronts per kv head.  The SCORE wavefront of head h (wavefront h) forms the scores of a chunk of 64
+// tokens (lane = token), keeps the running softmax and leaves the weights (x value scale, float16 hi + lo)
+// and the factors by which earlier sums shrink in LDS; the VALUE wavefront (wavefront KVH + h) scatters the
+// chunk's value coefficients into its dense tile and, one chunk behind, multiplies them by those weights on
+// the matrix cores.  The two workgroup barriers that order the staging area also order the hand-over
+// (weights are double-buffered).  Four wavefronts share a SIMD instead of two: the chains of dependent
+// LDS reads, transcendentals and products of one role run in the shadow of the other's.
+#define TRR_WAVE_BYTES (TRH_VT_BYTES + 2 * 4 * TRH_WT_PITCH)
+#define TRR_ALPHA_FLOATS 8          // per (buffer, head): four factors, then a flag "some factor differs from one"
+
+static size_t tri_roles_lds_bytes(int kvh, int gqa_pass) {
+  return 64 * sizeof(float) + (size_t)kvh * 64 * (gqa_pass * 8 + TRH_Q_PAD) + 64 +
+         4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRR_WAVE_BYTES + 2 * (size_t)kvh * TRR_ALPHA_FLOATS * sizeof(float);
+}
+
 template <int GQ, bool PAGED>
-__global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
+__global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int KVH = a.KVH;
   float* theta = (float*)lds_raw;                               // [64]
@@ -432,15 +442,19 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   constexpr int QROW = GQ * 8 + TRH_Q_PAD;                      // bytes of one pair's row of the query table
   unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // [4 arrays][KVH] x TRH_HEAD_PITCH
   unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
-  const int tid = threadIdx.x, lane = tid & 63, h = tid >> 6;   // wavefront = kv head
-  unsigned char* vt = tiles + (size_t)h * TRH_WAVE_BYTES;
-  unsigned char* wt = vt + TRH_VT_BYTES;
-  for (int i = lane; i < TRH_WAVE_BYTES / 4; i += 64) ((uint32_t*)vt)[i] = 0u;
+  float* alpha_lds = (float*)(tiles + (size_t)KVH * TRR_WAVE_BYTES);             // [2][KVH][TRR_ALPHA_FLOATS]
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const bool value_role = wv >= KVH;                            // wavefront-uniform
+  const int h = value_role ? wv - KVH : wv;
+  unsigned char* vt = tiles + (size_t)h * TRR_WAVE_BYTES;
+  unsigned char* wt0 = vt + TRH_VT_BYTES;                        // weight buffer i at wt0 + i * 4 * TRH_WT_PITCH
+  if (value_role) {   // every use leaves the tile zero again; weight rows of absent query heads stay zero
+    for (int i = lane; i < TRR_WAVE_BYTES / 4; i += 64) ((uint32_t*)vt)[i] = 0u;
+  }
   const int col_n = lane & 15, grp = lane >> 4;
   const int col_q = col_n & 3, col_e = (col_n >> 2) & 1;
   // a weight dword is (hi | lo << 16) of one token: the lane takes its half into its parity slot
   const uint32_t sel_w = (col_n >> 3) ? (col_e ? 0x03020c0cu : 0x0c0c0302u) : (col_e ? 0x01000c0cu : 0x0c0c0100u);
-  const unsigned char* wt_rd = wt + col_q * TRH_WT_PITCH + 16 * grp;
   const unsigned char* vt_rd = vt + col_n * TRH_VT_PITCH + 16 * grp;
   const int gqa = a.QH / KVH;
   const int b = blockIdx.y, split = blockIdx.x;
@@ -456,15 +470,20 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
   const bool kp_wide = a.kpos && a.kp_itype == AKV_I64;
   const unsigned char* kp_base = a.kpos ? (const unsigned char*)a.kpos : (const unsigned char*)a.theta;
 
-  // the thread's row of a chunk: token tid / KVH, head tid % KVH
-  const int my_t = tid / KVH, my_h = tid - my_t * KVH;
-  unsigned char* st_wr = stage + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
-  const unsigned char* st_rd = stage + (size_t)h * TRH_HEAD_PITCH + lane * 16;
+  // the thread's row of a chunk: token r / KVH, head r % KVH; the first KVH wavefronts fetch the key arrays,
+  // the others the value arrays
+  const int r = tid - (value_role ? KVH * 64 : 0);
+  const int my_t = r / KVH, my_h = r - my_t * KVH;
   const size_t arr = (size_t)KVH * TRH_HEAD_PITCH;
+  unsigned char* st_wr = stage + (value_role ? 2 * arr : 0) + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
+  const unsigned char* st_rd = stage + (value_role ? 2 * arr : 0) + (size_t)h * TRH_HEAD_PITCH + lane * 16;
   const int64_t last_row = ((int64_t)b * a.S + max(s1, (int64_t)1)) * KVH - 1;
+  const uint8_t* src_idx = value_role ? a.v_idx : a.k_idx;
+  const uint8_t* src_cf = value_role ? a.v_cf : a.k_cf;
+  const unsigned short* src_sc = (const unsigned short*)(value_role ? a.v_sc : a.k_sc);
 
-  struct tri_rows { uint32_t x[4][3]; unsigned short ksc, vsc; uint32_t kp_lo, kp_hi; };
-  auto fetch = [&](tri_rows& r, int64_t c0) {
+  struct tri_rows { uint32_t x[2][3]; unsigned short sc; uint32_t kp_lo, kp_hi; };
+  auto fetch = [&](tri_rows& rr, int64_t c0) {
     int64_t row;
     if (PAGED) {
       const int64_t tcl = max((int64_t)0, min(c0 + my_t, s1 - 1));           // tokens past the range: its last token
@@ -473,21 +492,18 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       phys = max((int64_t)0, min(phys, a.num_blocks - 1));                   // (an empty sequence reads a padding entry)
       row = ((phys * a.block_size) + (tcl - blk * a.block_size)) * KVH + my_h;
     } else {
-      row = min(((int64_t)b * a.S + c0) * KVH + tid, last_row);              // rows past the range: its last row
+      row = min(((int64_t)b * a.S + c0) * KVH + r, last_row);                // rows past the range: its last row
     }
-    const uint32_t* p0 = (const uint32_t*)(a.k_idx + row * 12);
-    const uint32_t* p1 = (const uint32_t*)(a.k_cf + row * 12);
-    const uint32_t* p2 = (const uint32_t*)(a.v_idx + row * 12);
-    const uint32_t* p3 = (const uint32_t*)(a.v_cf + row * 12);
+    const uint32_t* p0 = (const uint32_t*)(src_idx + row * 12);
+    const uint32_t* p1 = (const uint32_t*)(src_cf + row * 12);
 #pragma unroll
-    for (int w = 0; w < 3; ++w) { r.x[0][w] = p0[w]; r.x[1][w] = p1[w]; r.x[2][w] = p2[w]; r.x[3][w] = p3[w]; }
-    r.ksc = ((const unsigned short*)a.k_sc)[row];
-    r.vsc = ((const unsigned short*)a.v_sc)[row];
-    // the wavefront's own token positions (lane = token), as two dwords
+    for (int w = 0; w < 3; ++w) { rr.x[0][w] = p0[w]; rr.x[1][w] = p1[w]; }
+    rr.sc = src_sc[row];
+    // the score wavefront's own token positions (lane = token), as two dwords
     const int64_t tc = max((int64_t)0, min(c0 + lane, s1 - 1));
-    const int64_t pe = a.kpos ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
-    r.kp_lo = *(const uint32_t*)(kp_base + pe);
-    r.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
+    const int64_t pe = (a.kpos && !value_role) ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
+    rr.kp_lo = *(const uint32_t*)(kp_base + pe);
+    rr.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
   };
 
   for (int qg = 0; qg < gqa; qg += GQ) {
@@ -503,161 +519,206 @@ __global__ __launch_bounds__(512) void tri_decode_heads_kernel(tri_args a) {
       *(float*)((unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW + (q * 2 + (d & 1)) * 4) = v;
     }
     const uint32_t q_base = 64 * sizeof(float) + (uint32_t)h * 64 * QROW;
-    tri_float4 oacc[4];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
-    float m[GQ], l[GQ];
-#pragma unroll
-    for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
-
+    // One step of the staging pipeline, the same in both roles (two workgroup barriers): the chunk fetched
+    // during the previous step goes to the staging area, the next one is requested, the wavefront's own
+    // two entries per token come back.
     tri_rows nxt;
-    fetch(nxt, s0);
-    for (int64_t c0 = s0; c0 < s1; c0 += 64) {
-      // the chunk fetched during the previous step goes to the staging area, the next one is requested
-#pragma unroll
-      for (int A = 0; A < 4; ++A)
-        *(uint4*)(st_wr + A * arr) = make_uint4(nxt.x[A][0], nxt.x[A][1], nxt.x[A][2], A == 0 ? nxt.ksc : nxt.vsc);
-      const uint32_t kp_lo = nxt.kp_lo, kp_hi = nxt.kp_hi;
+    uint32_t kp_lo = 0, kp_hi = 0;
+    auto stage_step = [&](int64_t c0, uint4& e0, uint4& e1, uint32_t& other_sc) {
+      *(uint4*)(st_wr) = make_uint4(nxt.x[0][0], nxt.x[0][1], nxt.x[0][2], nxt.sc);
+      *(uint4*)(st_wr + arr) = make_uint4(nxt.x[1][0], nxt.x[1][1], nxt.x[1][2], nxt.sc);
+      kp_lo = nxt.kp_lo; kp_hi = nxt.kp_hi;
       __syncthreads();
       fetch(nxt, c0 + 64);
-      const uint4 e0 = *(const uint4*)(st_rd), e1 = *(const uint4*)(st_rd + arr);
-      const uint4 e2 = *(const uint4*)(st_rd + 2 * arr), e3 = *(const uint4*)(st_rd + 3 * arr);
+      e0 = *(const uint4*)(st_rd);
+      e1 = *(const uint4*)(st_rd + arr);
+      // (score wavefront: the value scale of its token, fourth dword of the value index entry)
+      other_sc = *(const uint32_t*)(st_rd + (value_role ? 0 : 2 * arr) + 12);
       __syncthreads();
-      const uint32_t ki[3] = {e0.x, e0.y, e0.z}, kc[3] = {e1.x, e1.y, e1.z};
-      const uint32_t vi[3] = {e2.x, e2.y, e2.z}, vc[3] = {e3.x, e3.y, e3.z};
-      const float ksc = __half2float(__ushort_as_half((unsigned short)e0.w));
-      const float vsc = __half2float(__ushort_as_half((unsigned short)e2.w));
+    };
+    fetch(nxt, s0);
 
-      const int64_t t = c0 + lane;
-      const bool valid = t < s1;
-      const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
-                       : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
-      const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
-      const float kscale = ksc * (inv_sqrt_d / 15.f);
-      float sc[GQ];
+    if (!value_role) {
+      float m[GQ], l[GQ];
 #pragma unroll
-      for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
-      // Per word of four pairs: the index bytes times 4 (a pair index is below 64, so the shift stays
-      // inside its byte) and the two nibbles of every coefficient byte in bytes of their own; a byte
-      // then becomes a float by one conversion.  A code c stands for (2c - 15)/15 x scale -- equal to
-      // the reference's fl(fl(c/7.5) - 1) x scale to a relative 1e-7 -- and scale/15 multiplies the
-      // finished sum instead of every coefficient.
-      uint32_t ki4[3], chi[3], clo[3];
+      for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
+      int buf = 0;
+      for (int64_t c0 = s0; c0 < s1; c0 += 64) {
+        uint4 e0, e1;
+        uint32_t vsc_raw;
+        stage_step(c0, e0, e1, vsc_raw);
+        const int64_t t = c0 + lane;
+        const bool valid = t < s1;
+        const uint32_t ki[3] = {e0.x, e0.y, e0.z}, kc[3] = {e1.x, e1.y, e1.z};
+        const float ksc = __half2float(__ushort_as_half((unsigned short)e0.w));
+        const float vsc = __half2float(__ushort_as_half((unsigned short)vsc_raw));
+        const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
+                         : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
+        const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
+        const float kscale = ksc * (inv_sqrt_d / 15.f);
+        float sc[GQ];
 #pragma unroll
-      for (int w = 0; w < 3; ++w) {
-        ki4[w] = (ki[w] & 0x3f3f3f3fu) << 2;
-        chi[w] = (kc[w] >> 4) & 0x0f0f0f0fu;
-        clo[w] = kc[w] & 0x0f0f0f0fu;
-      }
+        for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+        // Per word of four pairs: the index bytes times 4 (a pair index is below 64, so the shift stays
+        // inside its byte) and the two nibbles of every coefficient byte in bytes of their own; a byte
+        // then becomes a float by one conversion.  A code c stands for (2c - 15)/15 x scale -- equal to
+        // the reference's fl(fl(c/7.5) - 1) x scale to a relative 1e-7 -- and scale/15 multiplies the
+        // finished sum instead of every coefficient.
+        uint32_t ki4[3], chi[3], clo[3];
 #pragma unroll
-      for (int f = 0; f < 12; ++f) {
-        const uint32_t idx4 = (ki4[f >> 2] >> (8 * (f & 3))) & 255u;          // byte offset of theta[idx]
-        const float k0 = fmaf((float)((chi[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
-        const float k1 = fmaf((float)((clo[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
-        // (the dynamic LDS of this kernel starts at LDS address 0 and theta is its first object: the
-        // byte offset is the address, no base to add)
-        const float ph = __fmul_rn(delta, *(tri_lds_cfloat*)(uintptr_t)idx4);
-        float sn, cs;
-        tri_sincos(ph, sn, cs);
-        const float ka = k0 * cs - k1 * sn;
-        const float kb = k1 * cs + k0 * sn;
-        const uint32_t qrow = idx4 * (QROW / 4) + q_base;      // LDS address of the pair's row of this head
+        for (int w = 0; w < 3; ++w) {
+          ki4[w] = (ki[w] & 0x3f3f3f3fu) << 2;
+          chi[w] = (kc[w] >> 4) & 0x0f0f0f0fu;
+          clo[w] = kc[w] & 0x0f0f0f0fu;
+        }
+#pragma unroll
+        for (int f = 0; f < 12; ++f) {
+          const uint32_t idx4 = (ki4[f >> 2] >> (8 * (f & 3))) & 255u;          // byte offset of theta[idx]
+          const float k0 = fmaf((float)((chi[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
+          const float k1 = fmaf((float)((clo[f >> 2] >> (8 * (f & 3))) & 255u), 2.f, -15.f);
+          // (the dynamic LDS of this kernel starts at LDS address 0 and theta is its first object: the
+          // byte offset is the address, no base to add)
+          const float ph = __fmul_rn(delta, *(tri_lds_cfloat*)(uintptr_t)idx4);
+          float sn, cs;
+          tri_sincos(ph, sn, cs);
+          const float ka = k0 * cs - k1 * sn;
+          const float kb = k1 * cs + k0 * sn;
+          const uint32_t qrow = idx4 * (QROW / 4) + q_base;      // LDS address of the pair's row of this head
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) {
+            const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
+            sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+          }
+          // (with 128 registers per lane the query rows of all twelve pairs cannot be requested at once)
+          if ((f & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+        float p[GQ], alpha[GQ];
+        bool rescale = false;
+        const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
-          sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+          const float sv = valid ? sc[q] * kscale : -INFINITY;
+          const float mn = fmaxf(m[q], tri_wave_max(sv + bias));
+          alpha[q] = __expf(m[q] - mn);
+          rescale |= (mn != m[q]);
+          p[q] = valid ? __expf(sv - mn) : 0.f;
+          l[q] = l[q] * alpha[q] + p[q];
+          m[q] = mn;
         }
+        unsigned char* wt = wt0 + buf * 4 * TRH_WT_PITCH;
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) {
+          const float w = p[q] * vsc * TRI_WSCALE;
+          auto h2 = __builtin_amdgcn_cvt_pkrtz(w, 0.f);
+          auto l2 = __builtin_amdgcn_cvt_pkrtz(w - (float)h2[0], 0.f);
+          union { decltype(h2) hv; uint32_t u; } hb, lb;
+          hb.hv = h2; lb.hv = l2;
+          *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = (hb.u & 0xffffu) | (lb.u << 16);
+        }
+        if (lane < 5) {          // m is the same in every lane, and so are the factors
+          float* al = alpha_lds + ((size_t)buf * KVH + h) * TRR_ALPHA_FLOATS;
+          float av = rescale ? 1.f : 0.f;
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) av = lane == q ? alpha[q] : av;
+          if (lane < GQ || lane == 4) al[lane] = av;
+        }
+        buf ^= 1;
       }
-      float p[GQ], alpha[GQ];
-      bool rescale = false;
-      const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
+      __syncthreads();             // (the value wavefronts wait here for the weights of the last chunk)
 #pragma unroll
       for (int q = 0; q < GQ; ++q) {
-        const float sv = valid ? sc[q] * kscale : -INFINITY;
-        const float mn = fmaxf(m[q], tri_wave_max(sv + bias));
-        alpha[q] = __expf(m[q] - mn);
-        rescale |= (mn != m[q]);
-        p[q] = valid ? __expf(sv - mn) : 0.f;
-        l[q] = l[q] * alpha[q] + p[q];
-        m[q] = mn;
+        const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
+        const float lsum = akv_wave_sum(l[q]);
+        if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
       }
-      if (rescale) {  // wavefront-uniform: m is the same in every lane
-        float asel = alpha[0];
-        if (GQ == 4) asel = col_q == 1 ? alpha[1 % GQ] : col_q == 2 ? alpha[2 % GQ] : col_q == 3 ? alpha[3 % GQ] : asel;
+    } else {
+      tri_float4 oacc[4];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) oacc[mt] *= asel;
-      }
+      for (int mt = 0; mt < 4; ++mt) oacc[mt] = (tri_float4){0.f, 0.f, 0.f, 0.f};
+      // tile entries of the chunk whose weights are still being made
+      uint32_t voff[12], vval[12];
+      bool have_prev = false, prev_valid = false;
+      // weights of buffer bufc times the tile entries kept in voff / vval
+      auto consume = [&](int bufc) {
+        const float* al = alpha_lds + ((size_t)bufc * KVH + h) * TRR_ALPHA_FLOATS;
+        if (al[4] != 0.f) {      // wavefront-uniform
+          const float asel = al[GQ == 4 ? col_q : 0];
 #pragma unroll
-      for (int q = 0; q < GQ; ++q) {
-        const float w = p[q] * vsc * TRI_WSCALE;
-        auto h2 = __builtin_amdgcn_cvt_pkrtz(w, 0.f);
-        auto l2 = __builtin_amdgcn_cvt_pkrtz(w - (float)h2[0], 0.f);
-        union { decltype(h2) hv; uint32_t u; } hb, lb;
-        hb.hv = h2; lb.hv = l2;
-        *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = (hb.u & 0xffffu) | (lb.u << 16);
-      }
-      // tile entries of the lane's token: address and (2a - 15, 2b - 15) as a float16 pair, formed once
-      // (0x6400 + n is float16(1024 + n); minus 1039 is exact)
-      uint32_t voff[12];
-      uint32_t vval[12];
-#pragma unroll
-      for (int f = 0; f < 12; ++f) {
-        const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
-        const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
-        union { uint32_t u; tri_half2 hv; } cv;
-        cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
-        cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
-        vval[f] = cv.u;
-        voff[f] = idx * TRH_VT_PITCH + 4 * (lane & 31);
-      }
-#pragma unroll
-      for (int pass = 0; pass < 2; ++pass) {      // the tile holds 32 tokens
-        const bool mine = valid && (lane >> 5) == pass;
-        if (mine) {
-#pragma unroll
-          for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = vval[f];
+          for (int mt = 0; mt < 4; ++mt) oacc[mt] *= asel;
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const unsigned char* wt_rd = wt0 + bufc * 4 * TRH_WT_PITCH + col_q * TRH_WT_PITCH + 16 * grp;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const uint4 wr = *(const uint4*)(wt_rd + 64 * (2 * pass + ks));
-          union { uint32_t u[4]; tri_half8 hv; } bw;
-          bw.u[0] = __builtin_amdgcn_perm(wr.x, wr.x, sel_w);
-          bw.u[1] = __builtin_amdgcn_perm(wr.y, wr.y, sel_w);
-          bw.u[2] = __builtin_amdgcn_perm(wr.z, wr.z, sel_w);
-          bw.u[3] = __builtin_amdgcn_perm(wr.w, wr.w, sel_w);
+        for (int pass = 0; pass < 2; ++pass) {      // the tile holds 32 tokens
+          const bool mine = prev_valid && (lane >> 5) == pass;
+          if (mine) {
 #pragma unroll
-          for (int mt = 0; mt < 4; ++mt) {
-            union { uint4 u; tri_half8 hv; } av;
-            av.u = *(const uint4*)(vt_rd + mt * 16 * TRH_VT_PITCH + 64 * ks);
-            oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.hv, bw.hv, oacc[mt], 0, 0, 0);
+            for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = vval[f];
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) {
+            const uint4 wr = *(const uint4*)(wt_rd + 64 * (2 * pass + ks));
+            union { uint32_t u[4]; tri_half8 hv; } bw;
+            bw.u[0] = __builtin_amdgcn_perm(wr.x, wr.x, sel_w);
+            bw.u[1] = __builtin_amdgcn_perm(wr.y, wr.y, sel_w);
+            bw.u[2] = __builtin_amdgcn_perm(wr.z, wr.z, sel_w);
+            bw.u[3] = __builtin_amdgcn_perm(wr.w, wr.w, sel_w);
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+              union { uint4 u; tri_half8 hv; } av;
+              av.u = *(const uint4*)(vt_rd + mt * 16 * TRH_VT_PITCH + 64 * ks);
+              oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av.hv, bw.hv, oacc[mt], 0, 0, 0);
+            }
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          if (mine) {
+#pragma unroll
+            for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = 0u;
           }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (mine) {
+      };
+      int buf = 0;
+      for (int64_t c0 = s0; c0 < s1; c0 += 64) {
+        uint4 e0, e1;
+        uint32_t unused;
+        stage_step(c0, e0, e1, unused);
+        if (have_prev) consume(buf ^ 1);
+        // tile entries of the lane's token: address and (2a - 15, 2b - 15) as a float16 pair, formed once
+        // (0x6400 + n is float16(1024 + n); minus 1039 is exact)
+        const uint32_t vi[3] = {e0.x, e0.y, e0.z}, vc[3] = {e1.x, e1.y, e1.z};
 #pragma unroll
-          for (int f = 0; f < 12; ++f) *(uint32_t*)(vt + voff[f]) = 0u;
+        for (int f = 0; f < 12; ++f) {
+          const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
+          const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
+          union { uint32_t u; tri_half2 hv; } cv;
+          cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+          cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
+          vval[f] = cv.u;
+          voff[f] = idx * TRH_VT_PITCH + 4 * (lane & 31);
         }
+        have_prev = true;
+        prev_valid = c0 + lane < s1;
+        buf ^= 1;
       }
-    }
+      __syncthreads();             // the weights of the last chunk
+      if (have_prev) consume(buf ^ 1);
 #pragma unroll
-    for (int q = 0; q < GQ; ++q) {
-      const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
-      const float lsum = akv_wave_sum(l[q]);
+      for (int q = 0; q < GQ; ++q) {
+        const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float hi = oacc[mt][i];
-          const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
-          if (col_n < 8 && col_q == q)
-            a.part_acc[slot * 128 + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
-        }
-      if (lane == 0) { a.part_ml[slot * 2] = m[q]; a.part_ml[slot * 2 + 1] = lsum; }
+          for (int i = 0; i < 4; ++i) {
+            const float hi = oacc[mt][i];
+            const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
+            if (col_n < 8 && col_q == q)
+              a.part_acc[slot * 128 + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
+          }
+      }
     }
   }
 }
@@ -787,7 +848,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   if (dense && f12 && num_kv_heads <= 8) {
     // one workgroup per (token range, batch element), a wavefront per kv head
     const int gq = gqa % 4 == 0 ? 4 : 1;
-    const size_t lds = tri_heads_lds_bytes(num_kv_heads, gq);
+    const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq);
     if (lds <= 160 * 1024) {
       int cus = akv_cached_cu_count();
       if (cus <= 0) cus = 256;
@@ -806,8 +867,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
         configured = lds;
       }
       dim3 hgrid(a.nsplit, batch);
-      if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, false>), hgrid, num_kv_heads * 64, lds, stream, a);
-      else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, false>), hgrid, num_kv_heads * 64, lds, stream, a);
+      if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, false>), hgrid, num_kv_heads * 128, lds, stream, a);
+      else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, false>), hgrid, num_kv_heads * 128, lds, stream, a);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
       AKV_LAUNCH_CHECK("tri_reduce_kernel");
@@ -869,7 +930,7 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const bool aligned = ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
   const int gqa = num_q_heads / num_kv_heads;
   const int gq = gqa % 4 == 0 ? 4 : 1;
-  const size_t lds = tri_heads_lds_bytes(num_kv_heads, gq);
+  const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq);
   if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024)
     return akv_fail(AKV_ERR_UNSUPPORTED,
                     "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads and 4-byte "
@@ -916,8 +977,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
     configured = lds;
   }
   dim3 hgrid(a.nsplit, batch);
-  if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, true>), hgrid, num_kv_heads * 64, lds, stream, a);
-  else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, true>), hgrid, num_kv_heads * 64, lds, stream, a);
+  if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, true>), hgrid, num_kv_heads * 128, lds, stream, a);
+  else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, true>), hgrid, num_kv_heads * 128, lds, stream, a);
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
