@@ -62,16 +62,17 @@ __device__ __forceinline__ float tri_dequant(uint32_t code, float scale) {
   return __fmul_rn(__fsub_rn(__fdiv_rn((float)code, 7.5f), 1.0f), scale);
 }
 
-// sin and cos of a float32 angle of any size reached by positions x frequencies (|x| < ~1e6):
-// k = rint(x / 2 pi), remainder r = x - k 2 pi by two fused multiply-adds (2 pi = C1 + C2 with C1 the
-// nearest float: k C1 is exact inside the first one, and its result is exact too), then the hardware
-// sine and cosine, which take their argument in revolutions and are good to 1.3e-7 absolute on
-// [-1/2, 1/2] (measured against double precision over 2^22 arguments).
+// sin and cos of a float32 angle of any size reached by positions x frequencies (|x| < ~1e6), in
+// revolutions: 1 / 2 pi = H + L with H the nearest float; k = rint(fl(x H)); the fused multiply-add
+// x H - k is the exact product minus an integer, rounded once at the size of the remainder, and a second
+// one adds x L.  The remainder is good to 6e-8 revolutions (checked against 80-bit arithmetic over 2e6
+// arguments up to 1e6 rad; it can exceed 1/2 by the rounding of x H, which the hardware functions allow).
+// The hardware sine and cosine take revolutions and are good to 1.3e-7 absolute on [-1/2, 1/2] (measured
+// against double precision over 2^22 arguments).
 __device__ __forceinline__ void tri_sincos(float x, float& sn, float& cs) {
-  const float k = rintf(x * 0.15915494309189535f);
-  float r = fmaf(k, -6.2831854820251465f, x);
-  r = fmaf(k, 1.7484555e-07f, r);
-  const float f = r * 0.15915494309189535f;
+  const float k = rintf(x * 0.15915493667125702f);
+  float f = fmaf(x, 0.15915493667125702f, -k);
+  f = fmaf(x, 6.4206382432985265e-09f, f);
   sn = __builtin_amdgcn_sinf(f);
   cs = __builtin_amdgcn_cosf(f);
 }
@@ -400,6 +401,36 @@ __device__ __forceinline__ float tri_row16_max(float v) {
       : "+v"(v));
   return v;
 }
+// the same for four values at once: the four chains alternate, so no instruction reads the result of the
+// one before it and the idle cycles are not needed after the first
+__device__ __forceinline__ void tri_row16_max4(float& a, float& b, float& c, float& d) {
+  asm("s_nop 1\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %2, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %3, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %2, %2, %2 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %3, %3, %3 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %2, %2, %2 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %3, %3, %3 row_ror:1 row_mask:0xf bank_mask:0xf"
+      : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ __forceinline__ float tri_rows_max(float v) {
+  // the four rows: v_permlane32_swap / v_permlane16_swap fed the same value twice leave
+  // (rows 0,1,0,1 | 2,3,2,3) and (rows 0,0,2,2 | 1,1,3,3)
+  auto x = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(x[0]), __uint_as_float(x[1]));
+  auto y = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(y[0]), __uint_as_float(y[1]));
+}
 __device__ __forceinline__ float tri_wave_max(float v) {
   v = tri_row16_max(v);
   // the four rows: v_permlane32_swap / v_permlane16_swap fed the same value twice leave
@@ -428,18 +459,24 @@ typedef __attribute__((address_space(3))) const tri_f32x2 tri_lds_cfloat2;
 #define TRR_WAVE_BYTES (TRH_VT_BYTES + 2 * 4 * TRH_WT_PITCH)
 #define TRR_ALPHA_FLOATS 8          // per (buffer, head): four factors, then a flag "some factor differs from one"
 
-static size_t tri_roles_lds_bytes(int kvh, int gqa_pass) {
-  return 64 * sizeof(float) + (size_t)kvh * 64 * (gqa_pass * 8 + TRH_Q_PAD) + 64 +
+// bytes of one pair's row of the query table: float16 queries are kept as they are (GQ x (even, odd) halves; the
+// multiply-adds take them directly), others as float32 with 16 bytes of padding
+static constexpr int tri_qrow_bytes(int gqa_pass, bool q_half) { return q_half ? gqa_pass * 4 : gqa_pass * 8 + TRH_Q_PAD; }
+
+static size_t tri_roles_lds_bytes(int kvh, int gqa_pass, bool q_half) {
+  return 64 * sizeof(float) + (size_t)kvh * 64 * tri_qrow_bytes(gqa_pass, q_half) + 64 +
          4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRR_WAVE_BYTES + 2 * (size_t)kvh * TRR_ALPHA_FLOATS * sizeof(float);
 }
 
-template <int GQ, bool PAGED>
+typedef __attribute__((address_space(3))) const tri_half2 tri_lds_chalf2;
+
+template <int GQ, bool PAGED, bool QH16>
 __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int KVH = a.KVH;
   float* theta = (float*)lds_raw;                               // [64]
   float* q_lds = theta + 64;                                    // [KVH][64 pairs][GQ][even, odd]
-  constexpr int QROW = GQ * 8 + TRH_Q_PAD;                      // bytes of one pair's row of the query table
+  constexpr int QROW = tri_qrow_bytes(GQ, QH16);                // bytes of one pair's row of the query table
   unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // [4 arrays][KVH] x TRH_HEAD_PITCH
   unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
   float* alpha_lds = (float*)(tiles + (size_t)KVH * TRR_WAVE_BYTES);             // [2][KVH][TRR_ALPHA_FLOATS]
@@ -512,11 +549,16 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
       const int hh = i / (GQ * 128), rem = i - hh * (GQ * 128);
       const int q = rem >> 7, d = rem & 127;
       const int64_t off = ((int64_t)b * a.QH + (hh * gqa + qg + q)) * 128 + d;
-      float v;
-      if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
-      else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
-      else v = akv_elem<AKV_F32>::load(a.query, off);
-      *(float*)((unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW + (q * 2 + (d & 1)) * 4) = v;
+      unsigned char* row = (unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW;
+      if (QH16) {
+        *(unsigned short*)(row + (q * 2 + (d & 1)) * 2) = ((const unsigned short*)a.query)[off];
+      } else {
+        float v;
+        if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
+        else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
+        else v = akv_elem<AKV_F32>::load(a.query, off);
+        *(float*)(row + (q * 2 + (d & 1)) * 4) = v;
+      }
     }
     const uint32_t q_base = 64 * sizeof(float) + (uint32_t)h * 64 * QROW;
     // One step of the staging pipeline, the same in both roles (two workgroup barriers): the chunk fetched
@@ -570,6 +612,11 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
           ki4[w] = (ki[w] & 0x3f3f3f3fu) << 2;
           chi[w] = (kc[w] >> 4) & 0x0f0f0f0fu;
           clo[w] = kc[w] & 0x0f0f0f0fu;
+          // (kept opaque: otherwise the masks are folded into one bit-field extract per code and the
+          // conversion no longer selects its byte by itself)
+          asm("" : "+v"(ki4[w]));
+          asm("" : "+v"(chi[w]));
+          asm("" : "+v"(clo[w]));
         }
 #pragma unroll
         for (int f = 0; f < 12; ++f) {
@@ -586,8 +633,13 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
           const uint32_t qrow = idx4 * (QROW / 4) + q_base;      // LDS address of the pair's row of this head
 #pragma unroll
           for (int q = 0; q < GQ; ++q) {
-            const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
-            sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+            if (QH16) {
+              const tri_half2 qq = *(tri_lds_chalf2*)(uintptr_t)(qrow + 4 * q);
+              sc[q] = fmaf((float)qq.y, kb, fmaf((float)qq.x, ka, sc[q]));
+            } else {
+              const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
+              sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+            }
           }
           // (with 128 registers per lane the query rows of all twelve pairs cannot be requested at once)
           if ((f & 3) == 3) __builtin_amdgcn_sched_barrier(0);
@@ -595,13 +647,26 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
         float p[GQ], alpha[GQ];
         bool rescale = false;
         const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
+        float sv[GQ], mx[GQ];
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float sv = valid ? sc[q] * kscale : -INFINITY;
-          const float mn = fmaxf(m[q], tri_wave_max(sv + bias));
+          sv[q] = valid ? sc[q] * kscale : -INFINITY;
+          mx[q] = sv[q] + bias;
+        }
+        if (GQ == 4) {
+          tri_row16_max4(mx[0], mx[1 % GQ], mx[2 % GQ], mx[3 % GQ]);
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) mx[q] = tri_rows_max(mx[q]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) mx[q] = tri_wave_max(mx[q]);
+        }
+#pragma unroll
+        for (int q = 0; q < GQ; ++q) {
+          const float mn = fmaxf(m[q], mx[q]);
           alpha[q] = __expf(m[q] - mn);
           rescale |= (mn != m[q]);
-          p[q] = valid ? __expf(sv - mn) : 0.f;
+          p[q] = valid ? __expf(sv[q] - mn) : 0.f;
           l[q] = l[q] * alpha[q] + p[q];
           m[q] = mn;
         }
@@ -689,16 +754,20 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
         if (have_prev) consume(buf ^ 1);
         // tile entries of the lane's token: address and (2a - 15, 2b - 15) as a float16 pair, formed once
         // (0x6400 + n is float16(1024 + n); minus 1039 is exact)
+        // (the nibbles of a word of four coefficient bytes in bytes of their own; one byte permute then
+        // puts a pair's two codes into the low bytes of the two halves)
         const uint32_t vi[3] = {e0.x, e0.y, e0.z}, vc[3] = {e1.x, e1.y, e1.z};
+        const uint32_t lane_off = 4 * (lane & 31);
 #pragma unroll
         for (int f = 0; f < 12; ++f) {
           const uint32_t idx = (vi[f >> 2] >> (8 * (f & 3))) & 63u;
-          const uint32_t cf = (vc[f >> 2] >> (8 * (f & 3))) & 255u;
+          const uint32_t hiw = (vc[f >> 2] >> 4) & 0x0f0f0f0fu, low = vc[f >> 2] & 0x0f0f0f0fu;
+          const uint32_t pair = __builtin_amdgcn_perm(low, hiw, 0x0c040c00u + 0x00010001u * (f & 3));
           union { uint32_t u; tri_half2 hv; } cv;
-          cv.u = (((cf >> 4) | ((cf & 15u) << 16)) << 1) + 0x64006400u;
+          cv.u = (pair << 1) + 0x64006400u;
           cv.hv = cv.hv - (tri_half2){(_Float16)1039.f, (_Float16)1039.f};
           vval[f] = cv.u;
-          voff[f] = idx * TRH_VT_PITCH + 4 * (lane & 31);
+          voff[f] = idx * TRH_VT_PITCH + lane_off;
         }
         have_prev = true;
         prev_valid = c0 + lane < s1;
@@ -776,6 +845,29 @@ __global__ void tri_zero_kernel(float* out, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) out[i] = 0.f;
 }
 
+// launch of the all-heads kernel for (gq, qh, lds, hgrid, num_kv_heads, stream, a) of the caller; more than 64 KB
+// of dynamic LDS has to be allowed once per kernel
+template <int GQ, bool PAGED, bool QH16>
+static int tri_heads_launch(dim3 hgrid, int kvh, size_t lds, hipStream_t stream, const tri_args& a) {
+  static size_t configured = 0;
+  if (configured < lds) {
+    AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<GQ, PAGED, QH16>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    configured = lds;
+  }
+  AKV_LAUNCH_TIMED((tri_decode_heads_kernel<GQ, PAGED, QH16>), hgrid, kvh * 128, lds, stream, a);
+  return AKV_OK;
+}
+#define TRI_HEADS_LAUNCH(PAGED)                                                                                      \
+  do {                                                                                                               \
+    int rc_;                                                                                                         \
+    if (gq == 4) rc_ = qh ? tri_heads_launch<4, PAGED, true>(hgrid, num_kv_heads, lds, stream, a)                    \
+                          : tri_heads_launch<4, PAGED, false>(hgrid, num_kv_heads, lds, stream, a);                  \
+    else rc_ = qh ? tri_heads_launch<1, PAGED, true>(hgrid, num_kv_heads, lds, stream, a)                            \
+                  : tri_heads_launch<1, PAGED, false>(hgrid, num_kv_heads, lds, stream, a);                          \
+    if (rc_ != AKV_OK) return rc_;                                                                                   \
+  } while (0)
+
 static int tri_pick_splits(int batch, int kvh, int64_t S) {
   int cus = akv_cached_cu_count();
   if (cus <= 0) cus = 256;
@@ -848,7 +940,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   if (dense && f12 && num_kv_heads <= 8) {
     // one workgroup per (token range, batch element), a wavefront per kv head
     const int gq = gqa % 4 == 0 ? 4 : 1;
-    const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq);
+    const bool qh = q_dtype == AKV_F16;
+    const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
     if (lds <= 160 * 1024) {
       int cus = akv_cached_cu_count();
       if (cus <= 0) cus = 256;
@@ -859,16 +952,8 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
       if (n < 1) n = 1;
       a.nsplit = (int)n;
       a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
-      static size_t configured4 = 0, configured1 = 0;
-      size_t& configured = gq == 4 ? configured4 : configured1;
-      if (configured < lds) {
-        if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = lds;
-      }
       dim3 hgrid(a.nsplit, batch);
-      if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, false>), hgrid, num_kv_heads * 128, lds, stream, a);
-      else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, false>), hgrid, num_kv_heads * 128, lds, stream, a);
+      TRI_HEADS_LAUNCH(false);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
       AKV_LAUNCH_CHECK("tri_reduce_kernel");
@@ -930,7 +1015,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const bool aligned = ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
   const int gqa = num_q_heads / num_kv_heads;
   const int gq = gqa % 4 == 0 ? 4 : 1;
-  const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq);
+  const bool qh = q_dtype == AKV_F16;
+  const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
   if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024)
     return akv_fail(AKV_ERR_UNSUPPORTED,
                     "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads and 4-byte "
@@ -969,16 +1055,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
-  static size_t configured4 = 0, configured1 = 0;
-  size_t& configured = gq == 4 ? configured4 : configured1;
-  if (configured < lds) {
-    if (gq == 4) AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    else AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    configured = lds;
-  }
   dim3 hgrid(a.nsplit, batch);
-  if (gq == 4) AKV_LAUNCH_TIMED((tri_decode_heads_kernel<4, true>), hgrid, num_kv_heads * 128, lds, stream, a);
-  else AKV_LAUNCH_TIMED((tri_decode_heads_kernel<1, true>), hgrid, num_kv_heads * 128, lds, stream, a);
+  TRI_HEADS_LAUNCH(true);
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
