@@ -1091,11 +1091,14 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
     // The F-th largest key by a bitwise search (largest T with at least F keys >= T: one compare and a
     // population count per bit), then everything above it plus, of the keys equal to it, the lowest
     // lanes -- the order torch.topk's result has once it is sorted by index with ties to the lower index.
+    // (Once exactly F keys reach the threshold the remaining bits cannot change the set: the search stops there,
+    // after about half of its steps on keys without ties.)
     uint32_t T = 0;
-#pragma unroll
     for (int bit = 31; bit >= 0; --bit) {
       const uint32_t cand = T | (1u << bit);
-      if (__popcll(__ballot(key >= cand)) >= F) T = cand;
+      const int cnt = __popcll(__ballot(key >= cand));
+      if (cnt >= F) T = cand;
+      if (cnt == F) break;
     }
     const bool above = key > T, equal = key == T;
     const int need = F - __popcll(__ballot(above));
