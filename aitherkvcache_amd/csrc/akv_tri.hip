@@ -367,6 +367,77 @@ __global__ __launch_bounds__(256) void tri_decode_kernel(tri_args a) {
 }
 
 // ----------------------------------------------------------------------------------
+// TrigSeriesScorer.score alone (aither_kvcache/triattention/scorer.py:115-208): the logits [B][QH][S] as
+// float32, for callers that add a mask or look at the scores themselves (TriAttention.forward with an
+// attention mask, attention.py:148-166).  Lane = token, one pass per group of GQ query heads of the kv head;
+// the arithmetic is that of tri_decode_kernel's score phase.
+// ----------------------------------------------------------------------------------
+template <int GQ>
+__global__ __launch_bounds__(256) void tri_scores_kernel(tri_args a, float* __restrict__ out) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  float* theta = (float*)lds_raw;            // [D/2]
+  float* q_lds = theta + a.D / 2;            // [D/2][GQ][even, odd]
+  float* dq = q_lds + GQ * a.D;              // [256]: code / half - 1 with the reference's roundings
+  const int D = a.D, F = a.F, cb = a.cbits;
+  const int gqa = a.QH / a.KVH;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const bool valid = t < a.S;
+  const int64_t tc = valid ? t : a.S - 1;
+  const float inv_sqrt_d = 1.0f / sqrtf((float)D);
+  for (int i = threadIdx.x; i < D / 2; i += 256) theta[i] = a.theta[i];
+  dq[threadIdx.x] = __fsub_rn(__fdiv_rn((float)threadIdx.x, cb == 8 ? 127.5f : 7.5f), 1.0f);
+  const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)a.S;
+  const float kp = a.kpos ? (float)akv_load_index(a.kpos, a.kp_itype, (int64_t)b * a.S + tc) : (float)tc;
+  const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
+  const int64_t row = ((int64_t)b * a.S + tc) * a.KVH + h;
+  const float ksc = cb == 16 ? 1.f : __half2float(a.k_sc[row]);
+  for (int qg = 0; qg < gqa; qg += GQ) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < GQ * D; i += 256) {
+      const int q = i / D, d = i % D;
+      const int64_t off = ((int64_t)b * a.QH + (h * gqa + qg + q)) * D + d;
+      float v;
+      if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
+      else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
+      else v = akv_elem<AKV_F32>::load(a.query, off);
+      q_lds[((d >> 1) * GQ + q) * 2 + (d & 1)] = v;
+    }
+    __syncthreads();
+    float sc[GQ];
+#pragma unroll
+    for (int q = 0; q < GQ; ++q) sc[q] = 0.f;
+    for (int f = 0; f < F; ++f) {
+      const uint32_t idx = a.k_idx[row * F + f];
+      float k0, k1;
+      if (cb == 4) {
+        const uint32_t cf = a.k_cf[row * F + f];
+        k0 = __fmul_rn(dq[cf >> 4], ksc); k1 = __fmul_rn(dq[cf & 15u], ksc);
+      } else if (cb == 8) {
+        const uint8_t* pc = a.k_cf + (row * F + f) * 2;
+        k0 = __fmul_rn(dq[pc[0]], ksc); k1 = __fmul_rn(dq[pc[1]], ksc);
+      } else {
+        const __half* pc = (const __half*)a.k_cf + (row * F + f) * 2;
+        k0 = __half2float(pc[0]); k1 = __half2float(pc[1]);
+      }
+      float sn, cs;
+      tri_sincos(__fmul_rn(delta, theta[idx]), sn, cs);
+      const float ka = k0 * cs - k1 * sn;
+      const float kb = k1 * cs + k0 * sn;
+#pragma unroll
+      for (int q = 0; q < GQ; ++q) {
+        const float2 qq = *(const float2*)(q_lds + (idx * GQ + q) * 2);
+        sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+      }
+    }
+    if (valid) {
+#pragma unroll
+      for (int q = 0; q < GQ; ++q) out[((int64_t)b * a.QH + (h * gqa + qg + q)) * a.S + t] = sc[q] * inv_sqrt_d;
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------
 // head_dim 128, F = 12, up to 8 kv heads: one workgroup takes a token range for ALL kv heads
 // ----------------------------------------------------------------------------------
 // In the cache a token's rows of the kv heads lie side by side (12 bytes each), so a wavefront that
@@ -1060,6 +1131,42 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
+  return AKV_OK;
+}
+
+extern "C" int akv_tri_scores(const void* query, int q_dtype, const uint8_t* k_indices, const void* k_coeffs,
+                              const void* k_scales, const float* theta, const void* query_pos, int qp_itype,
+                              const void* key_positions, int kp_itype, float* out, int batch, int64_t seq_len,
+                              int num_q_heads, int num_kv_heads, int d, int num_freqs, int coeff_bits, int pre_rope,
+                              void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  AKV_REQUIRE(batch >= 0 && seq_len >= 0 && num_q_heads > 0 && num_kv_heads > 0, "akv_tri_scores: bad sizes");
+  AKV_REQUIRE(num_q_heads % num_kv_heads == 0, "akv_tri_scores: num_q_heads %% num_kv_heads != 0");
+  AKV_REQUIRE(d > 0 && d % 2 == 0 && d <= 512, "akv_tri_scores: head_dim=%d must be even and <= 512", d);
+  AKV_REQUIRE(num_freqs > 0 && num_freqs <= d / 2, "akv_tri_scores: num_freqs=%d out of range", num_freqs);
+  AKV_REQUIRE(coeff_bits == 4 || coeff_bits == 8 || coeff_bits == 16, "akv_tri_scores: coeff_bits=%d, must be 4, 8 or 16",
+              coeff_bits);
+  AKV_REQUIRE(akv_valid_dtype(q_dtype), "akv_tri_scores: bad dtype");
+  AKV_REQUIRE(!query_pos || akv_valid_itype(qp_itype), "akv_tri_scores: bad query_pos type");
+  AKV_REQUIRE(!key_positions || akv_valid_itype(kp_itype), "akv_tri_scores: bad key_positions type");
+  if (batch == 0 || seq_len == 0) return AKV_OK;
+  AKV_REQUIRE(query && out && theta && k_indices && k_coeffs, "akv_tri_scores: null pointer");
+  AKV_REQUIRE(coeff_bits == 16 || k_scales, "akv_tri_scores: null scales");
+  AKV_REQUIRE(coeff_bits != 16 || ((uintptr_t)k_coeffs & 1) == 0, "akv_tri_scores: float16 coefficients must be 2-byte aligned");
+  AKV_REQUIRE((seq_len + 255) / 256 < ((int64_t)1 << 31) && num_kv_heads < 65536 && batch < 65536, "akv_tri_scores: grid too large");
+  tri_args a = {};
+  a.query = query; a.q_dtype = q_dtype;
+  a.k_idx = k_indices; a.k_cf = (const uint8_t*)k_coeffs; a.k_sc = (const __half*)k_scales;
+  a.theta = theta; a.qpos = query_pos; a.qp_itype = qp_itype; a.kpos = key_positions; a.kp_itype = kp_itype;
+  a.B = batch; a.S = seq_len; a.QH = num_q_heads; a.KVH = num_kv_heads; a.D = d; a.F = num_freqs;
+  a.cbits = coeff_bits; a.post_rope = pre_rope ? 0 : 1;
+  const int gqa = num_q_heads / num_kv_heads;
+  const int gq = gqa % 4 == 0 ? 4 : 1;
+  const size_t lds = ((size_t)d / 2 + (size_t)gq * d + 256) * sizeof(float);
+  dim3 grid((unsigned)((seq_len + 255) / 256), num_kv_heads, batch);
+  if (gq == 4) tri_scores_kernel<4><<<grid, 256, lds, stream>>>(a, out);
+  else tri_scores_kernel<1><<<grid, 256, lds, stream>>>(a, out);
+  AKV_LAUNCH_CHECK("tri_scores_kernel");
   return AKV_OK;
 }
 

@@ -14,7 +14,8 @@ import torch
 
 from .. import _lib
 from .config import TriAttentionConfig
-from .encoder import SpectralEncoding, SpectralKVEncoder, packed_shape
+from .encoder import SpectralEncoding, SpectralKVEncoder, packed_shape, unpack_coefficients
+from .scorer import TrigSeriesScorer
 from .spectral import rope_frequencies
 
 
@@ -28,6 +29,7 @@ class TriAttention:
         self.gqa_ratio = config.gqa_ratio
         self.scale = 1.0 / math.sqrt(config.head_dim)
         self.encoder = SpectralKVEncoder(config)
+        self.scorer = TrigSeriesScorer(config, device=device)
         # float32 table evaluated on the host exactly as the reference does, then moved
         self._theta = rope_frequencies(config.head_dim, config.rope_base, device="cpu").to(device)
         self._workspace: Optional[torch.Tensor] = None
@@ -35,11 +37,85 @@ class TriAttention:
     def to(self, device: str) -> "TriAttention":
         self.device = device
         self._theta = self._theta.to(device)
+        self.scorer.to(device)
         return self
 
     def encode_kv(self, keys: torch.Tensor, values: torch.Tensor) -> Tuple[SpectralEncoding, SpectralEncoding]:
         """keys / values [B, S, num_kv_heads, head_dim] (keys before RoPE)."""
         return self.encoder.encode(keys), self.encoder.encode(values)
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                positions: Optional[torch.Tensor] = None,
+                attention_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Encode K / V, then attend every query position (reference: attention.py:116-182; its prefill form).
+        query [B, QH, S_q, D] or [B, QH, D]; key / value [B, S_kv, KVH, D] (keys before RoPE); positions [B, S_kv]
+        key positions (default 0..S_kv-1); query i sits at position i; attention_mask [B, S_q, S_kv] or
+        [B, 1, S_kv], added to the logits (-inf = masked) -> float32 [B, QH, S_q, D] (or [B, QH, D]).
+        Without a mask a query position is one decode_step; with one, the logits come from the scorer, mask and
+        softmax are torch ops and the weighted sum of the sparse value rows is a scatter-add."""
+        squeeze = query.dim() == 3
+        if squeeze:
+            query = query.unsqueeze(2)
+        B, QH, S_q, D = query.shape
+        k_enc, v_enc = self.encode_kv(key, value)
+        outs = []
+        for qi in range(S_q):
+            q_i = query[:, :, qi, :]
+            q_pos = torch.full((B,), qi, device=query.device, dtype=torch.int64)
+            if attention_mask is None:
+                outs.append(self.decode_step(q_i, k_enc, v_enc, q_pos, positions))
+                continue
+            scores = self.scorer.score(q_i, k_enc, q_pos, positions)
+            mask_i = attention_mask[:, qi:qi + 1, :] if attention_mask.dim() == 3 and attention_mask.shape[1] > 1 \
+                else attention_mask
+            weights = torch.softmax(scores + mask_i.to(scores.dtype), dim=-1)
+            outs.append(self._accumulate_values(weights, v_enc))
+        out = torch.stack(outs, dim=2)
+        return out.squeeze(2) if squeeze else out
+
+    def _accumulate_values(self, weights: torch.Tensor, v_enc: SpectralEncoding) -> torch.Tensor:
+        """sum_t weights[b, qh, t] * value row t of the query head's kv head, as float32 [B, QH, D]
+        (reference: attention.py:219-280)."""
+        B, QH, S = weights.shape
+        KVH = v_enc.indices.shape[2]
+        v0, v1 = unpack_coefficients(v_enc.packed, v_enc.scales, self.config.coeff_bits)       # [B, S, KVH, F]
+        heads = torch.arange(QH, device=weights.device) // (QH // KVH)
+        idx = v_enc.indices.long()[:, :, heads].permute(0, 2, 1, 3).reshape(B, QH, -1)           # [B, QH, S F]
+        w = weights.unsqueeze(-1)
+        out = torch.zeros(B, QH, self.head_dim, dtype=torch.float32, device=weights.device)
+        out.scatter_add_(-1, idx * 2, (w * v0[:, :, heads].permute(0, 2, 1, 3)).reshape(B, QH, -1))
+        out.scatter_add_(-1, idx * 2 + 1, (w * v1[:, :, heads].permute(0, 2, 1, 3)).reshape(B, QH, -1))
+        return out
+
+    @staticmethod
+    def reference_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                            rope_base: float = 1_000_000.0, positions_q: Optional[torch.Tensor] = None,
+                            positions_k: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Dense attention with explicit RoPE on the uncompressed tensors, for comparisons (reference:
+        attention.py:285-345): query [B, QH, D] and key [B, S, KVH, D] before RoPE, value [B, S, KVH, D];
+        positions default to S for the query and 0..S-1 for the keys -> float32 [B, QH, D].  Torch ops on the
+        tensors' device."""
+        B, QH, D = query.shape
+        S, KVH = key.shape[1], key.shape[2]
+        dev = query.device
+        if positions_q is None:
+            positions_q = torch.full((B,), S, device=dev)
+        if positions_k is None:
+            positions_k = torch.arange(S, device=dev).unsqueeze(0).expand(B, -1)
+        theta = rope_frequencies(D, rope_base, device="cpu").to(dev)
+
+        def rope(x, pos):                 # x [..., D], pos broadcastable to x.shape[:-1]
+            ang = pos.float().unsqueeze(-1) * theta
+            c, s = torch.cos(ang), torch.sin(ang)
+            xe, xo = x.float()[..., 0::2], x.float()[..., 1::2]
+            return torch.stack((xe * c - xo * s, xe * s + xo * c), dim=-1).flatten(-2)
+
+        q = rope(query, positions_q.view(B, 1))                                   # [B, QH, D]
+        k = rope(key, positions_k.view(B, S, 1))                                  # [B, S, KVH, D]
+        heads = torch.arange(QH, device=dev) // (QH // KVH)
+        scores = torch.einsum("bhd,bshd->bhs", q, k[:, :, heads]) / math.sqrt(D)
+        w = torch.softmax(scores, dim=-1)
+        return torch.einsum("bhs,bshd->bhd", w, value.float()[:, :, heads])
 
     def decode_step(self, query: torch.Tensor, k_enc: SpectralEncoding, v_enc: SpectralEncoding,
                     query_pos: Optional[torch.Tensor] = None,

@@ -94,3 +94,34 @@ class SpectralKVEncoder:
         out.scatter_(-1, idx * 2, v0)
         out.scatter_(-1, idx * 2 + 1, v1)
         return out
+
+    def encode_adaptive(self, x: torch.Tensor, min_energy_ratio: Optional[float] = None,
+                        max_freqs: Optional[int] = None):
+        """Encode with as many pairs as the most demanding vector of the batch needs to reach
+        `min_energy_ratio` of its pair energy, between num_freqs and max_freqs (reference: encoder.py:205-241).
+        Returns (encoding, pairs needed per vector)."""
+        from .spectral import pair_energy_profile
+        if min_energy_ratio is None:
+            min_energy_ratio = self.config.min_energy_ratio
+        if max_freqs is None:
+            max_freqs = self.num_pairs
+        prof = pair_energy_profile(x.float())
+        share = prof.cumsum(-1) / (prof.sum(-1, keepdim=True) + 1e-12)
+        needed = ((share >= min_energy_ratio).float().argmax(dim=-1) + 1).clamp(self.num_freqs, max_freqs)
+        return self.encode(x, num_freqs=int(needed.max().item())), needed
+
+    def compression_stats(self, x: torch.Tensor) -> dict:
+        """Compression ratio, retained energy, reconstruction error of `x` (reference: encoder.py:243-270)."""
+        from .spectral import spectral_concentration
+        dec = self.decode(self.encode(x)).float()
+        xf = x.float().to(dec.device)
+        return {
+            "num_freqs": self.num_freqs,
+            "coeff_bits": self.coeff_bits,
+            "bytes_per_token": self.config.bytes_per_kv_token,
+            "compression_ratio": self.config.compression_ratio,
+            "mse": (xf - dec).square().mean().item(),
+            "energy_ratio": spectral_concentration(xf, self.num_freqs).mean().item(),
+            "cosine_similarity": torch.nn.functional.cosine_similarity(
+                xf.reshape(-1, self.head_dim), dec.reshape(-1, self.head_dim), dim=-1).mean().item(),
+        }

@@ -303,6 +303,19 @@ int akv_tri_decode_step(const void* query, int q_dtype,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
+ * TrigSeriesScorer.score -- aither_kvcache/triattention/scorer.py:115-208: the pre-softmax logits alone,
+ * for callers that add a mask (TriAttention.forward, attention.py:148-166) or inspect the scores.
+ * Arguments as for akv_tri_decode_step; out [B][QH][S] float32, contiguous.
+ * ------------------------------------------------------------------------------- */
+int akv_tri_scores(const void* query, int q_dtype,
+                   const uint8_t* k_indices, const void* k_coeffs, const void* k_scales,
+                   const float* theta,
+                   const void* query_pos, int qp_itype,
+                   const void* key_positions, int kp_itype,
+                   float* out, int batch, int64_t seq_len, int num_q_heads, int num_kv_heads,
+                   int d, int num_freqs, int coeff_bits, int pre_rope, void* stream);
+
+/* ---------------------------------------------------------------------------------
  * TriAttention.decode_step over a paged spectral cache: what the reference does per sequence
  * with SpectralKVCache.fetch_sequence (aither_kvcache/triattention/cache.py:163-198; block
  * layout :9-15) followed by decode_step, for a whole batch and without the gather.

@@ -757,13 +757,16 @@ def tri_scores(query, k_idx, k_packed, k_scales, theta, query_pos=None, key_posi
 
 
 def tri_decode_step(query, k_enc, v_enc, theta, query_pos=None, key_positions=None, coeff_bits=4,
-                    pre_rope=True):
+                    pre_rope=True, mask=None):
     """TriAttention.decode_step, attention.py:186-280: scores -> softmax over S -> weighted
     scatter-add of the value coefficients into even/odd bins -> interleave.  k_enc / v_enc are
-    (indices, packed, scales) triples.  Returns float32 [B, QH, D]."""
+    (indices, packed, scales) triples.  `mask` [B, 1, S] is added to the logits first, which makes
+    this one query position of TriAttention.forward (attention.py:148-170).  Returns float32 [B, QH, D]."""
     query = np.asarray(query)
     B, QH, D = query.shape
     sc = tri_scores(query, *k_enc, theta, query_pos, key_positions, coeff_bits, pre_rope)
+    if mask is not None:
+        sc = (sc + np.asarray(mask, dtype=f32)).astype(f32)
     sc = sc - sc.max(axis=-1, keepdims=True)
     w = np.exp(sc)
     w = (w / w.sum(axis=-1, keepdims=True, dtype=f32)).astype(f32)

@@ -411,3 +411,90 @@ def test_width_argument_checks(dev):
     L = _lib.lib()
     rc = L.akv_tri_encode(x.data_ptr(), _lib.dtype_code(x), 20, 128, 128, 12, 5, x.data_ptr(), x.data_ptr(), x.data_ptr(), None)
     assert rc == _lib.AKV_ERR_INVALID
+
+
+# ---- the scorer alone, the prefill form, helpers ------------------------------------------------------
+def test_scorer_golden(golden, tri_widths, dev):
+    """TrigSeriesScorer.score against the reference's own logits: default width with explicit positions, and the
+    other widths / post-RoPE."""
+    from aitherkvcache_amd.triattention import TrigSeriesScorer
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=2, num_query_heads=8, rope_base=1e6)
+    sc = TrigSeriesScorer(cfg, device=str(dev)).score(t(golden["tri_q"], dev), enc(golden, "k", dev),
+                                                      t(golden["tri_qpos"], dev), t(golden["tri_kpos"], dev))
+    assert sc.dtype == torch.float32 and sc.shape == golden["tri_scores_explicit_pos"].shape
+    e = np.max(np.abs(sc.cpu().numpy() - golden["tri_scores_explicit_pos"]))
+    print(f"[tri scorer golden] {e:.2e}")
+    assert e <= TOL
+    g = tri_widths
+    for bits, pre in WIDTH_MODES:
+        cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=bits, num_kv_heads=2, num_query_heads=8,
+                                 rope_base=1e6, pre_rope=pre)
+        got = TrigSeriesScorer(cfg, device=str(dev)).score(t(g["q"], dev), _wenc(g, bits, "k", dev), t(g["qpos"], dev),
+                                                           t(g["kpos"], dev)).cpu().numpy()
+        assert np.max(np.abs(got - g[f"scores_b{bits}_{'pre' if pre else 'post'}"])) <= TOL
+
+
+@pytest.mark.parametrize("B,S,QH,KVH,D,F,bits", [(2, 700, 32, 8, 128, 12, 4), (2, 333, 6, 2, 32, 4, 8), (1, 70, 4, 4, 64, 32, 16)])
+def test_scorer_vs_oracle(dev, B, S, QH, KVH, D, F, bits):
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=bits, num_kv_heads=KVH, num_query_heads=QH, rope_base=1e4)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(S)
+    keys = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    k_enc, _ = tri.encode_kv(t(keys, dev), t(keys, dev))
+    q = rng.standard_normal((B, QH, D)).astype(np.float32)
+    qpos = rng.integers(S, 9000, size=B)
+    kpos = np.sort(rng.integers(0, 8000, size=(B, S)), axis=-1)
+    theta = tri._theta.cpu().numpy()
+    ke = tuple(x.cpu().numpy() for x in k_enc)
+    got = tri.scorer.score(t(q, dev), k_enc, t(qpos, dev), t(kpos, dev)).cpu().numpy()
+    assert np.max(np.abs(got - O.tri_scores(q, *ke, theta, qpos, kpos, bits))) <= TOL
+    got = tri.scorer.score(t(q, dev), k_enc).cpu().numpy()              # default positions
+    assert np.max(np.abs(got - O.tri_scores(q, *ke, theta, None, None, bits))) <= TOL
+    one = tri.scorer.score_single(t(q[:1], dev), SpectralEncoding(*(x[:1] for x in k_enc)), 1234).cpu().numpy()
+    assert np.max(np.abs(one - O.tri_scores(q[:1], *(x[:1] for x in ke), theta, np.array([1234]), None, bits))) <= TOL
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_forward_prefill_form_vs_oracle(dev, masked):
+    """TriAttention.forward: encode, then every query position i at position i against all keys, with and without an
+    additive (causal) mask; single-query form squeezed."""
+    B, S, Sq, QH, KVH, D, F = 2, 90, 5, 8, 2, 128, 12
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=F, num_kv_heads=KVH, num_query_heads=QH, rope_base=1e4)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(5)
+    keys = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    q = rng.standard_normal((B, QH, Sq, D)).astype(np.float32)
+    mask = None
+    if masked:
+        mask = np.zeros((B, Sq, S), np.float32)
+        for i in range(Sq):
+            mask[:, i, 40 + 10 * i:] = -np.inf
+    out = tri.forward(t(q, dev), t(keys, dev), t(vals, dev), attention_mask=None if mask is None else t(mask, dev))
+    assert out.shape == (B, QH, Sq, D) and out.dtype == torch.float32
+    ke, ve = O.spectral_encode(keys, F), O.spectral_encode(vals, F)
+    theta = tri._theta.cpu().numpy()
+    for i in range(Sq):
+        ref = O.tri_decode_step(q[:, :, i], ke, ve, theta, np.full((B,), i), None, 4, True,
+                                None if mask is None else mask[:, i:i + 1])
+        assert np.max(np.abs(out[:, :, i].cpu().numpy() - ref)) <= TOL
+    one = tri.forward(t(q[:, :, 0], dev), t(keys, dev), t(vals, dev))
+    assert one.shape == (B, QH, D) and torch.equal(one, tri.forward(t(q[:, :, :1], dev), t(keys, dev), t(vals, dev))[:, :, 0])
+
+
+def test_full_series_equals_rope_attention(dev):
+    """All pairs kept as fp16: the trigonometric series is RoPE attention (reference test_triattention.py:183-208)."""
+    B, S, QH, KVH, D = 2, 50, 4, 2, 32
+    cfg = TriAttentionConfig(head_dim=D, num_freqs=D // 2, coeff_bits=16, num_kv_heads=KVH, num_query_heads=QH, rope_base=1e4)
+    tri = TriAttention(cfg, device=str(dev))
+    g = torch.Generator(device=dev).manual_seed(1)
+    q = torch.randn(B, QH, D, device=dev, generator=g)
+    k = torch.randn(B, S, KVH, D, device=dev, generator=g).half()
+    v = torch.randn(B, S, KVH, D, device=dev, generator=g).half()
+    qpos = torch.tensor([60, 75], device=dev)
+    kpos = torch.arange(S, device=dev).unsqueeze(0).expand(B, -1)
+    out = tri.decode_step(q, *tri.encode_kv(k, v), qpos, kpos)
+    ref = TriAttention.reference_attention(q, k, v, 1e4, qpos, kpos)
+    assert torch.max(torch.abs(out - ref)).item() < 1e-3
+    stats = tri.encoder.compression_stats(k)
+    assert stats["cosine_similarity"] > 0.999 and stats["energy_ratio"] > 0.999

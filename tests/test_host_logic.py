@@ -351,3 +351,42 @@ def test_backend_format_selection_from_environment(monkeypatch):
     monkeypatch.setenv("AITHER_TQ_MODE", "")
     monkeypatch.setenv("AITHER_TQ_PRIMARY", "1")
     assert backend.primary_from_env()
+
+
+def test_tri_helpers_on_host_tensors():
+    """Spectral helpers, adaptive pair count and the dense RoPE attention helper are torch ops and run anywhere."""
+    from oracle import tq_oracle as O
+    from aitherkvcache_amd.triattention import SpectralKVEncoder, TriAttention, TriAttentionConfig
+    from aitherkvcache_amd.triattention.spectral import pair_energies, pair_energy_profile, spectral_concentration, topk_pairs
+    x = torch.tensor([[3.0, 4.0, 0.0, 1.0, 2.0, 0.0, 0.5, 0.5]])
+    assert torch.equal(pair_energies(x), torch.tensor([[25.0, 1.0, 4.0, 0.5]]))
+    idx, vals = topk_pairs(x, 2)
+    assert idx.dtype == torch.uint8 and idx.tolist() == [[0, 2]] and vals.tolist() == [[[3.0, 4.0], [2.0, 0.0]]]
+    assert abs(spectral_concentration(x, 2).item() - 29.0 / 30.5) < 1e-6
+    assert pair_energy_profile(x).tolist() == [[25.0, 4.0, 1.0, 0.5]]
+    cfg = TriAttentionConfig(head_dim=8, num_freqs=1, coeff_bits=16, num_kv_heads=1, num_query_heads=1, rope_base=1e4)
+    enc = SpectralKVEncoder(cfg)
+    e, needed = enc.encode_adaptive(x, min_energy_ratio=0.9)       # 25 / 30.5 < 0.9 <= 29 / 30.5
+    assert needed.tolist() == [2] and e.indices.tolist() == [[0, 2]]
+    st = enc.compression_stats(x)
+    assert st["num_freqs"] == 1 and abs(st["energy_ratio"] - 25.0 / 30.5) < 1e-6 and abs(st["mse"] - 5.5 / 8) < 1e-6
+    # dense RoPE attention against the oracle's dense attention on rotated tensors
+    rng = np.random.default_rng(0)
+    B, S, QH, KVH, D = 2, 9, 4, 2, 8
+    q, k, v = rng.standard_normal((B, QH, D)), rng.standard_normal((B, S, KVH, D)), rng.standard_normal((B, S, KVH, D))
+    got = TriAttention.reference_attention(torch.from_numpy(q).float(), torch.from_numpy(k).float(),
+                                           torch.from_numpy(v).float(), 1e4).numpy()
+    theta = O.rope_frequencies(D, 1e4).astype(np.float64)
+
+    def rope(x, pos):
+        ang = pos[..., None] * theta
+        xe, xo = x[..., 0::2], x[..., 1::2]
+        return np.stack((xe * np.cos(ang) - xo * np.sin(ang), xe * np.sin(ang) + xo * np.cos(ang)), -1).reshape(x.shape)
+
+    qr = rope(q, np.full((B, 1), float(S)))
+    kr = rope(k, np.broadcast_to(np.arange(S, dtype=np.float64)[None, :, None], (B, S, 1)))
+    for b in range(B):
+        for h in range(QH):
+            s = kr[b, :, h // 2] @ qr[b, h] / np.sqrt(D)
+            w = np.exp(s - s.max()); w /= w.sum()
+            assert np.max(np.abs(got[b, h] - w @ v[b, :, h // 2])) < 1e-5
