@@ -32,3 +32,49 @@ def get_codebook(d: int, bits: int) -> Tuple[np.ndarray, np.ndarray, float]:
 def get_theory_bounds(bits: int) -> Tuple[float, float]:
     """Distortion-rate bounds 4^-b <= MSE <= (3 pi / 2) 4^-b (reference: codebook.py:85-89)."""
     return 1.0 / 4 ** bits, (3 * math.pi / 2) / 4 ** bits
+
+
+def compute_codebook_scipy(d: int, bits: int, max_iter: int = 2000,
+                           tol: float = 1e-12) -> Tuple[np.ndarray, np.ndarray, float]:
+    """Lloyd-Max codebook computed from the coordinate density instead of the tables (reference:
+    codebook.py:92-175); needs scipy.  The density of one coordinate of a uniform point on S^(d-1) is taken as
+    N(0, 1/d) on [-5 sigma, 5 sigma] for d >= 64 and as the exact (1 - x^2)^((d-3)/2) law on [-1, 1] below.
+    Starts from equally spaced levels and alternates midpoints and conditional means until no level moves by more
+    than `tol`.  Returns (centroids, inner boundaries, total MSE = d x per-coordinate MSE).  A validation tool:
+    nothing on the hot path calls it."""
+    from scipy.integrate import quad
+    from scipy.special import gammaln
+    levels = 1 << bits
+    if d >= 64:
+        var = 1.0 / d
+        lo, hi = -5.0 * math.sqrt(var), 5.0 * math.sqrt(var)
+        norm = 1.0 / math.sqrt(2.0 * math.pi * var)
+
+        def pdf(x):
+            return norm * math.exp(-x * x / (2.0 * var))
+    else:
+        lo, hi = -1.0, 1.0
+        log_c = gammaln(d / 2) - 0.5 * math.log(math.pi) - gammaln((d - 1) / 2)
+
+        def pdf(x):
+            return 0.0 if abs(x) >= 1.0 else math.exp(log_c + 0.5 * (d - 3) * math.log(1.0 - x * x))
+
+    def edges(c):
+        return np.concatenate(([lo], (c[:-1] + c[1:]) / 2, [hi]))
+
+    step = (hi - lo) / levels
+    cen = lo + step * (np.arange(levels) + 0.5)
+    for _ in range(max_iter):
+        e = edges(cen)
+        new = np.empty(levels)
+        for i in range(levels):
+            a, b = e[i], e[i + 1]
+            mass = quad(pdf, a, b)[0] if b - a >= 1e-15 else 0.0
+            new[i] = quad(lambda x: x * pdf(x), a, b)[0] / mass if abs(mass) > 1e-15 else (a + b) / 2
+        moved = np.max(np.abs(new - cen))
+        cen = new
+        if moved < tol:
+            break
+    e = edges(cen)
+    mse = sum(quad(lambda x, c=cen[i]: (x - c) ** 2 * pdf(x), e[i], e[i + 1])[0] for i in range(levels))
+    return cen, (cen[:-1] + cen[1:]) / 2, float(mse * d)

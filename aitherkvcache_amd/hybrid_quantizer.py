@@ -88,6 +88,53 @@ _TQ35_D64 = {
 
 
 @functools.lru_cache(maxsize=None)
+# ---- host-side helpers of the reference's module (hybrid_quantizer.py:130-234,310-396): torch ops on whatever
+# device the tensor lives on.  The kernels do these steps in registers; callers that import the helpers keep working.
+def fwht_pow2(x: torch.Tensor) -> torch.Tensor:
+    """Unnormalised Walsh-Hadamard transform of the last axis (a power of two), written back into `x`."""
+    from .rotation import fast_hadamard_transform
+    x.copy_(fast_hadamard_transform(x))
+    return x
+
+
+def fwht_general(x: torch.Tensor) -> torch.Tensor:
+    """The same for any length: the axis is cut into descending powers of two (96 = 64 + 32) and each piece is
+    transformed on its own.  Returns a new tensor."""
+    from .rotation import fast_hadamard_transform
+    n, at, out = x.shape[-1], 0, []
+    while n > 0:
+        piece = 1 << (n.bit_length() - 1)
+        out.append(fast_hadamard_transform(x[..., at:at + piece]))
+        at, n = at + piece, n - piece
+    return torch.cat(out, dim=-1) if out else x.clone()
+
+
+def structured_hadamard(x: torch.Tensor, signs: torch.Tensor, normalized: bool = True,
+                        inverse: bool = False) -> torch.Tensor:
+    """H diag(signs) x (forward) or diag(signs) H x (inverse), divided by sqrt(dim) when `normalized`."""
+    y = fwht_general(x) * signs if inverse else fwht_general(x * signs)
+    return y / math.sqrt(x.shape[-1]) if normalized else y
+
+
+def pack_multibit(indices: torch.Tensor, bits: int) -> torch.Tensor:
+    """[..., dim] indices of `bits` bits (1..8) -> [..., ceil(dim bits / 8)] uint8, one MSB-first bit stream."""
+    dim = indices.shape[-1]
+    nbytes = -(-dim * bits // 8)
+    shifts = torch.arange(bits - 1, -1, -1, device=indices.device)
+    stream = ((indices.long().unsqueeze(-1) >> shifts) & 1).reshape(*indices.shape[:-1], dim * bits)
+    stream = torch.nn.functional.pad(stream, (0, nbytes * 8 - dim * bits))
+    weights = 1 << torch.arange(7, -1, -1, device=indices.device)
+    return (stream.reshape(*indices.shape[:-1], nbytes, 8) * weights).sum(-1).to(torch.uint8)
+
+
+def unpack_multibit(packed: torch.Tensor, dim: int, bits: int) -> torch.Tensor:
+    """Inverse of pack_multibit -> [..., dim] uint8."""
+    shifts = torch.arange(7, -1, -1, device=packed.device)
+    stream = ((packed.long().unsqueeze(-1) >> shifts) & 1).reshape(*packed.shape[:-1], packed.shape[-1] * 8)
+    weights = 1 << torch.arange(bits - 1, -1, -1, device=packed.device)
+    return (stream[..., :dim * bits].reshape(*packed.shape[:-1], dim, bits) * weights).sum(-1).to(torch.uint8)
+
+
 def _lloyd_on_grid(dim: int, bits: int) -> Tuple[np.ndarray, np.ndarray]:
     """Lloyd iteration on a 10,000-point grid over (-0.999, 0.999) weighted by the marginal
     density of a coordinate of a uniform point on S^{dim-1}, (1-x^2)^((dim-3)/2); at most 200

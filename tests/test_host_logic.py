@@ -390,3 +390,35 @@ def test_tri_helpers_on_host_tensors():
             s = kr[b, :, h // 2] @ qr[b, h] / np.sqrt(D)
             w = np.exp(s - s.max()); w /= w.sum()
             assert np.max(np.abs(got[b, h] - w @ v[b, :, h // 2])) < 1e-5
+
+
+def test_hybrid_module_helpers_against_the_oracle():
+    """fwht_pow2 / fwht_general / structured_hadamard / pack_multibit / unpack_multibit of the public module."""
+    from oracle import tq_oracle as O
+    from aitherkvcache_amd.hybrid_quantizer import (fwht_general, fwht_pow2, pack_multibit, structured_hadamard,
+                                                    unpack_multibit)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((5, 64)).astype(np.float32)
+    xt = torch.from_numpy(x.copy())
+    assert fwht_pow2(xt) is xt and np.allclose(xt.numpy(), O.fwht(x), rtol=1e-6, atol=1e-5)
+    y = rng.standard_normal((3, 96)).astype(np.float32)
+    got = fwht_general(torch.from_numpy(y)).numpy()
+    assert np.allclose(got[:, :64], O.fwht(y[:, :64]), atol=1e-5) and np.allclose(got[:, 64:], O.fwht(y[:, 64:]), atol=1e-5)
+    signs = np.where(rng.integers(0, 2, 64) > 0, 1.0, -1.0).astype(np.float32)
+    fwd = structured_hadamard(torch.from_numpy(x), torch.from_numpy(signs))
+    assert np.allclose(fwd.numpy(), O.structured_hadamard(x, signs), atol=1e-5)
+    back = structured_hadamard(fwd, torch.from_numpy(signs), inverse=True)
+    assert np.allclose(back.numpy(), x, atol=1e-5)
+    for bits, dim in ((1, 64), (2, 64), (3, 64), (4, 30), (3, 7)):
+        idx = rng.integers(0, 1 << bits, size=(4, dim)).astype(np.uint8)
+        p = pack_multibit(torch.from_numpy(idx), bits)
+        assert p.dtype == torch.uint8 and np.array_equal(p.numpy(), O.pack_multibit(idx, bits))
+        assert np.array_equal(unpack_multibit(p, dim, bits).numpy(), idx)
+
+
+def test_codebook_from_the_density_reproduces_the_tables():
+    from aitherkvcache_amd.codebook import compute_codebook_scipy
+    cen, bnd, mse = compute_codebook_scipy(128, 2, max_iter=200, tol=1e-10)
+    ref_c, ref_b, ref_mse = get_codebook(128, 2)
+    assert np.allclose(cen, ref_c, atol=1e-5) and np.allclose(bnd, ref_b, atol=1e-5) and abs(mse - ref_mse) < 2e-4   # (support cut at 5 sigma)
+    assert "GQA 4:1" in akv.triattention.TriAttentionConfig().summary()
