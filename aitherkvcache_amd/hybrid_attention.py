@@ -32,6 +32,7 @@ def hybrid_encode_and_store(htq, x: torch.Tensor, slot_mapping: torch.Tensor, ca
         raise ValueError(f"head_dim {head_dim} != {htq.head_dim}")
     if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
         x = x.float()
+    x = htq.to_group_order(x, head_axis=1)        # (a variance-ranked split: coordinates into group order first)
     if x.stride(-1) != 1:
         x = x.contiguous()
     slots = slot_mapping if slot_mapping.is_contiguous() else slot_mapping.contiguous()
@@ -67,6 +68,12 @@ class HybridPagedAttention:
         q = query
         if q.dtype not in (torch.float16, torch.bfloat16, torch.float32):
             q = q.float()
+        # A variance-ranked split stores every kv head's rows in that head's group order: the query heads of the
+        # kv head are moved into the same order (the dot products do not change), the outputs are moved back.
+        ranked = self._htq.group_order is not None
+        if ranked:
+            q = self._htq.to_group_order(q.reshape(num_seqs, num_kv_heads, -1, head_dim), head_axis=1) \
+                .reshape(num_seqs, num_q_heads, head_dim)
         if q.stride(-1) != 1:
             q = q.contiguous()
         out = torch.empty((num_seqs, num_q_heads, head_dim), dtype=q.dtype, device=dev)
@@ -92,6 +99,9 @@ class HybridPagedAttention:
             num_seqs, num_q_heads, num_kv_heads, block_size, min(k_cache.shape[0], v_cache.shape[0]),
             bt.shape[1], float(scale),
             ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev)))
+        if ranked:
+            out = self._htq.from_group_order(out.reshape(num_seqs, num_kv_heads, -1, head_dim), head_axis=1) \
+                .reshape(num_seqs, num_q_heads, head_dim)
         return out if out.dtype == query.dtype else out.to(query.dtype)
 
     def last_call_status(self) -> int:

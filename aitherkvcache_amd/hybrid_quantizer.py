@@ -234,16 +234,65 @@ class HybridTurboQuant:
         self._uniform_split = True
 
     def calibrate(self, sample_vectors: torch.Tensor) -> None:
-        """Variance-ranked per-head groups (reference: hybrid_quantizer.py:553-588).  The
-        kernels assume the uniform split; this mode is not built."""
-        raise NotImplementedError(
-            "variance-ranked calibrate() has no HIP kernel in this build; use calibrate_uniform()")
+        """Variance-ranked per-head groups (reference: hybrid_quantizer.py:553-588): per kv head the g0_dim
+        coordinates of largest mean square over the sample form group 0 (in descending order of that score), the
+        others group 1.  sample_vectors [num_samples, num_kv_heads, head_dim].
+        The kernels work on the uniform split; a ranked split is the same codec on permuted coordinates, so the
+        vectors are gathered into group order before they are encoded (`to_group_order`) and scattered back after
+        they are decoded -- one extra pass of torch ops per call that the uniform split does not pay."""
+        if sample_vectors.dim() != 3:
+            raise ValueError(f"Expected [num_samples, num_kv_heads, head_dim], got shape {list(sample_vectors.shape)}")
+        _, num_kv_heads, hdim = sample_vectors.shape
+        if hdim != self.head_dim:
+            raise ValueError(f"head_dim mismatch: expected {self.head_dim}, got {hdim}")
+        self._num_kv_heads = num_kv_heads
+        order = sample_vectors.float().square().mean(dim=0).sort(dim=-1, descending=True).indices.to(self.device)
+        self._group0_indices = order[:, :self._g0_dim].contiguous()
+        self._group1_indices = order[:, self._g0_dim:].contiguous()
+        self._calibrated = True
+        self._uniform_split = False
+
+    @property
+    def group_order(self) -> Optional[torch.Tensor]:
+        """[num_kv_heads, head_dim] coordinate order (group 0, then group 1) of a ranked split; None for the
+        uniform split, where the order is the identity."""
+        if not self._calibrated or self._uniform_split:
+            return None
+        return torch.cat([self._group0_indices, self._group1_indices], dim=-1)
+
+    def to_group_order(self, x: torch.Tensor, head_axis: Optional[int] = None) -> torch.Tensor:
+        """x [..., head_dim] with coordinates moved into group order.  head_axis names the axis that runs over the
+        kv heads; without one the flattened vectors cycle over the heads when their number is a multiple of
+        num_kv_heads and use head 0's order otherwise (the reference's rule, hybrid_quantizer.py:640-662)."""
+        return self._reorder(x, head_axis, inverse=False)
+
+    def from_group_order(self, x: torch.Tensor, head_axis: Optional[int] = None) -> torch.Tensor:
+        """Inverse of to_group_order."""
+        return self._reorder(x, head_axis, inverse=True)
+
+    def _reorder(self, x: torch.Tensor, head_axis: Optional[int], inverse: bool) -> torch.Tensor:
+        order = self.group_order
+        if order is None:
+            return x
+        order = order.to(x.device)
+        H, D = order.shape
+        if head_axis is not None:
+            xm = x.movedim(head_axis, -2)
+            if xm.shape[-2] != H:
+                raise ValueError(f"axis {head_axis} has {xm.shape[-2]} entries, calibrated for {H} kv heads")
+            idx = order.expand(xm.shape)
+        else:
+            flat = x.reshape(-1, D)
+            xm = flat.reshape(-1, H, D) if (H > 1 and flat.shape[0] % H == 0) else flat
+            idx = order.expand(xm.shape) if xm.dim() == 3 else order[0].expand(xm.shape)
+        out = torch.empty_like(xm).scatter_(-1, idx, xm) if inverse else torch.gather(xm, -1, idx)
+        return out.movedim(-2, head_axis) if head_axis is not None else out.reshape(x.shape)
 
     def _ensure_ready(self) -> None:
         if not self._calibrated:
             raise RuntimeError("HybridTurboQuant: must call calibrate() or calibrate_uniform() "
                                "before encode/decode.")
-        if self._table is None or not self._uniform_split:
+        if self._table is None:
             raise NotImplementedError(
                 f"HIP kernels exist for mode 'tq35' at head_dim 128 only (got {self.mode!r}, "
                 f"head_dim {self.head_dim})")
@@ -262,7 +311,7 @@ class HybridTurboQuant:
         batch = list(x.shape[:-1])
         if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
             x = x.float()
-        xf = x.reshape(-1, self.head_dim)
+        xf = self.to_group_order(x).reshape(-1, self.head_dim)
         if xf.stride(-1) != 1:
             xf = xf.contiguous()
         n = xf.shape[0]
@@ -287,7 +336,7 @@ class HybridTurboQuant:
         _lib.check(_lib.lib().akv_hybrid_decode(
             pf.data_ptr(), pf.stride(0) if n else self.layout.packed_dim, n, self._table.data_ptr(),
             out.data_ptr(), self.head_dim, _lib.stream_ptr(dev)))
-        return out.reshape(batch + [self.head_dim])
+        return self.from_group_order(out).reshape(batch + [self.head_dim])
 
     # -- analysis -----------------------------------------------------------------------------
     def validate(self, num_vectors: int = 10000) -> dict:

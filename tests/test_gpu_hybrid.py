@@ -385,3 +385,51 @@ def test_handoff_timeout_is_reported(golden, dev):
     assert attn.last_call_status() == 0
     ref = O.hybrid_paged_attention(q, kc.cpu().numpy(), vc.cpu().numpy(), tables, ctx, hp, 0.09, dtype=np.float64)
     assert np.max(np.abs(good.cpu().numpy().astype(np.float64) - ref)) <= 2e-3
+
+
+def test_ranked_calibration_is_the_codec_on_permuted_coordinates(golden, dev):
+    """calibrate(sample): encode / decode / paged attention equal the oracle's uniform-split codec applied to the
+    vectors in group order (what the reference's per-head gathers amount to, hybrid_quantizer.py:640-700)."""
+    kvh, qh = 2, 8
+    h = akv.HybridTurboQuant(device=str(dev))
+    rng = np.random.default_rng(11)
+    scale = np.stack([rng.permutation(128), rng.permutation(128)]).astype(np.float32) / 64.0 + 0.25     # [kvh, 128]
+    sample = torch.from_numpy((rng.standard_normal((400, kvh, 128)) * scale).astype(np.float32))
+    h.calibrate(sample.to(dev))
+    order = h.group_order.cpu().numpy()
+    assert order.shape == (kvh, 128) and all(sorted(order[i].tolist()) == list(range(128)) for i in range(kvh))
+    hp = params(golden)
+    x = (rng.standard_normal((60, kvh, 128)) * scale).astype(np.float16)
+    xg = np.take_along_axis(x, np.broadcast_to(order, x.shape), axis=-1)
+    packed = h.encode(t(x, dev)).cpu().numpy()
+    ref = O.hybrid_encode(xg.astype(np.float32), hp)
+    assert packed.shape == ref.shape and np.mean(np.any(packed != ref, axis=-1)) <= 0.02      # (boundary cases, as in the bulk test)
+    dec = h.decode(t(ref, dev)).cpu().numpy()
+    want = np.empty_like(dec)
+    np.put_along_axis(want, np.broadcast_to(order, dec.shape), O.hybrid_decode(ref, hp), axis=-1)
+    assert np.array_equal(dec, want)
+    # paged attention: cache written through hybrid_encode_and_store, queries and outputs in natural order
+    bs, nb, ctx = 16, 8, np.array([50, 17], dtype=np.int32)
+    kc = torch.zeros(nb, bs, kvh, 64, dtype=torch.uint8, device=dev)
+    vc = torch.zeros_like(kc)
+    keys = (rng.standard_normal((nb * bs, kvh, 128)) * scale).astype(np.float16)
+    vals = (rng.standard_normal((nb * bs, kvh, 128)) * scale).astype(np.float16)
+    slots = torch.arange(nb * bs, device=dev)
+    akv.hybrid_encode_and_store(h, t(keys, dev), slots, kc, block_size=bs)
+    akv.hybrid_encode_and_store(h, t(vals, dev), slots, vc, block_size=bs)
+    bt = np.array([[3, 0, 5, 6], [1, 2, 0, 0]], dtype=np.int32)
+    q = rng.standard_normal((2, qh, 128)).astype(np.float32)
+    out = akv.HybridPagedAttention(h, qh).forward(t(q, dev), kc, vc, t(bt, dev), t(ctx, dev), block_size=bs).cpu().numpy()
+    # oracle: rows decoded and moved back to natural order, dense float32 attention per sequence
+    def natural(cache):
+        d = O.hybrid_decode(cache.cpu().numpy(), hp)                                  # [nb, bs, kvh, 128] in group order
+        o = np.empty_like(d)
+        np.put_along_axis(o, np.broadcast_to(order, d.shape), d, axis=-1)
+        return o
+    kd, vd = natural(kc), natural(vc)
+    for s in range(2):
+        n = int(ctx[s])
+        rows = np.concatenate([np.arange(b * bs, (b + 1) * bs) for b in bt[s]])[:n]
+        kk, vv = kd.reshape(-1, kvh, 128)[rows], vd.reshape(-1, kvh, 128)[rows]
+        ref_o = O.dense_attention(q[s], kk, vv, 1.0 / np.sqrt(128.0))
+        assert np.max(np.abs(out[s] - ref_o)) <= 2e-4 * max(1.0, np.abs(ref_o).max())

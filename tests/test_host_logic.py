@@ -422,3 +422,33 @@ def test_codebook_from_the_density_reproduces_the_tables():
     ref_c, ref_b, ref_mse = get_codebook(128, 2)
     assert np.allclose(cen, ref_c, atol=1e-5) and np.allclose(bnd, ref_b, atol=1e-5) and abs(mse - ref_mse) < 2e-4   # (support cut at 5 sigma)
     assert "GQA 4:1" in akv.triattention.TriAttentionConfig().summary()
+
+
+def test_ranked_calibration_orders_coordinates_by_mean_square():
+    """HybridTurboQuant.calibrate: per kv head the 64 coordinates of largest mean square first, in descending order,
+    then the rest; to_group_order / from_group_order are inverse gathers with the reference's head rules."""
+    h = HybridTurboQuant(device="cpu")
+    rng = np.random.default_rng(7)
+    scale = rng.permutation(128).astype(np.float32) + 1.0                       # distinct scores
+    sample = torch.from_numpy(np.stack([np.ones((50, 128), np.float32) * scale,
+                                        np.ones((50, 128), np.float32) * scale[::-1]], axis=1))   # [50, 2, 128]
+    with pytest.raises(ValueError):
+        h.calibrate(sample[0])
+    h.calibrate(sample)
+    want0 = np.argsort(-scale, kind="stable")
+    assert h._group0_indices.shape == (2, 64) and h._group1_indices.shape == (2, 64)
+    assert np.array_equal(h._group0_indices[0].numpy(), want0[:64]) and np.array_equal(h._group1_indices[0].numpy(), want0[64:])
+    assert np.array_equal(h.group_order[1].numpy(), np.argsort(-scale[::-1], kind="stable"))
+    x = torch.from_numpy(rng.standard_normal((6, 2, 128)).astype(np.float32))
+    g = h.to_group_order(x, head_axis=1)
+    assert torch.equal(g[:, 0], x[:, 0][:, h.group_order[0]]) and torch.equal(g[:, 1], x[:, 1][:, h.group_order[1]])
+    assert torch.equal(h.from_group_order(g, head_axis=1), x)
+    # without a head axis: vectors cycle over the heads when their number is a multiple of the head count ...
+    assert torch.equal(h.to_group_order(x.reshape(12, 128)), g.reshape(12, 128))
+    # ... and use head 0's order otherwise
+    odd = x.reshape(12, 128)[:3]
+    assert torch.equal(h.to_group_order(odd), odd[:, h.group_order[0]])
+    assert torch.equal(h.from_group_order(h.to_group_order(odd)), odd)
+    u = HybridTurboQuant(device="cpu")
+    u.calibrate_uniform(4)
+    assert u.group_order is None and u.to_group_order(x) is x
