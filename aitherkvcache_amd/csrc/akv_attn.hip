@@ -51,9 +51,9 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
   const int s = blockIdx.x / groups, hg = blockIdx.x % groups;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int h = hg * 4 + wave;
-  // head_dim 128: the first half of this thread's column of Pi is requested before anything else, its
-  // round trip overlaps those of the partials
-  constexpr int PIPF = D == 128 ? 64 : 1;
+  // head_dim 128: this thread's column of Pi is requested before anything else, its round trip overlaps
+  // those of the partials (one wavefront per SIMD: the registers are there)
+  constexpr int PIPF = D == 128 ? 128 : 1;
   float pvr[PIPF];
   if constexpr (D == 128) {
 #pragma unroll
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
     // the first RED_PF partial accumulators are requested before anything is known about their
     // weights, so that their round trip overlaps the one of the (max, sum) pairs
-    constexpr int RED_PF = 16;
+    constexpr int RED_PF = D == 128 ? 32 : 16;
     float pre[RED_PF][DPL];
 #pragma unroll
     for (int u = 0; u < RED_PF; ++u) {
