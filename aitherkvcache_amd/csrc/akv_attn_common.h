@@ -153,6 +153,29 @@ __device__ __forceinline__ int akv_find_seq(const int32_t* __restrict__ prefix, 
   return lo;
 }
 
+// The same search for a whole wavefront with up to 63 sequences: lane i holds prefix[i] (one vector load at the
+// start of the kernel, `held`), the sequence is the number of entries 1..S that do not exceed g, and the bounds
+// of the sequence come out of the register -- no chain of dependent loads per segment.  More sequences than
+// that take the scalar search.
+__device__ __forceinline__ int akv_prefix_hold(const int32_t* __restrict__ prefix, int S) {
+  const int lane = threadIdx.x & 63;
+  return prefix[min(lane, S)];
+}
+__device__ __forceinline__ int akv_find_seq_held(const int32_t* __restrict__ prefix, int S, int held, int g,
+                                                 int& sb0, int& sb1) {
+  if (S <= 63) {
+    const int lane = threadIdx.x & 63;
+    const int s = __popcll(__ballot(lane >= 1 && lane <= S && held <= g));
+    sb0 = __builtin_amdgcn_readlane(held, s);
+    sb1 = __builtin_amdgcn_readlane(held, s + 1);
+    return s;
+  }
+  const int s = akv_find_seq(prefix, S, g);
+  sb0 = prefix[s];
+  sb1 = prefix[s + 1];
+  return s;
+}
+
 // merge (m, l, acc) <- (m, l, acc) (+) (ms, ls, accs)
 __device__ __forceinline__ void akv_lse_merge(float& m, float& l, float ms, float ls,
                                               float& alpha, float& beta) {

@@ -356,7 +356,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   // block, its second tile 16 positions further in.  bs32 is the same in every wavefront.
   const bool bs32 = a.block_size == 32;
   const int bs = bs32 ? 32 : 16;
-  const int total = a.prefix[a.S];
+  // (the block prefix of the batch in a register, one entry per lane: finding a segment's sequence and its
+  // bounds costs no chain of dependent loads)
+  const int held = akv_prefix_hold(a.prefix, a.S);
+  const int total = a.S <= 63 ? __builtin_amdgcn_readlane(held, a.S) : a.prefix[a.S];
   const int per = (total + G - 1) / G;
   const int g0 = blockIdx.x * per;
   const int g1 = min(total, g0 + per);
@@ -364,8 +367,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 
   int gcur = g0;
   while (gcur < g1) {
-    const int s = akv_find_seq(a.prefix, a.S, gcur);
-    const int sb0 = a.prefix[s], sb1 = a.prefix[s + 1];
+    int sb0, sb1;
+    const int s = akv_find_seq_held(a.prefix, a.S, held, gcur, sb0, sb1);
     const int blk_lo = gcur - sb0;
     const int blk_hi = min(g1, sb1) - sb0;
     const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
