@@ -208,6 +208,16 @@ def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
         one = tri.decode_step(t(q[b:b + 1], dev), SpectralEncoding(*(x[None] for x in k_enc)),
                               SpectralEncoding(*(x[None] for x in v_enc))).cpu().numpy()
         assert np.max(np.abs(one[0] - out[b])) <= 2e-6
+    # float16 queries stay float16 inside the kernel (its own query table), bfloat16 ones are widened
+    for qdt, npdt in ((torch.float16, np.float16),):
+        qh = q.astype(npdt)
+        out_h = tri.decode_step_paged(t(qh, dev), cache, bt, cl).cpu().numpy()
+        ref_h = O.tri_decode_step_paged(qh.astype(np.float32), arrays, tables, lens, BS, tri._theta.cpu().numpy())
+        assert np.max(np.abs(out_h - ref_h)) <= TOL
+    qb = torch.from_numpy(q).to(dev).bfloat16()
+    out_b = tri.decode_step_paged(qb, cache, bt, cl).cpu().numpy()
+    ref_b = O.tri_decode_step_paged(qb.float().cpu().numpy(), arrays, tables, lens, BS, tri._theta.cpu().numpy())
+    assert np.max(np.abs(out_b - ref_b)) <= TOL
 
 
 def test_paged_decode_without_table_columns(dev):
