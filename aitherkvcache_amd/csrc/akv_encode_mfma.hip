@@ -1,5 +1,5 @@
-// MFMA encode (norm -> rotate -> codebook search -> pack -> store) for float16 and bfloat16 input
-// at head_dim 128.
+// MFMA encode (norm -> rotate -> codebook search -> pack -> store) for float16, bfloat16 and float32
+// input at head_dim 128.
 //
 // The rotation is the only heavy arithmetic of the encode path (128 x 128 multiply-adds per
 // vector), so it runs on the matrix cores; everything else is arranged so that the matrix-core
@@ -11,7 +11,11 @@
 //         that ARE the four A operands (measured faster than the layout in which the four lanes
 //         of a row share each load).  float16 input is exact in the operand, so the vector is
 //         not normalised before the product: y = (sum_i Pi[j,i] x_i) * 1/(|x| + 1e-10), with one
-//         correctly rounded reciprocal per vector.
+//         correctly rounded reciprocal per vector.  float32 input is scaled by the power of two of the
+//         row's largest element and split into two float16 terms (hi + lo: every element to half a
+//         float32 ulp of itself, or to 2^-25 of the largest element where lo is subnormal); the product
+//         takes three MFMAs per tile (x_hi Pi_hi + x_hi Pi_lo + x_lo Pi_hi) and a wavefront step
+//         holds one M-tile instead of two, so that both terms of the rows fit the registers.
 //     B = Pi: float32 entries split into two float16 terms (hi + lo, scaled by 64 to stay clear
 //         of float16 subnormals), i.e. two MFMAs per tile and ~22 bits of the matrix.  N-tile nt,
 //         column col is output coordinate j = 8 col + nt.
@@ -128,9 +132,14 @@ __device__ __forceinline__ uint32_t em_cell(float y) {
   return __float_as_uint(fmaf(y, EM_CELL_S, EM_CELL_C)) & EM_CELL_MASK;
 }
 
-template <int BITS, bool PAGED, int XDT, bool DIRECT>
+// MT: M-tiles (16 vectors each) per wavefront step -- MT, or 1 for float32 input
+template <int BITS, bool PAGED, int XDT, bool DIRECT, int MT>
 __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
+  static_assert(MT <= MT && (XDT != AKV_F32 || MT == 1), "the LDS regions are sized for MT tiles");
+  constexpr int ROWS = 16 * MT;                       // vectors per wavefront step
+  constexpr int XB = XDT == AKV_F32 ? 4 : 2;          // bytes per input element
+  constexpr int NA = XDT == AKV_F32 ? 2 : 1;          // float16 terms of the input operand
   constexpr int NB = (1 << BITS) - 1;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -172,80 +181,87 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 
   unsigned char* wl = lds + EM_WAVE_OFF + wave * EM_WAVE_BYTES;
   int64_t* src_off = (int64_t*)wl;                    // address of the vector, or 0
-  int64_t* dst_p = (int64_t*)(wl + EM_ROWS * 8);      // address of the packed row, or 0
-  int64_t* dst_n = (int64_t*)(wl + EM_ROWS * 16);     // address of the norm
-  float* rinv = (float*)(wl + EM_ROWS * 24);          // 1/(|x| + 1e-10), scaled back by 1/EM_PSCALE; NaN rows flagged
+  int64_t* dst_p = (int64_t*)(wl + ROWS * 8);      // address of the packed row, or 0
+  int64_t* dst_n = (int64_t*)(wl + ROWS * 16);     // address of the norm
+  float* rinv = (float*)(wl + ROWS * 24);          // 1/(|x| + 1e-10), scaled back by 1/EM_PSCALE; NaN rows flagged
 
   const int64_t n_total = (PAGED && a.x2) ? 2 * a.n : a.n;      // a second tensor rides along (K and V of a step)
-  const int64_t steps = (n_total + EM_ROWS - 1) / EM_ROWS;
+  const int64_t steps = (n_total + ROWS - 1) / ROWS;
   const int64_t stride = (int64_t)gridDim.x * EM_WAVES;
 
   // A operands of one step straight from memory (zeros past the end): lane l resolves the source
   // row of vector base + l, the lanes of an M-tile pick the rows up through LDS
-  auto fetch = [&](em_half8 (&A)[EM_MT][4], int64_t step) {
+  // (a row's 32 elements of the lane as 16-byte pieces: four for 16-bit input -- the A operands themselves --
+  // eight for float32 input)
+  constexpr int NP = 4 * NA;
+  auto fetch = [&](uint4 (&R)[MT][NP], int64_t step) {
     if constexpr (DIRECT) {
       // contiguous rows whose byte offsets fit 31 bits: every lane forms its rows' addresses itself
       // (scalar base + 32-bit lane offset), no exchange through LDS
 #pragma unroll
-      for (int mt = 0; mt < EM_MT; ++mt) {
-        const uint32_t n = (uint32_t)step * EM_ROWS + 16 * mt + (lane & 15);
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint32_t n = (uint32_t)step * ROWS + 16 * mt + (lane & 15);
         if (n < (uint32_t)a.n) {
-          const uint4* p = (const uint4*)((const char*)a.x + (n * (uint32_t)a.xs0 + 32u * g) * 2u);
+          const uint4* p = (const uint4*)((const char*)a.x + (n * (uint32_t)a.xs0 + 32u * g) * (uint32_t)XB);
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks) {
-            union { uint4 u; em_half8 h; } cv;
-            cv.u = p[ks];
-            A[mt][ks] = cv.h;
-          }
+          for (int ks = 0; ks < NP; ++ks) R[mt][ks] = p[ks];
         } else {
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks) A[mt][ks] = (em_half8){0, 0, 0, 0, 0, 0, 0, 0};
+          for (int ks = 0; ks < NP; ++ks) R[mt][ks] = make_uint4(0u, 0u, 0u, 0u);
         }
       }
       return;
     }
-    int64_t n = step * EM_ROWS + lane;
+    int64_t n = step * ROWS + lane;
     int64_t so = 0;      // byte address of the vector, 0 = none
-    if (step < steps && n < n_total && lane < EM_ROWS) {
+    if (step < steps && n < n_total && lane < ROWS) {
       const bool second = PAGED && n >= a.n;
       if (second) n -= a.n;
       const char* xb = (const char*)(second ? a.x2 : a.x);
       if (PAGED) {
         const int64_t tok = n / a.heads, head = n - tok * a.heads;
-        so = (int64_t)(uintptr_t)(xb + 2 * (tok * a.xs0 + head * a.xs1));
+        so = (int64_t)(uintptr_t)(xb + XB * (tok * a.xs0 + head * a.xs1));
       } else {
-        so = (int64_t)(uintptr_t)(xb + 2 * n * a.xs0);
+        so = (int64_t)(uintptr_t)(xb + XB * n * a.xs0);
       }
     }
-    if (lane < EM_ROWS) src_off[lane] = so;
+    if (lane < ROWS) src_off[lane] = so;
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int64_t ro = src_off[16 * mt + (lane & 15)];
       if (ro != 0) {
-        const uint4* p = (const uint4*)(uintptr_t)(ro + 64 * g);
+        const uint4* p = (const uint4*)(uintptr_t)(ro + 32 * XB * g);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          union { uint4 u; em_half8 h; } cv;
-          cv.u = p[ks];
-          A[mt][ks] = cv.h;
-        }
+        for (int ks = 0; ks < NP; ++ks) R[mt][ks] = p[ks];
       } else {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) A[mt][ks] = (em_half8){0, 0, 0, 0, 0, 0, 0, 0};
+        for (int ks = 0; ks < NP; ++ks) R[mt][ks] = make_uint4(0u, 0u, 0u, 0u);
       }
     }
   };
 
   auto encode_step = [&](auto linear_tag, int64_t step) {
     constexpr bool LINEAR = decltype(linear_tag)::value;
-    em_half8 A[EM_MT][4];
-    fetch(A, step);
-    const int64_t base = step * EM_ROWS;
+    uint4 R[MT][NP];
+    fetch(R, step);
+    em_half8 A[MT][4];          // the operand (16-bit input), or its float16 hi term (float32 input)
+    em_half8 Alo[MT][4];        // float32 input: the lo term
+    if constexpr (XDT != AKV_F32) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          union { uint4 u; em_half8 h; } cv;
+          cv.u = R[mt][ks];
+          A[mt][ks] = cv.h;
+        }
+    }
+    const int64_t base = step * ROWS;
     // ---- lane l resolves the destination of vector base + l
     if constexpr (!DIRECT) {
       int64_t n = base + lane;
       int64_t dp = 0, dn = 0;      // byte addresses of the packed row and of the norm, 0 = skip
-      if (n < n_total && lane < EM_ROWS) {
+      if (n < n_total && lane < ROWS) {
         const bool second = PAGED && n >= a.n;
         if (second) n -= a.n;
         uint8_t* pb = second ? a.packed2 : a.packed;
@@ -265,19 +281,19 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           dn = (int64_t)(uintptr_t)(nb + n);
         }
       }
-      if (lane < EM_ROWS) {
+      if (lane < ROWS) {
         dst_p[lane] = dp;
         dst_n[lane] = dn;
       }
     }
-    float ss[EM_MT];
+    float ss[MT];
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt) ss[mt] = 0.f;
-    uint32_t unscale[EM_MT];     // float bits of the power of two taken out of each M-tile's rows
-    bool nonfinite[EM_MT];       // bfloat16 only: the row holds an infinity or a NaN
+    for (int mt = 0; mt < MT; ++mt) ss[mt] = 0.f;
+    uint32_t unscale[MT];     // float bits of the power of two taken out of each M-tile's rows
+    bool nonfinite[MT];       // bfloat16 only: the row holds an infinity or a NaN
     if constexpr (XDT == AKV_F16) {
 #pragma unroll
-      for (int mt = 0; mt < EM_MT; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) {
         unscale[mt] = 0x3f800000u;
         nonfinite[mt] = false;
 #pragma unroll
@@ -288,13 +304,62 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           for (int q = 0; q < 4; ++q) ss[mt] = __builtin_amdgcn_fdot2(cv.h2[q], cv.h2[q], ss[mt], false);
         }
       }
+    } else if constexpr (XDT == AKV_F32) {
+      // float32 rows: squared norm from the values themselves; then each row is scaled by the power of two
+      // that brings its largest element into [1, 2) and split into two float16 terms, both rounded to
+      // nearest: hi keeps 11 bits, x - hi is exact in float32 and has at most 12 significant bits and a sign,
+      // so lo is off by at most half a float32 ulp of the element (2^-25 of the largest element once lo is a
+      // float16 subnormal)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        uint32_t mx = 0u;
+#pragma unroll
+        for (int pc = 0; pc < NP; ++pc) {
+          const uint32_t w[4] = {R[mt][pc].x, R[mt][pc].y, R[mt][pc].z, R[mt][pc].w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            mx = max(mx, w[q] & 0x7fffffffu);
+            const float v = __uint_as_float(w[q]);
+            ss[mt] = fmaf(v, v, ss[mt]);
+          }
+        }
+        {   // largest magnitude of the row over its four lanes
+          auto r1 = __builtin_amdgcn_permlane32_swap(mx, mx, false, false);
+          mx = max(r1[0], r1[1]);
+          auto r2 = __builtin_amdgcn_permlane16_swap(mx, mx, false, false);
+          mx = max(r2[0], r2[1]);
+        }
+        uint32_t ef = mx >> 23;                      // exponent field of the largest element
+        nonfinite[mt] = ef == 255u;
+        if (ef == 0u || ef == 255u) ef = 127u;       // all (sub)zero, or not finite (flagged)
+        if (ef == 254u) ef = 253u;                   // keep the scale a normal number
+        const float sc = __uint_as_float((254u - ef) << 23);     // 2^(127 - ef)
+        unscale[mt] = ef << 23;                                   // 2^(ef - 127)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const float v[8] = {__uint_as_float(R[mt][2 * ks].x), __uint_as_float(R[mt][2 * ks].y),
+                              __uint_as_float(R[mt][2 * ks].z), __uint_as_float(R[mt][2 * ks].w),
+                              __uint_as_float(R[mt][2 * ks + 1].x), __uint_as_float(R[mt][2 * ks + 1].y),
+                              __uint_as_float(R[mt][2 * ks + 1].z), __uint_as_float(R[mt][2 * ks + 1].w)};
+          union { em_half8 h; em_half2 h2[4]; } hi, lo;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float x0 = v[2 * q] * sc, x1 = v[2 * q + 1] * sc;
+            const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+            hi.h2[q] = (em_half2){h0, h1};
+            lo.h2[q] = (em_half2){(_Float16)(x0 - (float)h0), (_Float16)(x1 - (float)h1)};
+          }
+          A[mt][ks] = hi.h;
+          Alo[mt][ks] = lo.h;
+        }
+      }
     } else {
       // bfloat16 rows: squared norm from the exact float32 values; then each row is scaled by the
       // power of two that brings its largest element into [1, 2) and converted to float16 -- exact
       // for every element within 2^14 of the largest (8 significant bits fit in 11), and off by at
       // most 2^-25 of the largest otherwise, far below the resolution of the codebook search
 #pragma unroll
-      for (int mt = 0; mt < EM_MT; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) {
         em_us2 mx2 = {0, 0};
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
@@ -337,37 +402,29 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         }
       }
     }
-    // lane l < EM_ROWS finishes vector l = 16 mt + row: transpose-reduce the partial sums over the
+    // lane l < ROWS finishes vector l = 16 mt + row: transpose-reduce the partial sums over the
     // four lanes of a row
     {
       const bool g1 = (g & 1) != 0;
-#if EM_MT == 4
-      const bool g2 = (g & 2) != 0;
-      const float a01 = (g1 ? ss[1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[1], 16, 64);
-      const float a23 = (g1 ? ss[3] : ss[2]) + __shfl_xor(g1 ? ss[2] : ss[3], 16, 64);
-      const float mine = (g2 ? a23 : a01) + __shfl_xor(g2 ? a01 : a23, 32, 64);
-#else
-      const float a01 = (g1 ? ss[1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[1], 16, 64);
-      const float mine = a01 + __shfl_xor(a01, 32, 64);     // lanes g and g + 2 both hold M-tile g & 1
-#endif
+      float mine;
+      if constexpr (MT == 1) {
+        const float a01 = ss[0] + __shfl_xor(ss[0], 16, 64);
+        mine = a01 + __shfl_xor(a01, 32, 64);                 // all four lanes of a row hold its sum
+      } else {
+        static_assert(MT <= 2, "two M-tiles at most");
+        const float a01 = (g1 ? ss[MT - 1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[MT - 1], 16, 64);
+        mine = a01 + __shfl_xor(a01, 32, 64);                 // lanes g and g + 2 both hold M-tile g & 1
+      }
       const float nrm = sqrtf(mine);
-#if EM_MT == 4
-      const uint32_t my_unscale = g == 0 ? unscale[0] : g == 1 ? unscale[1] : g == 2 ? unscale[2] : unscale[3];
-#else
-      const uint32_t my_unscale = g1 ? unscale[1] : unscale[0];
-#endif
+      const uint32_t my_unscale = (MT > 1 && g1) ? unscale[MT - 1] : unscale[0];
       const float r = (1.f / (nrm + 1e-10f)) * (1.f / EM_PSCALE) * __uint_as_float(my_unscale);
       // a vector with a NaN or an infinity rotates to NaN everywhere: every code is the last level.
       // (float16 squares cannot overflow, so there an infinite norm means an infinite element; a
       // finite bfloat16 row whose squares overflow has norm inf, unit vector 0 and y = 0 like the
       // reference: r is 0 and the scaled products are finite.)
-#if EM_MT == 4
-      const bool my_nonfinite = g == 0 ? nonfinite[0] : g == 1 ? nonfinite[1] : g == 2 ? nonfinite[2] : nonfinite[3];
-#else
-      const bool my_nonfinite = g1 ? nonfinite[1] : nonfinite[0];
-#endif
-      const bool nan_row = XDT == AKV_F16 ? !(nrm < INFINITY) : (my_nonfinite || nrm != nrm);
-      if (lane < EM_ROWS) {
+      const bool my_nonfinite = (MT > 1 && g1) ? nonfinite[MT - 1] : nonfinite[0];
+      const bool nan_row = XDT == AKV_F16 ? !(nrm < INFINITY) : (my_nonfinite || nrm != nrm);   // (float32 as bfloat16)
+      if (lane < ROWS) {
         rinv[lane] = nan_row ? __uint_as_float(0x7fc00000u) : r;
         if constexpr (DIRECT) {
           if ((uint32_t)base + lane < (uint32_t)a.n) a.norms[(uint32_t)base + lane] = nrm;
@@ -377,34 +434,36 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       }
     }
     // ---- rotate, search, pack
-    uint32_t packed[EM_MT][4];
+    uint32_t packed[MT][4];
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) packed[mt][i] = 0u;
-    em_float4 rv[EM_MT];
+    em_float4 rv[MT];
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       union { em_u32x4 u; em_float4 f; } cv;
-      cv.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_WAVE_OFF + wave * EM_WAVE_BYTES + EM_ROWS * 24 + (16 * mt + 4 * g) * 4);
+      cv.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_WAVE_OFF + wave * EM_WAVE_BYTES + ROWS * 24 + (16 * mt + 4 * g) * 4);
       rv[mt] = cv.f;
     }
     // N-tiles are software-pipelined: the matrix-core work of tile nt + 1 is issued together with
     // the search of tile nt (independent instruction streams in one basic block), so the vector
     // unit works in the shadow of the MFMAs.  The loop stays rolled (two tiles per pass): unrolled,
     // the scheduler would want every B operand in registers at once.
-    auto mfma_tile = [&](int nt, em_float4 (&acc)[EM_MT]) {
+    auto mfma_tile = [&](int nt, em_float4 (&acc)[MT]) {
 #pragma unroll
-      for (int mt = 0; mt < EM_MT; ++mt) acc[mt] = (em_float4){0.f, 0.f, 0.f, 0.f};
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = (em_float4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         union { em_u32x4 u; em_half8 h; } bh, bl;
         bh.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_B_OFF + ((nt * 4 + ks) * 64 + lane) * 16);
         bl.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_B_OFF + 32768 + ((nt * 4 + ks) * 64 + lane) * 16);
 #pragma unroll
-        for (int mt = 0; mt < EM_MT; ++mt) {
+        for (int mt = 0; mt < MT; ++mt) {
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bh.h, acc[mt], 0, 0, 0);
           acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[mt][ks], bl.h, acc[mt], 0, 0, 0);
+          if constexpr (XDT == AKV_F32)
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Alo[mt][ks], bh.h, acc[mt], 0, 0, 0);
         }
       }
     };
@@ -414,21 +473,21 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     auto tile_at = [&](int k) -> int {
       return BITS == 4 ? 6 - (k & ~1) + (k & 1) : BITS == 3 ? k : ((k + 4) & 7);
     };
-    auto search_tile = [&](const em_float4 (&acc)[EM_MT]) {
-      float y[EM_MT][4];
+    auto search_tile = [&](const em_float4 (&acc)[MT]) {
+      float y[MT][4];
 #pragma unroll
-      for (int mt = 0; mt < EM_MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) y[mt][i] = acc[mt][i] * rv[mt][i];
       if constexpr (!LINEAR) {
-        em_u32x2 e[EM_MT][4];
+        em_u32x2 e[MT][4];
 #pragma unroll
-        for (int mt = 0; mt < EM_MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             e[mt][i] = *(em_lds_u64*)(uintptr_t)em_cell(y[mt][i]);
 #pragma unroll
-        for (int mt = 0; mt < EM_MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t code = e[mt][i].x + ((__uint_as_float(e[mt][i].y) < y[mt][i]) ? 1u : 0u);
@@ -436,7 +495,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           }
       } else {
 #pragma unroll
-        for (int mt = 0; mt < EM_MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             uint32_t code = 0;
@@ -446,7 +505,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
           }
       }
     };
-    em_float4 accA[EM_MT], accB[EM_MT];
+    em_float4 accA[MT], accB[MT];
     mfma_tile(tile_at(0), accA);
 #pragma unroll 1
     for (int k = 0; k < 6; k += 2) {
@@ -456,7 +515,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       search_tile(accB);
       // issue order of the pass: one MFMA, then the vector and LDS work that fits in its shadow
 #pragma unroll
-      for (int q = 0; q < 16 * EM_MT; ++q) {
+      for (int q = 0; q < 8 * (NA + 1) * MT; ++q) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
         __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // VALU
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
@@ -465,7 +524,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     mfma_tile(tile_at(7), accB);
     search_tile(accA);
 #pragma unroll
-    for (int q = 0; q < 8 * EM_MT; ++q) {
+    for (int q = 0; q < 4 * (NA + 1) * MT; ++q) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -473,7 +532,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     search_tile(accB);
     // ---- store: lane (col, g) writes group col of rows 4g + i
 #pragma unroll
-    for (int mt = 0; mt < EM_MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int row = 16 * mt + 4 * g + i;
@@ -520,14 +579,16 @@ static bool em_disabled() {
 
 int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, int bits,
                         const void* rot_prep, hipStream_t stream) {
-  if (em_disabled() || d != 128 || (x_dtype != AKV_F16 && x_dtype != AKV_BF16)) return AKV_ERR_UNSUPPORTED;
+  if (em_disabled() || d != 128 || (x_dtype != AKV_F16 && x_dtype != AKV_BF16 && x_dtype != AKV_F32)) return AKV_ERR_UNSUPPORTED;
   // 16-byte loads of the input rows; aligned stores of the packed groups
-  if (((uintptr_t)a.x & 15) || ((uintptr_t)a.x2 & 15) || (a.xs0 & 7) || (paged && (a.xs1 & 7))) return AKV_ERR_UNSUPPORTED;
+  const int64_t xmask = x_dtype == AKV_F32 ? 3 : 7;        // elements per 16 bytes, minus one
+  if (((uintptr_t)a.x & 15) || ((uintptr_t)a.x2 & 15) || (a.xs0 & xmask) || (paged && (a.xs1 & xmask))) return AKV_ERR_UNSUPPORTED;
   const int64_t amask = bits == 4 ? 3 : bits == 2 ? 1 : 0;
   if (((uintptr_t)a.packed | (uintptr_t)a.packed2 | (uintptr_t)a.ps0 | (uintptr_t)a.ps1 | (uintptr_t)a.ps2) & amask) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const float*)rot_prep + (size_t)2 * d * d);
   const int64_t n_total = (paged && a.x2) ? 2 * a.n : a.n;
-  const int64_t steps = (n_total + EM_ROWS - 1) / EM_ROWS;
+  const int rows_per_step = x_dtype == AKV_F32 ? 16 : EM_ROWS;
+  const int64_t steps = (n_total + rows_per_step - 1) / rows_per_step;
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
   const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
@@ -535,15 +596,16 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   do {                                                                                               \
     static bool configured = false;                                                                  \
     if (!configured) {                                                                               \
-      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT, DR>,                 \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT)>, \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, EM_LDS_BYTES));        \
       configured = true;                                                                             \
     }                                                                                                \
-    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, DR>), grid, EM_THREADS, EM_LDS_BYTES, stream, a, bop); \
+    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT)>), grid, EM_THREADS, EM_LDS_BYTES, stream, a, bop); \
   } while (0)
-#define EM_LAUNCH_DT(BB, PG, DR) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16, DR); else EM_LAUNCH(BB, PG, AKV_BF16, DR); } while (0)
+#define EM_LAUNCH_DT(BB, PG, DR) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16, DR); else if (x_dtype == AKV_BF16) EM_LAUNCH(BB, PG, AKV_BF16, DR); else EM_LAUNCH(BB, PG, AKV_F32, DR); } while (0)
   // flat rows whose byte offsets stay below 2^31 take the variant with 32-bit lane offsets
-  const bool direct = !paged && a.n < ((int64_t)1 << 31) / (2 * a.xs0 > a.ps0 ? 2 * a.xs0 : a.ps0);
+  const int64_t xbytes = x_dtype == AKV_F32 ? 4 : 2;
+  const bool direct = !paged && a.n < ((int64_t)1 << 31) / (xbytes * a.xs0 > a.ps0 ? xbytes * a.xs0 : a.ps0);
   if (paged) {
     if (bits == 4) EM_LAUNCH_DT(4, true, false); else if (bits == 3) EM_LAUNCH_DT(3, true, false); else EM_LAUNCH_DT(2, true, false);
   } else if (direct) {

@@ -168,6 +168,18 @@ def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds, sweep=True
     res["kernel_mvec_s"] = n / kms / 1e3
     res["kernel_gbs"] = n * 324 / kms / 1e6
     res["kernel_frac_hbm"] = res["kernel_gbs"] / HBM_PEAK_GBS
+    # the same vectors as float32 input (512 B read + 68 B written per vector)
+    x32 = [v.float() for v in xs]
+
+    def enc32_step():
+        tq.encode(x32[st["i"] & 1])
+        st["i"] += 1
+    enc32_step()
+    kms32 = kernel_ms(torch, L, enc32_step, 32)
+    res["f32_input_kernel_mvec_s"] = n / kms32 / 1e3
+    res["f32_input_kernel_gbs"] = n * 580 / kms32 / 1e6
+    res["f32_input_kernel_frac_hbm"] = res["f32_input_kernel_gbs"] / HBM_PEAK_GBS
+    del x32
     # decode of the same vectors (68 B in, 256 B out per vector)
     coded = [tq.encode(v) for v in xs]
 

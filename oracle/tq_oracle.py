@@ -172,15 +172,20 @@ def rotate_unit_f64(x, rotation):
     return u @ rotation.astype(np.float64).T
 
 
-def boundary_ulp_distance(y64, boundaries):
-    """Distance from each float64 rotated value to the nearest decision boundary, in units of
-    the float32 ulp at that boundary (spacing of float32 at |b|; at b == 0 the spacing near
-    the values that actually occur, taken at 2**-24 relative to the typical |y|)."""
+def boundary_ulp_distance(y64, boundaries, floor=None):
+    """Distance from each float64 rotated value to the nearest decision boundary, in float32 ulps.
+    The ulp is taken at the largest of |boundary|, |value| and `floor`.  `floor` is the magnitude of
+    the largest term of the dot product that made the value: a float32 dot product resolves nothing
+    below one ulp of its largest term, so where the terms cancel (a value a few 1e-9 from the
+    boundary at 0 out of terms of 1e-2) the value's own ulp says nothing about what float32
+    arithmetic can decide."""
     b = np.asarray(boundaries, dtype=np.float64)
     d = np.abs(y64[..., None] - b)
     k = np.argmin(d, axis=-1)
     nearest = b[k]
     scale = np.maximum(np.abs(nearest), np.abs(y64))
+    if floor is not None:
+        scale = np.maximum(scale, np.asarray(floor, dtype=np.float64))
     ulp = np.spacing(np.maximum(scale, 1e-30).astype(f32)).astype(np.float64)
     return np.min(d, axis=-1) / ulp
 

@@ -72,6 +72,39 @@ def test_encode_bfloat16_wide_range_vs_oracle(golden, dev, bits):
     assert np.all(np.isinf(norms.cpu().numpy()))
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_encode_float32_wide_range_vs_oracle(golden, dev, bits):
+    """float32 rows are scaled by a power of two and split into two float16 terms for the matrix cores: rows of
+    very large, very small and mixed magnitudes, a zero row, odd row counts and strided rows must give the
+    oracle's codes (every differing code within the boundary allowance of check_codes)."""
+    rng = np.random.default_rng(177 + bits)
+    n = 20000 + 13
+    x = rng.standard_normal((n, 128)).astype(np.float32)
+    scale = np.exp2(rng.integers(-60, 60, size=n)).astype(np.float32)         # rows from 2^-60 to 2^60
+    x *= scale[:, None]
+    x[::7] *= np.exp2(rng.integers(-30, 1, size=(len(x[::7]), 128))).astype(np.float32)   # wide range inside a row
+    x[3] = 0.0
+    x[4] = 0.0
+    x[4, 17] = -3.25                                                           # one non-zero element
+    tq = make_tq(golden, dev, bits)
+    xt = torch.from_numpy(x).to(dev)
+    packed, norms = tq.encode(xt)
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, golden["rotation_d128_seed42"], bits)
+    # rows with a stride (a column slice of a wider tensor) and a leading batch shape
+    wide = torch.zeros(50, 3, 256, device=dev)
+    wide[..., 64:192] = xt[:150].reshape(50, 3, 128)
+    p2, n2 = tq.encode(wide[..., 64:192])
+    assert torch.equal(p2.reshape(150, -1), packed[:150]) and torch.equal(n2.reshape(150), norms[:150])
+    # overflowing squares, an infinity, a NaN
+    y = torch.full((3, 128), 2.0 ** 70, dtype=torch.float32)
+    y[1, 5] = float("inf")
+    y[2, 100] = float("nan")
+    packed, norms = tq.encode(y.to(dev))
+    codes = O._UNPACK[bits](packed.cpu().numpy(), 128)
+    assert np.all(codes[0] == (1 << bits) // 2 - 1) and np.all(codes[1] == (1 << bits) - 1) and np.all(codes[2] == (1 << bits) - 1)
+    assert np.all(np.isinf(norms.cpu().numpy()[:2])) and np.isnan(norms.cpu().numpy()[2])
+
+
 def test_head_dim_64(golden, dev):
     tq = make_tq(golden, dev, 4, d=64)
     x = golden["enc_x_d64"]
@@ -223,7 +256,7 @@ def test_k_and_v_in_one_launch_equal_two_launches(golden, dev, bits, dtype, toke
     """fused_kv_update_pair against two fused_kv_update calls (those are checked against the oracle
     above): byte-identical caches and norms.  Token counts that leave the K / V seam inside a step of the
     kernel, padding slots, slots beyond max_blocks, and the K / V halves of one serving cache tensor
-    (rows 4 bytes longer than the codes).  float32 input takes two launches inside the pair call."""
+    (rows 4 bytes longer than the codes)."""
     tq = make_tq(golden, dev, bits)
     H, NB, BS, P = 8, 40, 16, tq._packed_dim
     g = torch.Generator(device=dev).manual_seed(1000 * bits + tokens)

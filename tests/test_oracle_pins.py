@@ -348,3 +348,15 @@ def test_hybrid_margins_accept_the_oracle_and_catch_defects(golden):
     assert m["code_ulps"][0][7].max() > 1e3 and m["sign_ulps"][0][9].max() > 1e3
     assert m["code_ulps"][1][11].max() > 1e3 and abs(int(m["norm_steps"][1][13])) > 100
     assert m["code_ulps"][0][8].max() == 0 and m["sign_ulps"][1][9].max() == 0
+
+
+def test_boundary_distance_counts_ulps_of_the_largest_term_under_cancellation():
+    """A value 4e-9 above the boundary at 0 that came out of terms of 2e-2 is two float32 ulps of those terms
+    away from it, not millions of ulps of itself; away from cancellation the floor changes nothing."""
+    b = np.array([-0.02, 0.0, 0.02])
+    y = np.array([3.99e-9, 0.0200001])
+    plain = O.boundary_ulp_distance(y, b)
+    assert plain[0] > 1e6 and abs(plain[1] - 1e-7 / np.spacing(np.float32(0.0200001))) < 1e-3
+    floored = O.boundary_ulp_distance(y, b, floor=np.array([0.018, 0.018]))
+    assert abs(floored[0] - 3.99e-9 / np.spacing(np.float32(0.018))) < 1e-6 and floored[0] < 3
+    assert floored[1] == plain[1]

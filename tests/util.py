@@ -14,13 +14,19 @@ def kv_like(rng, shape, dtype=np.float16):
     return (g * s[..., None]).astype(dtype)
 
 
-def code_mismatch_report(codes_a, codes_b, y64, boundaries, oracle):
+def code_mismatch_report(codes_a, codes_b, y64, boundaries, oracle, unit64=None, R=None):
     """Where two code arrays differ, how far (in float32 ulps) the float64 rotated value is from
-    the nearest decision boundary.  Returns (count, max_ulps, histogram dict)."""
+    the nearest decision boundary.  With the unit vectors and the matrix given, the ulp is not taken
+    below that of the largest term R[j, i] * u[i] of the coordinate's dot product (cancellation).
+    Returns (count, max_ulps, histogram dict)."""
     diff = np.argwhere(codes_a != codes_b)
     if len(diff) == 0:
         return 0, 0.0, {}
-    ulps = oracle.boundary_ulp_distance(y64, boundaries)[tuple(diff.T)]
+    rows, cols = diff.T
+    floor = None
+    if unit64 is not None and R is not None:
+        floor = np.max(np.abs(np.asarray(R, dtype=np.float64)[cols] * unit64[rows]), axis=-1)
+    ulps = oracle.boundary_ulp_distance(y64[rows, cols], boundaries, floor)
     steps = np.abs(codes_a.astype(np.int64) - codes_b.astype(np.int64))[tuple(diff.T)]
     hist = {"<=1": int((ulps <= 1).sum()), "<=4": int(((ulps > 1) & (ulps <= 4)).sum()),
             "<=16": int(((ulps > 4) & (ulps <= 16)).sum()), ">16": int((ulps > 16).sum()),
@@ -35,8 +41,11 @@ def check_codes(packed, norms, x, R, bits, ref_packed=None, ref_norms=None, d=12
         ref_packed, ref_norms = O.encode(x, R, b, bits)
     ca = O._UNPACK[bits](packed.reshape(-1, packed.shape[-1]), d)
     cb = O._UNPACK[bits](ref_packed.reshape(-1, ref_packed.shape[-1]), d)
+    x64 = np.asarray(x).reshape(-1, d).astype(np.float64)
     y64 = O.rotate_unit_f64(np.asarray(x).reshape(-1, d), R)
-    n, max_ulps, hist = code_mismatch_report(ca, cb, y64, b, O)
+    with np.errstate(invalid="ignore", over="ignore"):
+        unit64 = x64 / (np.linalg.norm(x64, axis=-1, keepdims=True) + 1e-10)
+    n, max_ulps, hist = code_mismatch_report(ca, cb, y64, b, O, unit64, R)
     total = ca.size
     print(f"[codes] bits={bits} mismatching={n}/{total} max_ulps={max_ulps:.2f} hist={hist}")
     assert max_ulps <= MAX_ULPS, hist
