@@ -28,7 +28,7 @@
 //            builds, for each of the 8 coordinates, the 8-token k-slice; M-tile j row m is
 //            coordinate 8m + j.
 //
-// Dequantisation goes through tables in LDS indexed by a whole BYTE: entry (a<<4|b) is the fp16
+// Dequantisation goes through tables in LDS.  4-bit: indexed by a whole BYTE, entry (a<<4|b) is the fp16
 // pair (c[a], c[b]).  For K a byte holds two neighbouring coordinates of one token -- already a
 // k-pair; a K entry is 8 bytes, the hi pair and the lo pair (c = hi + lo to ~22 bits), fetched by
 // ONE LDS read (the LDS issues about one wavefront read per three to five cycles whatever its
@@ -39,11 +39,21 @@
 // table entry is replicated 32 times (address = entry * 256 + (lane & 31) * entry size), so lookups
 // never conflict on a bank.
 //
-// The 3-bit and 2-bit caches go through the same tables and the same products: their packed rows
-// are first spread to one code per NIBBLE in registers (a handful of shifts and masks per eight
-// codes, in whatever nibble order is cheapest), and the order is undone for free -- on the K side by
-// building the query operand in the same coordinate order, on the V side by the order in which the
-// accumulators are written out.
+// The 3-bit and 2-bit caches index tables of their own shape with the packed bits as they lie in memory (no
+// spreading to nibbles; the tq35 kernel below, whose parts mix code widths, does spread):
+//   3-bit  a group of eight codes is a big-endian 24-bit word (one byte permute); an index is a 6-bit FIELD of it.
+//          K: field = two neighbouring codes of a token, 64 entries of 8 bytes.  V: the codes at odd and at even
+//          positions of two neighbouring tokens are merged into two words of four fields (three operations
+//          each), 64 entries of 4 bytes.  An address costs two operations (field extract, shift-or) instead of
+//          one byte permute.
+//   2-bit  an index is a code BYTE.  K: four neighbouring codes of a token = the whole 16-byte A operand of one
+//          MFMA (hi pair, lo pair, hi pair, lo pair), 16 copies per entry (a 16-byte read is served 16 lanes at a
+//          time).  V: the same coordinate of FOUR tokens (tokens 4g, 4g+1 of both tiles, or 4g+2, 4g+3), 8-byte
+//          entries, 32 copies; the four halfwords of a tile are loaded two to a register and merged by bit-field
+//          inserts (16 operations for all 16 lookups of a chunk).  The weights are written in the same token
+//          order.  With 64 KB + 64 KB of tables the exchange buffers live in a third region (160 KB in all).
+// The order in which the coordinates reach the value product differs per format; it is undone for free by the order
+// in which the accumulators are written out (mf_vtile).  The query operand is in natural coordinate order for all.
 #include "akv_attn_common.h"
 #include "akv_nibble.h"
 
@@ -59,6 +69,11 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 // entry e of table B at 65536 + e*256:  [fp16(alpha c) pairs for V x 32 copies][128 bytes of exchange buffer]
 #define MF_TABB 65536u
 #define MF_XBUF 4096u                // distance of the two exchange buffers of a head slot
+// exchange units of the kernel for the uniform formats: stride and start (4- and 3-bit: the spare halves of table B
+// entries; 2-bit: 128-byte units after the tables)
+#define MF_XSTRIDE(bits) ((bits) == 2 ? 128u : 256u)
+#define MF_XBASE(bits) ((bits) == 2 ? 131072u : MF_TABB + 128u)
+#define MF_LDS_BYTES_2BIT (160 * 1024)
 #define MF_ALPHA_CANDIDATES 65536
 // words of the table block kept in the workspace
 #define MF_W_KHI 0
@@ -188,17 +203,17 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     }
   }
   __syncthreads();
-  // operand layout: [k-step n][lane (col, g)][e]: bytes 2(n%2) + e/4 of transcoded dword n/2, nibble e%2
-  // (4-bit: coordinate 32g + 4n + 2(e/4) + e%2); elements 2,3 and 6,7 repeat 0,1 and 4,5: they face
-  // the lo halves of the K table entries
+  // operand layout: [k-step n][lane (col, g)][e]: coordinate 32g + 4n + 2(e/4) + e%2 -- the four coordinates
+  // of k-step n are the two code bytes (4-bit), the two 6-bit fields (3-bit) or the one code byte (2-bit) the
+  // score wavefront looks up for that step; elements 2,3 and 6,7 repeat 0,1 and 4,5: they face the lo
+  // halves of the K table entries
   for (int n = tid >> 6; n < 8; n += 4) {
     const int lane = tid & 63;
     const int col = lane & 15, g = lane >> 4;
     unsigned short hbits[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int st = n >> 1, b = 2 * (n & 1) + (e >> 2), lo = e & 1;
-      const int dim = 32 * g + (bits == 4 ? mf_kcoord<4>(st, b, lo) : bits == 3 ? mf_kcoord<3>(st, b, lo) : mf_kcoord<2>(st, b, lo));
+      const int dim = 32 * g + 4 * n + 2 * (e >> 2) + (e & 1);
       float v = 0.f;
       if (col < 8) {
         if (col < gqa) v = __half2float(__float2half_rn(qr_lds[col][dim]));
@@ -240,6 +255,38 @@ __device__ __forceinline__ uint32_t mf_lut(uint32_t lanebits, uint32_t word, uin
 __device__ __forceinline__ mf_u32x2 mf_lut2(uint32_t lanebits, uint32_t word, uint32_t sel) {
   const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
   return *(mf_lds_cu64*)(uintptr_t)addr;
+}
+
+// 2-bit K lookup: the whole A operand of one MFMA (four coordinates of one code byte, hi and lo pairs)
+typedef __attribute__((address_space(3))) const mf_u32x4 mf_lds_cu128;
+__device__ __forceinline__ mf_u32x4 mf_lut4(uint32_t lanebits, uint32_t word, uint32_t sel) {
+  const uint32_t addr = __builtin_amdgcn_perm(word, lanebits, sel);
+  return *(mf_lds_cu128*)(uintptr_t)addr;
+}
+// 3-bit lookups: the table index is a 6-bit field (two codes) of a 24-bit word; address = field * 256 + lanebits
+__device__ __forceinline__ uint32_t mf_addr6(uint32_t lanebits, uint32_t word, int shift) {
+  return (__builtin_amdgcn_ubfe(word, (uint32_t)shift, 6u) << 8) | lanebits;
+}
+// K lookup number b (0..3) of a code word: 4-bit byte b, 3-bit field b from the top of the 24-bit word
+template <int BITS>
+__device__ __forceinline__ mf_u32x2 mf_klook(uint32_t lanebits, uint32_t word, int b) {
+  if constexpr (BITS == 3) return *(mf_lds_cu64*)(uintptr_t)mf_addr6(lanebits, word, 18 - 6 * b);
+  else return mf_lut2(lanebits, word, MF_SEL(b));
+}
+// V lookup number k (0..3) of a regrouped word: 4-bit byte k, 3-bit field k from the bottom
+template <int BITS>
+__device__ __forceinline__ uint32_t mf_vlook(uint32_t lanebits, uint32_t word, int k) {
+  if constexpr (BITS == 3) return *(mf_lds_cu32*)(uintptr_t)mf_addr6(lanebits, word, 6 * k);
+  else return mf_lut(lanebits, word, MF_SEL(k));
+}
+// M-tile of the value product that holds coordinate k of the lane's eight (the order in which the regrouping
+// of the code words hands the coordinates to the lookups)
+template <int BITS>
+__host__ __device__ constexpr int mf_vtile(int k) {
+  if (BITS == 4) return k;
+  if (BITS == 3) return 7 - k;
+  constexpr int t2[8] = {6, 2, 4, 0, 7, 3, 5, 1};
+  return t2[k];
 }
 
 __device__ __forceinline__ half8 mf_pack(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -320,8 +367,10 @@ struct mf_kraw {       // score wavefront, one 32-token chunk
   float nrm;           // lane < 32: K norm of token l, else V norm of token l - 32
 };
 typedef uint32_t mf_u32x3 __attribute__((ext_vector_type(3)));
+typedef uint16_t mf_u16x2 __attribute__((ext_vector_type(2)));
 struct mf_vraw {       // value wavefront
-  uint32_t v[8];       // V codes: token tau(g,e), the eight codes 8(l%16) .. 8(l%16)+7 (4 / 3 / 2 bytes)
+  uint32_t v[8];       // V codes: token tau(g,e), the eight codes 8(l%16) .. 8(l%16)+7 (4 / 3 bytes); 2-bit: v[2j + i],
+                       // tokens 4g + i (low half) and 4g + i + 2 (high half) of tile j, two bytes each
 };
 
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
@@ -340,15 +389,19 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   // flag hand-offs through LDS instead of the barrier, polled by the waiting side, were 5 % slower at
   // 4 bits: every poll is an LDS round trip on the critical path of its wavefront.)
   constexpr bool SYNC = true;
-  const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * 4u;   // V lookups: first halves of table B entries
-  const uint32_t lane4k = (uint32_t)(lane & 31) * 8u;             // K lookups: table A
+  // the copy of a table entry a lane reads (2-bit: 16 copies of 16-byte K entries and 32 of 8-byte V entries, else
+  // 32 copies of 8 and 4 bytes)
+  const uint32_t lane4v = MF_TABB + (uint32_t)(lane & 31) * (BITS == 2 ? 8u : 4u);   // 2-bit: whole entries of table B, else their first halves
+  const uint32_t lane4k = BITS == 2 ? (uint32_t)(lane & 15) * 16u : (uint32_t)(lane & 31) * 8u;               // table A
   // exchange buffers of this head slot: buffer b -> unit q = hs*2 + b = 16 entries' spare halves of table B
   //   weights (16 B per lane): entry 16q + lane/8, offset 128 + (lane%8)*16
   //   rescale (4 B per lane):  entry 16q + 8 + lane/32, offset 128 + (lane%32)*4
-  // (buffer 1 lies MF_XBUF bytes after buffer 0; the parity of the chunk is a compile-time constant
+  // (buffer 1 lies 16 entries after buffer 0; the parity of the chunk is a compile-time constant
   // at every use, so it folds into the offset field of the LDS instruction)
-  const uint32_t pb_addr = MF_TABB + (32u * hs + (uint32_t)(lane >> 3)) * 256u + 128u + (uint32_t)(lane & 7) * 16u;
-  const uint32_t rs_addr = MF_TABB + (32u * hs + 8u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)(lane & 31) * 4u;
+  // (2-bit: the V entries fill table B, the exchange units are 128-byte entries of a region of their own after it)
+  constexpr uint32_t XS = MF_XSTRIDE(BITS), XB0 = MF_XBASE(BITS), XPAR = 16u * XS;
+  const uint32_t pb_addr = XB0 + (32u * hs + (uint32_t)(lane >> 3)) * XS + (uint32_t)(lane & 7) * 16u;
+  const uint32_t rs_addr = XB0 + (32u * hs + 8u + (uint32_t)(lane >> 5)) * XS + (uint32_t)(lane & 31) * 4u;
 
 
   const int G = gridDim.x;
@@ -438,8 +491,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vns_head + npos * a.vns_pos
                                                      : hd * a.kns_head + npos * a.kns_pos);
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
-        const uint32_t nw_addr = MF_TABB + (32u * hs + 10u + (uint32_t)(lane >> 5)) * 256u + 128u + (uint32_t)ntok * 4u;
-        const uint32_t nr_addr = MF_TABB + (32u * hs + 10u) * 256u + 128u + (uint32_t)g * 16u;
+        const uint32_t nw_addr = XB0 + (32u * hs + 10u + (uint32_t)(lane >> 5)) * XS + (uint32_t)ntok * 4u;
+        const uint32_t nr_addr = XB0 + (32u * hs + 10u) * XS + (uint32_t)g * 16u;
         auto load_chunk = [&](mf_kraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
@@ -460,37 +513,63 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
         auto produce = [&](mf_kraw& r, int c, const uint32_t par) {
           float sv[8];
-          *(mf_lds_u32*)(uintptr_t)(nw_addr + MF_XBUF * par) = __float_as_uint(r.nrm);
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + XPAR * par) = __float_as_uint(r.nrm);
           {
-            // 8 steps (tile j, dword st): 4 table reads (hi and lo of each of the dword's 4 bytes) feed
-            // two MFMAs (bytes 0,1 and bytes 2,3); the reads of step n+2 are issued before the MFMAs of step n
-            uint32_t kw[8];       // one code per nibble, two codes per byte
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const uint32_t raw[4] = {r.k[j].x, r.k[j].y, r.k[j].z, r.k[j].w};
-              uint32_t sp[4];
-              mf_spread_row<BITS>(raw, sp);
-#pragma unroll
-              for (int d = 0; d < 4; ++d) kw[4 * j + d] = sp[d];
-            }
-            mf_u32x2 w[3][4];      // ring of three steps: two in flight behind the one multiplied
+            // 8 steps of two MFMAs; the table reads of step n+2 are issued before the MFMAs of step n.
+            //   4-bit: step = (tile j, dword st), 4 reads (one per code byte: hi and lo of two coordinates)
+            //   3-bit: step = (tile j, group of 8 codes as a big-endian 24-bit word), 4 reads (one per 6-bit field)
+            //   2-bit: step = (tile j, half of a dword), 2 reads (one per code byte: a whole MFMA operand)
             float4v acc[2];
             acc[0] = (float4v){0.f, 0.f, 0.f, 0.f};
             acc[1] = (float4v){0.f, 0.f, 0.f, 0.f};
+            if constexpr (BITS == 2) {
+              const uint32_t kw[4] = {r.k[0].x, r.k[0].y, r.k[1].x, r.k[1].y};
+              mf_u32x4 w[3][2];
 #pragma unroll
-            for (int n = 0; n < 2; ++n)
+              for (int n = 0; n < 2; ++n)
 #pragma unroll
-              for (int b = 0; b < 4; ++b) w[n][b] = mf_lut2(lane4k, kw[n], MF_SEL(b));
+                for (int b = 0; b < 2; ++b) w[n][b] = mf_lut4(lane4k, kw[n >> 1], MF_SEL(2 * (n & 1) + b));
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
-              if (n + 2 < 8) {
+              for (int n = 0; n < 8; ++n) {
+                if (n + 2 < 8) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) w[(n + 2) % 3][b] = mf_lut2(lane4k, kw[n + 2], MF_SEL(b));
+                  for (int b = 0; b < 2; ++b) w[(n + 2) % 3][b] = mf_lut4(lane4k, kw[(n + 2) >> 1], MF_SEL(2 * (n & 1) + b));
+                }
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+                  acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                      mf_pack(w[n % 3][b].x, w[n % 3][b].y, w[n % 3][b].z, w[n % 3][b].w), qb[2 * (n & 3) + b], acc[n >> 2], 0, 0, 0);
               }
-              acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(w[n % 3][0].x, w[n % 3][0].y, w[n % 3][1].x, w[n % 3][1].y), qb[2 * (n & 3)], acc[n >> 2], 0, 0, 0);
-              acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  mf_pack(w[n % 3][2].x, w[n % 3][2].y, w[n % 3][3].x, w[n % 3][3].y), qb[2 * (n & 3) + 1], acc[n >> 2], 0, 0, 0);
+            } else {
+              uint32_t kw[8];       // 4-bit: the code dwords; 3-bit: the 24-bit words
+#pragma unroll
+              for (int j = 0; j < 2; ++j) {
+                if constexpr (BITS == 4) {
+                  kw[4 * j + 0] = r.k[j].x; kw[4 * j + 1] = r.k[j].y; kw[4 * j + 2] = r.k[j].z; kw[4 * j + 3] = r.k[j].w;
+                } else {
+                  // group q = bytes 3q .. 3q+2 of the lane's twelve
+                  kw[4 * j + 0] = __builtin_amdgcn_perm(r.k[j].x, r.k[j].x, 0x0c000102u);
+                  kw[4 * j + 1] = __builtin_amdgcn_perm(r.k[j].y, r.k[j].x, 0x0c030405u);
+                  kw[4 * j + 2] = __builtin_amdgcn_perm(r.k[j].z, r.k[j].y, 0x0c020304u);
+                  kw[4 * j + 3] = __builtin_amdgcn_perm(r.k[j].z, r.k[j].z, 0x0c010203u);
+                }
+              }
+              mf_u32x2 w[3][4];      // ring of three steps: two in flight behind the one multiplied
+#pragma unroll
+              for (int n = 0; n < 2; ++n)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) w[n][b] = mf_klook<BITS>(lane4k, kw[n], b);
+#pragma unroll
+              for (int n = 0; n < 8; ++n) {
+                if (n + 2 < 8) {
+#pragma unroll
+                  for (int b = 0; b < 4; ++b) w[(n + 2) % 3][b] = mf_klook<BITS>(lane4k, kw[n + 2], b);
+                }
+                acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    mf_pack(w[n % 3][0].x, w[n % 3][0].y, w[n % 3][1].x, w[n % 3][1].y), qb[2 * (n & 3)], acc[n >> 2], 0, 0, 0);
+                acc[n >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    mf_pack(w[n % 3][2].x, w[n % 3][2].y, w[n % 3][3].x, w[n % 3][3].y), qb[2 * (n & 3) + 1], acc[n >> 2], 0, 0, 0);
+              }
             }
             __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
             load_chunk(r, c + 2);
@@ -500,7 +579,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               union { mf_u32x4 u; float f[4]; } kn;
-              kn.u = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 64u * j);
+              kn.u = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + 64u * j);
 #pragma unroll
               for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
             }
@@ -524,8 +603,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           m_run = m_new;
           float psum = 0.f;
           union { mf_u32x4 u[2]; float f[8]; } vn;
-          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u);
-          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + MF_XBUF * par) + 256u + 64u);
+          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS);
+          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS + 64u);
           float pw[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
@@ -536,23 +615,25 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           // weights as float16 hi + lo, two at a time: hi = pw truncated to float16, lo = pw - hi (exact
           // in float32, then truncated); columns [0,8) keep hi, columns [8,16) take the lo pair of the
           // column eight to their left (one row shift per packed pair)
+          // (2-bit: the value side's operand takes the tokens as 4g, 4g+1 of both tiles, then 4g+2, 4g+3 of both)
           union { mf_u32x4 u; uint32_t w[4]; } cv;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
+          for (int qq = 0; qq < 4; ++qq) {
+            const int q = BITS == 2 ? ((qq & 1) << 1 | (qq >> 1)) : qq;      // the pair of tokens operand dword qq holds
             auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q], pw[2 * q + 1]);
             auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q] - (float)h2[0], pw[2 * q + 1] - (float)h2[1]);
             union { decltype(h2) h; uint32_t u; } hb, lb;
             hb.h = h2;
             lb.h = l2;
             const uint32_t lo_left = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)lb.u, 0x118 /*row_shr:8*/, 0xf, 0xf, true);
-            cv.w[q] = col < 8 ? hb.u : lo_left;
+            cv.w[qq] = col < 8 ? hb.u : lo_left;
           }
           l_run = l_run * resc + psum;
           const float resc_left = mf_from_lo_cols(resc);
           const float resc_out = col < 8 ? resc : resc_left;
           // the buffer was last read for chunk c - 2, two barriers ago
-          *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par) = cv.u;
-          *(mf_lds_u32*)(uintptr_t)(rs_addr + MF_XBUF * par) = __float_as_uint(resc_out);
+          *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par) = cv.u;
+          *(mf_lds_u32*)(uintptr_t)(rs_addr + XPAR * par) = __float_as_uint(resc_out);
         };
 
         mf_kraw ra, rb;
@@ -602,11 +683,20 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             const unsigned char* vb = a.vp + mf_umul(pb[j], (uint32_t)a.vps_blk) + (j ? vtile1 : 0u);
+            if constexpr (BITS == 2) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {    // the token step rides in the uniform base
-              const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff);
-              if constexpr (BITS == 2) r.v[4 * j + i] = *(const uint16_t*)vr;
-              else r.v[4 * j + i] = *(const uint32_t*)vr;
+              for (int i = 0; i < 2; ++i) {
+                union { mf_u16x2 h; uint32_t u; } t;
+                t.h.x = *(const uint16_t*)(vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff));
+                t.h.y = *(const uint16_t*)(vb + (uint32_t)((i + 2) * (int)a.vps_pos) + mf_here(voff));
+                r.v[2 * j + i] = t.u;
+              }
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {    // the token step rides in the uniform base
+                const unsigned char* vr = vb + (uint32_t)(i * (int)a.vps_pos) + mf_here(voff);
+                r.v[4 * j + i] = *(const uint32_t*)vr;
+              }
             }
           }
         };
@@ -615,42 +705,69 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         // coordinates, the raw registers take the chunk after next (see the score side), and all 32
         // table lookups of the chunk are issued.  After the barrier only the weights are read and
         // the eight MFMAs run back to back.
-        uint32_t wv[4][4];    // step n -> byte n/2 of the dword, even (xe) or odd (xo) coordinate; M-tile n
+        // 4-bit and 3-bit: step n -> lookup n/2 of the regrouped word, even (xe) or odd (xo) position; M-tile n;
+        // four lookups (pairs of tokens) make an operand.  2-bit: a lookup is one coordinate of FOUR tokens, two
+        // make an operand; word n/2 of xe, bytes n%2 (tokens 4g, 4g+1 of both tiles) and n%2 + 2 (4g+2, 4g+3).
+        uint32_t wv[4][4];
         uint32_t xe[4], xo[4];
-        auto regroup = [&](mf_vraw& r, int c) {
+        auto vlook = [&](uint32_t (&dst)[4], int n) {
+          if constexpr (BITS == 2) {
 #pragma unroll
-          for (int p = 0; p < 4; ++p) {
-            uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
-            if constexpr (BITS == 3) {
-              const uint32_t na = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wa, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
-              const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wb, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
-              wa = mf_spread3(__builtin_amdgcn_perm(na, wa, sel3));
-              wb = mf_spread3(__builtin_amdgcn_perm(nb, wb, sel3));
-            } else if constexpr (BITS == 2) {
-              wa = mf_spread2(wa);
-              wb = mf_spread2(wb);
+            for (int p = 0; p < 2; ++p) {
+              const mf_u32x2 t = mf_lut2(lane4v, xe[n >> 1], MF_SEL((n & 1) + 2 * p));
+              dst[2 * p] = t.x;
+              dst[2 * p + 1] = t.y;
             }
-            xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
-            xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
+          } else {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) dst[p] = mf_vlook<BITS>(lane4v, (n & 1) ? xo[p] : xe[p], n >> 1);
+          }
+        };
+        auto regroup = [&](mf_vraw& r, int c) {
+          if constexpr (BITS == 2) {
+            // halves (a | c << 16) and (b | d << 16) of each tile: e = nibbles (a, b) of the codes at bit
+            // positions 0 mod 4, o = those at 2 mod 4; then the nibbles of the two tiles side by side
+            const uint32_t e0 = (r.v[0] & 0x33333333u) | ((r.v[1] << 2) & 0xccccccccu);
+            const uint32_t o0 = ((r.v[0] >> 2) & 0x33333333u) | (r.v[1] & 0xccccccccu);
+            const uint32_t e1 = (r.v[2] & 0x33333333u) | ((r.v[3] << 2) & 0xccccccccu);
+            const uint32_t o1 = ((r.v[2] >> 2) & 0x33333333u) | (r.v[3] & 0xccccccccu);
+            xe[0] = (e0 & 0x0f0f0f0fu) | ((e1 << 4) & 0xf0f0f0f0u);      // codes 3 and 7 of the lane's eight
+            xe[1] = ((e0 >> 4) & 0x0f0f0f0fu) | (e1 & 0xf0f0f0f0u);      // codes 1 and 5
+            xe[2] = (o0 & 0x0f0f0f0fu) | ((o1 << 4) & 0xf0f0f0f0u);      // codes 2 and 6
+            xe[3] = ((o0 >> 4) & 0x0f0f0f0fu) | (o1 & 0xf0f0f0f0u);      // codes 0 and 4
+          } else {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+              uint32_t wa = r.v[2 * p], wb = r.v[2 * p + 1];
+              if constexpr (BITS == 3) {
+                // the lane's three bytes as a big-endian 24-bit word (code 0 in bits 23:21), then the codes at
+                // odd positions (bits 0 mod 6) and at even positions (bits 3 mod 6) of the two tokens side by side
+                const uint32_t na = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wa, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
+                const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)wb, 0x101 /*row_shl:1*/, 0xf, 0xf, true);
+                wa = __builtin_amdgcn_perm(na, wa, sel3);
+                wb = __builtin_amdgcn_perm(nb, wb, sel3);
+                xe[p] = (wa & 0x001c71c7u) | ((wb << 3) & 0x00e38e38u);
+                xo[p] = ((wa >> 3) & 0x001c71c7u) | (wb & 0x00e38e38u);
+              } else {
+                xe[p] = (wa & 0xF0F0F0F0u) | ((wb >> 4) & 0x0F0F0F0Fu);
+                xo[p] = ((wa << 4) & 0xF0F0F0F0u) | (wb & 0x0F0F0F0Fu);
+              }
+            }
           }
           __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
           load_chunk(r, c + 1);                // a whole chunk period ahead of its use
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int n = 0; n < 4; ++n)
-#pragma unroll
-            for (int p = 0; p < 4; ++p) wv[n][p] = mf_lut(lane4v, (n & 1) ? xo[p] : xe[p], MF_SEL(n >> 1));
+          for (int n = 0; n < 4; ++n) vlook(wv[n], n);
         };
         auto consume = [&](int c, const uint32_t par) {
           // second half of the lookups: in flight while the weights arrive and the first four MFMAs run
           uint32_t wl[4][4];
 #pragma unroll
-          for (int n = 4; n < 8; ++n)
-#pragma unroll
-            for (int p = 0; p < 4; ++p) wl[n - 4][p] = mf_lut(lane4v, (n & 1) ? xo[p] : xe[p], MF_SEL(n >> 1));
+          for (int n = 4; n < 8; ++n) vlook(wl[n - 4], n);
           union { half8 h; mf_u32x4 u; } cv;
-          cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + MF_XBUF * par);
-          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + MF_XBUF * par));
+          cv.u = *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par);
+          const float resc = __uint_as_float(*(mf_lds_cu32*)(uintptr_t)(rs_addr + XPAR * par));
           if (__builtin_amdgcn_ballot_w64(resc != 1.f) != 0) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
@@ -689,10 +806,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           float* dst = a.part_acc + slot * 128 + 32 * g;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            *(float4*)(dst + 8 * i) = make_float4(o[mf_vtile_of_coord<BITS>(0)][i], o[mf_vtile_of_coord<BITS>(1)][i],
-                                                  o[mf_vtile_of_coord<BITS>(2)][i], o[mf_vtile_of_coord<BITS>(3)][i]);
-            *(float4*)(dst + 8 * i + 4) = make_float4(o[mf_vtile_of_coord<BITS>(4)][i], o[mf_vtile_of_coord<BITS>(5)][i],
-                                                      o[mf_vtile_of_coord<BITS>(6)][i], o[mf_vtile_of_coord<BITS>(7)][i]);
+            *(float4*)(dst + 8 * i) = make_float4(o[mf_vtile<BITS>(0)][i], o[mf_vtile<BITS>(1)][i],
+                                                  o[mf_vtile<BITS>(2)][i], o[mf_vtile<BITS>(3)][i]);
+            *(float4*)(dst + 8 * i + 4) = make_float4(o[mf_vtile<BITS>(4)][i], o[mf_vtile<BITS>(5)][i],
+                                                      o[mf_vtile<BITS>(6)][i], o[mf_vtile<BITS>(7)][i]);
           }
         }
       }
@@ -706,17 +823,40 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
   // ---- tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) reads the entry's three words once
   // and writes 8 of its 32 copies with 16-byte stores
+  // The words of the workspace block are pairs indexed by two nibbles (first code << 4 | second code).
   {
     const int e = threadIdx.x >> 2, qt = threadIdx.x & 3;
-    const uint32_t khi = x.lut[MF_W_KHI + e], klo = x.lut[MF_W_KLO + e], vhi = x.lut[MF_W_VHI + e];
-    uint4* ka = (uint4*)(lds_raw + e * 256 + qt * 64);                  // K copies 8qt .. 8qt+7 (8 bytes each)
-    uint4* va = (uint4*)(lds_raw + MF_TABB + e * 256 + qt * 32);        // V copies 8qt .. 8qt+7 (4 bytes each)
+    uint4* ka = (uint4*)(lds_raw + e * 256 + qt * 64);
+    uint4* va = (uint4*)(lds_raw + MF_TABB + e * 256 + qt * (BITS == 2 ? 64 : 32));
+    if constexpr (BITS == 2) {
+      // entry = one code byte.  K: four coordinates (codes from the top bits down) as (hi pair, lo pair) twice,
+      // 16 copies of 16 bytes.  V: the same coordinate of four tokens (codes from the bottom bits up), 32
+      // copies of 8 bytes.
+      const int k01 = ((e >> 6) << 4) | ((e >> 4) & 3), k23 = (((e >> 2) & 3) << 4) | (e & 3);
+      const uint4 kq = make_uint4(x.lut[MF_W_KHI + k01], x.lut[MF_W_KLO + k01], x.lut[MF_W_KHI + k23], x.lut[MF_W_KLO + k23]);
+      const int v01 = ((e & 3) << 4) | ((e >> 2) & 3), v23 = (((e >> 4) & 3) << 4) | (e >> 6);
+      const uint32_t va01 = x.lut[MF_W_VHI + v01], va23 = x.lut[MF_W_VHI + v23];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ka[i] = make_uint4(khi, klo, khi, klo);
+      for (int i = 0; i < 4; ++i) ka[i] = kq;                            // K copies 4qt .. 4qt+3
 #pragma unroll
-    for (int i = 0; i < 2; ++i) va[i] = make_uint4(vhi, vhi, vhi, vhi);
+      for (int i = 0; i < 4; ++i) va[i] = make_uint4(va01, va23, va01, va23);   // V copies 8qt .. 8qt+7
+    } else {
+      // 4-bit: entry = one code byte (two codes).  3-bit: entry = a 6-bit field, K (first code << 3 | second
+      // code) of one token, V (code of the odd token << 3 | code of the even token) of one coordinate; 64 entries.
+      int ke = e, ve = e;
+      if constexpr (BITS == 3) {
+        ke = (((e >> 3) & 7) << 4) | (e & 7);
+        ve = ((e & 7) << 4) | ((e >> 3) & 7);
+      }
+      const uint32_t khi = x.lut[MF_W_KHI + ke], klo = x.lut[MF_W_KLO + ke], vhi = x.lut[MF_W_VHI + ve];
+      if (BITS == 4 || e < 64) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ka[i] = make_uint4(khi, klo, khi, klo);    // K copies 8qt .. 8qt+7 (8 bytes each)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) va[i] = make_uint4(vhi, vhi, vhi, vhi);    // V copies 8qt .. 8qt+7 (4 bytes each)
+      }
+    }
   }
-  if (threadIdx.x < 8) *(uint2*)(lds_raw + MF_TABB + (32u * threadIdx.x + 12u) * 256u + 128u) = make_uint2(0u, 0u);
   __syncthreads();
   if ((wave >> 3) == 0) mf_role_main<0, BITS>(a, x, wave & 7);
   else mf_role_main<1, BITS>(a, x, wave & 7);
@@ -797,12 +937,12 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   if (!configured) {
     AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
     AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
+    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES_2BIT));
     configured = true;
   }
   if (bits == 4) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<4>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
   else if (bits == 3) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<3>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
-  else AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<2>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
+  else AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<2>, grid, MF_THREADS, MF_LDS_BYTES_2BIT, stream, a, x);
   AKV_LAUNCH_CHECK("akv_attn_mfma_kernel");
   return AKV_OK;
 }
