@@ -364,7 +364,7 @@ __device__ __forceinline__ void mf_barrier() {
 
 struct mf_kraw {       // score wavefront, one 32-token chunk
   uint4 k[2];          // K code rows: tile j, token l%16, the lane's quarter of the row (16 / 12 / 8 bytes)
-  float nrm;           // lane < 32: K norm of token l, else V norm of token l - 32
+  float nrm;           // one of the chunk's norms (any head of the pass; see the score role)
 };
 typedef uint32_t mf_u32x3 __attribute__((ext_vector_type(3)));
 typedef uint16_t mf_u16x2 __attribute__((ext_vector_type(2)));
@@ -480,22 +480,35 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         }
         float m_run = -INFINITY, l_run = 0.f;
         const uint32_t koff = (uint32_t)(hd * a.kps_head + col * a.kps_pos + (BITS == 4 ? 16 : BITS == 3 ? 12 : 8) * g);
-        // norms travel one per lane (lanes [0,32): K norm of token l, lanes [32,64): V norm of token
-        // l - 32), prefetched with the codes, and are spread to the accumulator layout through the
-        // spare halves of table B entries 16q + 10 (K) and 16q + 11 (V)
-        const int ntok = lane & 31;
-        const bool nrm_is_v = lane >= 32;
+        // Norms: the 32 K norms and 32 V norms a head needs per chunk lie 4 bytes apiece, one head stride apart.
+        // Read per head they would be 64 addresses in sixteen or more 128-byte lines per load instruction; the
+        // score wavefronts of the pass share the work instead: with n active head slots the 64 n norms of a
+        // chunk are numbered [kind][token][head] and wavefront hs takes numbers 64 hs .. 64 hs + 63 (n = 8 and
+        // dense norms: eight tokens x eight heads, two lines).  They are prefetched with the codes, written
+        // into every head's exchange unit at the END of the step before the one that uses them (entries
+        // 16q + 10 (K) and 16q + 11 (V) of the unit, 32 floats each) and read back after the barrier in the
+        // accumulator layout.
+        const int nact = min(MF_HEADS, a.KVH - hbase);
+        const int nidx = 64 * hs + lane;
+        const int nhead = nidx % nact, nrest = nidx / nact;
+        const int ntok = nrest & 31;
+        const bool nrm_is_v = nrest >= 32;
+        const int nh = hbase + nhead;
+        const int nhd = a.hgroup > 1 ? nh / a.hgroup : nh;
         const float* nrm_base = nrm_is_v ? a.vn : a.kn;
         const uint32_t nrm_blk = (uint32_t)(nrm_is_v ? a.vns_blk : a.kns_blk);
         const int npos = bs32 ? ntok : (ntok & 15);        // position of token ntok inside its block
-        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? hd * a.vns_head + npos * a.vns_pos
-                                                     : hd * a.kns_head + npos * a.kns_pos);
+        const uint32_t nrm_off = (uint32_t)(nrm_is_v ? nhd * a.vns_head + npos * a.vns_pos
+                                                     : nhd * a.kns_head + npos * a.kns_pos);
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
-        const uint32_t nw_addr = XB0 + (32u * hs + 10u + (uint32_t)(lane >> 5)) * XS + (uint32_t)ntok * 4u;
+        const uint32_t nw_addr = XB0 + (32u * (uint32_t)nhead + 10u + (nrm_is_v ? 1u : 0u)) * XS + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = XB0 + (32u * hs + 10u) * XS + (uint32_t)g * 16u;
         auto load_chunk = [&](mf_kraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
+          // the norm first: it is wanted one step before the rows, and loads complete in the order of issue
+          r.nrm = nrm_base[mf_umul(ntok >= 16 ? pb[1] : pb[0], nrm_blk) + nrm_off];
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             const unsigned char* kr = a.kp + mf_umul(pb[j], (uint32_t)a.kps_blk) + (j ? ktile1 : 0u) + mf_here(koff);
@@ -509,11 +522,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
               r.k[j].x = t.x; r.k[j].y = t.y;
             }
           }
-          r.nrm = nrm_base[mf_umul(ntok >= 16 ? pb[1] : pb[0], nrm_blk) + nrm_off];
         };
-        auto produce = [&](mf_kraw& r, int c, const uint32_t par) {
+        // (`rn` holds the next chunk: its norms go out at the end of this step, behind the barrier that ends it)
+        auto produce = [&](mf_kraw& r, const mf_kraw& rn, int c, const uint32_t par) {
           float sv[8];
-          *(mf_lds_u32*)(uintptr_t)(nw_addr + XPAR * par) = __float_as_uint(r.nrm);
           {
             // 8 steps of two MFMAs; the table reads of step n+2 are issued before the MFMAs of step n.
             //   4-bit: step = (tile j, dword st), 4 reads (one per code byte: hi and lo of two coordinates)
@@ -634,6 +646,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           // the buffer was last read for chunk c - 2, two barriers ago
           *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + XPAR * par) = __float_as_uint(resc_out);
+          // the other parity's norm entries were last read in the step before this one
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + XPAR * (par ^ 1u)) = __float_as_uint(rn.nrm);
         };
 
         mf_kraw ra, rb;
@@ -642,19 +656,20 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_sched_barrier(0);     // queue order = chunk order, as in the loop
         load_chunk(rb, 1);
         __builtin_amdgcn_sched_barrier(0);
+        *(mf_lds_u32*)(uintptr_t)nw_addr = __float_as_uint(ra.nrm);     // norms of chunk 0, ahead of the first barrier
         // pairs of chunks with the same loads on every path (an early exit from the middle of the
         // body would make the compiler wait for the newest prefetch at the top of every iteration)
         int c = 0;
         for (; c + 1 < nchunks; c += 2) {
           if (c - win_c0 >= MF_WIN) load_window(c);
           if constexpr (SYNC) mf_barrier();
-          produce(ra, c, 0);
+          produce(ra, rb, c, 0);
           if constexpr (SYNC) mf_barrier();
-          produce(rb, c + 1, 1);
+          produce(rb, ra, c + 1, 1);
         }
         if (c < nchunks) {
           if constexpr (SYNC) mf_barrier();
-          produce(ra, c, 0);      // odd tail, already in ra
+          produce(ra, rb, c, 0);      // odd tail, already in ra
         }
         if constexpr (SYNC) mf_barrier();
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
