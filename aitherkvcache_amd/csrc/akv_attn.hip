@@ -36,38 +36,49 @@ __global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
 }
 
 // ----------------------------------------------------------------------------------
-// reduce: one workgroup per (sequence, group of 4 query heads).  Wavefront w merges the
-// partials of head 4*group + w; then all 256 threads apply the inverse rotation, one load of
-// Pi[k][j] serving two heads.
+// reduce: a workgroup takes (sequence, group of 4 query heads) items, blockIdx.x, + gridDim.x, ...
+// Wavefront w merges the partials of head 4*group + w; then all 256 threads apply the inverse
+// rotation, one load of Pi[k][j] serving two heads.  At head_dim 128 a thread keeps its column of
+// Pi in registers across its items: with one workgroup per item a batch of 256 sequences x 32 heads
+// read the 64 KB matrix 4096 times (43 us for the kernel; 2048 items on 512 workgroups: see the host side).
 // ----------------------------------------------------------------------------------
 template <int D, int ODT>
-__global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
+__global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
     const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
-    const float* __restrict__ part_ml, const float* __restrict__ Pi, int S, int QH, int G,
+    const float* __restrict__ part_ml, const float* __restrict__ Pi, const uint4* __restrict__ bop, int S, int QH, int G,
     void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status) {
   constexpr int DPL = D / 64;
-  __shared__ float a_lds[4][D];
+  __shared__ __align__(16) float a_lds[4][D];
   const int groups = (QH + 3) / 4;
-  const int s = blockIdx.x / groups, hg = blockIdx.x % groups;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int h = hg * 4 + wave;
-  // head_dim 128: this thread's column of Pi is requested before anything else, its round trip overlaps
-  // those of the partials (one wavefront per SIMD: the registers are there)
-  constexpr int PIPF = D == 128 ? 128 : 1;
-  float pvr[PIPF];
+  // head_dim 128: the inverse rotation runs on the matrix cores.  Wavefront w owns N-tiles 2w and 2w + 1 of the
+  // matrix operand (output coordinates 8 col + N-tile: lane col ends up with the neighbouring coordinates
+  // 8 col + 2w and + 1); its 16 operand registers per term are requested before anything else and stay for
+  // all items of the workgroup.  (On the vector unit, with a column of the matrix per thread, the rotation was
+  // 22 of the kernel's 39 us for 256 sequences x 32 heads.)
+  akv_half8 bh[2][4], bl[2][4];
   if constexpr (D == 128) {
 #pragma unroll
-    for (int k = 0; k < PIPF; ++k) pvr[k] = Pi[(size_t)k * D + (threadIdx.x & 127)];
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int idx = ((2 * wave + t) * 4 + ks) * 64 + lane;
+        bh[t][ks] = akv_as_half8(bop[idx]);
+        bl[t][ks] = akv_as_half8(bop[2048 + idx]);
+      }
   }
-  const int b0 = prefix[s], b1 = prefix[s + 1];
   // a main kernel whose bounded wait gave up has produced garbage: say so in every output
   const float poison = status[0] != 0u ? __uint_as_float(0x7fc00000u) : 0.f;
-  if (b1 <= b0) {
+  for (int item = blockIdx.x; item < S * groups; item += gridDim.x) {
+  const int s = item / groups, hg = item % groups;
+  const int h = hg * 4 + wave;
+  const int b0 = prefix[s], b1 = prefix[s + 1];
+  if (b1 <= b0) {        // (the same for the whole workgroup)
     if (h < QH) {
 #pragma unroll
       for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, s * os_seq + h * os_head + lane * DPL + i, poison);
     }
-    return;
+    continue;
   }
   if (h < QH) {
     const int total = prefix[S];
@@ -75,13 +86,19 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
     // the first RED_PF partial accumulators are requested before anything is known about their
     // weights, so that their round trip overlaps the one of the (max, sum) pairs
+    // (only slots that exist are read: a batch of many short sequences has one or two per head)
     constexpr int RED_PF = D == 128 ? 32 : 16;
     float pre[RED_PF][DPL];
 #pragma unroll
     for (int u = 0; u < RED_PF; ++u) {
-      const size_t slot = (size_t)(min(w_lo + u, w_hi) + s) * QH + h;
+      if (w_lo + u <= w_hi) {
+        const size_t slot = (size_t)(w_lo + u + s) * QH + h;
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) pre[u][i] = part_acc[slot * D + lane * DPL + i];
+        for (int i = 0; i < DPL; ++i) pre[u][i] = part_acc[slot * D + lane * DPL + i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) pre[u][i] = 0.f;
+      }
     }
     // lanes over slots: global max and sum; with at most 64 slots (the usual case) lane u keeps the
     // weight of slot w_lo + u and the second pass takes it from there
@@ -143,6 +160,45 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     for (int i = 0; i < DPL; ++i) a_lds[wave][lane * DPL + i] = 0.f;
   }
   __syncthreads();
+  if constexpr (D == 128) {
+    // A operand: row r = head r % 4 of the item (rows 4..15 repeat them and are not used), contracted coordinates
+    // 32 kg + 8 ks + e of the merged vector; result: lane (col, 0) holds heads 0..3 for output coordinates
+    // 8 col + 2 wave and + 1
+    const int r = lane & 15, kg = lane >> 4;
+    float v[4][8];
+    float m = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const float4 x0 = *(const float4*)&a_lds[r & 3][32 * kg + 8 * ks];
+      const float4 x1 = *(const float4*)&a_lds[r & 3][32 * kg + 8 * ks + 4];
+      v[ks][0] = x0.x; v[ks][1] = x0.y; v[ks][2] = x0.z; v[ks][3] = x0.w;
+      v[ks][4] = x1.x; v[ks][5] = x1.y; v[ks][6] = x1.z; v[ks][7] = x1.w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(v[ks][e]));
+    }
+    const uint32_t ex = akv_row_exponent(akv_rows_max(m));
+    const float sc = akv_row_scale(ex);
+    akv_float4v acc[2];
+    acc[0] = (akv_float4v){0.f, 0.f, 0.f, 0.f};
+    acc[1] = (akv_float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      akv_half8 hi, lo;
+      akv_split8(v[ks], sc, hi, lo);
+      acc[0] = akv_mfma3(hi, lo, bh[0][ks], bl[0][ks], acc[0]);
+      acc[1] = akv_mfma3(hi, lo, bh[1][ks], bl[1][ks], acc[1]);
+    }
+    const float usc = akv_row_unscale(ex) * (1.f / 64.f);     // lane i < 4: the factor of head i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float ui = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(usc), i));
+      const int hq = hg * 4 + i;
+      if (kg == 0 && hq < QH) {
+        akv_elem<ODT>::store(out, s * os_seq + hq * os_head + 8 * r + 2 * wave, acc[0][i] * ui + poison);
+        akv_elem<ODT>::store(out, s * os_seq + hq * os_head + 8 * r + 2 * wave + 1, acc[1][i] * ui + poison);
+      }
+    }
+  } else {
   // inverse rotation: thread t owns coordinates (t % 128) * JP .. of heads 2 * (t / 128) and + 1
   constexpr int JT = 128;                 // threads along the coordinate axis
   constexpr int JP = D / JT > 0 ? D / JT : 1;   // coordinates per thread (D=256 -> 2)
@@ -153,15 +209,8 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
     for (int q = 0; q < 2; ++q)
 #pragma unroll
       for (int i = 0; i < JP; ++i) o[q][i] = 0.f;
-    if constexpr (D == 128) {
-#pragma unroll
-      for (int k = 0; k < PIPF; ++k) {
-        o[0][0] = fmaf(a_lds[2 * pr][k], pvr[k], o[0][0]);
-        o[1][0] = fmaf(a_lds[2 * pr + 1][k], pvr[k], o[1][0]);
-      }
-    }
 #pragma unroll 64
-    for (int k = (D == 128 ? PIPF : 0); k < D; ++k) {
+    for (int k = 0; k < D; ++k) {
       const float a0v = a_lds[2 * pr][k], a1v = a_lds[2 * pr + 1][k];
 #pragma unroll
       for (int i = 0; i < JP; ++i) {
@@ -179,6 +228,9 @@ __global__ __launch_bounds__(256) void akv_attn_reduce_kernel(
           akv_elem<ODT>::store(out, s * os_seq + hq * os_head + jt * JP + i, o[q][i] + poison);
       }
     }
+  }
+  }
+  __syncthreads();       // the merged vectors are read until here; the next item overwrites them
   }
 }
 
@@ -389,13 +441,16 @@ static int akv_launch_attn_general(const akv_attn_args& a, int grid, hipStream_t
 }
 
 template <int D>
-static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, int G, void* out,
+static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, const uint4* bop, int G, void* out,
                              int64_t os_seq, int64_t os_head, const uint32_t* status, hipStream_t stream) {
-  const int grid = a.S * ((a.QH + 3) / 4);
+  // at most three workgroups per CU (what its registers admit at once); a workgroup loops over its items
+  const int items = a.S * ((a.QH + 3) / 4);
+  const int cus = akv_cached_cu_count();
+  const int grid = items < 3 * (cus > 0 ? cus : 256) ? items : 3 * (cus > 0 ? cus : 256);
   switch (odt) {
-    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
-    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
-    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
   }
   AKV_LAUNCH_CHECK("akv_attn_reduce_kernel");
   return AKV_OK;
@@ -478,9 +533,9 @@ static int akv_paged_attn_impl(
 #undef AKV_CASE
   }
   if (rc) return rc;
-  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
-  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
-  return akv_launch_reduce<256>(out_dtype, a, Pi, Gused, out, os_seq, os_head, ws.status, stream);
+  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, stream);
+  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(128)), Gused, out, os_seq, os_head, ws.status, stream);
+  return akv_launch_reduce<256>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, stream);
 }
 
 extern "C" int akv_paged_attn(

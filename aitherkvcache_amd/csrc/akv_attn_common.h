@@ -186,3 +186,52 @@ __device__ __forceinline__ void akv_lse_merge(float& m, float& l, float ms, floa
   l = alpha * l + beta * ls;
   m = mn;
 }
+
+// ----------------------------------------------------------------------------------
+// 128 x 128 rotations of a few float32 rows on the matrix cores (query rotation of the prologue,
+// inverse rotation of the reduce).  The matrix comes as the float16 hi + lo operand tables of the
+// prepared-rotation buffer (entries x 64; [hi | lo][8 N-tiles][4 k-steps][64 lanes] x 16 bytes, lane
+// (col, g) = output coordinate 8 col + N-tile, contracted coordinates 32 g + 8 k-step + e).  A row is
+// scaled by a power of two that brings its largest element to [1, 2) (exact), split into two float16
+// terms rounded to nearest, and a tile is three products: hi.hi + hi.lo + lo.hi (~22 bits).
+// ----------------------------------------------------------------------------------
+typedef _Float16 akv_half8 __attribute__((ext_vector_type(8)));
+typedef float akv_float4v __attribute__((ext_vector_type(4)));
+
+// max over the four 16-lane rows of a wavefront, for every column (lane % 16)
+__device__ __forceinline__ float akv_rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+// biased exponent used to scale a row whose largest magnitude is m (clamped so that both factors are normal)
+__device__ __forceinline__ uint32_t akv_row_exponent(float m) {
+  const uint32_t e = (__float_as_uint(m) >> 23) & 0xffu;
+  return e < 1u ? 1u : (e > 253u ? 253u : e);
+}
+__device__ __forceinline__ float akv_row_scale(uint32_t e) { return __uint_as_float((254u - e) << 23); }     // 2^(127 - e)
+__device__ __forceinline__ float akv_row_unscale(uint32_t e) { return __uint_as_float(e << 23); }             // 2^(e - 127)
+// eight scaled values as two float16 operands
+__device__ __forceinline__ void akv_split8(const float (&v)[8], float sc, akv_half8& hi, akv_half8& lo) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float x = v[e] * sc;
+    const _Float16 h = (_Float16)x;
+    hi[e] = h;
+    lo[e] = (_Float16)(x - (float)h);
+  }
+}
+__device__ __forceinline__ akv_half8 akv_as_half8(uint4 u) {
+  union { uint4 u; akv_half8 h; } cv;
+  cv.u = u;
+  return cv.h;
+}
+// acc += (hi + lo) . (bh + bl) without the lo.lo term
+__device__ __forceinline__ akv_float4v akv_mfma3(akv_half8 hi, akv_half8 lo, akv_half8 bh, akv_half8 bl, akv_float4v acc) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, bh, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, bl, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, bh, acc, 0, 0, 0);
+  return acc;
+}
+

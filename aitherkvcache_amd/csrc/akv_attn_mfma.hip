@@ -98,23 +98,25 @@ struct akv_mfma_extra {
 // ----------------------------------------------------------------------------------
 template <int QDT>
 __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
-    const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
+    const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const uint4* __restrict__ bop,
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
-    uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits) {
-  __shared__ __align__(16) float q_lds[128][8];   // [input coordinate][query head of the group], zero-padded
+    uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits, int nqb) {
+  __shared__ __align__(16) float q_lds[8][132];   // [query head of the group][input coordinate], zero-padded heads
   __shared__ float qr_lds[8][128];
   __shared__ int32_t scratch[257];
   __shared__ float best_err[256];
   __shared__ float best_alpha[256];
   const int tid = threadIdx.x;
+  // blocks [0, nqb): query rotation, (sequence, kv head) items blockIdx.x, + nqb, ...; block nqb: block prefix;
+  // block nqb + 1: tables
   const int nq = S * KVH;
-  if ((int)blockIdx.x == nq) {
+  if ((int)blockIdx.x == nqb) {
     if (tid == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
-  if ((int)blockIdx.x == nq + 1) {
+  if ((int)blockIdx.x == nqb + 1) {
     // The tables depend on the codebook only.  They are kept in the workspace together with
     // the centroids they were built from and a marker; when those match, nothing is rebuilt.
     __shared__ int stale;
@@ -163,43 +165,65 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     if (tid == 0) lut[MF_W_MARK] = MF_MARK + (uint32_t)bits;
     return;
   }
-  const int s = blockIdx.x / KVH, h = blockIdx.x % KVH;
   const int gqa = QH / KVH;
-  // thread (dim, half): partial dot products over 64 of the 128 input coordinates for every query
-  // head of the group.  Its 64 matrix entries are requested first, together with the queries, so that
-  // the two round trips to memory overlap instead of following each other across the barrier.
-  const int dim = tid & 127, half = tid >> 7;
-  float pvr[64];
+  // q' = Pi q on the matrix cores: A = the queries of the kv head (row r = query head r % 8), B = the float16
+  // hi + lo operand of the encode kernel (lane (col, g): output coordinate 8 col + N-tile, input coordinates
+  // 32 g + 8 ks + e).  Wavefront w owns N-tiles 2w and 2w + 1; their operand registers are requested first and
+  // stay for all items of the block.  (On the vector unit, with the queries broadcast from LDS, this kernel took
+  // 23 us for 256 sequences x 8 kv heads.)
+  const int lane = tid & 63, wave = tid >> 6;
+  akv_half8 bh[2][4], bl[2][4];
 #pragma unroll
-  for (int jj = 0; jj < 64; ++jj) pvr[jj] = PiT[(half * 64 + jj) * 128 + dim];
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int idx = ((2 * wave + t) * 4 + ks) * 64 + lane;
+      bh[t][ks] = akv_as_half8(bop[idx]);
+      bl[t][ks] = akv_as_half8(bop[2048 + idx]);
+    }
+  for (int item = blockIdx.x; item < nq; item += nqb) {
+  const int s = item / KVH, h = item % KVH;
   for (int i = tid; i < 8 * 128; i += 256) {
     const int q = i >> 7, j = i & 127;
-    q_lds[j][q] = q < gqa ? akv_elem<QDT>::load(query, s * qs_seq + (h * gqa + q) * qs_head + j) : 0.f;
+    q_lds[q][j] = q < gqa ? akv_elem<QDT>::load(query, s * qs_seq + (h * gqa + q) * qs_head + j) : 0.f;
   }
   __syncthreads();
   {
-    float part[8];
+    const int r = lane & 15, kg = lane >> 4;
+    float v[4][8];
+    float m = 0.f;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) part[q] = 0.f;
+    for (int ks = 0; ks < 4; ++ks) {
+      const float4 x0 = *(const float4*)&q_lds[r & 7][32 * kg + 8 * ks];
+      const float4 x1 = *(const float4*)&q_lds[r & 7][32 * kg + 8 * ks + 4];
+      v[ks][0] = x0.x; v[ks][1] = x0.y; v[ks][2] = x0.z; v[ks][3] = x0.w;
+      v[ks][4] = x1.x; v[ks][5] = x1.y; v[ks][6] = x1.z; v[ks][7] = x1.w;
 #pragma unroll
-    for (int jj = 0; jj < 64; ++jj) {
-      const int j = half * 64 + jj;
-      const float pv = pvr[jj];
-      const float4 qa = *(const float4*)&q_lds[j][0];
-      const float4 qc = *(const float4*)&q_lds[j][4];
-      part[0] = fmaf(pv, qa.x, part[0]); part[1] = fmaf(pv, qa.y, part[1]);
-      part[2] = fmaf(pv, qa.z, part[2]); part[3] = fmaf(pv, qa.w, part[3]);
-      part[4] = fmaf(pv, qc.x, part[4]); part[5] = fmaf(pv, qc.y, part[5]);
-      part[6] = fmaf(pv, qc.z, part[6]); part[7] = fmaf(pv, qc.w, part[7]);
+      for (int e = 0; e < 8; ++e) m = fmaxf(m, fabsf(v[ks][e]));
     }
-    if (half == 1) {
+    const uint32_t ex = akv_row_exponent(akv_rows_max(m));
+    const float sc = akv_row_scale(ex);
+    akv_float4v acc[2];
+    acc[0] = (akv_float4v){0.f, 0.f, 0.f, 0.f};
+    acc[1] = (akv_float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int q = 0; q < 8; ++q) qr_lds[q][dim] = part[q];
+    for (int ks = 0; ks < 4; ++ks) {
+      akv_half8 hi, lo;
+      akv_split8(v[ks], sc, hi, lo);
+      acc[0] = akv_mfma3(hi, lo, bh[0][ks], bl[0][ks], acc[0]);
+      acc[1] = akv_mfma3(hi, lo, bh[1][ks], bl[1][ks], acc[1]);
     }
-    __syncthreads();
-    if (half == 0) {
+    // lane (col, kg) holds query heads 4 kg + i (kg < 2) at output coordinates 8 col + 2 wave and + 1
+    const float usc = akv_row_unscale(ex) * (qscale / 64.f);     // lane q < 8: the factor of query head q
 #pragma unroll
-      for (int q = 0; q < 8; ++q) qr_lds[q][dim] = (qr_lds[q][dim] + part[q]) * qscale;
+    for (int i = 0; i < 4; ++i) {
+      const float u0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(usc), i));
+      const float u1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(usc), 4 + i));
+      if (kg < 2) {
+        const float ui = kg == 0 ? u0 : u1;
+        qr_lds[4 * kg + i][8 * r + 2 * wave] = acc[0][i] * ui;
+        qr_lds[4 * kg + i][8 * r + 2 * wave + 1] = acc[1][i] * ui;
+      }
     }
   }
   __syncthreads();
@@ -227,6 +251,8 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     o.x = hbits[0] | (hbits[1] << 16); o.y = hbits[2] | (hbits[3] << 16);
     o.z = hbits[4] | (hbits[5] << 16); o.w = hbits[6] | (hbits[7] << 16);
     qop[((size_t)(s * KVH + h) * 8 + n) * 64 + lane] = o;
+  }
+  __syncthreads();     // q_lds and qr_lds are rewritten by the next item
   }
 }
 
@@ -943,8 +969,12 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   x.status = ws.status;
   x.spin_limit = g_spin_limit;
   const float qscale = a.scale * 1.4426950408889634f;   // scores come out in the log2 domain
-  const int pgrid = a.S * a.KVH + 2;
-#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, PiT, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, x.status, qscale, bits)
+  // rotation blocks: one per (sequence, kv head) up to six per CU (what its registers admit at once), then they loop
+  const int cus = akv_cached_cu_count();
+  const int nqb = a.S * a.KVH < 6 * (cus > 0 ? cus : 256) ? a.S * a.KVH : 6 * (cus > 0 ? cus : 256);
+  const int pgrid = nqb + 2;
+  const uint4* bop = (const uint4*)(PiT + 128 * 128);    // the encode kernel's operand follows Pi and PiT in the prepared buffer
+#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, bop, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, x.status, qscale, bits, nqb)
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
