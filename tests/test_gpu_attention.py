@@ -87,11 +87,12 @@ def oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, bits, block_size=16, P=No
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
-@pytest.mark.parametrize("qh,kvh", [(32, 8), (8, 8), (6, 2), (16, 2), (32, 2), (24, 2), (9, 1), (40, 2)])
+@pytest.mark.parametrize("qh,kvh", [(32, 8), (8, 8), (6, 2), (16, 2), (32, 2), (24, 2), (9, 1), (40, 2), (16, 16), (24, 12), (48, 6)])
 def test_ragged_batch_vs_oracle(golden, dev, bits, qh, kvh):
     """Ragged contexts (0, 1, partial block, many blocks), permuted non-contiguous tables, GQA
     ratios 4 / 1 / 3 / 8, and 16 / 12 / 9 / 20 (a kv head presented as two or three groups of query
-    heads on the matrix-core kernel)."""
+    heads on the matrix-core kernel); 16 and 12 kv heads, and 6 kv heads as 12 groups, take two passes of
+    eight head slots on that kernel, the second with eight or four active slots."""
     tq = make_tq(golden, dev, bits)
     rng = np.random.default_rng(200 + bits + qh)
     NB = 96
