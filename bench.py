@@ -19,6 +19,8 @@ having been written by the encode-on-write kernel.  One JSON line is printed:
   encode     the encode-on-write kernel: Mvec/s on 2**20 vectors, the latency of one 256-token
              step (K and V, 8 heads), and `sweep`: kernel duration for 2**12 .. 2**22 vectors with the
              smallest size that reaches 60 % of the HBM peak (`vectors_at_60pct_hbm`)
+  hbm_reference  what torch's own sum (read) and copy (read + write) kernels stream on this box over
+             360 MB, the size of the headline step's cache: context for the fraction of the nominal peak
 
 Algorithmic bytes per context token = 8 heads x (64 B codes + 4 B norm) x (K and V) = 1088 B
 (104 / 72 / 128 B x 8 for 3-bit / 2-bit / tq35), plus queries, outputs and block tables.
@@ -125,6 +127,27 @@ def kernel_ms(torch, L, fn, steps):
         raise RuntimeError(L.akv_last_error().decode())
     assert n.value == steps, (n.value, steps)
     return ms.value
+
+
+def hbm_reference(torch, dev):
+    """What the image's own streaming kernels reach on this box for a buffer of the workload's size (360 MB, two
+    buffers alternated): torch's sum (read only) and a device-to-device copy (read + write), in TB/s."""
+    n = 90 * 1024 * 1024
+    xs = [torch.empty(n, dtype=torch.float32, device=dev).normal_() for _ in range(2)]
+    y = torch.empty_like(xs[0])
+    st = {"i": 0}
+
+    def rd():
+        st["i"] += 1
+        xs[st["i"] & 1].sum()
+
+    def cp():
+        st["i"] += 1
+        y.copy_(xs[st["i"] & 1])
+    precondition(torch, rd, PRECONDITION_S / 2)
+    t_rd = timed(torch, rd, 20, 5)
+    t_cp = timed(torch, cp, 20, 5)
+    return {"bytes": n * 4, "torch_sum_read_tbs": n * 4 / t_rd / 1e9, "device_copy_read_plus_write_tbs": 2 * n * 4 / t_cp / 1e9}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -484,6 +507,8 @@ def main():
                        "sample": "numpy oracle encode of 65,536 vectors (config 0)"}
     out["cpu_baseline"] = cpu_obj
     out["encode"] = enc
+    if not args.no_sweep:
+        out["hbm_reference"] = hbm_reference(torch, dev)
     print(json.dumps(out))
 
 
