@@ -120,6 +120,34 @@ def test_ragged_batch_vs_oracle(golden, dev, bits, qh, kvh):
     assert np.max(np.abs(out32.cpu().numpy() - ref)) <= 1e-3
 
 
+@pytest.mark.parametrize("bits", [4, 3])
+def test_batch_of_many_sequences_vs_oracle(golden, dev, bits):
+    """330 sequences of 0..90 tokens x 32 query heads: more (sequence, kv head) and (sequence, four heads) items
+    than the rotation blocks of the prologue and the workgroups of the reduce kernel, which then take several
+    items each; more than 63 sequences also take the scalar search for a segment's sequence."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(900 + bits)
+    NB, S, qh, kvh = 64, 330, 32, 8
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, kvh, bits)
+    ctx = rng.integers(0, 91, size=S).astype(np.int64)
+    ctx[:4] = [0, 1, 16, 90]
+    width = 8
+    tables = np.full((S, width), -3, dtype=np.int64)
+    for s_, c_ in enumerate(ctx):
+        nb = -(-int(c_) // 16)
+        tables[s_, :nb] = rng.permutation(NB)[:nb]
+    q = rng.standard_normal((S, qh, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, num_query_heads=qh)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), block_size=16, num_kv_heads=kvh)
+    ref = oracle_out(q, kp, kn, vp, vn, tables, ctx, golden, bits)
+    got = out.cpu().numpy().astype(np.float64)
+    print(f"[attn many sequences] bits={bits} max|diff|={np.max(np.abs(got - ref)):.2e}")
+    assert np.all(got[0] == 0)
+    assert within_tol(got, ref)
+    out32 = attn.forward(t(q.astype(np.float32), dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev), 16, kvh)
+    assert np.max(np.abs(out32.cpu().numpy() - ref)) <= 1e-3
+
+
 def test_serving_layout_strided_views(golden, dev):
     """K/V as views of one uint8 [blocks, 2, bs, heads, 68] tensor (row pitch 68 bytes) and norms
     as a slice of a [layers, blocks, bs, heads] tensor."""
