@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TurboQuant hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode4|decode3|decode2|tq35|tri|encode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode4|decode4_b256|decode3|decode2|tq35|tri|encode]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The default workload is the headline one: paged decode attention over a tq-t4nc cache
@@ -59,7 +59,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="decode4",
-                    choices=["decode4", "decode3", "decode2", "tq35", "tri", "encode"])
+                    choices=["decode4", "decode4_b256", "decode3", "decode2", "tq35", "tri", "encode"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the encode size sweep (a profiler run then sees the encode kernel at 2**20 vectors only)")
@@ -379,11 +379,16 @@ def main():
            "scaling": "weak", "vs_baseline": None, "data": "synthetic", "unit": "GB/s"}
     cpu_obj = None
 
-    if args.workload in ("decode4", "decode3", "decode2", "tq35"):
+    if args.workload in ("decode4", "decode4_b256", "decode3", "decode2", "tq35"):
         if args.workload == "decode4":
             rng = np.random.default_rng(2)
             ctx = rng.integers(1024, 40961, size=16).astype(np.int64)
             name = "config 2: paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 16, ctx U[1k,40k], block 16, seed 2"
+            bits, per_tok, tq = 4, 1088, tq4
+        elif args.workload == "decode4_b256":
+            # a serving batch of many short sequences: the prologue and reduce kernels weigh as much as the main one
+            ctx = np.full(256, 256, dtype=np.int64)
+            name = "paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 256 x 256 tokens, block 16, seed 2"
             bits, per_tok, tq = 4, 1088, tq4
         else:
             ctx = np.full(64, 8192, dtype=np.int64)
@@ -395,7 +400,7 @@ def main():
                 tq.calibrate_uniform(8)
             else:
                 tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
-        seed = 2 if args.workload == "decode4" else 3
+        seed = 2 if args.workload in ("decode4", "decode4_b256") else 3
         # two copies of the cache, alternated, so that no step finds its data in the 256 MB
         # last-level cache left by the previous one
         ws = [decode_workload(torch, akv, dev, tq, bits, seed + 100 * i, len(ctx), ctx) for i in range(2)]
