@@ -103,20 +103,21 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
     uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits, int nqb) {
   __shared__ __align__(16) float q_lds[8][132];   // [query head of the group][input coordinate], zero-padded heads
-  __shared__ float qr_lds[8][128];
+  __shared__ float qr_lds[8][132];     // (rows 4 banks apart: the eight heads of a coordinate are read together)
   __shared__ int32_t scratch[257];
   __shared__ float best_err[256];
   __shared__ float best_alpha[256];
   const int tid = threadIdx.x;
-  // blocks [0, nqb): query rotation, (sequence, kv head) items blockIdx.x, + nqb, ...; block nqb: block prefix;
-  // block nqb + 1: tables
+  // block 0: block prefix; block 1: tables (first, so that they start at once and do not wait for a free slot
+  // behind the rotation blocks); blocks [2, 2 + nqb): query rotation, (sequence, kv head) items blockIdx.x - 2,
+  // + nqb, ...
   const int nq = S * KVH;
-  if ((int)blockIdx.x == nqb) {
+  if ((int)blockIdx.x == 0) {
     if (tid == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
     return;
   }
-  if ((int)blockIdx.x == nqb + 1) {
+  if ((int)blockIdx.x == 1) {
     // The tables depend on the codebook only.  They are kept in the workspace together with
     // the centroids they were built from and a marker; when those match, nothing is rebuilt.
     __shared__ int stale;
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
       bh[t][ks] = akv_as_half8(bop[idx]);
       bl[t][ks] = akv_as_half8(bop[2048 + idx]);
     }
-  for (int item = blockIdx.x; item < nq; item += nqb) {
+  for (int item = (int)blockIdx.x - 2; item < nq; item += nqb) {
   const int s = item / KVH, h = item % KVH;
   for (int i = tid; i < 8 * 128; i += 256) {
     const int q = i >> 7, j = i & 127;
