@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
     const float* __restrict__ part_ml, const float* __restrict__ Pi, const uint4* __restrict__ bop, int S, int QH, int G,
     void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status) {
   constexpr int DPL = D / 64;
-  __shared__ __align__(16) float a_lds[4][D];
+  __shared__ __align__(16) float a_lds[4][D + 8];    // (rows 8 banks apart: the four heads are read together)
   const int groups = (QH + 3) / 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // head_dim 128: the inverse rotation runs on the matrix cores.  Wavefront w owns N-tiles 2w and 2w + 1 of the
