@@ -142,3 +142,48 @@ class TQPagedAttention:
         """0 when the most recent forward() ran clean; bit 0 set when a bounded hand-off wait inside
         its main kernel gave up (the outputs of that call are NaN).  Synchronises the stream."""
         return _lib.attn_status(self._workspace)
+
+
+class _RotationHolder:
+    """What TQPagedAttention reads from a quantizer, for callers that bring the rotation and the codebook
+    themselves."""
+
+    def __init__(self, rotation: torch.Tensor, centroids: torch.Tensor, head_dim: int, bits: int):
+        from .packing import packed_size
+        self.rotation = rotation
+        self.centroids = centroids.to(torch.float32).contiguous()
+        self.head_dim = head_dim
+        self.bits = bits
+        self.num_levels = 1 << bits
+        self._packed_dim = packed_size(head_dim, bits)
+
+    def prepared_rotation(self):
+        from .quantizer import prepared_rotation_for
+        return prepared_rotation_for(self.rotation)
+
+
+class TQPagedAttentionRef:
+    """Constructor and forward() of the reference's pure-PyTorch class (fused_attention.py:53-185): rotation
+    [head_dim, head_dim], centroids [2**bits], an explicit score scale, fixed head counts and block size.
+    Here it runs the same HIP kernels as TQPagedAttention (there is no CPU path: tensors must live on the GPU);
+    the results are those the golden vectors of the reference's class are checked against."""
+
+    def __init__(self, rotation: torch.Tensor, centroids: torch.Tensor, scale: float, num_kv_heads: int,
+                 num_query_heads: int, head_dim: int, block_size: int, bits: int = 4):
+        self.rotation = rotation
+        self.centroids = centroids
+        self.scale = scale
+        self.num_kv_heads = num_kv_heads
+        self.num_query_heads = num_query_heads
+        self.gqa_ratio = num_query_heads // num_kv_heads
+        self.head_dim = head_dim
+        self.block_size = block_size
+        self.bits = bits
+        self._impl = TQPagedAttention(_RotationHolder(rotation, centroids, head_dim, bits), num_query_heads)
+        self._impl.scale = float(scale)
+
+    def forward(self, query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens) -> torch.Tensor:
+        """query [num_seqs, num_query_heads, head_dim] -> same shape and dtype."""
+        return self._impl.forward(query, k_packed, k_norms, v_packed, v_norms, block_tables, context_lens,
+                                  block_size=self.block_size, num_kv_heads=self.num_kv_heads)
+

@@ -117,6 +117,38 @@ class TriAttention:
         w = torch.softmax(scores, dim=-1)
         return torch.einsum("bhs,bshd->bhd", w, value.float()[:, :, heads])
 
+    def benchmark(self, batch_size: int = 1, seq_len: int = 2048, num_trials: int = 10) -> dict:
+        """Times encode_kv, decode_step and the dense reference_attention on random data of the configured shape
+        and compares the two results (reference: attention.py:347-405).  Wall-clock per call in milliseconds, the
+        device synchronised around every timed loop."""
+        import time
+        dev = torch.device(self.device)
+        D, QH, KVH = self.head_dim, self.num_query_heads, self.num_kv_heads
+        q = torch.randn(batch_size, QH, D, device=dev)
+        k = torch.randn(batch_size, seq_len, KVH, D, device=dev)
+        v = torch.randn(batch_size, seq_len, KVH, D, device=dev)
+        kpos = torch.arange(seq_len, device=dev).unsqueeze(0).expand(batch_size, -1).contiguous()
+        qpos = torch.full((batch_size,), seq_len, device=dev)
+
+        def timed(fn):
+            res = fn()
+            torch.cuda.synchronize(dev)
+            t0 = time.perf_counter()
+            for _ in range(num_trials):
+                res = fn()
+            torch.cuda.synchronize(dev)
+            return res, (time.perf_counter() - t0) / num_trials * 1e3
+
+        (k_enc, v_enc), enc_ms = timed(lambda: self.encode_kv(k, v))
+        out, dec_ms = timed(lambda: self.decode_step(q, k_enc, v_enc, qpos, kpos))
+        ref, ref_ms = timed(lambda: self.reference_attention(q, k, v, self.config.rope_base))
+        cos = torch.nn.functional.cosine_similarity(out.reshape(-1, D).float(), ref.reshape(-1, D).float(), dim=-1)
+        return {"encode_ms": enc_ms, "decode_ms": dec_ms, "reference_ms": ref_ms,
+                "speedup": ref_ms / dec_ms if dec_ms > 0 else float("inf"),
+                "compression_ratio": self.config.kv_compression_ratio,
+                "cosine_similarity": cos.mean().item(), "mse": (out.float() - ref.float()).square().mean().item(),
+                "seq_len": seq_len, "batch_size": batch_size}
+
     def decode_step(self, query: torch.Tensor, k_enc: SpectralEncoding, v_enc: SpectralEncoding,
                     query_pos: Optional[torch.Tensor] = None,
                     key_positions: Optional[torch.Tensor] = None) -> torch.Tensor:

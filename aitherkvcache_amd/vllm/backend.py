@@ -49,6 +49,8 @@ def __getattr__(name):
         cls = _make_backend_class()
     elif name == "TurboQuantImpl":
         cls = _get_impl_class()
+    elif name == "TQGPUCache":                 # defined in .cache here; the reference keeps it in this module
+        from .cache import TQGPUCache as cls
     else:
         raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
     globals()[name] = cls

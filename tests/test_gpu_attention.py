@@ -61,6 +61,27 @@ def test_golden_outputs(golden, dev, bits, itype):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_reference_named_class_golden_outputs(golden, dev, bits):
+    """TQPagedAttentionRef takes the rotation, the codebook and the scale as the reference's class of that name
+    does; its results are the reference's golden outputs."""
+    from aitherkvcache_amd.fused_attention import TQPagedAttentionRef
+    tq = make_tq(golden, dev, bits)
+    ref_attn = TQPagedAttentionRef(tq.rotation, tq.centroids, 1.0 / math.sqrt(128), num_kv_heads=2, num_query_heads=8,
+                                   head_dim=128, block_size=16, bits=bits)
+    out = ref_attn.forward(t(golden["attn_q"], dev), t(golden[f"attn_kp_b{bits}"], dev),
+                           t(golden[f"attn_kn_b{bits}"], dev), t(golden[f"attn_vp_b{bits}"], dev),
+                           t(golden[f"attn_vn_b{bits}"], dev), t(golden["attn_tables"], dev), t(golden["attn_ctx"], dev))
+    got = out.cpu().numpy().astype(np.float32)
+    assert np.max(np.abs(got - golden[f"attn_out_b{bits}"].astype(np.float32))) <= TOL
+    # the scale is the caller's: twice the scale is not the same attention
+    other = TQPagedAttentionRef(tq.rotation, tq.centroids, 2.0 / math.sqrt(128), 2, 8, 128, 16, bits)
+    out2 = other.forward(t(golden["attn_q"], dev), t(golden[f"attn_kp_b{bits}"], dev),
+                         t(golden[f"attn_kn_b{bits}"], dev), t(golden[f"attn_vp_b{bits}"], dev),
+                         t(golden[f"attn_vn_b{bits}"], dev), t(golden["attn_tables"], dev), t(golden["attn_ctx"], dev))
+    assert float((out2.float() - out.float()).abs().max()) > 1e-2
+
+
 def build_cache(rng, tq, dev, num_blocks, kvh, bits, block_size=16, pad=0):
     """Random K/V written through the HIP encode-on-write kernel.  Returns device tensors and the
     host copies the oracle reads."""

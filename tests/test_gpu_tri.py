@@ -508,3 +508,18 @@ def test_full_series_equals_rope_attention(dev):
     assert torch.max(torch.abs(out - ref)).item() < 1e-3
     stats = tri.encoder.compression_stats(k)
     assert stats["cosine_similarity"] > 0.999 and stats["energy_ratio"] > 0.999
+
+
+@pytest.mark.gpu
+def test_benchmark_method_reports_times_and_quality(dev):
+    """TriAttention.benchmark runs encode, decode step and the dense reference on random data; random vectors have
+    no spectral concentration, so only the shape of the report and sane ranges are asserted."""
+    from aitherkvcache_amd.triattention import TriAttention, TriAttentionConfig
+    tri = TriAttention(TriAttentionConfig(head_dim=128, num_freqs=12, num_kv_heads=2, num_query_heads=8), device=str(dev))
+    rep = tri.benchmark(batch_size=2, seq_len=300, num_trials=2)
+    assert set(rep) == {"encode_ms", "decode_ms", "reference_ms", "speedup", "compression_ratio", "cosine_similarity",
+                        "mse", "seq_len", "batch_size"}
+    assert rep["encode_ms"] > 0 and rep["decode_ms"] > 0 and rep["reference_ms"] > 0
+    assert rep["seq_len"] == 300 and rep["batch_size"] == 2 and rep["compression_ratio"] > 5
+    assert -1.0 <= rep["cosine_similarity"] <= 1.0 and rep["mse"] >= 0
+

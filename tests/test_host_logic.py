@@ -452,3 +452,36 @@ def test_ranked_calibration_orders_coordinates_by_mean_square():
     u = HybridTurboQuant(device="cpu")
     u.calibrate_uniform(4)
     assert u.group_order is None and u.to_group_order(x) is x
+
+
+def test_tri_pair_series_and_dct_helpers():
+    """The pairwise series equals the dot product of explicitly rotated vectors (the identity the scorer rests on);
+    the DCT matrix is orthogonal, equals scipy's orthonormal DCT-II and inverts."""
+    import scipy.fft
+    from aitherkvcache_amd.triattention.spectral import (dct, dct_matrix, idct, rope_frequencies, rope_phase_matrix,
+                                                           trig_series_coefficients)
+    rng = np.random.default_rng(5)
+    B, S, D = 2, 7, 16
+    q = torch.from_numpy(rng.standard_normal((B, 1, D)))
+    k = torch.from_numpy(rng.standard_normal((B, S, D)))
+    theta = rope_frequencies(D, 1e4, dtype=torch.float64)
+    qpos = torch.tensor([11, 3]); kpos = torch.from_numpy(rng.integers(0, 20, size=(B, S)))
+    c, s_ = trig_series_coefficients(q.expand(B, S, D), k)
+    cp, sp = rope_phase_matrix(qpos, kpos, theta)
+    series = (c * cp + s_ * sp).sum(-1)
+
+    def rope(x, pos):
+        ang = pos.double().unsqueeze(-1) * theta
+        xe, xo = x[..., 0::2], x[..., 1::2]
+        return torch.stack((xe * torch.cos(ang) - xo * torch.sin(ang), xe * torch.sin(ang) + xo * torch.cos(ang)), -1).flatten(-2)
+    direct = (rope(q, qpos.view(B, 1)) * rope(k, kpos)).sum(-1)
+    assert float((series - direct).abs().max()) < 1e-12
+    idx = torch.tensor([1, 6]).expand(B, S, 2)
+    c2, s2 = trig_series_coefficients(q.expand(B, S, D), k, idx)
+    assert torch.equal(c2, c[..., [1, 6]]) and torch.equal(s2, s_[..., [1, 6]])
+    Dm = dct_matrix(12, dtype=torch.float64)
+    assert float((Dm @ Dm.T - torch.eye(12, dtype=torch.float64)).abs().max()) < 1e-14
+    x = torch.from_numpy(rng.standard_normal((3, 12)))
+    assert np.max(np.abs(dct(x).numpy() - scipy.fft.dct(x.numpy(), type=2, norm="ortho", axis=-1))) < 1e-13
+    assert float((idct(dct(x, Dm), Dm) - x).abs().max()) < 1e-13
+
