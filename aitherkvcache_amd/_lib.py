@@ -66,6 +66,7 @@ SIGNATURES = {
     "akv_paged_attn_status": (_i, [_p, C.POINTER(C.c_int), _p]),
     "akv_debug_set_handoff_spin_limit": (_i, [_i]),
     "akv_debug_set_attn_stream": (_i, [_i]),
+    "akv_debug_read_probe": (_i, [_p, _sz, _p, _p]),
     "akv_hybrid_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
                                      _p, _i64, _i64, _i64, _i, _i64, _p]),

@@ -151,6 +151,38 @@ extern "C" int akv_rotation_prepare(const float* rotation, int d, void* prep, si
 }
 
 // ----------------------------------------------------------------------------------
+// Read probe: what a kernel that does nothing but read reaches on this device.  Every lane sums 16-byte loads
+// of a contiguous buffer (a wavefront covers 1 KB per instruction, four loads in flight per lane) and one value
+// per workgroup is written so that the loads stay.  Timed like the dominant kernels (akv_profile_*).
+// ----------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void akv_read_probe_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  uint32_t acc = 0;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc += (a.x ^ a.y) + (a.z ^ a.w) + (b.x ^ b.y) + (b.z ^ b.w) + (c.x ^ c.y) + (c.z ^ c.w) + (d.x ^ d.y) + (d.z ^ d.w);
+  }
+  for (; i < n16; i += stride) {
+    const uint4 a = src[i];
+    acc += (a.x ^ a.y) + (a.z ^ a.w);
+  }
+  acc = (uint32_t)akv_wave_sum((float)(acc & 0xffffu));
+  if ((threadIdx.x & 63) == 0) atomicAdd(&sink[blockIdx.x & 63], acc);
+}
+
+extern "C" int akv_debug_read_probe(const void* src, size_t bytes, void* sink256, void* stream_) {
+  AKV_REQUIRE(src && sink256, "akv_debug_read_probe: null pointer");
+  AKV_REQUIRE(((uintptr_t)src & 15) == 0 && bytes >= 16, "akv_debug_read_probe: src must be 16-byte aligned and hold 16 bytes or more");
+  hipStream_t stream = (hipStream_t)stream_;
+  const int cus = akv_cached_cu_count();
+  const int grid = 2 * (cus > 0 ? cus : 256);     // measured best on the MI355X: 6.1 TB/s over 360 MB (1, 3, 4, 8, 16 per CU: 6.0, 5.8, 5.0, 4.8, 3.7)
+  AKV_LAUNCH_TIMED(akv_read_probe_kernel, grid, 256, 0, stream, (const uint4*)src, bytes / 16, (uint32_t*)sink256);
+  AKV_LAUNCH_CHECK("akv_read_probe_kernel");
+  return AKV_OK;
+}
+
+// ----------------------------------------------------------------------------------
 // quantize + pack / unpack + lookup   (triton_ops.py:220-259)
 // ----------------------------------------------------------------------------------
 template <int BITS>

@@ -19,7 +19,7 @@ having been written by the encode-on-write kernel.  One JSON line is printed:
   encode     the encode-on-write kernel: Mvec/s on 2**20 vectors, the latency of one 256-token
              step (K and V, 8 heads), and `sweep`: kernel duration for 2**12 .. 2**22 vectors with the
              smallest size that reaches 60 % of the HBM peak (`vectors_at_60pct_hbm`)
-  hbm_reference  what torch's own sum (read) and copy (read + write) kernels stream on this box over
+  hbm_reference  what a kernel that only reads (the library's read probe), torch's sum and a copy stream on this box over
              360 MB, the size of the headline step's cache: context for the fraction of the nominal peak
 
 Algorithmic bytes per context token = 8 heads x (64 B codes + 4 B norm) x (K and V) = 1088 B
@@ -129,9 +129,10 @@ def kernel_ms(torch, L, fn, steps):
     return ms.value
 
 
-def hbm_reference(torch, dev):
-    """What the image's own streaming kernels reach on this box for a buffer of the workload's size (360 MB, two
-    buffers alternated): torch's sum (read only) and a device-to-device copy (read + write), in TB/s."""
+def hbm_reference(torch, dev, L):
+    """What plain streaming kernels reach on this box for a buffer of the workload's size (360 MB, two buffers
+    alternated), in TB/s: the library's read probe (16-byte loads, nothing else; kernel time like the dominant
+    kernels'), torch's sum (read only) and a device-to-device copy (read + write)."""
     n = 90 * 1024 * 1024
     xs = [torch.empty(n, dtype=torch.float32, device=dev).normal_() for _ in range(2)]
     y = torch.empty_like(xs[0])
@@ -144,10 +145,19 @@ def hbm_reference(torch, dev):
     def cp():
         st["i"] += 1
         y.copy_(xs[st["i"] & 1])
+    from aitherkvcache_amd import _lib
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+
+    def probe():
+        st["i"] += 1
+        x = xs[st["i"] & 1]
+        _lib.check(L.akv_debug_read_probe(x.data_ptr(), n * 4, sink.data_ptr(), _lib.stream_ptr(dev)))
     precondition(torch, rd, PRECONDITION_S / 2)
     t_rd = timed(torch, rd, 20, 5)
     t_cp = timed(torch, cp, 20, 5)
-    return {"bytes": n * 4, "torch_sum_read_tbs": n * 4 / t_rd / 1e9, "device_copy_read_plus_write_tbs": 2 * n * 4 / t_cp / 1e9}
+    t_pr = kernel_ms(torch, L, probe, 32)
+    return {"bytes": n * 4, "read_probe_kernel_tbs": n * 4 / t_pr / 1e9, "torch_sum_read_tbs": n * 4 / t_rd / 1e9,
+            "device_copy_read_plus_write_tbs": 2 * n * 4 / t_cp / 1e9}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -513,7 +523,7 @@ def main():
     out["cpu_baseline"] = cpu_obj
     out["encode"] = enc
     if not args.no_sweep:
-        out["hbm_reference"] = hbm_reference(torch, dev)
+        out["hbm_reference"] = hbm_reference(torch, dev, L)
     print(json.dumps(out))
 
 

@@ -237,6 +237,12 @@ int akv_debug_set_handoff_spin_limit(int polls);
  * environment) selects the streaming one where it applies; results are the same to rounding. */
 int akv_debug_set_attn_stream(int on);
 
+/* A kernel that only reads: `bytes` of device memory at `src` (16-byte aligned) are summed, one word per
+ * workgroup goes to `sink256` (256 bytes of device memory).  For benchmarks: timed through akv_profile_* like
+ * the dominant kernels, it says what a plain streaming read reaches on the device at hand, next to the 8 TB/s
+ * the roofline figures are quoted against.  No counterpart in the reference. */
+int akv_debug_read_probe(const void* src, size_t bytes, void* sink256, void* stream);
+
 /* ---------------------------------------------------------------------------------
  * HybridTurboQuant, mode tq35 with calibrate_uniform() groups (dims 0..63 at 3-bit MSE,
  * dims 64..127 at 2-bit MSE, each with a 1-bit QJL residual sketch and fp16 norms inside
