@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import aitherkvcache_amd as akv
-from aitherkvcache_amd import triton_ops
+from aitherkvcache_amd import _lib, triton_ops
 from oracle import tq_oracle as O
 from tests.util import kv_like, code_mismatch_report, check_codes, MAX_ULPS
 
@@ -475,3 +475,21 @@ def test_gpu_cache_encode_spill_warm(golden, dev):
     assert not cache.has_spilled(3) and cache.has_spilled(0)
     cache.spill_blocks(torch.empty(0, dtype=torch.long))
     cache.warm_blocks(torch.empty(0, dtype=torch.long))
+
+
+def test_read_probe_sums_what_it_reads(dev):
+    """The read probe of the benchmarks: every 16-byte piece is read exactly once (the folded sum of the words
+    of a known buffer comes out), sizes that are no multiple of the unrolled step included."""
+    L = _lib.lib()
+    for n16 in (1, 255, 4096 * 37 + 5):
+        words = torch.arange(4 * n16, dtype=torch.int64, device=dev) % 251
+        buf = words.to(torch.int32).contiguous()
+        sink = torch.zeros(64, dtype=torch.int32, device=dev)
+        _lib.check(L.akv_debug_read_probe(buf.data_ptr(), 16 * n16, sink.data_ptr(), _lib.stream_ptr(dev)))
+        w = words.view(n16, 4)
+        per_piece = (w[:, 0] ^ w[:, 1]) + (w[:, 2] ^ w[:, 3])
+        # a lane folds its 32-bit sum to 16 bits before the wavefront adds up in float32; small values keep that exact
+        assert int(sink.sum().item()) == int(per_piece.sum().item())
+    with pytest.raises(ValueError):
+        _lib.check(L.akv_debug_read_probe(0, 16, sink.data_ptr(), _lib.stream_ptr(dev)))
+
