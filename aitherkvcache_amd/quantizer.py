@@ -47,6 +47,9 @@ class PreparedRotation:
         if rotation.shape != (d, d):
             raise ValueError(f"rotation must be square, got {tuple(rotation.shape)}")
         self.head_dim = d
+        # (the tensor the key below is taken from stays referenced: while this object lives, e.g. in the cache of
+        # prepared_rotation_for, its address cannot be handed to another tensor that would then match the key)
+        self._origin = rotation
         self.source = rotation.detach().to(torch.float32).contiguous()
         L = _lib.lib()
         nbytes = L.akv_rotation_prepared_bytes(d)
