@@ -65,7 +65,6 @@ SIGNATURES = {
                                    _p]),
     "akv_paged_attn_status": (_i, [_p, C.POINTER(C.c_int), _p]),
     "akv_debug_set_handoff_spin_limit": (_i, [_i]),
-    "akv_debug_set_attn_stream": (_i, [_i]),
     "akv_debug_read_probe": (_i, [_p, _sz, _p, _p]),
     "akv_hybrid_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
@@ -173,6 +172,14 @@ def attn_status(workspace: Optional[torch.Tensor]) -> int:
         return 0
     flags = C.c_int(0)
     check(lib().akv_paged_attn_status(workspace.data_ptr(), C.byref(flags), stream_ptr(workspace.device)))
+    return flags.value
+
+
+def attn_status_static(device) -> int:
+    """Status word of the most recent akv_paged_attn_static call on `device` (the built-in scratch array)."""
+    flags = C.c_int(0)
+    with torch.cuda.device(device):
+        check(lib().akv_paged_attn_status(None, C.byref(flags), stream_ptr(device)))
     return flags.value
 
 

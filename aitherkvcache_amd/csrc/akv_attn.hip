@@ -396,12 +396,6 @@ bool akv_attn_mfma_applicable(const akv_attn_args& a, int d, int bits);
 int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
                       const akv_attn_args& a, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream);
 
-// streaming kernel for the dense 4-bit layout (akv_attn_stream.hip)
-size_t akv_attn_stream_extra_bytes(int S);
-bool akv_attn_stream_applicable(const akv_attn_args& a, int d, int bits);
-int akv_attn_stream_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head, const float* PiT,
-                        const akv_attn_args& a, int bits, const akv_attn_ws& ws, void* extra_ws, int grid, hipStream_t stream);
-
 extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int d) {
   if (num_seqs < 0 || num_q_heads <= 0 || d <= 0) return 0;
   // the number of kv heads is not known here; it is at most the number of query heads
@@ -409,9 +403,16 @@ extern "C" size_t akv_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, 
          akv_attn_mfma_extra_bytes(num_seqs, num_q_heads);
 }
 
+static void* akv_static_scratch_of_current_device();   // null before the first akv_paged_attn_static call there
+
 extern "C" int akv_paged_attn_status(const void* workspace, int* flags, void* stream_) {
-  AKV_REQUIRE(workspace != nullptr && flags != nullptr, "akv_paged_attn_status: null pointer");
+  AKV_REQUIRE(flags != nullptr, "akv_paged_attn_status: null pointer");
   hipStream_t stream = (hipStream_t)stream_;
+  if (workspace == nullptr) {
+    // the built-in scratch array of akv_paged_attn_static on the current device
+    workspace = akv_static_scratch_of_current_device();
+    if (workspace == nullptr) { *flags = 0; return AKV_OK; }
+  }
   uint32_t word = 0;
   AKV_HIP(hipMemcpyAsync(&word, (const char*)workspace + AKV_WS_LUT_BYTES, sizeof(word), hipMemcpyDeviceToHost, stream));
   AKV_HIP(hipStreamSynchronize(stream));
@@ -513,10 +514,7 @@ static int akv_paged_attn_impl(
 
   int rc;
   int Gused = G;
-  if (akv_attn_stream_applicable(a, d, bits)) {
-    Gused = G / AKV_ATTN_WG_PER_CU;   // one 16-wavefront workgroup per CU (its rings and table fill the LDS)
-    rc = akv_attn_stream_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
-  } else if (akv_attn_mfma_applicable(a, d, bits)) {
+  if (akv_attn_mfma_applicable(a, d, bits)) {
     Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
     rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
   } else {
@@ -573,6 +571,12 @@ extern "C" int akv_paged_attn(
 #define AKV_STATIC_MAX_DEVICES 64
 static __device__ __align__(256) unsigned char akv_attn_scratch[AKV_STATIC_SCRATCH_BYTES];
 static void* g_attn_scratch_ptr[AKV_STATIC_MAX_DEVICES];
+
+static void* akv_static_scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= AKV_STATIC_MAX_DEVICES) return nullptr;
+  return __atomic_load_n(&g_attn_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+}
 
 extern "C" size_t akv_paged_attn_static_scratch_bytes(void) { return AKV_STATIC_SCRATCH_BYTES; }
 

@@ -530,6 +530,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
         const uint32_t nw_addr = XB0 + (32u * (uint32_t)nhead + 10u + (nrm_is_v ? 1u : 0u)) * XS + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = XB0 + (32u * hs + 10u) * XS + (uint32_t)g * 16u;
+        // what a lane hands over: a key norm as it is, a value norm as log2 |v| clamped below at -60 (a zero
+        // vector then weighs 2^-60 of its codes: nothing at any output precision; NaN and negative norms,
+        // which only rows outside a context can hold, come out as -60 as well)
+        auto norm_out = [&](float n) { return nrm_is_v ? fmaxf(__builtin_amdgcn_logf(n), -60.f) : n; };
         auto load_chunk = [&](mf_kraw& r, int c) {
           uint32_t pb[2];
           chunk_blocks(c, pb[0], pb[1]);
@@ -623,7 +627,20 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
               for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
             }
           }
+          // The value norms arrive as log2 |v| (clamped below at -60, see the hand-over of the norms) and the
+          // running maximum is kept over score + log2 |v|: the weight p |v| of a token is then exp2 of a
+          // non-positive number, at most 1 whatever the size of the norms, and fits the float16 operand of the
+          // value product with the same relative precision for tiny and for huge value vectors.  The
+          // denominator sums the plain p = exp2(score - max) in the same frame (at most 2^60 each); the frame
+          // cancels between numerator and denominator and travels as `m` of the partial result.
+          union { mf_u32x4 u[2]; float f[8]; } vn;
+          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS);
+          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS + 64u);
+          float tv[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) tv[i] = sv[i] + vn.f[i];
           if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
+            // (a row past the context may hold anything, NaN norms included: both sums are overwritten)
             const int tok0 = blk_lo * bs + 32 * c;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
@@ -631,25 +648,21 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
               for (int i = 0; i < 4; ++i) {
                 const int tok = tok0 + 16 * j + 4 * g + i;
                 const bool ok = (tok < t_end) && (j == 0 || bs32 || 2 * c + 1 < nblk);
-                if (!ok) sv[4 * j + i] = -INFINITY;
+                if (!ok) { sv[4 * j + i] = -INFINITY; tv[4 * j + i] = -INFINITY; }
               }
           }
           // running softmax in the log2 domain (scale * log2 e is folded into the query operand)
-          float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+          float mx = fmaxf(fmaxf(fmaxf(tv[0], tv[1]), fmaxf(tv[2], tv[3])), fmaxf(fmaxf(tv[4], tv[5]), fmaxf(tv[6], tv[7])));
           mx = mf_rows_max(mx);
           const float m_new = fmaxf(m_run, mx);
           const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
           m_run = m_new;
           float psum = 0.f;
-          union { mf_u32x4 u[2]; float f[8]; } vn;
-          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS);
-          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS + 64u);
           float pw[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);    // 0 for masked tokens
-            psum += p;
-            pw[i] = p * vn.f[i];
+            psum += __builtin_amdgcn_exp2f(sv[i] - m_new);            // 0 for masked tokens
+            pw[i] = __builtin_amdgcn_exp2f(tv[i] - m_new);            // p |v| <= 1; 0 for masked tokens
           }
           // weights as float16 hi + lo, two at a time: hi = pw truncated to float16, lo = pw - hi (exact
           // in float32, then truncated); columns [0,8) keep hi, columns [8,16) take the lo pair of the
@@ -674,7 +687,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + XPAR * par) = __float_as_uint(resc_out);
           // the other parity's norm entries were last read in the step before this one
-          *(mf_lds_u32*)(uintptr_t)(nw_addr + XPAR * (par ^ 1u)) = __float_as_uint(rn.nrm);
+          *(mf_lds_u32*)(uintptr_t)(nw_addr + XPAR * (par ^ 1u)) = __float_as_uint(norm_out(rn.nrm));
         };
 
         mf_kraw ra, rb;
@@ -683,7 +696,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_sched_barrier(0);     // queue order = chunk order, as in the loop
         load_chunk(rb, 1);
         __builtin_amdgcn_sched_barrier(0);
-        *(mf_lds_u32*)(uintptr_t)nw_addr = __float_as_uint(ra.nrm);     // norms of chunk 0, ahead of the first barrier
+        *(mf_lds_u32*)(uintptr_t)nw_addr = __float_as_uint(norm_out(ra.nrm));     // norms of chunk 0, ahead of the first barrier
         // pairs of chunks with the same loads on every path (an early exit from the middle of the
         // body would make the compiler wait for the newest prefetch at the top of every iteration)
         int c = 0;

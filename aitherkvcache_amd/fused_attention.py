@@ -103,14 +103,15 @@ class TQPagedAttention:
         for name, t in (("k_packed", k_packed), ("v_packed", v_packed)):
             if t.dtype != torch.uint8 or t.stride(-1) != 1 or t.shape[-1] < self.packed_dim:
                 raise ValueError(f"{name} must be uint8 with contiguous rows of >= {self.packed_dim} bytes")
+        if _static_out is not None and (k_norms.dtype != torch.float32 or v_norms.dtype != torch.float32):
+            raise ValueError("forward_no_alloc needs float32 norms (a conversion would allocate)")
         k_norms = k_norms if k_norms.dtype == torch.float32 else k_norms.float()
         v_norms = v_norms if v_norms.dtype == torch.float32 else v_norms.float()
         bt = block_tables if block_tables.stride(-1) == 1 else block_tables.contiguous()
         cl = context_lens if context_lens.is_contiguous() else context_lens.contiguous()
         num_blocks = min(k_packed.shape[0], k_norms.shape[0], v_packed.shape[0], v_norms.shape[0])
         if _static_out is not None:
-            if (q is not query or k_norms.dtype != torch.float32 or v_norms.dtype != torch.float32
-                    or bt is not block_tables or cl is not context_lens):
+            if q is not query or bt is not block_tables or cl is not context_lens:
                 raise ValueError("forward_no_alloc needs inputs that take no conversion")
             _lib.check(_lib.lib().akv_paged_attn_static(
                 q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
@@ -123,7 +124,9 @@ class TQPagedAttention:
                 out.data_ptr(), _lib.dtype_code(out), out.stride(0), out.stride(1),
                 num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, bt.shape[1], self.scale,
                 _lib.stream_ptr(dev)))
+            self._last_static = dev
             return out
+        self._last_static = None
         ws = self._get_workspace(num_seqs, dev)
         _lib.check(_lib.lib().akv_paged_attn(
             q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
@@ -139,8 +142,10 @@ class TQPagedAttention:
         return out if out.dtype == query.dtype else out.to(query.dtype)
 
     def last_call_status(self) -> int:
-        """0 when the most recent forward() ran clean; bit 0 set when a bounded hand-off wait inside
-        its main kernel gave up (the outputs of that call are NaN).  Synchronises the stream."""
+        """0 when the most recent forward() / forward_no_alloc() ran clean; bit 0 set when a bounded hand-off
+        wait inside its main kernel gave up (the outputs of that call are NaN).  Synchronises the stream."""
+        if getattr(self, "_last_static", None) is not None:
+            return _lib.attn_status_static(self._last_static)       # the library's built-in scratch array
         return _lib.attn_status(self._workspace)
 
 

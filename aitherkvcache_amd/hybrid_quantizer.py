@@ -9,8 +9,9 @@ of a half travel as fp16 inside the 64-byte row (hybrid_quantizer.py:92-123,706-
 
 encode / decode are HIP kernels (one wavefront per vector, butterflies across lanes); the
 codebooks and sign vectors are built on the host at construction, as in the reference.
-Only `tq35` with `calibrate_uniform()` has kernels; `tq25` and variance-ranked `calibrate()`
-are recognised (layout arithmetic works) but raise NotImplementedError when used.
+Only `tq35` has kernels.  `calibrate_uniform()` is the configuration they are written for;
+`calibrate(sample)` runs the same kernels on coordinates permuted into group order.  `tq25` is
+recognised (layout arithmetic works) but raises NotImplementedError when used.
 """
 from __future__ import annotations
 
@@ -87,7 +88,6 @@ _TQ35_D64 = {
 }
 
 
-@functools.lru_cache(maxsize=None)
 # ---- host-side helpers of the reference's module (hybrid_quantizer.py:130-234,310-396): torch ops on whatever
 # device the tensor lives on.  The kernels do these steps in registers; callers that import the helpers keep working.
 def fwht_pow2(x: torch.Tensor) -> torch.Tensor:
@@ -135,6 +135,7 @@ def unpack_multibit(packed: torch.Tensor, dim: int, bits: int) -> torch.Tensor:
     return (stream[..., :dim * bits].reshape(*packed.shape[:-1], dim, bits) * weights).sum(-1).to(torch.uint8)
 
 
+@functools.lru_cache(maxsize=None)
 def _lloyd_on_grid(dim: int, bits: int) -> Tuple[np.ndarray, np.ndarray]:
     """Lloyd iteration on a 10,000-point grid over (-0.999, 0.999) weighted by the marginal
     density of a coordinate of a uniform point on S^{dim-1}, (1-x^2)^((dim-3)/2); at most 200

@@ -224,18 +224,13 @@ int akv_paged_attn_static(const void* query, int q_dtype, int64_t qs_seq, int64_
  * each other through counters with BOUNDED waits, so that a kernel always finishes; a wait
  * that gives up marks the call, whose outputs are then all NaN.  This waits for `stream` and
  * copies the mark to *flags (host pointer): 0 = clean, bit 0 = a hand-off wait gave up.
+ * workspace == NULL asks about the most recent akv_paged_attn_static call on the current device
+ * (0 when there has been none).
  * akv_debug_set_handoff_spin_limit changes the number of polls such a wait makes (negative =
  * the default, 65536); it exists so that a test can exercise the failure path from the host
  * (0 polls: every wait gives up at once, every kernel still runs to its end). */
 int akv_paged_attn_status(const void* workspace, int* flags, void* stream);
 int akv_debug_set_handoff_spin_limit(int polls);
-/* Two matrix-core kernels can serve a dense 4-bit cache of eight kv heads ([blocks][block_size][8][64]
- * codes, [blocks][block_size][8] norms, 16-byte aligned, at most 8 query heads per kv head): the general one,
- * which loads rows into registers, and a streaming one, which fetches whole 8 KB tiles straight into LDS
- * (HBM traffic exactly the algorithmic bytes).  Sustained, both take the same time; in short bursts the
- * general one is faster and is the default.  akv_debug_set_attn_stream(1) (or AKV_ATTN_STREAM=1 in the
- * environment) selects the streaming one where it applies; results are the same to rounding. */
-int akv_debug_set_attn_stream(int on);
 
 /* A kernel that only reads: `bytes` of device memory at `src` (16-byte aligned) are summed, one word per
  * workgroup goes to `sink256` (256 bytes of device memory).  For benchmarks: timed through akv_profile_* like

@@ -183,7 +183,8 @@ def test_paged_attention_ragged_batch_with_stale_rows(golden, dev, qh, kvh, bs):
 def test_config3_shape_properties(golden, dev):
     """tq35 at the benchmark shape (32Q/8KV, 64 sequences x 8192 tokens, block 16), too large for the
     oracle: with one value row everywhere the output must be that row decoded, whatever the scores
-    and wherever the workgroup cuts fall; then one whole sequence with random values against the oracle."""
+    and wherever the workgroup cuts fall; then one whole sequence, run alone, with random values against the
+    oracle; then eight sequences of the full-batch launch with random values against the oracle."""
     h = akv.HybridTurboQuant(device=str(dev))
     h.calibrate_uniform(num_kv_heads=8)
     hp = params(golden)
@@ -222,6 +223,14 @@ def test_config3_shape_properties(golden, dev):
     got = o.cpu().numpy().astype(np.float64)
     print(f"[hybrid attn config 3] one sequence max|diff|={np.max(np.abs(got - ref)):.2e}")
     assert np.all(np.abs(got - ref) <= 2e-3 + 2.0 ** -11 * np.abs(ref))
+    # the whole batch in ONE launch with random values: eight sequences spread over it, the ragged and the
+    # one-token one among them, each against the oracle (a wrong table column or partial slot shows here)
+    full = attn.forward(t(q, dev), kc, vc_r, t(tables, dev), t(ctx, dev), scale=scale).cpu().numpy().astype(np.float64)
+    kc_h, vc_h = kc.cpu().numpy(), vc_r.cpu().numpy()
+    for s_ in (0, 5, 17, 18, 31, 32, 47, 63):
+        r_ = O.hybrid_paged_attention(q[s_:s_ + 1], kc_h, vc_h, tables[s_:s_ + 1], ctx[s_:s_ + 1], hp, scale,
+                                      dtype=np.float64)[0]
+        assert np.all(np.abs(full[s_] - r_) <= 2e-3 + 2.0 ** -11 * np.abs(r_)), f"sequence {s_} of the full batch"
 
 
 def test_hybrid_decode_step_custom_op(golden, dev):

@@ -401,6 +401,11 @@ def test_hybrid_module_helpers_against_the_oracle():
     x = rng.standard_normal((5, 64)).astype(np.float32)
     xt = torch.from_numpy(x.copy())
     assert fwht_pow2(xt) is xt and np.allclose(xt.numpy(), O.fwht(x), rtol=1e-6, atol=1e-5)
+    # H H = N I: a second call on the SAME tensor must transform it again (nothing is cached per argument)
+    assert fwht_pow2(xt) is xt and np.allclose(xt.numpy(), 64.0 * x, rtol=1e-5, atol=1e-4)
+    ones = torch.ones(4)
+    assert fwht_pow2(ones).tolist() == [4.0, 0.0, 0.0, 0.0] and fwht_pow2(ones).tolist() == [4.0, 4.0, 4.0, 4.0]
+    assert not hasattr(fwht_pow2, "cache_info")
     y = rng.standard_normal((3, 96)).astype(np.float32)
     got = fwht_general(torch.from_numpy(y)).numpy()
     assert np.allclose(got[:, :64], O.fwht(y[:, :64]), atol=1e-5) and np.allclose(got[:, 64:], O.fwht(y[:, 64:]), atol=1e-5)
