@@ -46,7 +46,8 @@ template <int D, int ODT>
 __global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
     const int32_t* __restrict__ prefix, const float* __restrict__ part_acc,
     const float* __restrict__ part_ml, const float* __restrict__ Pi, const uint4* __restrict__ bop, int S, int QH, int G,
-    void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status) {
+    void* __restrict__ out, int64_t os_seq, int64_t os_head, const uint32_t* __restrict__ status,
+    const int32_t* __restrict__ seqw) {
   constexpr int DPL = D / 64;
   __shared__ __align__(16) float a_lds[4][D + 8];    // (rows 8 banks apart: the four heads are read together)
   const int groups = (QH + 3) / 4;
@@ -72,8 +73,20 @@ __global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
   for (int item = blockIdx.x; item < S * groups; item += gridDim.x) {
   const int s = item / groups, hg = item % groups;
   const int h = hg * 4 + wave;
-  const int b0 = prefix[s], b1 = prefix[s + 1];
-  if (b1 <= b0) {        // (the same for the whole workgroup)
+  // workgroups of the main kernel whose ranges meet the sequence: from the record of the matrix-core
+  // kernel's prologue (seqw), else from the equal cut of the block axis
+  int b0 = 0, b1 = 0, w_lo, w_hi;
+  if (seqw != nullptr) {
+    w_lo = seqw[2 * s];
+    w_hi = seqw[2 * s + 1];
+  } else {
+    b0 = prefix[s];
+    b1 = prefix[s + 1];
+    const int per = (prefix[S] + G - 1) / G;
+    w_lo = per > 0 ? b0 / per : 0;
+    w_hi = b1 > b0 ? (b1 - 1) / per : w_lo - 1;
+  }
+  if (w_hi < w_lo) {        // an empty sequence (the same for the whole workgroup)
     if (h < QH) {
 #pragma unroll
       for (int i = 0; i < DPL; ++i) akv_elem<ODT>::store(out, s * os_seq + h * os_head + lane * DPL + i, poison);
@@ -81,9 +94,6 @@ __global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
     continue;
   }
   if (h < QH) {
-    const int total = prefix[S];
-    const int per = (total + G - 1) / G;
-    const int w_lo = b0 / per, w_hi = (b1 - 1) / per;
     // the first RED_PF partial accumulators are requested before anything is known about their
     // weights, so that their round trip overlaps the one of the (max, sum) pairs
     // (only slots that exist are read: a batch of many short sequences has one or two per head)
@@ -443,15 +453,15 @@ static int akv_launch_attn_general(const akv_attn_args& a, int grid, hipStream_t
 
 template <int D>
 static int akv_launch_reduce(int odt, const akv_attn_args& a, const float* Pi, const uint4* bop, int G, void* out,
-                             int64_t os_seq, int64_t os_head, const uint32_t* status, hipStream_t stream) {
+                             int64_t os_seq, int64_t os_head, const uint32_t* status, const int32_t* seqw, hipStream_t stream) {
   // at most three workgroups per CU (what its registers admit at once); a workgroup loops over its items
   const int items = a.S * ((a.QH + 3) / 4);
   const int cus = akv_cached_cu_count();
   const int grid = items < 3 * (cus > 0 ? cus : 256) ? items : 3 * (cus > 0 ? cus : 256);
   switch (odt) {
-    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
-    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
-    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status); break;
+    case AKV_F16: akv_attn_reduce_kernel<D, AKV_F16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status, seqw); break;
+    case AKV_BF16: akv_attn_reduce_kernel<D, AKV_BF16><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status, seqw); break;
+    default: akv_attn_reduce_kernel<D, AKV_F32><<<grid, 256, 0, stream>>>(a.prefix, a.part_acc, a.part_ml, Pi, bop, a.S, a.QH, G, out, os_seq, os_head, status, seqw); break;
   }
   AKV_LAUNCH_CHECK("akv_attn_reduce_kernel");
   return AKV_OK;
@@ -514,7 +524,9 @@ static int akv_paged_attn_impl(
 
   int rc;
   int Gused = G;
+  const int32_t* seqw = nullptr;      // set by the matrix-core path, whose prologue cuts the block axis itself
   if (akv_attn_mfma_applicable(a, d, bits)) {
+    seqw = ws.seqw;
     Gused = G / AKV_ATTN_WG_PER_CU;   // one 8-wavefront workgroup per CU (64 KiB table, up to 256 VGPRs)
     rc = akv_attn_mfma_run(query, q_dtype, qs_seq, qs_head, PiT, a, bits, ws, (char*)workspace + ws.bytes, Gused, stream);
   } else {
@@ -531,9 +543,9 @@ static int akv_paged_attn_impl(
 #undef AKV_CASE
   }
   if (rc) return rc;
-  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, stream);
-  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(128)), Gused, out, os_seq, os_head, ws.status, stream);
-  return akv_launch_reduce<256>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, stream);
+  if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
+  if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(128)), Gused, out, os_seq, os_head, ws.status, seqw, stream);
+  return akv_launch_reduce<256>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
 }
 
 extern "C" int akv_paged_attn(

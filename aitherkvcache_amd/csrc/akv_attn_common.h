@@ -58,7 +58,9 @@ static inline size_t akv_align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct akv_attn_ws {
   uint32_t* lut;     // AKV_WS_LUT_BYTES of cached tables (matrix-core kernels)
   uint32_t* status;  // AKV_WS_STATUS_BYTES
-  int32_t* wgdesc;   // [G][8] start record of every workgroup of the streaming kernel (written by its prologue)
+  int32_t* wgdesc;   // [G][8] record of every workgroup of the matrix-core kernel: its range [g0, g1) of the global
+                     // block axis (written by that kernel's prologue; see akv_attn_partition)
+  int32_t* seqw;     // [S][2] first and last workgroup whose range meets the sequence (same prologue)
   int32_t* prefix;   // [S + 1] exclusive prefix of blocks per sequence; prefix[S] = total
   float* qrot;       // [S][QH][acc_floats] transformed queries
   float* part_acc;   // [G + S][QH][acc_floats]
@@ -73,6 +75,8 @@ static inline akv_attn_ws akv_attn_ws_layout(void* base, int S, int QH, int acc_
   size_t off = AKV_WS_HEADER_BYTES;
   w.wgdesc = (int32_t*)((char*)base + off);
   off += akv_align256((size_t)G * 8 * 4);
+  w.seqw = (int32_t*)((char*)base + off);
+  off += akv_align256((size_t)(S > 0 ? S : 1) * 2 * 4);
   w.prefix = (int32_t*)((char*)base + off);
   off += akv_align256((size_t)(S + 1) * 4);
   w.qrot = (float*)((char*)base + off);
@@ -141,6 +145,106 @@ __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, 
     run += akv_seq_blocks(context_lens, cl_itype, s, block_size, max_blocks_per_seq);
   }
   if (tid == 255) prefix[S] = base + inc;
+}
+
+// ----------------------------------------------------------------------------------
+// Partition of the global block axis among the G workgroups of the matrix-core kernel, written by one
+// workgroup of 256 threads after the prefix scan (same workgroup; `prefix` is read back from memory).
+//
+// A workgroup whose range crosses a sequence boundary starts twice (query operand, block ids, first rows, a
+// partial chunk at both ends): measured, such workgroups finish 5 us after the others and ARE the tail of
+// the launch.  So when the batch has few sequences (at most 64 in all, the non-empty ones at most G / 4) every
+// sequence gets whole workgroups: the smallest lambda (chunks per workgroup) with sum_s ceil(c_s / lambda) <= G
+// is found by bisection (the sum is non-increasing in lambda), sequence s takes k_s = ceil(c_s / lambda)
+// consecutive workgroups and splits its c_s chunks evenly among them; left-over workgroups get an empty range.
+// Otherwise the axis is cut into G equal ranges as before.  Either way workgroups and sequences both advance
+// monotonically along the axis, so slot = workgroup + sequence stays unique, and seqw[s] = (first, last
+// workgroup that meets sequence s), which the reduce kernel reads instead of dividing by the range length.
+// `cb` = blocks per chunk of the main kernel (2 for blocks of 16 tokens, 1 for blocks of 32).
+// ----------------------------------------------------------------------------------
+__device__ __forceinline__ void akv_attn_partition(const int32_t* prefix, int S, int G, int cb, int32_t* wgdesc,
+                                                   int32_t* seqw, int32_t* lds /*[>= 136]*/) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  __threadfence_block();
+  __syncthreads();                      // the prefix written by this workgroup is readable by all of it
+  const int total = prefix[S];
+  int32_t* p_wfirst = lds;              // [65] first workgroup of each sequence; [S] = workgroups in use
+  int32_t* p_pref = lds + 65;           // [65] block prefix
+  int32_t* p_mode = lds + 130;          // [0] 1 = whole workgroups per sequence
+  if (tid < 64) {
+    int aligned = 0;
+    if (S <= 64) {
+      const int b0 = lane < S ? prefix[lane] : total, b1 = lane < S ? prefix[lane + 1] : total;
+      const int c = (b1 - b0 + cb - 1) / cb;                     // chunks of the lane's sequence
+      p_pref[lane] = b0;
+      if (lane == 0) p_pref[64] = total;
+      int sumc = c;
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) sumc += __shfl_xor(sumc, m, 64);
+      const int nz = __popcll(__ballot(c > 0));
+      aligned = (nz >= 1 && nz * 4 <= G) ? 1 : 0;
+      if (aligned) {
+        int lo = (sumc + G - 1) / G, hi = (sumc + (G - nz) - 1) / (G - nz);      // hi is always feasible
+        if (lo < 1) lo = 1;
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          int tot = (c + mid - 1) / mid;
+#pragma unroll
+          for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
+          if (tot <= G) hi = mid; else lo = mid + 1;
+        }
+        const int k = (c + lo - 1) / lo;
+        int inc = k;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int up = __shfl_up(inc, d, 64);
+          if (lane >= d) inc += up;
+        }
+        p_wfirst[lane] = inc - k;
+        if (lane == 63) p_wfirst[64] = inc;
+      }
+    }
+    if (lane == 0) p_mode[0] = aligned;
+  }
+  __syncthreads();
+  const int aligned = p_mode[0];
+  const int per = (total + G - 1) / G;
+  for (int w = tid; w < G; w += blockDim.x) {
+    int g0 = 0, g1 = 0;
+    if (aligned) {
+      if (w < p_wfirst[64]) {
+        // the last s with p_wfirst[s] <= w (entries are non-decreasing; a sequence without workgroups shares the
+        // next one's entry and is passed over; entries of lanes past the batch equal the number in use)
+        int cnt = 0;
+        for (int i = 0; i < 64; ++i) cnt += (p_wfirst[i] <= w) ? 1 : 0;
+        const int s = cnt - 1;
+        const int b0 = p_pref[s], b1 = p_pref[s + 1];
+        const int k = p_wfirst[s + 1] - p_wfirst[s];
+        const int c = (b1 - b0 + cb - 1) / cb;
+        const int pc = (c + k - 1) / k;
+        g0 = min(b1, b0 + (w - p_wfirst[s]) * pc * cb);
+        g1 = min(b1, g0 + pc * cb);
+      }
+    } else {
+      g0 = min(total, w * per);
+      g1 = min(total, g0 + per);
+    }
+    wgdesc[w * 8] = g0;
+    wgdesc[w * 8 + 1] = g1;
+  }
+  for (int s = tid; s < S; s += blockDim.x) {
+    int w_lo, w_hi;
+    if (aligned) {
+      w_lo = p_wfirst[s];
+      w_hi = p_wfirst[s + 1] - 1;
+    } else {
+      const int b0 = prefix[s], b1 = prefix[s + 1];
+      w_lo = per > 0 ? b0 / per : 0;
+      w_hi = (per > 0 && b1 > b0) ? (b1 - 1) / per : w_lo - 1;
+    }
+    seqw[2 * s] = w_lo;
+    seqw[2 * s + 1] = w_hi;
+  }
 }
 
 // largest s with prefix[s] <= g  (prefix non-decreasing, prefix[0] = 0, g < prefix[S])

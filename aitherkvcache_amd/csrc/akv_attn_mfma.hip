@@ -89,6 +89,7 @@ static_assert(MF_W_WORDS * 4 <= AKV_WS_LUT_BYTES, "table block must fit the work
 struct akv_mfma_extra {
   const uint32_t* lut;   // table block, MF_W_* (workspace header)
   const uint4* qop;      // [S][KVH][8 k-steps][64 lanes] half8 as uint4 (workspace)
+  const int32_t* wgdesc; // [G][8]: range [g0, g1) of the global block axis of every workgroup (workspace)
   uint32_t* status;      // status words of the call (workspace header)
   int spin_limit;        // polls a hand-off wait makes before it gives up
 };
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const uint4* __restrict__ bop,
     const float* __restrict__ centroids, int S, int QH, int KVH, const void* context_lens,
     int cl_itype, int block_size, int64_t max_blocks_per_seq, int32_t* prefix,
-    uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits, int nqb) {
+    uint4* __restrict__ qop, uint32_t* __restrict__ lut, uint32_t* __restrict__ status, float qscale, int bits, int nqb,
+    int32_t* __restrict__ wgdesc, int32_t* __restrict__ seqw, int G) {
   __shared__ __align__(16) float q_lds[8][132];   // [query head of the group][input coordinate], zero-padded heads
   __shared__ float qr_lds[8][132];     // (rows 4 banks apart: the eight heads of a coordinate are read together)
   __shared__ int32_t scratch[257];
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
   if ((int)blockIdx.x == 0) {
     if (tid == 0) status[0] = 0u;
     akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
+    akv_attn_partition(prefix, S, G, block_size == 32 ? 1 : 2, wgdesc, seqw, scratch);
     return;
   }
   if ((int)blockIdx.x == 1) {
@@ -431,7 +434,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   const uint32_t rs_addr = XB0 + (32u * hs + 8u + (uint32_t)(lane >> 5)) * XS + (uint32_t)(lane & 31) * 4u;
 
 
-  const int G = gridDim.x;
   // blocks of 16 tokens: a chunk (32 tokens, two 16-token tiles) is two blocks; blocks of 32: one
   // block, its second tile 16 positions further in.  bs32 is the same in every wavefront.
   const bool bs32 = a.block_size == 32;
@@ -439,10 +441,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   // (the block prefix of the batch in a register, one entry per lane: finding a segment's sequence and its
   // bounds costs no chain of dependent loads)
   const int held = akv_prefix_hold(a.prefix, a.S);
-  const int total = a.S <= 63 ? __builtin_amdgcn_readlane(held, a.S) : a.prefix[a.S];
-  const int per = (total + G - 1) / G;
-  const int g0 = blockIdx.x * per;
-  const int g1 = min(total, g0 + per);
+  // the workgroup's range of the global block axis, as the prologue cut it (whole workgroups per sequence
+  // when the batch has few sequences, equal ranges otherwise)
+  const int g0 = x.wgdesc[8 * blockIdx.x], g1 = x.wgdesc[8 * blockIdx.x + 1];
   const int gqa = a.QH / a.KVH;
 
   int gcur = g0;
@@ -980,6 +981,7 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   akv_mfma_extra x;
   x.lut = ws.lut;
   x.qop = (const uint4*)extra_ws;
+  x.wgdesc = ws.wgdesc;
   x.status = ws.status;
   x.spin_limit = g_spin_limit;
   const float qscale = a.scale * 1.4426950408889634f;   // scores come out in the log2 domain
@@ -988,7 +990,7 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   const int nqb = a.S * a.KVH < 6 * (cus > 0 ? cus : 256) ? a.S * a.KVH : 6 * (cus > 0 ? cus : 256);
   const int pgrid = nqb + 2;
   const uint4* bop = (const uint4*)(PiT + 128 * 128);    // the encode kernel's operand follows Pi and PiT in the prepared buffer
-#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, bop, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, x.status, qscale, bits, nqb)
+#define MF_PRO(DT) akv_attn_mfma_prologue_kernel<DT><<<pgrid, 256, 0, stream>>>(query, qs_seq, qs_head, bop, a.centroids, a.S, a.QH, a.KVH, a.context_lens, a.cl_itype, a.block_size, a.max_blocks_per_seq, prefix, (uint4*)x.qop, (uint32_t*)x.lut, x.status, qscale, bits, nqb, ws.wgdesc, ws.seqw, grid)
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");

@@ -61,6 +61,8 @@ def parse():
     ap.add_argument("--workload", default="decode4",
                     choices=["decode4", "decode4_b256", "decode3", "decode2", "tq35", "tri", "encode"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the 3-bit / 2-bit / tq35 / TriAttention workloads that the default run reports beside the headline one")
     ap.add_argument("--no-sweep", action="store_true",
                     help="skip the encode size sweep (a profiler run then sees the encode kernel at 2**20 vectors only)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -239,7 +241,32 @@ def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds, sweep=True
             reps += 1
         dt = (time.perf_counter() - t0) / reps
         res["cpu_mvec_s"] = 65536 / dt / 1e6
+        res["parity_config0"] = encode_parity_config0(torch, tq, dev, R)
     return res, tq
+
+
+def encode_parity_config0(torch, tq, dev, R):
+    """The 65,536 vectors of the CPU round-trip configuration (numpy PCG64 seed 0: N(0,1) entries times a
+    lognormal(0, 0.5) norm, fp16) through the HIP encode and decode kernels, against the oracle: codes that
+    differ, counted, with the distance of their float64 rotated value from the decision boundary in float32
+    ulps as a histogram; norms; reconstruction error of the round trip."""
+    from oracle import tq_oracle as O
+    rng = np.random.default_rng(0)
+    g = rng.standard_normal((65536, 128), dtype=np.float32)
+    sc = rng.lognormal(0.0, 0.5, size=65536).astype(np.float32)
+    x = (g * sc[:, None]).astype(np.float16)
+    xd = torch.from_numpy(x).to(dev)
+    packed, norms = tq.encode(xd)
+    rep = O.encode_parity_report(packed.cpu().numpy(), norms.cpu().numpy(), x, R, 4)
+    xh = tq.decode(packed, norms).float().cpu().numpy().astype(np.float64)
+    x64 = x.astype(np.float64)
+    rep["round_trip_mse"] = float(np.mean((xh - x64) ** 2))
+    rep["round_trip_mse_over_mean_sq_norm"] = float(np.sum((xh - x64) ** 2) / np.sum(x64 ** 2))
+    c, _, _ = O.get_codebook(128, 4)
+    ref = O.decode(packed.cpu().numpy(), norms.cpu().numpy(), R, c, 4).astype(np.float64)
+    rep["decode_max_abs_diff_vs_oracle"] = float(np.max(np.abs(xh - ref)))
+    rep["vectors"] = 65536
+    return rep
 
 
 def decode_workload(torch, akv, dev, tq, bits_or_mode, seed, num_seqs, ctx):
@@ -357,6 +384,147 @@ def encode_sweep(torch, akv, L, tq, dev, gen):
     return rows, reached
 
 
+DECODE_DTYPE = "fp16 hi+lo MFMA operands (keys and queries carry 22 bits, values 11), f32 accumulate and softmax"
+
+
+def traffic_fields(workload):
+    """`traffic` of a roofline object: not measured in this run (counters need a profiler), read from the
+    committed counter runs."""
+    t = measured_traffic(workload)
+    return {"traffic": t, "traffic_source": None if t is None else "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / "
+                                                                    "WRITE_SIZE runs of this command, committed; not measured in this run)"}
+
+
+def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_seconds, cores):
+    """One paged decode-attention workload: (result fields, roofline, cpu_baseline or None)."""
+    if workload == "decode4":
+        rng = np.random.default_rng(2)
+        ctx = rng.integers(1024, 40961, size=16).astype(np.int64)
+        name = "config 2: paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 16, ctx U[1k,40k], block 16, seed 2"
+        bits, per_tok, tq = 4, 1088, tq4
+    elif workload == "decode4_b256":
+        # a serving batch of many short sequences: the prologue and reduce kernels weigh as much as the main one
+        ctx = np.full(256, 256, dtype=np.int64)
+        name = "paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 256 x 256 tokens, block 16, seed 2"
+        bits, per_tok, tq = 4, 1088, tq4
+    else:
+        ctx = np.full(64, 8192, dtype=np.int64)
+        bits = {"decode3": 3, "decode2": 2, "tq35": "tq35"}[workload]
+        per_tok = {"decode3": 8 * 104, "decode2": 8 * 72, "tq35": 8 * 128}[workload]
+        name = f"config 3: paged decode attention, {workload}, 32Q/8KV d=128, batch 64 x 8192, block 16, seed 3"
+        if bits == "tq35":
+            tq = akv.HybridTurboQuant(device=str(dev))
+            tq.calibrate_uniform(8)
+        else:
+            tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
+    seed = 2 if workload in ("decode4", "decode4_b256") else 3
+    # two copies of the cache, alternated, so that no step finds its data in the 256 MB
+    # last-level cache left by the previous one
+    ws = [decode_workload(torch, akv, dev, tq, bits, seed + 100 * i, len(ctx), ctx) for i in range(2)]
+    if bits == "tq35":
+        attn = akv.HybridPagedAttention(tq, 32)
+        calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["vp"], w["tables"], w["ctx"], scale=1 / math.sqrt(128))
+                 for w in ws]
+    else:
+        attn = akv.TQPagedAttention(tq, 32)
+        calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["kn"], w["vp"], w["vn"], w["tables"], w["ctx"])
+                 for w in ws]
+    state = {"i": 0}
+
+    def step():
+        calls[state["i"] & 1]()
+        state["i"] += 1
+
+    tokens = int(ctx.sum())
+    algo_bytes = tokens * per_tok + 2 * len(ctx) * 32 * 128 * 2 + ws[0]["tables"].numel() * 4
+    ms = timed(torch, step, steps, warmup)
+    kms = kernel_ms(torch, L, step, max(20, steps))
+    res = dict(metric="tq-t4nc paged-decode attn GB/s" if workload == "decode4" else f"{workload} paged-decode attn GB/s",
+               value=algo_bytes / ms / 1e6, ms_per_step=ms, dtype=DECODE_DTYPE,
+               config={"workload": name, "context_tokens": tokens, "algorithmic_bytes_per_step": algo_bytes,
+                       "cache_copies_alternated": 2, "preconditioning_s": PRECONDITION_S})
+    achieved = tokens * per_tok / kms / 1e6
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            **traffic_fields(workload), "kernel": "main decode-attention kernel", "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": tokens * per_tok}
+    cpu_obj = None
+    if cpu and bits == "tq35":
+        toks, secs, what = cpu_hybrid_baseline(ws[0], tq, cpu_seconds)
+        cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+                   "sample": f"numpy float32 oracle (hybrid_decode of every addressed row, dense softmax "
+                             f"attention) on {what} = {toks} context tokens"}
+    elif cpu:
+        toks, secs, seqs = cpu_attention_baseline(ws[0], tq, bits, cpu_seconds)
+        cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+                   "sample": f"numpy float32 oracle (gather, unpack, codebook, einsum, softmax, einsum, inverse "
+                             f"rotation) on whole sequences {seqs} of the batch = {toks} context tokens"}
+    del ws, calls, attn
+    torch.cuda.empty_cache()
+    return res, roof, cpu_obj
+
+
+def run_tri(torch, L, dev, steps, warmup, cpu, cpu_seconds, cores):
+    from aitherkvcache_amd.triattention import TriAttention, TriAttentionConfig
+    cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=8, num_query_heads=32,
+                             rope_base=1e6)
+    tri = TriAttention(cfg, device=str(dev))
+    gen = torch.Generator(device=dev).manual_seed(4)
+    B, S = 8, 32768
+    std = (torch.arange(64, device=dev) + 1.0) ** -0.75
+    sets = []
+    for _ in range(3):     # three copies alternated: one copy (109 MB) would sit in the last-level cache
+        keys = (torch.randn(B, S, 8, 64, 2, device=dev, generator=gen) * std[:, None]).reshape(B, S, 8, 128).half()
+        vals = torch.randn(B, S, 8, 128, device=dev, generator=gen).half()
+        sets.append(tri.encode_kv(keys, vals))
+        del keys, vals
+    # queries in the model's dtype (fp16, like the keys and values of this configuration); the same step with
+    # float32 queries is reported beside it
+    q32 = torch.randn(B, 32, 128, device=dev, generator=gen)
+    q = q32.half()
+    state = {"i": 0, "q": q}
+
+    def step():
+        k_enc, v_enc = sets[state["i"] % 3]
+        tri.decode_step(state["q"], k_enc, v_enc)
+        state["i"] += 1
+
+    algo_bytes = B * S * 8 * 52
+    ms = timed(torch, step, steps, warmup)
+    kms = kernel_ms(torch, L, step, max(20, steps))
+    state["q"] = q32
+    kms32 = kernel_ms(torch, L, step, max(20, steps))
+    state["q"] = q
+    res = dict(metric="TriAttention decode_step GB/s", value=algo_bytes / ms / 1e6, ms_per_step=ms,
+               dtype="f32 scores and softmax, fp16 hi/lo MFMA operands for the value sums",
+               config={"workload": "config 4: TriAttention decode_step, F=12 int4, 32Q/8KV d=128, batch 8 x 32768, "
+                                   "fp16 queries, seed 4",
+                       "algorithmic_bytes_per_step": algo_bytes, "cache_copies_alternated": 3,
+                       "preconditioning_s": PRECONDITION_S, "kernel_ms_float32_queries": kms32})
+    achieved = algo_bytes / kms / 1e6
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            **traffic_fields("tri"), "kernel": "tri_decode_heads_kernel<4>", "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": algo_bytes}
+    cpu_obj = None
+    if cpu:
+        from oracle import tq_oracle as O
+        k_enc, v_enc = sets[0]
+        S_s = 2048
+        ke = tuple(t[:1, :S_s].cpu().numpy() for t in k_enc)
+        ve = tuple(t[:1, :S_s].cpu().numpy() for t in v_enc)
+        th = tri._theta.cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < cpu_seconds or reps < 1:
+            O.tri_decode_step(q[:1].cpu().numpy(), ke, ve, th)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        cpu_obj = {"value": S_s * 8 * 52 / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+                   "sample": f"numpy oracle of decode_step on batch element 0, first {S_s} tokens"}
+    del sets
+    torch.cuda.empty_cache()
+    return res, roof, cpu_obj
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -366,7 +534,6 @@ def main():
     import torch
     import aitherkvcache_amd as akv
     from aitherkvcache_amd import _lib
-    from aitherkvcache_amd.triattention import TriAttention, TriAttentionConfig
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a HIP device")
@@ -390,124 +557,14 @@ def main():
     cpu_obj = None
 
     if args.workload in ("decode4", "decode4_b256", "decode3", "decode2", "tq35"):
-        if args.workload == "decode4":
-            rng = np.random.default_rng(2)
-            ctx = rng.integers(1024, 40961, size=16).astype(np.int64)
-            name = "config 2: paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 16, ctx U[1k,40k], block 16, seed 2"
-            bits, per_tok, tq = 4, 1088, tq4
-        elif args.workload == "decode4_b256":
-            # a serving batch of many short sequences: the prologue and reduce kernels weigh as much as the main one
-            ctx = np.full(256, 256, dtype=np.int64)
-            name = "paged decode attention, tq-t4nc, 32Q/8KV d=128, batch 256 x 256 tokens, block 16, seed 2"
-            bits, per_tok, tq = 4, 1088, tq4
-        else:
-            ctx = np.full(64, 8192, dtype=np.int64)
-            bits = {"decode3": 3, "decode2": 2, "tq35": "tq35"}[args.workload]
-            per_tok = {"decode3": 8 * 104, "decode2": 8 * 72, "tq35": 8 * 128}[args.workload]
-            name = f"config 3: paged decode attention, {args.workload}, 32Q/8KV d=128, batch 64 x 8192, block 16, seed 3"
-            if bits == "tq35":
-                tq = akv.HybridTurboQuant(device=str(dev))
-                tq.calibrate_uniform(8)
-            else:
-                tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
-        seed = 2 if args.workload in ("decode4", "decode4_b256") else 3
-        # two copies of the cache, alternated, so that no step finds its data in the 256 MB
-        # last-level cache left by the previous one
-        ws = [decode_workload(torch, akv, dev, tq, bits, seed + 100 * i, len(ctx), ctx) for i in range(2)]
-        if bits == "tq35":
-            attn = akv.HybridPagedAttention(tq, 32)
-            calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["vp"], w["tables"], w["ctx"], scale=1 / math.sqrt(128))
-                     for w in ws]
-        else:
-            attn = akv.TQPagedAttention(tq, 32)
-            calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["kn"], w["vp"], w["vn"], w["tables"], w["ctx"])
-                     for w in ws]
-        state = {"i": 0}
-
-        def step():
-            calls[state["i"] & 1]()
-            state["i"] += 1
-
-        tokens = int(ctx.sum())
-        algo_bytes = tokens * per_tok + 2 * len(ctx) * 32 * 128 * 2 + ws[0]["tables"].numel() * 4
-        ms = timed(torch, step, args.steps, args.warmup)
-        kms = kernel_ms(torch, L, step, max(20, args.steps))
-        out.update(metric="tq-t4nc paged-decode attn GB/s" if args.workload == "decode4"
-                   else f"{args.workload} paged-decode attn GB/s",
-                   value=algo_bytes / ms / 1e6, ms_per_step=ms,
-                   dtype="fp16 hi+lo MFMA operands (keys and queries carry 22 bits, values 11), f32 accumulate and softmax",
-                   config={"workload": name, "context_tokens": tokens, "algorithmic_bytes_per_step": algo_bytes,
-                           "cache_copies_alternated": 2, "preconditioning_s": PRECONDITION_S})
-        achieved = tokens * per_tok / kms / 1e6
-        out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
-                           "kernel": "main decode-attention kernel", "kernel_ms": kms}
-        if cpu and bits == "tq35":
-            toks, secs, what = cpu_hybrid_baseline(ws[0], tq, args.cpu_seconds)
-            cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-                       "sample": f"numpy float32 oracle (hybrid_decode of every addressed row, dense softmax "
-                                 f"attention) on {what} = {toks} context tokens"}
-        elif cpu:
-            toks, secs, seqs = cpu_attention_baseline(ws[0], tq, bits, args.cpu_seconds)
-            cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-                       "sample": f"numpy float32 oracle (gather, unpack, codebook, einsum, softmax, einsum, inverse "
-                                 f"rotation) on whole sequences {seqs} of the batch = {toks} context tokens"}
+        res, roof, cpu_obj = run_decode(torch, akv, L, dev, args.workload, tq4, args.steps, args.warmup, cpu,
+                                        args.cpu_seconds, cores)
+        out.update(res)
+        out["roofline"] = roof
     elif args.workload == "tri":
-        cfg = TriAttentionConfig(head_dim=128, num_freqs=12, coeff_bits=4, num_kv_heads=8, num_query_heads=32,
-                                 rope_base=1e6)
-        tri = TriAttention(cfg, device=str(dev))
-        gen = torch.Generator(device=dev).manual_seed(4)
-        B, S = 8, 32768
-        std = (torch.arange(64, device=dev) + 1.0) ** -0.75
-        sets = []
-        for _ in range(3):     # three copies alternated: one copy (109 MB) would sit in the last-level cache
-            keys = (torch.randn(B, S, 8, 64, 2, device=dev, generator=gen) * std[:, None]).reshape(B, S, 8, 128).half()
-            vals = torch.randn(B, S, 8, 128, device=dev, generator=gen).half()
-            sets.append(tri.encode_kv(keys, vals))
-            del keys, vals
-        # queries in the model's dtype (fp16, like the keys and values of this configuration); the same step with
-        # float32 queries is reported beside it
-        q32 = torch.randn(B, 32, 128, device=dev, generator=gen)
-        q = q32.half()
-        state = {"i": 0, "q": q}
-
-        def step():
-            k_enc, v_enc = sets[state["i"] % 3]
-            tri.decode_step(state["q"], k_enc, v_enc)
-            state["i"] += 1
-
-        algo_bytes = B * S * 8 * 52
-        ms = timed(torch, step, args.steps, args.warmup)
-        kms = kernel_ms(torch, L, step, max(20, args.steps))
-        state["q"] = q32
-        kms32 = kernel_ms(torch, L, step, max(20, args.steps))
-        state["q"] = q
-        out.update(metric="TriAttention decode_step GB/s", value=algo_bytes / ms / 1e6, ms_per_step=ms,
-                   dtype="f32 scores and softmax, fp16 hi/lo MFMA operands for the value sums",
-                   config={"workload": "config 4: TriAttention decode_step, F=12 int4, 32Q/8KV d=128, batch 8 x 32768, "
-                                       "fp16 queries, seed 4",
-                           "algorithmic_bytes_per_step": algo_bytes, "cache_copies_alternated": 3,
-                           "preconditioning_s": PRECONDITION_S, "kernel_ms_float32_queries": kms32})
-        achieved = algo_bytes / kms / 1e6
-        out["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic("tri"),
-                           "kernel": "tri_decode_heads_kernel<4>",
-                           "kernel_ms": kms}
-        if cpu:
-            from oracle import tq_oracle as O
-            k_enc, v_enc = sets[0]
-            S_s = 2048
-            ke = tuple(t[:1, :S_s].cpu().numpy() for t in k_enc)
-            ve = tuple(t[:1, :S_s].cpu().numpy() for t in v_enc)
-            th = tri._theta.cpu().numpy()
-            t0 = time.perf_counter()
-            reps = 0
-            while time.perf_counter() - t0 < args.cpu_seconds or reps < 1:
-                O.tri_decode_step(q[:1].cpu().numpy(), ke, ve, th)
-                reps += 1
-            dt = (time.perf_counter() - t0) / reps
-            cpu_obj = {"value": S_s * 8 * 52 / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-                       "sample": f"numpy oracle of decode_step on batch element 0, first {S_s} tokens"}
+        res, roof, cpu_obj = run_tri(torch, L, dev, args.steps, args.warmup, cpu, args.cpu_seconds, cores)
+        out.update(res)
+        out["roofline"] = roof
     else:  # encode as the measured step
         n = enc["vectors"]
         out.update(metric="tq-t4nc encode GB/s", value=n * 324 / (n / enc["mvec_s"] / 1e3) / 1e6,
@@ -516,12 +573,27 @@ def main():
                    config={"workload": "TurboQuant.encode of 2**20 fp16 vectors x 128 (324 B per vector)",
                            "preconditioning_s": PRECONDITION_S})
         out["roofline"] = {"bound": "hbm", "achieved": enc["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": enc["kernel_frac_hbm"], "traffic": measured_traffic("encode"), "kernel": "encode kernel"}
+                           "frac": enc["kernel_frac_hbm"], **traffic_fields("encode"), "kernel": "encode kernel"}
         if cpu:
             cpu_obj = {"value": enc.get("cpu_mvec_s", 0) * 324 / 1e3, "unit": "GB/s", "cores": cores, "kind": "port",
                        "sample": "numpy oracle encode of 65,536 vectors (config 0)"}
     out["cpu_baseline"] = cpu_obj
     out["encode"] = enc
+    if args.workload == "decode4" and not args.no_secondary:
+        # the other benchmark configurations, same method (two or three cache copies alternated, sustained
+        # clocks, kernel time from dispatch time stamps), no CPU leg
+        sec = {}
+        for wl in ("decode3", "decode2", "tq35"):
+            r, roof, _ = run_decode(torch, akv, L, dev, wl, tq4, args.steps, args.warmup, False, 0.0, cores)
+            sec[wl] = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "step_gbs": r["value"],
+                       "kernel_ms": roof["kernel_ms"], "algorithmic_bytes_per_launch": roof["algorithmic_bytes_per_launch"],
+                       "frac": roof["frac"], "traffic": roof["traffic"], "traffic_source": roof["traffic_source"]}
+        r, roof, _ = run_tri(torch, L, dev, args.steps, args.warmup, False, 0.0, cores)
+        sec["tri"] = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "step_gbs": r["value"],
+                      "kernel_ms": roof["kernel_ms"], "kernel_ms_float32_queries": r["config"]["kernel_ms_float32_queries"],
+                      "algorithmic_bytes_per_launch": roof["algorithmic_bytes_per_launch"], "frac": roof["frac"],
+                      "traffic": roof["traffic"], "traffic_source": roof["traffic_source"]}
+        out["secondary"] = sec
     if not args.no_sweep:
         out["hbm_reference"] = hbm_reference(torch, dev, L)
     print(json.dumps(out))

@@ -190,6 +190,50 @@ def boundary_ulp_distance(y64, boundaries, floor=None):
     return np.min(d, axis=-1) / ulp
 
 
+def code_mismatch_report(codes_a, codes_b, y64, boundaries, unit64=None, R=None):
+    """Where two code arrays differ, how far (in float32 ulps) the float64 rotated value is from
+    the nearest decision boundary.  With the unit vectors and the matrix given, the ulp is not taken
+    below that of the largest term R[j, i] * u[i] of the coordinate's dot product (cancellation).
+    Returns (count, max_ulps, histogram dict)."""
+    diff = np.argwhere(codes_a != codes_b)
+    if len(diff) == 0:
+        return 0, 0.0, {}
+    rows, cols = diff.T
+    floor = None
+    if unit64 is not None and R is not None:
+        floor = np.max(np.abs(np.asarray(R, dtype=np.float64)[cols] * unit64[rows]), axis=-1)
+    ulps = boundary_ulp_distance(y64[rows, cols], boundaries, floor)
+    steps = np.abs(codes_a.astype(np.int64) - codes_b.astype(np.int64))[tuple(diff.T)]
+    hist = {"<=1": int((ulps <= 1).sum()), "<=4": int(((ulps > 1) & (ulps <= 4)).sum()),
+            "<=16": int(((ulps > 4) & (ulps <= 16)).sum()), ">16": int((ulps > 16).sum()),
+            "max_code_step": int(steps.max())}
+    return len(diff), float(ulps.max()), hist
+
+
+def encode_parity_report(packed, norms, x, rotation, bits):
+    """Codes and norms of some encoder against encode() of this file on the same vectors: how many codes
+    differ, the histogram of the distances (float32 ulps) of their float64 rotated values from the
+    decision boundary, and the largest relative difference of the norms."""
+    d = rotation.shape[0]
+    _, b, _ = get_codebook(d, bits)
+    ref_packed, ref_norms = encode(x, rotation, b, bits)
+    ca = _UNPACK[bits](np.asarray(packed).reshape(-1, packed.shape[-1]), d)
+    cb = _UNPACK[bits](ref_packed.reshape(-1, ref_packed.shape[-1]), d)
+    x64 = np.asarray(x).reshape(-1, d).astype(np.float64)
+    y64 = rotate_unit_f64(np.asarray(x).reshape(-1, d), rotation)
+    with np.errstate(invalid="ignore", over="ignore"):
+        unit64 = x64 / (np.linalg.norm(x64, axis=-1, keepdims=True) + 1e-10)
+    n, max_ulps, hist = code_mismatch_report(ca, cb, y64, b, unit64, rotation)
+    nr = np.asarray(ref_norms).reshape(-1).astype(np.float64)
+    ng = np.asarray(norms).reshape(-1).astype(np.float64)
+    nz = nr > 0
+    rel = float(np.max(np.abs(ng[nz] - nr[nz]) / nr[nz])) if nz.any() else 0.0
+    full = {"<=1": 0, "<=4": 0, "<=16": 0, ">16": 0}
+    full.update({k: v for k, v in hist.items() if k in full})
+    return {"codes": int(ca.size), "mismatching": int(n), "max_ulps_from_boundary": max_ulps,
+            "ulp_histogram": full, "max_code_step": int(hist.get("max_code_step", 0)), "norm_max_rel_diff": rel}
+
+
 def encode(x, rotation, boundaries, bits) -> Tuple[np.ndarray, np.ndarray]:
     """TurboQuant.encode, quantizer.py:122-166 (torch path :203-207)."""
     x = np.asarray(x)

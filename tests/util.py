@@ -15,23 +15,8 @@ def kv_like(rng, shape, dtype=np.float16):
 
 
 def code_mismatch_report(codes_a, codes_b, y64, boundaries, oracle, unit64=None, R=None):
-    """Where two code arrays differ, how far (in float32 ulps) the float64 rotated value is from
-    the nearest decision boundary.  With the unit vectors and the matrix given, the ulp is not taken
-    below that of the largest term R[j, i] * u[i] of the coordinate's dot product (cancellation).
-    Returns (count, max_ulps, histogram dict)."""
-    diff = np.argwhere(codes_a != codes_b)
-    if len(diff) == 0:
-        return 0, 0.0, {}
-    rows, cols = diff.T
-    floor = None
-    if unit64 is not None and R is not None:
-        floor = np.max(np.abs(np.asarray(R, dtype=np.float64)[cols] * unit64[rows]), axis=-1)
-    ulps = oracle.boundary_ulp_distance(y64[rows, cols], boundaries, floor)
-    steps = np.abs(codes_a.astype(np.int64) - codes_b.astype(np.int64))[tuple(diff.T)]
-    hist = {"<=1": int((ulps <= 1).sum()), "<=4": int(((ulps > 1) & (ulps <= 4)).sum()),
-            "<=16": int(((ulps > 4) & (ulps <= 16)).sum()), ">16": int((ulps > 16).sum()),
-            "max_code_step": int(steps.max())}
-    return len(diff), float(ulps.max()), hist
+    """The oracle's account of differing codes (count, max_ulps, histogram dict)."""
+    return oracle.code_mismatch_report(codes_a, codes_b, y64, boundaries, unit64, R)
 
 
 def check_codes(packed, norms, x, R, bits, ref_packed=None, ref_norms=None, d=128):
