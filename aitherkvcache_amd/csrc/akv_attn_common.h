@@ -55,11 +55,22 @@ static inline size_t akv_align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // status word 0: nonzero when a bounded wait inside the main kernel of the most recent call gave up
 // (cleared by the prologue, set with a plain vector store, turned into NaN outputs by the reduce)
 #define AKV_STATUS_HANDOFF_TIMEOUT 1u
+// record of a workgroup (int32 words): its range [g0, g1) of the global block axis; then its first segment: the
+// sequence (-1: not recorded, the kernel searches the prefix), the sequence's first and one-past-last global
+// block, its context length in tokens (clamped to the table width)
+#define AKV_WGREC 8
+#define AKV_WGREC_G0 0
+#define AKV_WGREC_G1 1
+#define AKV_WGREC_SEQ 2
+#define AKV_WGREC_SB0 3
+#define AKV_WGREC_SB1 4
+#define AKV_WGREC_CTX 5
 struct akv_attn_ws {
   uint32_t* lut;     // AKV_WS_LUT_BYTES of cached tables (matrix-core kernels)
   uint32_t* status;  // AKV_WS_STATUS_BYTES
-  int32_t* wgdesc;   // [G][8] record of every workgroup of the matrix-core kernel: its range [g0, g1) of the global
-                     // block axis (written by that kernel's prologue; see akv_attn_partition)
+  int32_t* wgdesc;   // [G][AKV_WGREC] record of every workgroup of the matrix-core kernel: its range of the global
+                     // block axis and what its first segment starts from (written by that kernel's prologue; see
+                     // akv_attn_partition)
   int32_t* seqw;     // [S][2] first and last workgroup whose range meets the sequence (same prologue)
   int32_t* prefix;   // [S + 1] exclusive prefix of blocks per sequence; prefix[S] = total
   float* qrot;       // [S][QH][acc_floats] transformed queries
@@ -74,7 +85,7 @@ static inline akv_attn_ws akv_attn_ws_layout(void* base, int S, int QH, int acc_
   w.status = (uint32_t*)((char*)base + AKV_WS_LUT_BYTES);
   size_t off = AKV_WS_HEADER_BYTES;
   w.wgdesc = (int32_t*)((char*)base + off);
-  off += akv_align256((size_t)G * 8 * 4);
+  off += akv_align256((size_t)G * AKV_WGREC * 4);
   w.seqw = (int32_t*)((char*)base + off);
   off += akv_align256((size_t)(S > 0 ? S : 1) * 2 * 4);
   w.prefix = (int32_t*)((char*)base + off);
@@ -148,8 +159,8 @@ __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, 
 }
 
 // ----------------------------------------------------------------------------------
-// Partition of the global block axis among the G workgroups of the matrix-core kernel, written by one
-// workgroup of 256 threads after the prefix scan (same workgroup; `prefix` is read back from memory).
+// Block prefix of the batch and partition of the global block axis among the G workgroups of the matrix-core
+// kernel, written by one workgroup of 256 threads.
 //
 // A workgroup whose range crosses a sequence boundary starts twice (query operand, block ids, first rows, a
 // partial chunk at both ends): measured, such workgroups finish 5 us after the others and ARE the tail of
@@ -162,62 +173,108 @@ __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, 
 // workgroup that meets sequence s), which the reduce kernel reads instead of dividing by the range length.
 // `cb` = blocks per chunk of the main kernel (2 for blocks of 16 tokens, 1 for blocks of 32).
 // ----------------------------------------------------------------------------------
-__device__ __forceinline__ void akv_attn_partition(const int32_t* prefix, int S, int G, int cb, int32_t* wgdesc,
-                                                   int32_t* seqw, int32_t* lds /*[>= 136]*/) {
+__device__ __forceinline__ void akv_attn_partition(int32_t* prefix, int S, int G, int cb, int32_t* wgdesc, int32_t* seqw,
+                                                   int32_t* lds /*[>= 257]*/, const void* context_lens, int cl_itype,
+                                                   int block_size, int64_t max_blocks_per_seq) {
   const int tid = threadIdx.x, lane = tid & 63;
-  __threadfence_block();
-  __syncthreads();                      // the prefix written by this workgroup is readable by all of it
-  const int total = prefix[S];
-  int32_t* p_wfirst = lds;              // [65] first workgroup of each sequence; [S] = workgroups in use
-  int32_t* p_pref = lds + 65;           // [65] block prefix
-  int32_t* p_mode = lds + 130;          // [0] 1 = whole workgroups per sequence
-  if (tid < 64) {
-    int aligned = 0;
-    if (S <= 64) {
-      const int b0 = lane < S ? prefix[lane] : total, b1 = lane < S ? prefix[lane + 1] : total;
-      const int c = (b1 - b0 + cb - 1) / cb;                     // chunks of the lane's sequence
-      p_pref[lane] = b0;
-      if (lane == 0) p_pref[64] = total;
-      int sumc = c;
-#pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) sumc += __shfl_xor(sumc, m, 64);
-      const int nz = __popcll(__ballot(c > 0));
-      aligned = (nz >= 1 && nz * 4 <= G) ? 1 : 0;
-      if (aligned) {
-        int lo = (sumc + G - 1) / G, hi = (sumc + (G - nz) - 1) / (G - nz);      // hi is always feasible
-        if (lo < 1) lo = 1;
-        while (lo < hi) {
-          const int mid = (lo + hi) >> 1;
-          int tot = (c + mid - 1) / mid;
-#pragma unroll
-          for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
-          if (tot <= G) hi = mid; else lo = mid + 1;
-        }
-        const int k = (c + lo - 1) / lo;
-        int inc = k;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const int up = __shfl_up(inc, d, 64);
-          if (lane >= d) inc += up;
-        }
-        p_wfirst[lane] = inc - k;
-        if (lane == 63) p_wfirst[64] = inc;
-      }
+  int32_t* p_wfirst = lds;              // [65] first workgroup of each sequence; [64] = workgroups in use
+  int32_t* p_pref = lds + 65;           // [65] block prefix; [64] = total
+  int32_t* p_ctx = lds + 130;           // [64] context length in tokens (clamped to the table width)
+  int32_t* p_mode = lds + 194;          // [0] 1 = whole workgroups per sequence, [1] = total blocks
+  if (S > 64) {
+    // many sequences: the general scan, equal ranges, first segments found by the main kernel itself
+    akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, lds);
+    __threadfence_block();
+    __syncthreads();                    // the prefix written by this workgroup is readable by all of it
+    const int total = prefix[S];
+    const int per = (total + G - 1) / G;
+    for (int w = tid; w < G; w += blockDim.x) {
+      int32_t* rec = wgdesc + (size_t)w * AKV_WGREC;
+      const int g0 = min(total, w * per);
+      rec[AKV_WGREC_G0] = g0;
+      rec[AKV_WGREC_G1] = min(total, g0 + per);
+      rec[AKV_WGREC_SEQ] = -1;
     }
-    if (lane == 0) p_mode[0] = aligned;
+    for (int s = tid; s < S; s += blockDim.x) {
+      const int b0 = prefix[s], b1 = prefix[s + 1];
+      const int w_lo = per > 0 ? b0 / per : 0;
+      seqw[2 * s] = w_lo;
+      seqw[2 * s + 1] = (per > 0 && b1 > b0) ? (b1 - 1) / per : w_lo - 1;
+    }
+    return;
+  }
+  // at most 64 sequences: one wavefront holds the batch, lane = sequence
+  if (tid < 64) {
+    int n = 0, ctx = 0;
+    if (lane < S) {
+      ctx = (int)akv_seq_tokens(context_lens, cl_itype, lane, block_size, max_blocks_per_seq);
+      n = (ctx + block_size - 1) / block_size;
+    }
+    int inc = n;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(inc, d, 64);
+      if (lane >= d) inc += up;
+    }
+    const int total = __shfl(inc, 63, 64);
+    const int b0 = inc - n;
+    if (lane < S) prefix[lane] = b0;
+    if (lane == 0) prefix[S] = total;
+    p_pref[lane] = b0;
+    p_ctx[lane] = ctx;
+    const int c = (n + cb - 1) / cb;                             // chunks of the lane's sequence
+    int sumc = c;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) sumc += __shfl_xor(sumc, m, 64);
+    const int nz = __popcll(__ballot(c > 0));
+    const int aligned = (nz >= 1 && nz * 4 <= G) ? 1 : 0;
+    if (aligned) {
+      int lo = (sumc + G - 1) / G, hi = (sumc + (G - nz) - 1) / (G - nz);      // hi is always feasible
+      if (lo < 1) lo = 1;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        int tot = (c + mid - 1) / mid;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
+        if (tot <= G) hi = mid; else lo = mid + 1;
+      }
+      const int k = (c + lo - 1) / lo;
+      int kinc = k;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(kinc, d, 64);
+        if (lane >= d) kinc += up;
+      }
+      p_wfirst[lane] = kinc - k;
+      if (lane == 63) p_wfirst[64] = kinc;
+      if (lane < S) {
+        seqw[2 * lane] = kinc - k;
+        seqw[2 * lane + 1] = kinc - 1;
+      }
+    } else if (lane < S) {
+      const int per = (total + G - 1) / G;
+      const int w_lo = per > 0 ? b0 / per : 0;
+      seqw[2 * lane] = w_lo;
+      seqw[2 * lane + 1] = (per > 0 && n > 0) ? (b0 + n - 1) / per : w_lo - 1;
+    }
+    if (lane == 0) {
+      p_pref[64] = total;
+      p_mode[0] = aligned;
+      p_mode[1] = total;
+    }
   }
   __syncthreads();
-  const int aligned = p_mode[0];
+  const int aligned = p_mode[0], total = p_mode[1];
   const int per = (total + G - 1) / G;
   for (int w = tid; w < G; w += blockDim.x) {
-    int g0 = 0, g1 = 0;
+    int g0 = 0, g1 = 0, s = -1;
     if (aligned) {
       if (w < p_wfirst[64]) {
         // the last s with p_wfirst[s] <= w (entries are non-decreasing; a sequence without workgroups shares the
         // next one's entry and is passed over; entries of lanes past the batch equal the number in use)
         int cnt = 0;
         for (int i = 0; i < 64; ++i) cnt += (p_wfirst[i] <= w) ? 1 : 0;
-        const int s = cnt - 1;
+        s = cnt - 1;
         const int b0 = p_pref[s], b1 = p_pref[s + 1];
         const int k = p_wfirst[s + 1] - p_wfirst[s];
         const int c = (b1 - b0 + cb - 1) / cb;
@@ -228,22 +285,21 @@ __device__ __forceinline__ void akv_attn_partition(const int32_t* prefix, int S,
     } else {
       g0 = min(total, w * per);
       g1 = min(total, g0 + per);
+      if (g0 < g1) {
+        int cnt = 0;
+        for (int i = 0; i < 64; ++i) cnt += (i < S && p_pref[i] <= g0) ? 1 : 0;
+        s = cnt - 1;      // the last sequence that starts at or before g0 (an empty one shares its successor's start)
+      }
     }
-    wgdesc[w * 8] = g0;
-    wgdesc[w * 8 + 1] = g1;
-  }
-  for (int s = tid; s < S; s += blockDim.x) {
-    int w_lo, w_hi;
-    if (aligned) {
-      w_lo = p_wfirst[s];
-      w_hi = p_wfirst[s + 1] - 1;
-    } else {
-      const int b0 = prefix[s], b1 = prefix[s + 1];
-      w_lo = per > 0 ? b0 / per : 0;
-      w_hi = (per > 0 && b1 > b0) ? (b1 - 1) / per : w_lo - 1;
+    int32_t* rec = wgdesc + (size_t)w * AKV_WGREC;
+    rec[AKV_WGREC_G0] = g0;
+    rec[AKV_WGREC_G1] = g1;
+    rec[AKV_WGREC_SEQ] = g0 < g1 ? s : -1;
+    if (g0 < g1) {
+      rec[AKV_WGREC_SB0] = p_pref[s];
+      rec[AKV_WGREC_SB1] = p_pref[s + 1];
+      rec[AKV_WGREC_CTX] = p_ctx[s];
     }
-    seqw[2 * s] = w_lo;
-    seqw[2 * s + 1] = w_hi;
   }
 }
 

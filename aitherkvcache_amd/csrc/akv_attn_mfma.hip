@@ -89,7 +89,7 @@ static_assert(MF_W_WORDS * 4 <= AKV_WS_LUT_BYTES, "table block must fit the work
 struct akv_mfma_extra {
   const uint32_t* lut;   // table block, MF_W_* (workspace header)
   const uint4* qop;      // [S][KVH][8 k-steps][64 lanes] half8 as uint4 (workspace)
-  const int32_t* wgdesc; // [G][8]: range [g0, g1) of the global block axis of every workgroup (workspace)
+  const int32_t* wgdesc; // [G][AKV_WGREC] record of every workgroup (workspace)
   uint32_t* status;      // status words of the call (workspace header)
   int spin_limit;        // polls a hand-off wait makes before it gives up
 };
@@ -116,8 +116,8 @@ __global__ __launch_bounds__(256) void akv_attn_mfma_prologue_kernel(
   const int nq = S * KVH;
   if ((int)blockIdx.x == 0) {
     if (tid == 0) status[0] = 0u;
-    akv_block_prefix_scan(context_lens, cl_itype, S, block_size, max_blocks_per_seq, prefix, scratch);
-    akv_attn_partition(prefix, S, G, block_size == 32 ? 1 : 2, wgdesc, seqw, scratch);
+    akv_attn_partition(prefix, S, G, block_size == 32 ? 1 : 2, wgdesc, seqw, scratch, context_lens, cl_itype, block_size,
+                       max_blocks_per_seq);
     return;
   }
   if ((int)blockIdx.x == 1) {
@@ -403,11 +403,19 @@ struct mf_vraw {       // value wavefront
                        // tokens 4g + i (low half) and 4g + i + 2 (high half) of tile j, two bytes each
 };
 
+// What a wavefront starts from: the workgroup's record and the first window of block ids of its first segment
+// (lane i: block blk_lo + i of the segment, clamped to the segment's last), fetched at the kernel's entry
+struct mf_start {
+  int g0, g1;              // the workgroup's range of the global block axis
+  int s, sb0, sb1, ctx;    // first segment: sequence (-1: search the prefix), its first and one-past-last global block, its tokens
+  int pbwin;
+};
+
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
 // separate instantiations entered through one uniform branch, so that neither keeps the other's
 // loop-invariant registers alive.
 template <int ROLE, int BITS>
-__device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs) {
+__device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs, const mf_start& st) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
   // One workgroup barrier per chunk orders everything: in interval k the score wavefronts produce the
@@ -443,16 +451,30 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   const int held = akv_prefix_hold(a.prefix, a.S);
   // the workgroup's range of the global block axis, as the prologue cut it (whole workgroups per sequence
   // when the batch has few sequences, equal ranges otherwise)
-  const int g0 = x.wgdesc[8 * blockIdx.x], g1 = x.wgdesc[8 * blockIdx.x + 1];
+  const int g0 = st.g0, g1 = st.g1;
+  // the window of block ids: lane i of pbwin holds the physical id of block (2 * win_c0 + i) of the segment
+  // (win_c0 + i for blocks of 32).  `fresh`: it holds window 0 of the first segment, from the kernel's entry.
+  int pbwin = st.pbwin, win_c0 = 0;
+  bool fresh = st.s >= 0;
   const int gqa = a.QH / a.KVH;
 
   int gcur = g0;
   while (gcur < g1) {
-    int sb0, sb1;
-    const int s = akv_find_seq_held(a.prefix, a.S, held, gcur, sb0, sb1);
+    // the first segment starts from the workgroup's record (scalar loads that the kernel's entry has already
+    // brought in), later ones -- a range that crosses into the next sequence -- search the held prefix
+    int s, sb0, sb1;
+    int64_t ctx;
+    if (gcur == g0 && st.s >= 0) {
+      s = st.s;
+      sb0 = st.sb0;
+      sb1 = st.sb1;
+      ctx = st.ctx;
+    } else {
+      s = akv_find_seq_held(a.prefix, a.S, held, gcur, sb0, sb1);
+      ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
+    }
     const int blk_lo = gcur - sb0;
     const int blk_hi = min(g1, sb1) - sb0;
-    const int64_t ctx = akv_seq_tokens(a.context_lens, a.cl_itype, s, bs, a.max_blocks_per_seq);
     const int t_end = (int)min((int64_t)blk_hi * bs, ctx);
     gcur = sb0 + blk_hi;
     const int nblk = blk_hi - blk_lo;
@@ -479,7 +501,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       // A window of 64 ids serves MF_WIN chunks plus the two-chunk lookahead of the prefetch.  Its
       // reload drains every outstanding load (once per MF_WIN chunks); the chunk loop itself issues
       // the same loads on every path, so its waits stay counted waits for the chunk that is due.
-      int pbwin = 0, win_c0 = 0;
       auto load_window = [&](int c0) {
         const int bi = min(blk_lo + (bs32 ? c0 : 2 * c0) + lane, blk_hi - 1);
         pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + bi), a.num_blocks);
@@ -493,7 +514,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         p0 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w0);
         p1 = (uint32_t)__builtin_amdgcn_readlane(pbwin, w1);
       };
-      load_window(0);
+      if (!fresh) load_window(0);
+      fresh = false;
 
       if constexpr (ROLE == 0) {
         // =========================== score wavefront ===========================
@@ -877,6 +899,25 @@ template <int BITS>
 __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
+  // ---- the workgroup's record (scalar loads) and, from it, the first window of 64 block ids of its first
+  // segment: both requested here, ahead of the table fill, so that the two dependent trips to memory that every
+  // wavefront would otherwise start with after the fill run beside it
+  mf_start st;
+  {
+    const int32_t* rec = x.wgdesc + (size_t)blockIdx.x * AKV_WGREC;
+    st.g0 = rec[AKV_WGREC_G0];
+    st.g1 = rec[AKV_WGREC_G1];
+    st.s = rec[AKV_WGREC_SEQ];
+    st.sb0 = rec[AKV_WGREC_SB0];
+    st.sb1 = rec[AKV_WGREC_SB1];
+    st.ctx = rec[AKV_WGREC_CTX];
+    st.pbwin = 0;
+    if (st.g0 < st.g1 && st.s >= 0) {
+      const int blk_lo = st.g0 - st.sb0, blk_hi = min(st.g1, st.sb1) - st.sb0;
+      const int bi = min(blk_lo + (int)(threadIdx.x & 63), blk_hi - 1);
+      st.pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, st.s * a.bt_stride + bi), a.num_blocks);
+    }
+  }
   // ---- tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) reads the entry's three words once
   // and writes 8 of its 32 copies with 16-byte stores
   // The words of the workspace block are pairs indexed by two nibbles (first code << 4 | second code).
@@ -914,8 +955,8 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
     }
   }
   __syncthreads();
-  if ((wave >> 3) == 0) mf_role_main<0, BITS>(a, x, wave & 7);
-  else mf_role_main<1, BITS>(a, x, wave & 7);
+  if ((wave >> 3) == 0) mf_role_main<0, BITS>(a, x, wave & 7, st);
+  else mf_role_main<1, BITS>(a, x, wave & 7, st);
 }
 
 // ----------------------------------------------------------------------------------
