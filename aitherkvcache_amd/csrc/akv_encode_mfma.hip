@@ -145,8 +145,10 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = lane & 15, g = lane >> 4;
 
-  // ---- workgroup set-up: B operand, boundaries, cell table
-  {
+  // ---- workgroup set-up: B operand, boundaries, cell table (called after the wavefront has requested the rows
+  // of its first step, so that their trip to memory runs beside the fill: a call of one serving step is a single
+  // step per wavefront and nothing else)
+  auto setup = [&]() {
     uint4* b_lds = (uint4*)(lds + EM_B_OFF);
     for (int i = threadIdx.x; i < EM_B_BYTES / 16; i += EM_THREADS) b_lds[i] = bop[i];
     float* bnd = (float*)(lds + EM_BND_OFF);
@@ -175,8 +177,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       if (cnt > 1) atomicOr(par, 1u);
     }
     __syncthreads();
-  }
-  const bool linear_search = ((const uint32_t*)(lds + EM_PAR_OFF))[0] != 0;   // uniform
+  };
   const float* bnd = (const float*)(lds + EM_BND_OFF);
 
   unsigned char* wl = lds + EM_WAVE_OFF + wave * EM_WAVE_BYTES;
@@ -198,6 +199,16 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     if constexpr (DIRECT) {
       // contiguous rows whose byte offsets fit 31 bits: every lane forms its rows' addresses itself
       // (scalar base + 32-bit lane offset), no exchange through LDS
+      if ((uint32_t)step * ROWS + ROWS <= (uint32_t)a.n) {      // a whole step (all but the last): nothing to check
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const uint32_t n = (uint32_t)step * ROWS + 16 * mt + (lane & 15);
+          const uint4* p = (const uint4*)((const char*)a.x + (n * (uint32_t)a.xs0 + 32u * g) * (uint32_t)XB);
+#pragma unroll
+          for (int ks = 0; ks < NP; ++ks) R[mt][ks] = p[ks];
+        }
+        return;
+      }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const uint32_t n = (uint32_t)step * ROWS + 16 * mt + (lane & 15);
@@ -240,10 +251,8 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     }
   };
 
-  auto encode_step = [&](auto linear_tag, int64_t step) {
+  auto encode_step = [&](auto linear_tag, int64_t step, uint4 (&R)[MT][NP]) {
     constexpr bool LINEAR = decltype(linear_tag)::value;
-    uint4 R[MT][NP];
-    fetch(R, step);
     em_half8 A[MT][4];          // the operand (16-bit input), or its float16 hi term (float32 input)
     em_half8 Alo[MT][4];        // float32 input: the lo term
     if constexpr (XDT != AKV_F32) {
@@ -404,6 +413,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     }
     // lane l < ROWS finishes vector l = 16 mt + row: transpose-reduce the partial sums over the
     // four lanes of a row
+    bool any_nan;       // some vector of the step holds a NaN or an infinity (the same in every lane)
     {
       const bool g1 = (g & 1) != 0;
       float mine;
@@ -424,6 +434,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       // reference: r is 0 and the scaled products are finite.)
       const bool my_nonfinite = (MT > 1 && g1) ? nonfinite[MT - 1] : nonfinite[0];
       const bool nan_row = XDT == AKV_F16 ? !(nrm < INFINITY) : (my_nonfinite || nrm != nrm);   // (float32 as bfloat16)
+      any_nan = __ballot(nan_row && lane < ROWS) != 0;
       if (lane < ROWS) {
         rinv[lane] = nan_row ? __uint_as_float(0x7fc00000u) : r;
         if constexpr (DIRECT) {
@@ -531,6 +542,28 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
     }
     search_tile(accB);
     // ---- store: lane (col, g) writes group col of rows 4g + i
+    auto put = [&](uint8_t* prow, uint32_t v) {
+      if (BITS == 4) {
+        *(uint32_t*)(prow + 4 * col) = v;
+      } else if (BITS == 3) {
+        prow[3 * col] = (uint8_t)(v >> 16);
+        prow[3 * col + 1] = (uint8_t)(v >> 8);
+        prow[3 * col + 2] = (uint8_t)v;
+      } else {
+        *(uint16_t*)(prow + 2 * col) = (uint16_t)v;
+      }
+    };
+    if (DIRECT && !any_nan && (uint32_t)base + ROWS <= (uint32_t)a.n) {
+      // a whole step of finite vectors (all but a few): the row's address is a scalar (step and row number)
+      // plus the lane's own offset (its row quarter and group), nothing is checked
+      const uint32_t lane_off = (uint32_t)(4 * g) * (uint32_t)a.ps0;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          put(a.packed + (uint64_t)((uint32_t)base + 16 * mt + i) * (uint32_t)a.ps0 + lane_off, packed[mt][i]);
+      return;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -548,23 +581,26 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         }
         uint32_t v = packed[mt][i];
         if (!(rv[mt][i] == rv[mt][i])) v = 0xffffffffu;     // NaN vector: last level everywhere
-        if (BITS == 4) {
-          *(uint32_t*)(prow + 4 * col) = v;
-        } else if (BITS == 3) {
-          prow[3 * col] = (uint8_t)(v >> 16);
-          prow[3 * col + 1] = (uint8_t)(v >> 8);
-          prow[3 * col + 2] = (uint8_t)v;
-        } else {
-          *(uint16_t*)(prow + 2 * col) = (uint16_t)v;
-        }
+        put(prow, v);
       }
   };
 
-  // (two wavefronts share a SIMD: one computes while the other waits for its rows)
+  // the rows of a step are requested at the end of the step before it (the first: before the set-up)
+  const int64_t first = (int64_t)wave * gridDim.x + blockIdx.x;
+  uint4 R[MT][NP];
+  fetch(R, first);
+  setup();
+  const bool linear_search = ((const uint32_t*)(lds + EM_PAR_OFF))[0] != 0;   // uniform
   if (__builtin_expect(!linear_search, 1)) {
-    for (int64_t step = (int64_t)wave * gridDim.x + blockIdx.x; step < steps; step += stride) encode_step(std::false_type{}, step);
+    for (int64_t step = first; step < steps; step += stride) {
+      encode_step(std::false_type{}, step, R);
+      fetch(R, step + stride);
+    }
   } else {
-    for (int64_t step = (int64_t)wave * gridDim.x + blockIdx.x; step < steps; step += stride) encode_step(std::true_type{}, step);
+    for (int64_t step = first; step < steps; step += stride) {
+      encode_step(std::true_type{}, step, R);
+      fetch(R, step + stride);
+    }
   }
 }
 
