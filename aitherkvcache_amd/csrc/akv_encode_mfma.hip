@@ -623,20 +623,30 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   if (((uintptr_t)a.packed | (uintptr_t)a.packed2 | (uintptr_t)a.ps0 | (uintptr_t)a.ps1 | (uintptr_t)a.ps2) & amask) return AKV_ERR_UNSUPPORTED;
   const uint4* bop = (const uint4*)((const float*)rot_prep + (size_t)2 * d * d);
   const int64_t n_total = (paged && a.x2) ? 2 * a.n : a.n;
-  const int rows_per_step = x_dtype == AKV_F32 ? 16 : EM_ROWS;
+  const int cus = akv_cached_cu_count();
+  // A call too small to give every CU a step of 32 vectors (one serving step: 4,096 vectors) runs the form with 16
+  // vectors per wavefront step: twice the workgroups, half the chain of products and searches that its one busy
+  // wavefront per workgroup walks through alone.
+  const bool narrow = paged && x_dtype != AKV_F32 && (n_total + EM_ROWS - 1) / EM_ROWS < cus;
+  const int rows_per_step = (x_dtype == AKV_F32 || narrow) ? 16 : EM_ROWS;
   const int64_t steps = (n_total + rows_per_step - 1) / rows_per_step;
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
-  const int grid = (int)(steps < akv_cached_cu_count() ? steps : akv_cached_cu_count());
-#define EM_LAUNCH(BB, PG, DT, DR)                                                                       \
+  const int grid = (int)(steps < cus ? steps : cus);
+#define EM_LAUNCH_MT(BB, PG, DT, DR, MM)                                                              \
   do {                                                                                               \
     static bool configured = false;                                                                  \
     if (!configured) {                                                                               \
-      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT)>, \
+      AKV_HIP(hipFuncSetAttribute((const void*)akv_encode_mfma_kernel<BB, PG, DT, DR, MM>,            \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, EM_LDS_BYTES));        \
       configured = true;                                                                             \
     }                                                                                                \
-    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT)>), grid, EM_THREADS, EM_LDS_BYTES, stream, a, bop); \
+    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, DR, MM>), grid, EM_THREADS, EM_LDS_BYTES, stream, a, bop); \
+  } while (0)
+#define EM_LAUNCH(BB, PG, DT, DR)                                                                     \
+  do {                                                                                               \
+    if (DT == AKV_F32 || (PG && narrow)) EM_LAUNCH_MT(BB, PG, DT, DR, 1);                             \
+    else EM_LAUNCH_MT(BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT));                                   \
   } while (0)
 #define EM_LAUNCH_DT(BB, PG, DR) do { if (x_dtype == AKV_F16) EM_LAUNCH(BB, PG, AKV_F16, DR); else if (x_dtype == AKV_BF16) EM_LAUNCH(BB, PG, AKV_BF16, DR); else EM_LAUNCH(BB, PG, AKV_F32, DR); } while (0)
   // flat rows whose byte offsets stay below 2^31 take the variant with 32-bit lane offsets
@@ -651,6 +661,7 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   }
 #undef EM_LAUNCH_DT
 #undef EM_LAUNCH
+#undef EM_LAUNCH_MT
   AKV_LAUNCH_CHECK("akv_encode_mfma_kernel");
   return AKV_OK;
 }

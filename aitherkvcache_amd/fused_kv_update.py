@@ -20,6 +20,7 @@ logger = logging.getLogger("aither.turboquant.fused_kv_update")
 
 HAS_HIP = _lib.available()
 HAS_TRITON = HAS_HIP
+_DTYPE_OK = (torch.float16, torch.bfloat16, torch.float32)
 
 __all__ = ["fused_tq4_kv_update", "fused_kv_update", "fused_encode_and_store", "HAS_TRITON", "HAS_HIP"]
 
@@ -109,9 +110,79 @@ def fused_kv_update_pair(key, value, slot_mapping, k_packed, k_norms, v_packed, 
         block_size, max_blocks, _lib.stream_ptr(dev)))
 
 
+class _StorePlan:
+    """What fused_encode_and_store needs for one (cache object, layer) once its tensors have been validated: the
+    per-layer views, their strides and the prepared rotation.  A serving loop calls the function once per layer and
+    step with the same cache; re-deriving views, shapes and strides each time costs more host time than the
+    kernel runs.  A plan is valid while the cache object still holds the same tensors and the same quantizer
+    matrix; the step's own tensors (key, value, slot_mapping) are checked on every call."""
+
+    __slots__ = ("kp_all", "kn_all", "vp_all", "vn_all", "tq", "rot", "rot_version", "views", "prep", "bnd", "fixed",
+                 "tail", "dev", "max_blocks", "block_size")
+
+    def __init__(self, tq_cache, layer_idx):
+        tq = tq_cache.tq
+        self.kp_all, self.kn_all = tq_cache.k_packed, tq_cache.k_norms
+        self.vp_all, self.vn_all = tq_cache.v_packed, tq_cache.v_norms
+        self.tq, self.rot, self.rot_version = tq, tq.rotation, tq.rotation._version
+        kp, kn, vp, vn = (t[layer_idx] for t in (self.kp_all, self.kn_all, self.vp_all, self.vn_all))
+        self.views = (kp, kn, vp, vn)
+        self.dev = _lib.require_gpu(kp, kn, vp, vn, tq.rotation, tq.boundaries_inner)
+        head_dim = tq.head_dim
+        same = (kp.shape == vp.shape and kp.stride() == vp.stride() and kn.shape == vn.shape
+                and kn.stride() == vn.stride() and kp.dtype == torch.uint8 and vp.dtype == torch.uint8
+                and kn.dtype == torch.float32 and vn.dtype == torch.float32 and kp.stride(-1) == 1
+                and kp.shape[-1] >= packed_size(head_dim, tq.bits) and hasattr(tq, "prepared_rotation")
+                and head_dim > 0 and (head_dim & (head_dim - 1)) == 0)
+        self.fixed = None
+        if not same:
+            return
+        self.prep = tq.prepared_rotation()
+        b = tq.boundaries_inner
+        self.bnd = b if (b.dtype == torch.float32 and b.is_contiguous()) else b.float().contiguous()
+        self.block_size = tq_cache.block_size
+        self.max_blocks = tq_cache.max_blocks or kp.shape[0]
+        self.tail = (kp.shape[2], head_dim)
+        self.fixed = (self.prep.ptr, self.bnd.data_ptr(), tq.bits, kp.data_ptr(), vp.data_ptr(), kp.stride(0),
+                      kp.stride(1), kp.stride(2), kn.data_ptr(), vn.data_ptr(), kn.stride(0), kn.stride(1),
+                      kn.stride(2), self.block_size, self.max_blocks)
+
+    def valid_for(self, tq_cache) -> bool:
+        tq = tq_cache.tq
+        return (tq_cache.k_packed is self.kp_all and tq_cache.v_packed is self.vp_all
+                and tq_cache.k_norms is self.kn_all and tq_cache.v_norms is self.vn_all and tq is self.tq
+                and tq.rotation is self.rot and tq.rotation._version == self.rot_version
+                and tq_cache.block_size == self.block_size
+                and (tq_cache.max_blocks or self.views[0].shape[0]) == self.max_blocks)
+
+
 def fused_encode_and_store(tq_cache, layer_idx: int, key, value, slot_mapping) -> None:
     """K and V for one layer into a cache object with attributes tq, k_packed, k_norms,
     v_packed, v_norms, block_size, max_blocks (reference: fused_kv_update.py:412-468)."""
+    plans = tq_cache.__dict__.get("_akv_store_plans") if hasattr(tq_cache, "__dict__") else None
+    if plans is None:
+        plans = {}
+        try:
+            tq_cache._akv_store_plans = plans
+        except AttributeError:
+            pass
+    plan = plans.get(layer_idx)
+    if plan is None or plan.fixed is None or not plan.valid_for(tq_cache):
+        plan = _StorePlan(tq_cache, layer_idx)
+        plans[layer_idx] = plan
+    f = plan.fixed
+    if (f is not None and key.dtype in _DTYPE_OK and value.dtype is key.dtype and key.dim() == 3
+            and key.shape[1:] == plan.tail and value.shape == key.shape and key.stride(2) == 1
+            and key.stride() == value.stride() and key.device == plan.dev and value.device == plan.dev
+            and slot_mapping.device == plan.dev and slot_mapping.is_contiguous()
+            and slot_mapping.shape[0] == key.shape[0]):
+        if key.shape[0] == 0:
+            return
+        _lib.check(_lib.lib().akv_encode_paged_kv(
+            key.data_ptr(), value.data_ptr(), _lib.dtype_code(key), key.shape[0], plan.tail[0], plan.tail[1],
+            key.stride(0), key.stride(1), slot_mapping.data_ptr(), _lib.itype_code(slot_mapping), f[0], f[1], f[2],
+            f[3], f[4], f[5], f[6], f[7], f[8], f[9], f[10], f[11], f[12], f[13], f[14], _lib.stream_ptr(plan.dev)))
+        return
     tq = tq_cache.tq
     prep = tq.prepared_rotation() if hasattr(tq, "prepared_rotation") else None
     fused_kv_update_pair(key, value, slot_mapping, tq_cache.k_packed[layer_idx], tq_cache.k_norms[layer_idx],
