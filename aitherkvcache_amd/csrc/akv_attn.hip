@@ -16,7 +16,7 @@ __global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
     const void* __restrict__ query, int64_t qs_seq, int64_t qs_head, const float* __restrict__ PiT,
     int S, int QH, int D, const void* context_lens, int cl_itype, int block_size,
     int64_t max_blocks_per_seq, int32_t* prefix, float* __restrict__ qrot, uint32_t* __restrict__ status) {
-  __shared__ float q_lds[256];
+  __shared__ float q_lds[512];
   __shared__ int32_t scratch[257];
   const int b = blockIdx.x;
   if (b == S * QH) {
@@ -26,12 +26,12 @@ __global__ __launch_bounds__(256) void akv_attn_prologue_kernel(
   }
   const int s = b / QH, h = b % QH;
   const int tid = threadIdx.x;
-  if (tid < D) q_lds[tid] = akv_elem<QDT>::load(query, s * qs_seq + h * qs_head + tid);
+  for (int t = tid; t < D; t += 256) q_lds[t] = akv_elem<QDT>::load(query, s * qs_seq + h * qs_head + t);
   __syncthreads();
-  if (tid < D) {
+  for (int t = tid; t < D; t += 256) {
     float acc = 0.f;
-    for (int j = 0; j < D; ++j) acc = fmaf(PiT[(size_t)j * D + tid], q_lds[j], acc);
-    qrot[((size_t)s * QH + h) * D + tid] = acc;
+    for (int j = 0; j < D; ++j) acc = fmaf(PiT[(size_t)j * D + t], q_lds[j], acc);
+    qrot[((size_t)s * QH + h) * D + t] = acc;
   }
 }
 
@@ -251,14 +251,15 @@ __global__ __launch_bounds__(256, 3) void akv_attn_reduce_kernel(
 // weights staged in the wavefront's own LDS slice).  The query heads of a kv head are taken
 // GQ at a time (GQ = 4 when the GQA ratio is a multiple of 4, else 1).
 // ----------------------------------------------------------------------------------
-#define AKV_ATTN_WAVES 8
+#define AKV_ATTN_WAVES 8      // wavefronts of a workgroup (4 at head_dim 512, where a wavefront's staging area is four times as large)
+template <int D> constexpr int akv_attn_gen_waves() { return D >= 512 ? 4 : AKV_ATTN_WAVES; }
 
 template <int D, int BITS, int GQ>
 struct akv_attn_gen_cfg {
   static constexpr int ROWDW = D * BITS / 32;
   static constexpr int VROW = ROWDW + 1;  // padded row stride in dwords
   static constexpr size_t wave_floats = 64 * GQ + 64 * VROW;
-  static size_t lds_bytes(int QH) { return ((size_t)QH * D + AKV_ATTN_WAVES * wave_floats + 16) * 4; }
+  static size_t lds_bytes(int QH) { return ((size_t)QH * D + akv_attn_gen_waves<D>() * wave_floats + 16) * 4; }
 };
 
 template <int D, int BITS, int GQ>
@@ -273,7 +274,7 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* p_lds = wave_base + wave * cfg::wave_floats;      // [64][GQ]
   uint32_t* v_lds = (uint32_t*)(p_lds + 64 * GQ);          // [64][VROW]
-  float* cen = wave_base + AKV_ATTN_WAVES * cfg::wave_floats;
+  float* cen = wave_base + akv_attn_gen_waves<D>() * cfg::wave_floats;
 
   if (threadIdx.x < (1 << BITS)) cen[threadIdx.x] = a.centroids[threadIdx.x];
 
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(512) void akv_attn_general_kernel(akv_attn_args a) 
       q_lds[i] = a.qrot[(size_t)s * a.QH * D + i];
     __syncthreads();
 
-    for (int h = wave; h < a.KVH; h += AKV_ATTN_WAVES) {
+    for (int h = wave; h < a.KVH; h += akv_attn_gen_waves<D>()) {
       for (int qg = 0; qg < gqa; qg += GQ) {
         float m[GQ], l[GQ], acc[GQ][DPL];
 #pragma unroll
@@ -438,7 +439,7 @@ static int akv_launch_attn_general_gq(const akv_attn_args& a, int grid, hipStrea
   AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_general_kernel<D, BITS, GQ>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   akv_profile_mark_begin(stream);
-  akv_attn_general_kernel<D, BITS, GQ><<<grid, 512, lds, stream>>>(a);
+  akv_attn_general_kernel<D, BITS, GQ><<<grid, 64 * akv_attn_gen_waves<D>(), lds, stream>>>(a);
   akv_profile_mark_end(stream);
   AKV_LAUNCH_CHECK("akv_attn_general_kernel");
   return AKV_OK;
@@ -488,8 +489,8 @@ static int akv_paged_attn_impl(
   AKV_REQUIRE(akv_valid_itype(bt_itype) && akv_valid_itype(cl_itype), "akv_paged_attn: bad index type");
   AKV_REQUIRE(block_size > 0 && max_blocks_per_seq >= 0, "akv_paged_attn: bad block_size / table width");
   AKV_REQUIRE(bits >= 2 && bits <= 4, "akv_paged_attn: bits=%d not in {2,3,4}", bits);
-  if (!(d == 64 || d == 128 || d == 256))
-    return akv_fail(AKV_ERR_UNSUPPORTED, "akv_paged_attn: head_dim=%d not in {64,128,256}", d);
+  if (!(d == 64 || d == 128 || d == 256 || d == 512))
+    return akv_fail(AKV_ERR_UNSUPPORTED, "akv_paged_attn: head_dim=%d not in {64,128,256,512}", d);
   if (num_seqs == 0) return AKV_OK;
   AKV_REQUIRE(query && out && rot_prep && centroids && context_lens, "akv_paged_attn: null pointer");
   AKV_REQUIRE(max_blocks_per_seq == 0 || (k_packed && k_norms && v_packed && v_norms && block_tables),
@@ -540,12 +541,14 @@ static int akv_paged_attn_impl(
     AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
     AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
     AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+    AKV_CASE(512, 2) AKV_CASE(512, 3) AKV_CASE(512, 4)
 #undef AKV_CASE
   }
   if (rc) return rc;
   if (d == 64) return akv_launch_reduce<64>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
   if (d == 128) return akv_launch_reduce<128>(out_dtype, a, Pi, (const uint4*)((const char*)rot_prep + AKV_PREP_DECODE_OFFSET(128)), Gused, out, os_seq, os_head, ws.status, seqw, stream);
-  return akv_launch_reduce<256>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
+  if (d == 256) return akv_launch_reduce<256>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
+  return akv_launch_reduce<512>(out_dtype, a, Pi, nullptr, Gused, out, os_seq, os_head, ws.status, seqw, stream);
 }
 
 extern "C" int akv_paged_attn(

@@ -136,7 +136,7 @@ extern "C" size_t akv_rotation_prepared_bytes(int d) { return akv_prep_floats(d)
 extern "C" int akv_rotation_prepare(const float* rotation, int d, void* prep, size_t prep_bytes,
                                     void* stream) {
   AKV_REQUIRE(rotation && prep, "akv_rotation_prepare: null pointer");
-  AKV_REQUIRE(d == 64 || d == 128 || d == 256, "akv_rotation_prepare: head_dim %d not in {64,128,256}", d);
+  AKV_REQUIRE(d == 64 || d == 128 || d == 256 || d == 512, "akv_rotation_prepare: head_dim %d not in {64,128,256,512}", d);
   AKV_REQUIRE(prep_bytes >= akv_rotation_prepared_bytes(d), "akv_rotation_prepare: prep buffer too small");
   AKV_REQUIRE(((uintptr_t)prep & 255) == 0, "akv_rotation_prepare: prep must be 256-byte aligned");
   dim3 grid(d / 32, d / 32);
@@ -301,7 +301,7 @@ __device__ __forceinline__ void akv_rotate_tile(const float* __restrict__ m_lds,
 }
 
 template <int D> struct akv_gen_cfg {
-  static constexpr int KT = (D <= 128) ? D : 64;  // matrix rows staged at a time (<= 64 KiB)
+  static constexpr int KT = (D <= 128) ? D : (D == 256 ? 64 : 32);  // matrix rows staged at a time (<= 64 KiB)
   static constexpr size_t mat_floats = (size_t)KT * D;
   static constexpr size_t in_floats = (size_t)AKV_GEN_WAVES * AKV_GEN_VPW * D;
   static constexpr size_t code_bytes = (size_t)AKV_GEN_WAVES * AKV_GEN_VPW * D;
@@ -541,6 +541,7 @@ static int akv_encode_dispatch(int d, int bits, int dt, const akv_gen_args& a, v
   AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
   AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
   AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+  AKV_CASE(512, 2) AKV_CASE(512, 3) AKV_CASE(512, 4)
 #undef AKV_CASE
   return akv_fail(AKV_ERR_UNSUPPORTED, "encode: no kernel for head_dim=%d bits=%d", d, bits);
 }
@@ -550,8 +551,8 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
                         const void* rot_prep, hipStream_t stream);
 
 static int akv_check_codec_args(const char* fn, int d, int bits) {
-  if (!(d == 64 || d == 128 || d == 256))
-    return akv_fail(AKV_ERR_UNSUPPORTED, "%s: head_dim=%d not in {64,128,256}", fn, d);
+  if (!(d == 64 || d == 128 || d == 256 || d == 512))
+    return akv_fail(AKV_ERR_UNSUPPORTED, "%s: head_dim=%d not in {64,128,256,512}", fn, d);
   if (bits < 2 || bits > 4) return akv_fail(AKV_ERR_INVALID, "%s: bits=%d not in {2,3,4}", fn, bits);
   return AKV_OK;
 }
@@ -655,6 +656,7 @@ static int akv_decode_dispatch(int d, int bits, int out_dtype, const akv_gen_arg
   AKV_CASE(64, 2) AKV_CASE(64, 3) AKV_CASE(64, 4)
   AKV_CASE(128, 2) AKV_CASE(128, 3) AKV_CASE(128, 4)
   AKV_CASE(256, 2) AKV_CASE(256, 3) AKV_CASE(256, 4)
+  AKV_CASE(512, 2) AKV_CASE(512, 3) AKV_CASE(512, 4)
 #undef AKV_CASE
   return akv_fail(AKV_ERR_UNSUPPORTED, "decode: no kernel for head_dim=%d bits=%d", d, bits);
 }

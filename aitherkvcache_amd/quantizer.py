@@ -20,7 +20,7 @@ from .codebook import get_codebook, get_theory_bounds
 from .packing import packed_size
 from .rotation import random_orthogonal, randomized_hadamard_matrix
 
-_KERNEL_HEAD_DIMS = (64, 128, 256)
+_KERNEL_HEAD_DIMS = (64, 128, 256, 512)
 
 
 @dataclass

@@ -117,6 +117,49 @@ def test_head_dim_64(golden, dev):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("d", [256, 512])
+def test_wide_heads_codec_and_attention_vs_oracle(dev, bits, d):
+    """head_dim 256 and 512 (the reference's quantizer takes every power of two, quantizer.py:78-81, and its
+    backend lists 512, vllm/backend.py:308-309): flat encode / decode, the paged write and decode attention
+    against the oracle, with the matrix the quantizer itself draws for the dimension."""
+    tq = akv.TurboQuant(head_dim=d, bits=bits, device=str(dev))
+    R = tq.rotation.cpu().numpy()
+    rng = np.random.default_rng(d + bits)
+    x = kv_like(rng, (300, d))
+    packed, norms = tq.encode(torch.from_numpy(x).to(dev))
+    assert packed.shape == (300, d * bits // 8)
+    check_codes(packed.cpu().numpy(), norms.cpu().numpy(), x, R, bits, d=d)
+    c, b, _ = O.get_codebook(d, bits)
+    dec = tq.decode(packed, norms).cpu().numpy().astype(np.float32)
+    ref = O.decode(packed.cpu().numpy(), norms.cpu().numpy(), R, c, bits)
+    assert np.max(np.abs(dec - ref.astype(np.float32))) <= 2e-3 * max(1.0, np.abs(ref).max() / 4)
+    # paged write + decode attention (GQA 4:1, ragged contexts, permuted tables)
+    NB, BS, KVH, QH = 12, 16, 2, 8
+    P = tq._packed_dim
+    keys, vals = kv_like(rng, (NB * BS, KVH, d)), kv_like(rng, (NB * BS, KVH, d))
+    kp = torch.zeros(NB, BS, KVH, P, dtype=torch.uint8, device=dev)
+    vp = torch.zeros_like(kp)
+    kn = torch.zeros(NB, BS, KVH, device=dev)
+    vn = torch.zeros_like(kn)
+    slots = torch.from_numpy(rng.permutation(NB * BS)).to(dev)
+    akv.fused_kv_update(torch.from_numpy(keys).to(dev), slots, kp, kn, tq.rotation, tq.boundaries_inner, bits, BS)
+    akv.fused_kv_update(torch.from_numpy(vals).to(dev), slots, vp, vn, tq.rotation, tq.boundaries_inner, bits, BS)
+    ref_p = np.zeros((NB, BS, KVH, P), np.uint8)
+    ref_n = np.zeros((NB, BS, KVH), np.float32)
+    O.kv_update(keys, slots.cpu().numpy(), ref_p, ref_n, R, b, BS, 0, bits)
+    assert np.mean(kp.cpu().numpy() == ref_p) > 0.9999 and np.allclose(kn.cpu().numpy(), ref_n, rtol=1e-6)
+    ctx = np.array([0, 1, 17, 150, NB * BS], dtype=np.int64)
+    tables = np.stack([rng.permutation(NB) for _ in ctx]).astype(np.int32)
+    q = rng.standard_normal((len(ctx), QH, d)).astype(np.float16)
+    out = akv.TQPagedAttention(tq, QH).forward(torch.from_numpy(q).to(dev), kp, kn, vp, vn,
+                                               torch.from_numpy(tables).to(dev), torch.from_numpy(ctx).to(dev))
+    want = O.paged_attention(q, kp.cpu().numpy(), kn.cpu().numpy(), vp.cpu().numpy(), vn.cpu().numpy(), tables, ctx,
+                             R, c, bits, dtype=np.float64, cast_output=False)
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.all(got[0] == 0) and np.all(np.abs(got - want) <= 2e-3 + 2.0 ** -11 * np.abs(want))
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("n", [1, 31, 33, 4097])
 def test_encode_ragged_sizes_vs_oracle(golden, dev, bits, n):
     tq = make_tq(golden, dev, bits)
