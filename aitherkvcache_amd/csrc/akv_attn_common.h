@@ -164,7 +164,7 @@ __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, 
 //
 // A workgroup whose range crosses a sequence boundary starts twice (query operand, block ids, first rows, a
 // partial chunk at both ends): measured, such workgroups finish 5 us after the others and ARE the tail of
-// the launch.  So when the batch has few sequences (at most 64 in all, the non-empty ones at most G / 4) every
+// the launch.  So when the batch has few sequences (at most 64 in all, the non-empty ones at most G / 8) every
 // sequence gets whole workgroups: the smallest lambda (chunks per workgroup) with sum_s ceil(c_s / lambda) <= G
 // is found by bisection (the sum is non-increasing in lambda), sequence s takes k_s = ceil(c_s / lambda)
 // consecutive workgroups and splits its c_s chunks evenly among them; left-over workgroups get an empty range.
@@ -227,7 +227,7 @@ __device__ __forceinline__ void akv_attn_partition(int32_t* prefix, int S, int G
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) sumc += __shfl_xor(sumc, m, 64);
     const int nz = __popcll(__ballot(c > 0));
-    const int aligned = (nz >= 1 && nz * 4 <= G) ? 1 : 0;
+    const int aligned = (nz >= 1 && nz * 8 <= G) ? 1 : 0;
     if (aligned) {
       int lo = (sumc + G - 1) / G, hi = (sumc + (G - nz) - 1) / (G - nz);      // hi is always feasible
       if (lo < 1) lo = 1;

@@ -656,3 +656,33 @@ def test_value_norms_far_outside_the_float16_range(golden, dev, bits, case):
     print(f"[attn value norms {case}] bits={bits} max|out|={np.abs(ref).max():.3e} max relative diff={rel:.2e}")
     assert rel <= 5e-4
     assert attn.last_call_status() == 0
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+@pytest.mark.parametrize("S,empty_every", [(40, 0), (33, 2), (64, 0), (64, 3), (65, 0), (20, 0), (32, 0), (1, 0)])
+def test_partition_of_the_block_axis_by_batch_shape(golden, dev, bits, S, empty_every):
+    """The three ways the prologue cuts the block axis among the workgroups -- whole workgroups per sequence (few
+    non-empty sequences), equal ranges with the sequences held by one wavefront (up to 64 sequences), equal
+    ranges through the general scan (more) -- with empty sequences in between, sequences of one token and
+    lengths that leave the last workgroup of a sequence a single block: every sequence against the oracle."""
+    tq = make_tq(golden, dev, bits)
+    rng = np.random.default_rng(8800 + 7 * S + bits + empty_every)
+    NB, KVH, QH = 400, 8, 32
+    kp, kn, vp, vn = build_cache(rng, tq, dev, NB, KVH, bits)
+    ctx = rng.integers(1, 2500, size=S).astype(np.int64)
+    ctx[rng.integers(0, S)] = 1
+    ctx[rng.integers(0, S)] = 16 * 33 + 1
+    if empty_every:
+        ctx[::empty_every] = 0
+    width = int(-(-ctx.max() // 16))
+    tables = np.full((S, width), -9, dtype=np.int32)
+    for s_, c_ in enumerate(ctx):
+        nb = -(-int(c_) // 16)
+        tables[s_, :nb] = rng.integers(0, NB, size=nb)        # blocks may repeat between sequences: only reads
+    q = rng.standard_normal((S, QH, 128)).astype(np.float16)
+    attn = akv.TQPagedAttention(tq, QH)
+    out = attn.forward(t(q, dev), kp, kn, vp, vn, t(tables, dev), t(ctx, dev)).cpu().numpy()
+    refs = oracle_rows_of_batch(q, kp, kn, vp, vn, np.maximum(tables, 0), ctx, golden, bits, range(S))
+    for s_, r_ in refs.items():
+        assert within_tol(out[s_], r_), f"sequence {s_} of {S} (ctx {ctx[s_]})"
+    assert attn.last_call_status() == 0
