@@ -228,7 +228,9 @@ int akv_paged_attn_static(const void* query, int q_dtype, int64_t qs_seq, int64_
  * (0 when there has been none).
  * akv_debug_set_handoff_spin_limit changes the number of polls such a wait makes (negative =
  * the default, 65536); it exists so that a test can exercise the failure path from the host
- * (0 polls: every wait gives up at once, every kernel still runs to its end). */
+ * (0 polls: every wait gives up at once, every kernel still runs to its end).  The akv_debug_* and
+ * akv_profile_* switches are process-global words read at each launch and are not synchronised: set them
+ * from one thread while no call of another thread is being issued. */
 int akv_paged_attn_status(const void* workspace, int* flags, void* stream);
 int akv_debug_set_handoff_spin_limit(int polls);
 
