@@ -160,6 +160,25 @@ __device__ __forceinline__ int64_t akv_load_index(const void* p, int itype, int6
 }
 
 // ----------------------------------------------------------------------------------
+// device: float32 operations that stay rounded one by one.  (The "_rn" helpers of the HIP headers are
+// plain operators, which the compiler is free to fuse into multiply-adds; a product made here carries
+// no permission to be fused, so a sum that takes it sees the rounded product, as in code that runs
+// one tensor operation after the other.)
+// ----------------------------------------------------------------------------------
+__device__ __forceinline__ float akv_mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float akv_add_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a + b;
+}
+__device__ __forceinline__ float akv_sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+
+// ----------------------------------------------------------------------------------
 // device: wavefront (64-lane) reductions; every lane receives the result
 // ----------------------------------------------------------------------------------
 __device__ __forceinline__ float akv_wave_sum(float v) {

@@ -38,15 +38,15 @@ __device__ __forceinline__ void hyb_encode_group(float xv, int lane, const float
                                                  const float* cen, const float* bnd,
                                                  uint8_t* codes, uint8_t* signs, uint8_t* row,
                                                  int row_off) {
-  const float ss = akv_wave_sum(__fmul_rn(xv, xv));
+  const float ss = akv_wave_sum(akv_mul_rn(xv, xv));
   const float nrm = sqrtf(ss);
-  const float unit = __fdiv_rn(xv, __fadd_rn(nrm, 1e-10f));
-  const float rot = __fmul_rn(hyb_fwht64(__fmul_rn(unit, had[lane]), lane), 0.125f);
+  const float unit = __fdiv_rn(xv, akv_add_rn(nrm, 1e-10f));
+  const float rot = akv_mul_rn(hyb_fwht64(akv_mul_rn(unit, had[lane]), lane), 0.125f);
   const uint32_t code = akv_search<MB>(rot, bnd);
-  const float mse_hat = __fmul_rn(__fmul_rn(hyb_fwht64(cen[code], lane), had[lane]), 0.125f);
-  const float res = __fsub_rn(unit, mse_hat);
-  const float rn = sqrtf(akv_wave_sum(__fmul_rn(res, res)));
-  const float proj = __fmul_rn(hyb_fwht64(__fmul_rn(res, qjl[lane]), lane), 0.125f);
+  const float mse_hat = akv_mul_rn(akv_mul_rn(hyb_fwht64(cen[code], lane), had[lane]), 0.125f);
+  const float res = akv_sub_rn(unit, mse_hat);
+  const float rn = sqrtf(akv_wave_sum(akv_mul_rn(res, res)));
+  const float proj = akv_mul_rn(hyb_fwht64(akv_mul_rn(res, qjl[lane]), lane), 0.125f);
   codes[lane] = (uint8_t)code;
   signs[lane] = proj >= 0.f ? 1 : 0;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -107,9 +107,10 @@ __global__ __launch_bounds__(256) void hyb_encode_kernel(hyb_enc_args a) {
 // operation, the order of the butterflies and the order of the sums are those of the kernel above
 // (and of the reference); only the division is a reciprocal with one correction step.
 // ----------------------------------------------------------------------------------
-// (The "_rn" arithmetic helpers of the HIP headers are plain operators, which the compiler may fuse
-// into multiply-adds; the reference rounds every operation.  Where a product that is not exact feeds
-// a sum, it passes through hyb_rounded(), an empty asm statement the optimiser cannot see through.)
+// (The reference rounds every operation: the products come from akv_mul_rn, which the compiler may not
+// fuse into a multiply-add.  Where a product that is not exact feeds a tree of sums it also passes
+// through hyb_rounded(), an empty asm statement the optimiser cannot see through, so the tree is not
+// reassociated around it either.)
 __device__ __forceinline__ float hyb_rounded(float x) {
   asm volatile("" : "+v"(x));
   return x;
@@ -121,8 +122,8 @@ __device__ __forceinline__ void hyb_fwht64_regs(float (&v)[64]) {
     for (int i = 0; i < 64; ++i)
       if ((i & h) == 0) {
         const float lo = v[i], hi = v[i + h];
-        v[i] = __fadd_rn(lo, hi);
-        v[i + h] = __fsub_rn(lo, hi);
+        v[i] = akv_add_rn(lo, hi);
+        v[i + h] = akv_sub_rn(lo, hi);
       }
 }
 // sum in the order of the wavefront reduction (partners 32, 16, ..., 1 apart)
@@ -130,7 +131,7 @@ __device__ __forceinline__ float hyb_tree_sum64(float (&t)[64]) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1)
 #pragma unroll
-    for (int i = 0; i < m; ++i) t[i] = __fadd_rn(t[i], t[i + m]);
+    for (int i = 0; i < m; ++i) t[i] = akv_add_rn(t[i], t[i + m]);
   return t[0];
 }
 __device__ __forceinline__ void hyb_put_byte(uint32_t* words, int k, uint32_t byte) { words[k >> 2] |= byte << (8 * (k & 3)); }
@@ -166,20 +167,20 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
     }
   }
 #pragma unroll
-  for (int j = 0; j < 64; ++j) v[j] = hyb_rounded(__fmul_rn(u[j], u[j]));
+  for (int j = 0; j < 64; ++j) v[j] = hyb_rounded(akv_mul_rn(u[j], u[j]));
   const float nrm = sqrtf(hyb_tree_sum64(v));
-  const float den = __fadd_rn(nrm, 1e-10f);
+  const float den = akv_add_rn(nrm, 1e-10f);
   const float rcp = __frcp_rn(den);
   const bool plain = !(den < INFINITY);
 #pragma unroll
   for (int j = 0; j < 64; ++j) {
     // x / den: reciprocal, then one correction step (the correctly rounded quotient but for rare ties)
-    const float q0 = __fmul_rn(u[j], rcp);
+    const float q0 = akv_mul_rn(u[j], rcp);
     const float e = fmaf(-q0, den, u[j]);
     // (an infinite or NaN norm: x * (1 / den) alone already is what the division gives)
     const float q = plain ? q0 : fmaf(e, rcp, q0);
     u[j] = q;
-    v[j] = __fmul_rn(q, had[j]);
+    v[j] = akv_mul_rn(q, had[j]);
   }
   hyb_fwht64_regs(v);
 #pragma unroll
@@ -191,7 +192,7 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
       uint32_t g24 = 0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const uint32_t c = akv_search<3>(__fmul_rn(v[8 * g + i], 0.125f), bnd);
+        const uint32_t c = akv_search<3>(akv_mul_rn(v[8 * g + i], 0.125f), bnd);
         g24 |= c << (21 - 3 * i);
         v[8 * g + i] = cen[c];
       }
@@ -205,7 +206,7 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
       uint32_t b = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t c = akv_search<2>(__fmul_rn(v[4 * k + i], 0.125f), bnd);
+        const uint32_t c = akv_search<2>(akv_mul_rn(v[4 * k + i], 0.125f), bnd);
         b |= c << (6 - 2 * i);
         v[4 * k + i] = cen[c];
       }
@@ -215,19 +216,19 @@ __device__ __forceinline__ void hyb_encode_group_lane(const void* x, int64_t off
   hyb_fwht64_regs(v);
 #pragma unroll
   for (int j = 0; j < 64; ++j) {
-    const float mse_hat = __fmul_rn(__fmul_rn(v[j], had[j]), 0.125f);
-    u[j] = __fsub_rn(u[j], mse_hat);              // residual
-    v[j] = hyb_rounded(__fmul_rn(u[j], u[j]));
+    const float mse_hat = akv_mul_rn(akv_mul_rn(v[j], had[j]), 0.125f);
+    u[j] = akv_sub_rn(u[j], mse_hat);              // residual
+    v[j] = hyb_rounded(akv_mul_rn(u[j], u[j]));
   }
   const float rn = sqrtf(hyb_tree_sum64(v));
 #pragma unroll
-  for (int j = 0; j < 64; ++j) v[j] = __fmul_rn(u[j], qjl[j]);
+  for (int j = 0; j < 64; ++j) v[j] = akv_mul_rn(u[j], qjl[j]);
   hyb_fwht64_regs(v);
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     uint32_t b = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) b |= (__fmul_rn(v[8 * k + i], 0.125f) >= 0.f ? 1u : 0u) << (7 - i);
+    for (int i = 0; i < 8; ++i) b |= (akv_mul_rn(v[8 * k + i], 0.125f) >= 0.f ? 1u : 0u) << (7 - i);
     hyb_put_byte(words + CW, k, b);
   }
   words[CW + 2] = (uint32_t)__half_as_ushort(__float2half_rn(nrm)) | ((uint32_t)__half_as_ushort(__float2half_rn(rn)) << 16);
@@ -270,13 +271,13 @@ __device__ __forceinline__ float hyb_decode_group(const uint8_t* row, int lane, 
                                                   const float* qjl, const float* cen, float kappa) {
   constexpr int MSE_BYTES = 64 * MB / 8;
   const uint32_t code = akv_stream_code<MB>(lane, [&](int o) { return (uint32_t)row[o]; });
-  const float mse_hat = __fmul_rn(__fmul_rn(hyb_fwht64(cen[code], lane), had[lane]), 0.125f);
+  const float mse_hat = akv_mul_rn(akv_mul_rn(hyb_fwht64(cen[code], lane), had[lane]), 0.125f);
   const uint32_t bit = (row[MSE_BYTES + (lane >> 3)] >> (7 - (lane & 7))) & 1u;
   const float sg = bit ? kappa : -kappa;
-  const float qjl_hat = __fmul_rn(__fmul_rn(hyb_fwht64(sg, lane), qjl[lane]), 0.125f);
+  const float qjl_hat = akv_mul_rn(akv_mul_rn(hyb_fwht64(sg, lane), qjl[lane]), 0.125f);
   const float n = hyb_half_bits_to_float(row[MSE_BYTES + 8] | (row[MSE_BYTES + 9] << 8));
   const float rn = hyb_half_bits_to_float(row[MSE_BYTES + 10] | (row[MSE_BYTES + 11] << 8));
-  return __fmul_rn(__fadd_rn(mse_hat, __fmul_rn(qjl_hat, rn)), n);
+  return akv_mul_rn(akv_add_rn(mse_hat, akv_mul_rn(qjl_hat, rn)), n);
 }
 
 __global__ __launch_bounds__(256) void hyb_decode_kernel(const uint8_t* __restrict__ packed,
@@ -320,9 +321,9 @@ __device__ __forceinline__ void hyb_decode_group_lane(const uint32_t* words, con
   const float rn = hyb_half_bits_to_float(words[CW + 2] >> 16);
 #pragma unroll
   for (int j = 0; j < 64; ++j) {
-    const float mse_hat = __fmul_rn(__fmul_rn(v[j], had[j]), 0.125f);
-    const float qjl_hat = __fmul_rn(__fmul_rn(w[j], qjl[j]), 0.125f);
-    v[j] = __fmul_rn(__fadd_rn(mse_hat, hyb_rounded(__fmul_rn(qjl_hat, rn))), n);
+    const float mse_hat = akv_mul_rn(akv_mul_rn(v[j], had[j]), 0.125f);
+    const float qjl_hat = akv_mul_rn(akv_mul_rn(w[j], qjl[j]), 0.125f);
+    v[j] = akv_mul_rn(akv_add_rn(mse_hat, hyb_rounded(akv_mul_rn(qjl_hat, rn))), n);
   }
   float4* o4 = (float4*)out;
 #pragma unroll

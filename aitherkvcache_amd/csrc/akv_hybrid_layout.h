@@ -25,7 +25,7 @@ __device__ __forceinline__ float hyb_fwht64(float v, int lane) {
 #pragma unroll
   for (int h = 1; h < 64; h <<= 1) {
     const float o = __shfl_xor(v, h, AKV_WAVE);
-    v = (lane & h) ? __fsub_rn(o, v) : __fadd_rn(v, o);
+    v = (lane & h) ? akv_sub_rn(o, v) : akv_add_rn(v, o);
   }
   return v;
 }

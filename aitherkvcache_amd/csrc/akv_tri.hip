@@ -1183,7 +1183,8 @@ template <int XDT>
 __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict__ x, int64_t n, int d, int64_t xs,
                                                          int F, int cbits, uint8_t* __restrict__ indices,
                                                          uint8_t* __restrict__ coeffs, __half* __restrict__ scales) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: the vector index and the search stay scalar
   const int P = d >> 1;
   const bool have = lane < P;
   for (int64_t v = (int64_t)blockIdx.x * 4 + wave; v < n; v += (int64_t)gridDim.x * 4) {
@@ -1192,7 +1193,7 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
       x0 = akv_elem<XDT>::load(x, v * xs + 2 * lane);
       x1 = akv_elem<XDT>::load(x, v * xs + 2 * lane + 1);
     }
-    const float e = __fadd_rn(__fmul_rn(x0, x0), __fmul_rn(x1, x1));
+    const float e = akv_add_rn(akv_mul_rn(x0, x0), akv_mul_rn(x1, x1));
     // non-negative floats and NaNs order like their bit patterns; lanes beyond the last pair sort last
     const uint32_t key = have ? (__float_as_uint(e) & 0x7fffffffu) + 1u : 0u;
     // The F-th largest key by a bitwise search (largest T with at least F keys >= T: one compare and a
@@ -1230,8 +1231,8 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
       ((__half*)coeffs)[(v * F + pos) * 2 + 1] = __float2half_rn(x1);
     } else if (keep) {
       const float half_code = cbits == 8 ? 127.5f : 7.5f, top = cbits == 8 ? 255.f : 15.f;
-      const float c0 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x0, scale), 1.0f), half_code));
-      const float c1 = rintf(__fmul_rn(__fadd_rn(__fdiv_rn(x1, scale), 1.0f), half_code));
+      const float c0 = rintf(akv_mul_rn(akv_add_rn(__fdiv_rn(x0, scale), 1.0f), half_code));
+      const float c1 = rintf(akv_mul_rn(akv_add_rn(__fdiv_rn(x1, scale), 1.0f), half_code));
       // clamp(0, top) then the cast to uint8; a NaN becomes 0 as in torch's float -> uint8 conversion on the CPU
       const uint32_t q0 = c0 != c0 ? 0u : (uint32_t)fminf(fmaxf(c0, 0.f), top);
       const uint32_t q1 = c1 != c1 ? 0u : (uint32_t)fminf(fmaxf(c1, 0.f), top);

@@ -160,6 +160,30 @@ def test_spectral_encode_vs_oracle(dev, dtype, D, F):
     assert e0.indices.shape == (0, F)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_spectral_encode_energies_a_rounding_apart(dev, bits):
+    """float32 pairs on the unit circle: every energy is 1 up to the last places, so which pairs are kept
+    depends on each square and their sum being rounded on its own, as the reference's pow(2).sum(-1) does
+    (a fused multiply-add moves the result by a place and changes the selection)."""
+    D, F, n = 128, 12, 20000
+    rng = np.random.default_rng(77 + bits)
+    ang = rng.uniform(0, 2 * np.pi, (n, D // 2))
+    x = np.stack([np.cos(ang), np.sin(ang)], -1).astype(np.float32).reshape(n, D)
+    x *= np.float32(2.0) ** rng.integers(-3, 4, (n, 1)).astype(np.float32)       # exact scalings of whole rows
+    a, b = x[:, 0::2].astype(np.float64), x[:, 1::2].astype(np.float64)
+    plain = (x[:, 0::2] * x[:, 0::2] + x[:, 1::2] * x[:, 1::2]).astype(np.float32)
+    fused = (a * a + (x[:, 1::2] * x[:, 1::2]).astype(np.float64)).astype(np.float32)
+    assert np.mean(plain != fused) > 0.05                  # the case is present in the data
+    xt = torch.from_numpy(x).to(dev)
+    tri = TriAttention(TriAttentionConfig(head_dim=D, num_freqs=F, coeff_bits=bits, num_kv_heads=1, num_query_heads=1),
+                       device=str(dev))
+    e = tri.encoder.encode(xt)
+    ri, rp, rs = O.spectral_encode(x, F, bits)
+    assert np.array_equal(e.indices.cpu().numpy(), ri)
+    assert np.array_equal(e.packed.cpu().numpy(), rp)
+    assert np.array_equal(e.scales.cpu().numpy(), rs)
+
+
 @pytest.mark.parametrize("KVH,QH,bt_dtype,BS", [(8, 32, torch.int32, 16), (2, 8, torch.int64, 16), (4, 4, torch.int32, 16),
                                                  (8, 32, torch.int64, 32), (1, 4, torch.int32, 8), (16, 16, torch.int32, 16)])
 def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
