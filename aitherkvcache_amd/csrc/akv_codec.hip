@@ -291,10 +291,11 @@ __device__ __forceinline__ void akv_rotate_tile(const float* __restrict__ m_lds,
       const float4 u = *(const float4*)(in_lds + v * D + k0 + k);
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
-        acc[v][i] = fmaf(m[0][i], u.x, acc[v][i]);
-        acc[v][i] = fmaf(m[1][i], u.y, acc[v][i]);
-        acc[v][i] = fmaf(m[2][i], u.z, acc[v][i]);
-        acc[v][i] = fmaf(m[3][i], u.w, acc[v][i]);
+        // four terms are summed on their own and then added: the running sum is rounded once per four terms
+        // instead of four times (at head_dim 256 and 512 a single chain of fused multiply-adds drifted up to
+        // 18 float32 units in the last place of the largest term away from the exact sum)
+        const float quad = fmaf(m[0][i], u.x, fmaf(m[1][i], u.y, fmaf(m[2][i], u.z, m[3][i] * u.w)));
+        acc[v][i] += quad;
       }
     }
   }
