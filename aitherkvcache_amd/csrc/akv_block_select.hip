@@ -94,9 +94,13 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const float* __restrict_
   }
 }
 
-// larger float <-> larger unsigned
+// larger float <-> larger unsigned; the two zeros share a key (they compare equal, so the lower column wins
+// between them like between any equal scores) and a NaN of either sign ranks above everything, +inf included,
+// as torch.topk ranks it
 __device__ __forceinline__ uint32_t bs_key(float v) {
-  const uint32_t u = __float_as_uint(v);
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
+  if (u == 0x80000000u) u = 0u;
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

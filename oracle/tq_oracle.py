@@ -446,8 +446,9 @@ def block_select(scores, block_tables, context_lens, block_size, max_selected, n
                  num_recent_blocks=2):
     """select_blocks, block_selector.py:182-236: sink and recent columns forced in, top-k of the
     rest (k = min(max_selected, table width)), kept in column order, physical ids gathered,
-    zero padding up to max_selected; context = min(ctx, k * block_size).  Among equal scores the
-    lower column wins here (torch.topk leaves that open)."""
+    zero padding up to max_selected; context = min(ctx, k * block_size).  Among equal scores (the
+    two zeros are equal) the lower column wins here (torch.topk leaves that open); a NaN score ranks
+    above everything, +inf included, as torch.topk ranks it."""
     scores = np.asarray(scores, dtype=f32)
     S, B = scores.shape
     ctx = np.asarray(context_lens)
@@ -459,7 +460,10 @@ def block_select(scores, block_tables, context_lens, block_size, max_selected, n
     sel[mandatory] = np.inf
     sel[~valid] = -np.inf
     k = min(max_selected, B)
-    top = np.sort(np.argsort(-sel, axis=1, kind="stable")[:, :k], axis=1)
+    nan = np.isnan(sel)
+    finite_key = np.where(nan, np.inf, sel)
+    order = np.stack([np.lexsort((np.arange(B), -finite_key[s], ~nan[s])) for s in range(S)]) if S else np.zeros((0, B), int)
+    top = np.sort(order[:, :k], axis=1)
     fbt = np.take_along_axis(np.asarray(block_tables), top, axis=1)
     if k < max_selected:
         fbt = np.concatenate([fbt, np.zeros((S, max_selected - k), dtype=fbt.dtype)], axis=1)

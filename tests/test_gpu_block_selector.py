@@ -100,6 +100,28 @@ def test_selector_class_and_large_table(bsel, dev):
         assert np.array_equal(fbt.cpu().numpy(), obt) and np.array_equal(fcl.cpu().numpy(), ocl)
 
 
+def test_selection_with_signed_zeros_and_nan_scores(dev):
+    """Scores quantised to a few levels hold both zeros: they are equal keys (the lower column wins, as between
+    any equal scores); a NaN ranks above everything (torch.topk's order, block_selector.py:205-207)."""
+    rng = np.random.default_rng(11)
+    S, B = 6, 300
+    sc = (np.round(rng.standard_normal((S, B)) * 3) / 3).astype(np.float32)
+    assert np.any(np.signbit(sc) & (sc == 0)) and np.any(~np.signbit(sc) & (sc == 0))
+    sc[rng.random((S, B)) < 0.02] = np.nan
+    sc[0, 5] = -np.nan
+    ctx = np.array([B * 16, B * 16 - 5, 40 * 16, 1, 0, 150 * 16 + 1], dtype=np.int64)
+    table = rng.integers(0, 1 << 20, size=(S, B)).astype(np.int64)
+    nb = (ctx + 15) // 16
+    for ms, sinks, recents in ((30, 2, 2), (7, 0, 0), (100, 3, 1), (B + 4, 1, 1)):
+        fbt, fcl = select_blocks(t(sc, dev), t(table, dev), t(ctx, dev), 16, ms, sinks, recents)
+        obt, ocl = O.block_select(sc, table, ctx, 16, ms, sinks, recents)
+        assert np.array_equal(fcl.cpu().numpy(), ocl)
+        k = min(ms, B)
+        for s in range(S):
+            m = min(k, int(nb[s]))
+            assert np.array_equal(fbt[s, :m].cpu().numpy(), obt[s, :m]), (ms, s)
+
+
 def test_sparse_attention_end_to_end(golden, dev):
     """Encode -> representatives -> selection -> attention equals attention over the selected blocks alone."""
     tq = akv.TurboQuant(head_dim=128, bits=4, device=str(dev))

@@ -199,3 +199,38 @@ def test_block_scores_and_selection_golden(bsel):
     for s in range(3):
         m = min(30, int(nb[s]))
         assert np.array_equal(fbt[s, :m], bsel["cls_fbt"][s, :m])
+
+
+def test_block_select_orders_nan_and_zeros_like_topk():
+    """torch.topk, which the reference's selection is (block_selector.py:205-207), ranks a NaN above everything
+    and treats the two zeros as equal: the oracle's selection on scores with NaNs, +-0 and otherwise distinct
+    values equals topk's wherever topk's answer does not depend on its choice among equal keys."""
+    import torch
+    rng = np.random.default_rng(5)
+    compared = 0
+    for _ in range(300):
+        S, B, bs = 3, int(rng.integers(1, 80)), 16
+        ms, sinks, recents = int(rng.integers(1, B + 3)), int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        sc = (rng.permutation(S * B).reshape(S, B) - S * B // 2).astype(np.float32)      # distinct; one of them is 0
+        sc[rng.random((S, B)) < 0.1] = np.nan
+        sc[sc == 0] = -0.0 if rng.random() < 0.5 else 0.0
+        ctx = rng.integers(0, B * bs + 1, S).astype(np.int64)
+        table = np.tile(np.arange(B), (S, 1)).astype(np.int64)           # ids = columns: the selection can be read off
+        fbt, _ = O.block_select(sc, table, ctx, bs, ms, sinks, recents)
+        t = torch.from_numpy(sc.copy())
+        nb = (torch.from_numpy(ctx) + bs - 1) // bs
+        col = torch.arange(B)[None]
+        valid = col < nb[:, None]
+        t[((col < sinks) | (col >= nb[:, None] - recents)) & valid] = float("inf")
+        t[~valid] = float("-inf")
+        k = min(ms, B)
+        idx = t.topk(k, dim=1, sorted=False)[1].sort(dim=1)[0].numpy()
+        for s in range(S):
+            row = t[s].numpy().astype(np.float64)
+            key = np.where(np.isnan(row), np.inf, np.clip(row, -1e300, 1e300))      # NaN above +inf
+            kth = np.sort(key)[::-1][k - 1]
+            if int(np.sum(key >= kth)) != k:
+                continue                                             # topk chooses among equal keys at the cut
+            assert np.array_equal(np.sort(idx[s]), fbt[s, :k]), (row, idx[s], fbt[s])
+            compared += 1
+    assert compared > 300
