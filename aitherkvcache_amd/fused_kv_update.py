@@ -114,17 +114,20 @@ class _StorePlan:
     """What fused_encode_and_store needs for one (cache object, layer) once its tensors have been validated: the
     per-layer views, their strides and the prepared rotation.  A serving loop calls the function once per layer and
     step with the same cache; re-deriving views, shapes and strides each time costs more host time than the
-    kernel runs.  A plan is valid while the cache object still holds the same tensors and the same quantizer
-    matrix; the step's own tensors (key, value, slot_mapping) are checked on every call."""
+    kernel runs.  A plan is valid while the cache object still holds the same tensors (same objects, same
+    storage) and the same quantizer (matrix, boundaries and bit width, by object and version counter); the
+    step's own tensors (key, value, slot_mapping) are checked on every call."""
 
     __slots__ = ("kp_all", "kn_all", "vp_all", "vn_all", "tq", "rot", "rot_version", "views", "prep", "bnd", "fixed",
-                 "tail", "dev", "max_blocks", "block_size")
+                 "tail", "dev", "max_blocks", "block_size", "b_src", "b_version", "bits", "ptrs")
 
     def __init__(self, tq_cache, layer_idx):
         tq = tq_cache.tq
         self.kp_all, self.kn_all = tq_cache.k_packed, tq_cache.k_norms
         self.vp_all, self.vn_all = tq_cache.v_packed, tq_cache.v_norms
         self.tq, self.rot, self.rot_version = tq, tq.rotation, tq.rotation._version
+        self.b_src, self.b_version, self.bits = tq.boundaries_inner, tq.boundaries_inner._version, tq.bits
+        self.ptrs = (self.kp_all.data_ptr(), self.kn_all.data_ptr(), self.vp_all.data_ptr(), self.vn_all.data_ptr())
         kp, kn, vp, vn = (t[layer_idx] for t in (self.kp_all, self.kn_all, self.vp_all, self.vn_all))
         self.views = (kp, kn, vp, vn)
         self.dev = _lib.require_gpu(kp, kn, vp, vn, tq.rotation, tq.boundaries_inner)
@@ -152,6 +155,10 @@ class _StorePlan:
         return (tq_cache.k_packed is self.kp_all and tq_cache.v_packed is self.vp_all
                 and tq_cache.k_norms is self.kn_all and tq_cache.v_norms is self.vn_all and tq is self.tq
                 and tq.rotation is self.rot and tq.rotation._version == self.rot_version
+                and tq.boundaries_inner is self.b_src and self.b_src._version == self.b_version and tq.bits == self.bits
+                # (a tensor can be given other storage in place: set_, resize_)
+                and (self.kp_all.data_ptr(), self.kn_all.data_ptr(), self.vp_all.data_ptr(),
+                     self.vn_all.data_ptr()) == self.ptrs
                 and tq_cache.block_size == self.block_size
                 and (tq_cache.max_blocks or self.views[0].shape[0]) == self.max_blocks)
 

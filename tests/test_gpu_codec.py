@@ -292,6 +292,60 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+def test_fused_encode_and_store_follows_changes_of_the_cache_object(golden, dev):
+    """The function keeps what it has derived from a cache object per layer; everything that may change
+    behind it -- cache tensors replaced or given other storage in place, the quantizer's matrix or boundaries
+    replaced or rewritten in place, the block limit, the step's dtype / shape / slot dtype -- must be seen on the
+    next call.  Every state is compared with fused_kv_update_pair on the same inputs."""
+    class Cache:
+        pass
+    c = Cache()
+    c.tq = make_tq(golden, dev, 4)
+    c.block_size, c.max_blocks = 16, 6
+    L, NB, H = 2, 6, 2
+    c.k_packed = torch.zeros(L, NB, 16, H, 64, dtype=torch.uint8, device=dev)
+    c.v_packed = torch.zeros_like(c.k_packed)
+    c.k_norms = torch.zeros(L, NB, 16, H, device=dev)
+    c.v_norms = torch.zeros_like(c.k_norms)
+    g = torch.Generator(device=dev).manual_seed(3)
+
+    def step(layer, tokens=9, dtype=torch.float16, slot_dtype=torch.int64):
+        k = torch.randn(tokens, H, 128, device=dev, generator=g).to(dtype)
+        v = torch.randn(tokens, H, 128, device=dev, generator=g).to(dtype)
+        slots = (torch.randperm(NB * 16 + 8, device=dev, generator=g)[:tokens] - 4).to(slot_dtype)
+        akv.fused_encode_and_store(c, layer, k, v, slots)
+        want = [torch.zeros_like(x[layer]) for x in (c.k_packed, c.k_norms, c.v_packed, c.v_norms)]
+        akv.fused_kv_update_pair(k, v, slots, want[0], want[1], want[2], want[3], c.tq.rotation, c.tq.boundaries_inner,
+                                 c.tq.bits, block_size=c.block_size, max_blocks=c.max_blocks)
+        written = want[1] != 0
+        for got, w in zip((c.k_packed, c.k_norms, c.v_packed, c.v_norms), want):
+            assert torch.equal(got[layer][written], w[written])
+        return int(written.sum())
+
+    assert step(0) > 0 and step(1) > 0 and step(0) > 0
+    step(0, dtype=torch.bfloat16)
+    step(0, dtype=torch.float32, slot_dtype=torch.int32)
+    step(1, tokens=1)
+    c.max_blocks = 3                                           # fewer blocks may be written
+    c.k_norms.zero_(); c.v_norms.zero_()
+    step(0, tokens=40)
+    assert torch.all(c.k_norms[0, 3:] == 0)
+    c.max_blocks = 6
+    c.k_packed = torch.zeros_like(c.k_packed)                  # another tensor object
+    c.k_norms = torch.zeros_like(c.k_norms)
+    step(0)
+    c.v_packed.set_(torch.zeros_like(c.v_packed))              # the same object over other storage
+    step(0)
+    c.tq.boundaries_inner.mul_(0.5)                            # rewritten in place
+    step(1)
+    c.tq.boundaries_inner = c.tq.boundaries_inner * 2.0        # replaced
+    step(1)
+    c.tq.rotation = c.tq.rotation.flip(0).contiguous()         # another matrix
+    step(0)
+    c.tq.rotation.copy_(torch.from_numpy(golden["rotation_d128_seed42"]).to(dev))
+    step(0)
+
+
 @pytest.mark.parametrize("bits", [2, 3, 4])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("tokens", [1, 37, 256])
