@@ -119,7 +119,7 @@ class _StorePlan:
     step's own tensors (key, value, slot_mapping) are checked on every call."""
 
     __slots__ = ("kp_all", "kn_all", "vp_all", "vn_all", "tq", "rot", "rot_version", "views", "prep", "bnd", "fixed",
-                 "tail", "dev", "max_blocks", "block_size", "b_src", "b_version", "bits", "ptrs")
+                 "tail", "dev", "max_blocks", "block_size", "b_src", "b_version", "bits", "ptrs", "layer")
 
     def __init__(self, tq_cache, layer_idx):
         tq = tq_cache.tq
@@ -127,9 +127,10 @@ class _StorePlan:
         self.vp_all, self.vn_all = tq_cache.v_packed, tq_cache.v_norms
         self.tq, self.rot, self.rot_version = tq, tq.rotation, tq.rotation._version
         self.b_src, self.b_version, self.bits = tq.boundaries_inner, tq.boundaries_inner._version, tq.bits
-        self.ptrs = (self.kp_all.data_ptr(), self.kn_all.data_ptr(), self.vp_all.data_ptr(), self.vn_all.data_ptr())
         kp, kn, vp, vn = (t[layer_idx] for t in (self.kp_all, self.kn_all, self.vp_all, self.vn_all))
         self.views = (kp, kn, vp, vn)
+        self.layer = layer_idx
+        self.ptrs = self._storage()
         self.dev = _lib.require_gpu(kp, kn, vp, vn, tq.rotation, tq.boundaries_inner)
         head_dim = tq.head_dim
         same = (kp.shape == vp.shape and kp.stride() == vp.stride() and kn.shape == vn.shape
@@ -150,6 +151,18 @@ class _StorePlan:
                       kp.stride(1), kp.stride(2), kn.data_ptr(), vn.data_ptr(), kn.stride(0), kn.stride(1),
                       kn.stride(2), self.block_size, self.max_blocks)
 
+    def _storage(self):
+        """Where the layer's four tensors lie now.  A container that is one tensor per kind is asked for its own
+        address (its per-layer view cannot move without it); a list of per-layer tensors must still hold the
+        very tensor the view was taken from."""
+        out = []
+        for box, view in zip((self.kp_all, self.kn_all, self.vp_all, self.vn_all), self.views):
+            if isinstance(box, torch.Tensor):
+                out.append(box.data_ptr())
+            else:
+                out.append(view.data_ptr() if box[self.layer] is view else -1)
+        return tuple(out)
+
     def valid_for(self, tq_cache) -> bool:
         tq = tq_cache.tq
         return (tq_cache.k_packed is self.kp_all and tq_cache.v_packed is self.vp_all
@@ -157,8 +170,7 @@ class _StorePlan:
                 and tq.rotation is self.rot and tq.rotation._version == self.rot_version
                 and tq.boundaries_inner is self.b_src and self.b_src._version == self.b_version and tq.bits == self.bits
                 # (a tensor can be given other storage in place: set_, resize_)
-                and (self.kp_all.data_ptr(), self.kn_all.data_ptr(), self.vp_all.data_ptr(),
-                     self.vn_all.data_ptr()) == self.ptrs
+                and self._storage() == self.ptrs
                 and tq_cache.block_size == self.block_size
                 and (tq_cache.max_blocks or self.views[0].shape[0]) == self.max_blocks)
 

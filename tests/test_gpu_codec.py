@@ -344,6 +344,12 @@ def test_fused_encode_and_store_follows_changes_of_the_cache_object(golden, dev)
     step(0)
     c.tq.rotation.copy_(torch.from_numpy(golden["rotation_d128_seed42"]).to(dev))
     step(0)
+    c.k_packed = [c.k_packed[i].clone() for i in range(L)]     # a list of per-layer tensors, as the serving cache keeps them
+    c.k_norms = [c.k_norms[i].clone() for i in range(L)]
+    step(0)
+    step(1)
+    c.k_packed[0] = torch.zeros_like(c.k_packed[0])            # one element replaced inside the same list
+    step(0)
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
