@@ -119,7 +119,7 @@ class _StorePlan:
     step's own tensors (key, value, slot_mapping) are checked on every call."""
 
     __slots__ = ("kp_all", "kn_all", "vp_all", "vn_all", "tq", "rot", "rot_version", "views", "prep", "bnd", "fixed",
-                 "tail", "dev", "max_blocks", "block_size", "b_src", "b_version", "bits", "ptrs", "layer")
+                 "tail", "dev", "max_blocks", "block_size", "b_src", "b_version", "bits", "ptrs", "layer", "boxed")
 
     def __init__(self, tq_cache, layer_idx):
         tq = tq_cache.tq
@@ -130,6 +130,7 @@ class _StorePlan:
         kp, kn, vp, vn = (t[layer_idx] for t in (self.kp_all, self.kn_all, self.vp_all, self.vn_all))
         self.views = (kp, kn, vp, vn)
         self.layer = layer_idx
+        self.boxed = all(isinstance(t, torch.Tensor) for t in (self.kp_all, self.kn_all, self.vp_all, self.vn_all))
         self.ptrs = self._storage()
         self.dev = _lib.require_gpu(kp, kn, vp, vn, tq.rotation, tq.boundaries_inner)
         head_dim = tq.head_dim
@@ -152,25 +153,30 @@ class _StorePlan:
                       kn.stride(2), self.block_size, self.max_blocks)
 
     def _storage(self):
-        """Where the layer's four tensors lie now.  A container that is one tensor per kind is asked for its own
-        address (its per-layer view cannot move without it); a list of per-layer tensors must still hold the
-        very tensor the view was taken from."""
+        """Where the layer's four tensors lie now, or None when one of them has been replaced.  A container that is
+        one tensor per kind is asked for its own address (its per-layer view cannot move without it); a list of
+        per-layer tensors must still hold the very tensor the view was taken from."""
+        if self.boxed:
+            return (self.kp_all.data_ptr(), self.kn_all.data_ptr(), self.vp_all.data_ptr(), self.vn_all.data_ptr())
         out = []
         for box, view in zip((self.kp_all, self.kn_all, self.vp_all, self.vn_all), self.views):
             if isinstance(box, torch.Tensor):
                 out.append(box.data_ptr())
+            elif box[self.layer] is view:
+                out.append(view.data_ptr())
             else:
-                out.append(view.data_ptr() if box[self.layer] is view else -1)
+                return None
         return tuple(out)
 
     def valid_for(self, tq_cache) -> bool:
         tq = tq_cache.tq
+        b = self.b_src
         return (tq_cache.k_packed is self.kp_all and tq_cache.v_packed is self.vp_all
                 and tq_cache.k_norms is self.kn_all and tq_cache.v_norms is self.vn_all and tq is self.tq
-                and tq.rotation is self.rot and tq.rotation._version == self.rot_version
-                and tq.boundaries_inner is self.b_src and self.b_src._version == self.b_version and tq.bits == self.bits
-                # (a tensor can be given other storage in place: set_, resize_)
-                and self._storage() == self.ptrs
+                and tq.rotation is self.rot and self.rot._version == self.rot_version
+                and tq.boundaries_inner is b and b._version == self.b_version and tq.bits == self.bits
+                # (a tensor can be given other storage in place: set_, resize_, an assignment to .data)
+                and self.ptrs is not None and self._storage() == self.ptrs
                 and tq_cache.block_size == self.block_size
                 and (tq_cache.max_blocks or self.views[0].shape[0]) == self.max_blocks)
 

@@ -350,6 +350,10 @@ def test_fused_encode_and_store_follows_changes_of_the_cache_object(golden, dev)
     step(1)
     c.k_packed[0] = torch.zeros_like(c.k_packed[0])            # one element replaced inside the same list
     step(0)
+    c.k_norms[1].data = torch.zeros_like(c.k_norms[1])         # an element given other storage
+    step(1)
+    c.v_norms.data = torch.zeros_like(c.v_norms)
+    step(1)
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4])
