@@ -37,6 +37,12 @@ class TurboQuantConfig:
     use_triton: bool = True
 
 
+def _rotation_key(rotation: torch.Tensor):
+    """What tells one matrix from another without reading it: where it lies, how it is laid out there (a
+    transposed view shares address and version with its base) and how often it has been written."""
+    return (rotation.data_ptr(), rotation._version, rotation.stride(), rotation.dtype, str(rotation.device))
+
+
 class PreparedRotation:
     """Device buffer with the layouts of the rotation the kernels read (Pi, Pi^T and the MFMA
     operand tiles), produced by akv_rotation_prepare."""
@@ -56,10 +62,10 @@ class PreparedRotation:
         self.buffer = torch.empty(nbytes, dtype=torch.uint8, device=rotation.device)
         _lib.check(L.akv_rotation_prepare(self.source.data_ptr(), d, self.buffer.data_ptr(), nbytes,
                                           _lib.stream_ptr(rotation.device)))
-        self._key = (rotation.data_ptr(), rotation._version)
+        self._key = _rotation_key(rotation)
 
     def matches(self, rotation: torch.Tensor) -> bool:
-        return self._key == (rotation.data_ptr(), rotation._version)
+        return self._key == _rotation_key(rotation)
 
     @property
     def ptr(self) -> int:
@@ -70,10 +76,10 @@ _PREPARED_CACHE: dict = {}
 
 
 def prepared_rotation_for(rotation: torch.Tensor) -> PreparedRotation:
-    """Prepared form of an arbitrary rotation tensor, cached per storage address and version
+    """Prepared form of an arbitrary rotation tensor, cached per storage address, layout and version
     (used by the entry points that receive `rotation` as an argument, like
     fused_tq4_kv_update)."""
-    key = (rotation.data_ptr(), rotation._version, str(rotation.device))
+    key = _rotation_key(rotation)
     hit = _PREPARED_CACHE.get(key)
     if hit is None:
         if len(_PREPARED_CACHE) > 64:

@@ -292,6 +292,40 @@ def test_fused_encode_and_store(golden, dev):
     assert torch.all(c.k_packed[0] == 0) and int((c.k_norms[1] != 0).sum()) == 8
 
 
+def test_rotation_argument_is_told_apart_by_layout_and_contents(golden, dev):
+    """fused_kv_update keeps the prepared form of the matrix it is handed.  A transposed view shares address and
+    version counter with its base; a matrix rewritten in place keeps its address; a new matrix may be given the
+    address of a freed one: each call must encode with the matrix it was handed."""
+    tq = make_tq(golden, dev, 4)
+    R = golden["rotation_d128_seed42"]
+    rng = np.random.default_rng(12)
+    x = kv_like(rng, (64, 2, 128))
+    slots = torch.arange(64, device=dev)
+    _, bnd, _ = O.get_codebook(128, 4)
+
+    def run(rot):
+        packed = torch.zeros(4, 16, 2, 64, dtype=torch.uint8, device=dev)
+        norms = torch.zeros(4, 16, 2, device=dev)
+        akv.fused_kv_update(torch.from_numpy(x).to(dev), slots, packed, norms, rot, tq.boundaries_inner, 4, 16)
+        ref_p = np.zeros((4, 16, 2, 64), np.uint8)
+        ref_n = np.zeros((4, 16, 2), np.float32)
+        Rh = rot.detach().float().cpu().numpy()
+        O.kv_update(x, slots.cpu().numpy(), ref_p, ref_n, Rh, bnd, 16, 0, 4)
+        assert np.mean(packed.cpu().numpy() == ref_p) > 0.999, "encoded with another matrix"
+
+    rot = torch.from_numpy(R).to(dev)
+    run(rot)
+    run(rot.t())                         # same address, same version, other layout
+    run(rot)
+    rot.copy_(rot.flip(0))               # same address, rewritten
+    run(rot)
+    for seed in range(3):                # fresh matrices that may land on a freed one's address
+        q, _ = np.linalg.qr(np.random.default_rng(seed).standard_normal((128, 128)))
+        fresh = torch.from_numpy(q.astype(np.float32)).to(dev)
+        run(fresh)
+        del fresh
+
+
 def test_fused_encode_and_store_follows_changes_of_the_cache_object(golden, dev):
     """The function keeps what it has derived from a cache object per layer; everything that may change
     behind it -- cache tensors replaced or given other storage in place, the quantizer's matrix or boundaries
