@@ -364,6 +364,38 @@ __device__ __forceinline__ float mf_rows_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// Row shifts that write ONE bank (four neighbouring lanes) of every row of sixteen; the other lanes keep `old`.
+// mf_to_bank<K>: lane 4K + c of a row receives `src` of lane c.
+template <int K>
+__device__ __forceinline__ float mf_to_bank(float old, float src) {
+  static_assert(K >= 1 && K <= 3, "bank 0 holds its own values");
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), 0x110 + 4 * K /*row_shr:4K*/, 0xf, 1 << K, false));
+}
+// mf_dpp_bank<CTRL, K>: lanes of bank K receive `src` through the row operation CTRL, the others keep `old`
+template <int CTRL, int K>
+__device__ __forceinline__ float mf_dpp_bank(float old, float src) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), CTRL, 0xf, 1 << K, false));
+}
+// mf_pair_from_bank<Q>: lanes 0..3 of a row receive `hi` of lanes 4Q + c, lanes 8..11 receive `lo` of lanes 4Q + c,
+// every other lane zero (quad_perm 0,1,2,3 is the shift by nothing)
+template <int Q>
+__device__ __forceinline__ uint32_t mf_pair_from_bank(uint32_t hi, uint32_t lo) {
+  constexpr int hi_ctrl = Q == 0 ? 0xE4 : 0x100 + 4 * Q;                                            // row_shl:4Q
+  constexpr int lo_ctrl = Q == 2 ? 0xE4 : (Q < 2 ? 0x110 + (8 - 4 * Q) : 0x100 + (4 * Q - 8));      // row_shr:8-4Q / row_shl:4Q-8
+  int w = __builtin_amdgcn_update_dpp(0, (int)hi, hi_ctrl, 0xf, 0x1, false);
+  w = __builtin_amdgcn_update_dpp(w, (int)lo, lo_ctrl, 0xf, 0x4, false);
+  return (uint32_t)w;
+}
+// sum / maximum over the four banks of a row (every lane gets the result of the lanes c, c + 4, c + 8, c + 12)
+__device__ __forceinline__ float mf_banks_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124 /*row_ror:4*/, 0xf, 0xf, false)));
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128 /*row_ror:8*/, 0xf, 0xf, false)));
+}
+__device__ __forceinline__ float mf_banks_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124 /*row_ror:4*/, 0xf, 0xf, false));
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128 /*row_ror:8*/, 0xf, 0xf, false));
+}
+
 // Pairwise hand-off between the score and the value wavefront of a head slot (tq35 kernel; the kernel
 // for the uniform formats orders its chunks with workgroup barriers instead): two counters in LDS,
 // `ready` (chunks whose weights are written) and `done` (chunks whose weights have been read), both
@@ -414,7 +446,7 @@ struct mf_start {
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
 // separate instantiations entered through one uniform branch, so that neither keeps the other's
 // loop-invariant registers alive.
-template <int ROLE, int BITS>
+template <int ROLE, int BITS, bool PACK4>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs, const mf_start& st) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
@@ -553,6 +585,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
         const uint32_t nw_addr = XB0 + (32u * (uint32_t)nhead + 10u + (nrm_is_v ? 1u : 0u)) * XS + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = XB0 + (32u * hs + 10u) * XS + (uint32_t)g * 16u;
+        // (packed form: the lane's bank kb = token pair; its two norms are eight of those sixteen bytes)
+        const int kb = (lane >> 2) & 3;
+        const uint32_t nr2_addr = nr_addr + 64u * (uint32_t)(kb >> 1) + 8u * (uint32_t)(kb & 1);
         // what a lane hands over: a key norm as it is, a value norm as log2 |v| clamped below at -60 (a zero
         // vector then weighs 2^-60 of its codes: nothing at any output precision; NaN and negative norms,
         // which only rows outside a context can hold, come out as -60 as well)
@@ -640,6 +675,27 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
             load_chunk(r, c + 2);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (PACK4) {
+              // At most four query heads per kv head: only columns 0..3 (the float16 roundings of the queries) and
+              // 8..11 (their remainders) of a row of sixteen lanes carry sums, eight per lane.  Everything from
+              // here to the weights runs on a PACKED copy instead: lane 4k + c of a row takes the token pair k
+              // (values 2k, 2k + 1 of the eight) of head c -- the first term from lane c, the second from lane
+              // 8 + c, by row shifts that write one bank of four lanes each.  Two sums, two norm products, four
+              // exponentials (a quarter of the rate of ordinary vector instructions) and one float16 split per lane
+              // and chunk in place of eight, eight, sixteen and four.
+#pragma unroll
+              for (int jj = 0; jj < 2; ++jj) {
+                float hi = acc[0][jj];                                              // bank 0: its own values 0, 1
+                hi = mf_dpp_bank<0x114 /*row_shr:4*/, 1>(hi, acc[0][2 + jj]);
+                hi = mf_dpp_bank<0x118 /*row_shr:8*/, 2>(hi, acc[1][jj]);
+                hi = mf_dpp_bank<0x11c /*row_shr:12*/, 3>(hi, acc[1][2 + jj]);
+                float lo = acc[1][jj];                                              // bank 2: its own values 4, 5
+                lo = mf_dpp_bank<0x108 /*row_shl:8*/, 0>(lo, acc[0][jj]);
+                lo = mf_dpp_bank<0x104 /*row_shl:4*/, 1>(lo, acc[0][2 + jj]);
+                lo = mf_dpp_bank<0x114 /*row_shr:4*/, 3>(lo, acc[1][2 + jj]);
+                sv[jj] = hi + lo;
+              }
+            } else {
             // columns c and c + 8 carry the hi and lo part of the same query head; only lanes of
             // columns [0,8) keep a meaningful softmax state (the others see the lo part alone)
 #pragma unroll
@@ -649,6 +705,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
 #pragma unroll
               for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
             }
+            }
           }
           // The value norms arrive as log2 |v| (clamped below at -60, see the hand-over of the norms) and the
           // running maximum is kept over score + log2 |v|: the weight p |v| of a token is then exp2 of a
@@ -656,10 +713,29 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           // value product with the same relative precision for tiny and for huge value vectors.  The
           // denominator sums the plain p = exp2(score - max) in the same frame (at most 2^60 each); the frame
           // cancels between numerator and denominator and travels as `m` of the partial result.
+          float tv[8];
+          if constexpr (PACK4) {
+            // the lane's token pair: key norms and log2 of the value norms, eight bytes each
+            union { mf_u32x2 u; float f[2]; } kn, vn;
+            kn.u = *(mf_lds_cu64*)(uintptr_t)(nr2_addr + XPAR * par);
+            vn.u = *(mf_lds_cu64*)(uintptr_t)(nr2_addr + XPAR * par + XS);
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+              sv[jj] *= kn.f[jj];
+              tv[jj] = sv[jj] + vn.f[jj];
+            }
+            if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
+              // (a row past the context may hold anything, NaN norms included: both sums are overwritten)
+              const int tok0 = blk_lo * bs + 32 * c + 16 * (kb >> 1) + 4 * g + 2 * (kb & 1);
+              const bool tile_ok = (kb >> 1) == 0 || bs32 || 2 * c + 1 < nblk;
+#pragma unroll
+              for (int jj = 0; jj < 2; ++jj)
+                if (!(tile_ok && tok0 + jj < t_end)) { sv[jj] = -INFINITY; tv[jj] = -INFINITY; }
+            }
+          } else {
           union { mf_u32x4 u[2]; float f[8]; } vn;
           vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS);
           vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS + 64u);
-          float tv[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) tv[i] = sv[i] + vn.f[i];
           if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
@@ -674,7 +750,36 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
                 if (!ok) { sv[4 * j + i] = -INFINITY; tv[4 * j + i] = -INFINITY; }
               }
           }
+          }
           // running softmax in the log2 domain (scale * log2 e is folded into the query operand)
+          union { mf_u32x4 u; uint32_t w[4]; } cv;
+          float resc_out;
+          if constexpr (PACK4) {
+            // every lane of a row knows the running maximum of its head c; the sum is kept per lane (its own
+            // pair's share) and added up over the banks when the segment ends
+            float mx = fmaxf(tv[0], tv[1]);
+            mx = mf_rows_max(mf_banks_max(mx));
+            const float m_new = fmaxf(m_run, mx);
+            const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
+            m_run = m_new;
+            const float psum = __builtin_amdgcn_exp2f(sv[0] - m_new) + __builtin_amdgcn_exp2f(sv[1] - m_new);   // 0 for masked tokens
+            const float w0 = __builtin_amdgcn_exp2f(tv[0] - m_new), w1 = __builtin_amdgcn_exp2f(tv[1] - m_new);   // p |v| <= 1
+            l_run = l_run * resc + psum;
+            // the pair as float16 hi + lo (hi = truncated, lo = the exact float32 difference, truncated)
+            auto h2 = __builtin_amdgcn_cvt_pkrtz(w0, w1);
+            auto l2 = __builtin_amdgcn_cvt_pkrtz(w0 - (float)h2[0], w1 - (float)h2[1]);
+            union { decltype(h2) h; uint32_t u; } hb, lb;
+            hb.h = h2;
+            lb.h = l2;
+            // operand dword qq of a lane = token pair q(qq): columns 0..3 take the hi pair from bank q of their row,
+            // columns 8..11 the lo pair; the other columns belong to no query head and hold zeros
+            // (2-bit: the value side's operand takes the tokens as 4g, 4g+1 of both tiles, then 4g+2, 4g+3 of both)
+            cv.w[0] = mf_pair_from_bank<0>(hb.u, lb.u);
+            cv.w[1] = mf_pair_from_bank<BITS == 2 ? 2 : 1>(hb.u, lb.u);
+            cv.w[2] = mf_pair_from_bank<BITS == 2 ? 1 : 2>(hb.u, lb.u);
+            cv.w[3] = mf_pair_from_bank<3>(hb.u, lb.u);
+            resc_out = resc;
+          } else {
           float mx = fmaxf(fmaxf(fmaxf(tv[0], tv[1]), fmaxf(tv[2], tv[3])), fmaxf(fmaxf(tv[4], tv[5]), fmaxf(tv[6], tv[7])));
           mx = mf_rows_max(mx);
           const float m_new = fmaxf(m_run, mx);
@@ -691,7 +796,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           // in float32, then truncated); columns [0,8) keep hi, columns [8,16) take the lo pair of the
           // column eight to their left (one row shift per packed pair)
           // (2-bit: the value side's operand takes the tokens as 4g, 4g+1 of both tiles, then 4g+2, 4g+3 of both)
-          union { mf_u32x4 u; uint32_t w[4]; } cv;
 #pragma unroll
           for (int qq = 0; qq < 4; ++qq) {
             const int q = BITS == 2 ? ((qq & 1) << 1 | (qq >> 1)) : qq;      // the pair of tokens operand dword qq holds
@@ -705,7 +809,8 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           }
           l_run = l_run * resc + psum;
           const float resc_left = mf_from_lo_cols(resc);
-          const float resc_out = col < 8 ? resc : resc_left;
+          resc_out = col < 8 ? resc : resc_left;
+          }
           // the buffer was last read for chunk c - 2, two barriers ago
           *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par) = cv.u;
           *(mf_lds_u32*)(uintptr_t)(rs_addr + XPAR * par) = __float_as_uint(resc_out);
@@ -738,6 +843,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
         float lsum = l_run;
         lsum = mf_rows_sum(lsum);
+        if constexpr (PACK4) lsum = mf_banks_sum(lsum);      // every lane of a row summed its own token pair
         if (active && col < gqa && g == 0) {
           const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
           a.part_ml[slot * 2] = m_run * 0.6931471805599453f;   // back to the natural-log domain
@@ -895,7 +1001,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   }
 }
 
-template <int BITS>
+template <int BITS, bool PACK4>
 __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
@@ -955,8 +1061,8 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
     }
   }
   __syncthreads();
-  if ((wave >> 3) == 0) mf_role_main<0, BITS>(a, x, wave & 7, st);
-  else mf_role_main<1, BITS>(a, x, wave & 7, st);
+  if ((wave >> 3) == 0) mf_role_main<0, BITS, PACK4>(a, x, wave & 7, st);
+  else mf_role_main<1, BITS, PACK4>(a, x, wave & 7, st);
 }
 
 // ----------------------------------------------------------------------------------
@@ -1035,16 +1141,23 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
+  // at most four query heads per kv head (or group): the score wavefronts work on packed scores
+  const bool pack4 = a.QH / a.KVH <= 4;
   static bool configured = false;
   if (!configured) {
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES));
-    AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, MF_LDS_BYTES_2BIT));
+#define MF_CFG(B, P, L) AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<B, P>, hipFuncAttributeMaxDynamicSharedMemorySize, L))
+    MF_CFG(4, false, MF_LDS_BYTES); MF_CFG(4, true, MF_LDS_BYTES);
+    MF_CFG(3, false, MF_LDS_BYTES); MF_CFG(3, true, MF_LDS_BYTES);
+    MF_CFG(2, false, MF_LDS_BYTES_2BIT); MF_CFG(2, true, MF_LDS_BYTES_2BIT);
+#undef MF_CFG
     configured = true;
   }
-  if (bits == 4) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<4>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
-  else if (bits == 3) AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<3>, grid, MF_THREADS, MF_LDS_BYTES, stream, a, x);
-  else AKV_LAUNCH_TIMED(akv_attn_mfma_kernel<2>, grid, MF_THREADS, MF_LDS_BYTES_2BIT, stream, a, x);
+#define MF_RUN(B, L) do { if (pack4) AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, true>), grid, MF_THREADS, L, stream, a, x); \
+                         else AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, false>), grid, MF_THREADS, L, stream, a, x); } while (0)
+  if (bits == 4) MF_RUN(4, MF_LDS_BYTES);
+  else if (bits == 3) MF_RUN(3, MF_LDS_BYTES);
+  else MF_RUN(2, MF_LDS_BYTES_2BIT);
+#undef MF_RUN
   AKV_LAUNCH_CHECK("akv_attn_mfma_kernel");
   return AKV_OK;
 }
