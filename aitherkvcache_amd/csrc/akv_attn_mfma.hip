@@ -1513,71 +1513,63 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
               sv[4 * j + i] = raw + mf_from_hi_cols(raw);
             }
           }
-          // value-side factors of the lane's eight tokens
-          float vn0[8], vr0[8], vn1[8], vr1[8];
+          // From here on the wavefront works on a PACKED copy of the scores: the group has four query heads, so only
+          // columns 0..3 of a row of sixteen lanes hold scores, eight per lane.  Lane 4k + c takes the token pair k
+          // (values 2k, 2k + 1) of head c: two exponentials, eight weight products and four float16 splits per lane
+          // and chunk in place of eight, thirty-two and sixteen; every lane then writes its own pair straight into
+          // the operand fragments of the value side.
+          const int kb = col >> 2, c4 = col & 3;
+          float ps[2];
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            union { mf_u32x4 u; float f[4]; } t0, t1, t2, t3;
-            const uint32_t base = nr_addr + 4096u * par + 512u + 256u * j;
-            t0.u = *(mf_lds_u128*)(uintptr_t)(base);
-            t1.u = *(mf_lds_u128*)(uintptr_t)(base + 64u);
-            t2.u = *(mf_lds_u128*)(uintptr_t)(base + 128u);
-            t3.u = *(mf_lds_u128*)(uintptr_t)(base + 192u);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { vn0[4 * j + i] = t0.f[i]; vr0[4 * j + i] = t1.f[i]; vn1[4 * j + i] = t2.f[i]; vr1[4 * j + i] = t3.f[i]; }
+          for (int jj = 0; jj < 2; ++jj)
+            ps[jj] = mf_to_bank<3>(mf_to_bank<2>(mf_to_bank<1>(sv[jj], sv[2 + jj]), sv[4 + jj]), sv[6 + jj]);
+          // value-side factors of the lane's token pair (tile kb / 2, tokens 4g + 2 (kb % 2) + {0, 1})
+          union { mf_u32x2 u; float f[2]; } vn0, vr0, vn1, vr1;
+          {
+            const uint32_t base = nr_addr + 4096u * par + 512u + 256u * (uint32_t)(kb >> 1) + 8u * (uint32_t)(kb & 1);
+            vn0.u = *(mf_lds_cu64*)(uintptr_t)(base);
+            vr0.u = *(mf_lds_cu64*)(uintptr_t)(base + 64u);
+            vn1.u = *(mf_lds_cu64*)(uintptr_t)(base + 128u);
+            vr1.u = *(mf_lds_cu64*)(uintptr_t)(base + 192u);
           }
           if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens (whose rows may hold anything)
-            const int tok0 = blk_lo * bs + 32 * c;
+            const int tok0 = blk_lo * bs + 32 * c + 16 * (kb >> 1) + 4 * g + 2 * (kb & 1);
+            const bool tile_ok = (kb >> 1) == 0 || bs32 || 2 * c + 1 < nblk;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const int tok = tok0 + 16 * j + 4 * g + i;
-                const bool ok = (tok < t_end) && (j == 0 || bs32 || 2 * c + 1 < nblk);
-                if (!ok) { sv[4 * j + i] = -INFINITY; vn0[4 * j + i] = 0.f; vr0[4 * j + i] = 0.f; vn1[4 * j + i] = 0.f; vr1[4 * j + i] = 0.f; }
-              }
+            for (int jj = 0; jj < 2; ++jj)
+              if (!(tile_ok && tok0 + jj < t_end)) { ps[jj] = -INFINITY; vn0.f[jj] = 0.f; vr0.f[jj] = 0.f; vn1.f[jj] = 0.f; vr1.f[jj] = 0.f; }
           }
-          float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-          mx = mf_rows_max(mx);
+          const float mx = mf_rows_max(mf_banks_max(fmaxf(ps[0], ps[1])));
           const float m_new = fmaxf(m_run, mx);
           const float resc = __builtin_amdgcn_exp2f(m_run - m_new);
           m_run = m_new;
-          float psum = 0.f;
-          float pw[4][8];
+          float pw[4][2];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float p = __builtin_amdgcn_exp2f(sv[i] - m_new);
-            psum += p;
-            pw[0][i] = p * vn0[i];
-            pw[1][i] = pw[0][i] * vr0[i];
-            pw[2][i] = p * vn1[i];
-            pw[3][i] = pw[2][i] * vr1[i];
+          for (int jj = 0; jj < 2; ++jj) {
+            const float p = __builtin_amdgcn_exp2f(ps[jj] - m_new);
+            pw[0][jj] = p * vn0.f[jj];
+            pw[1][jj] = pw[0][jj] * vr0.f[jj];
+            pw[2][jj] = p * vn1.f[jj];
+            pw[3][jj] = pw[2][jj] * vr1.f[jj];
+            ps[jj] = p;
           }
-          l_run = l_run * resc + psum;
+          l_run = l_run * resc + (ps[0] + ps[1]);       // the lane's own pair; summed over the banks when the segment ends
           mf_wait_ge(fl_addr + 4u, c >= 2 ? T + (uint32_t)c - 1u : T, a.status, a.spin_limit);
-          if (col < 4) {
-            // weight operand of pass P (0 = C: sets A0, A1; 1 = S: sets B0, B1): column 4 t + col holds the
-            // fp16 part of set t of query head col, column 8 + 4 t + col its remainder; column k of the
-            // tile is read by lane 16 g + k
+          // weight operand of pass P (0 = C: sets A0, A1; 1 = S: sets B0, B1): column 4 t + c holds the fp16 part of
+          // set t of query head c, column 8 + 4 t + c its remainder; column k of the tile is read by lane 16 g + k,
+          // whose sixteen bytes are the token pairs 0..3: this lane supplies dword kb of each
 #pragma unroll
-            for (int X = 0; X < 4; ++X) {
-              union { mf_u32x4 u; uint32_t w[4]; } hi, lo;
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[X][2 * q], pw[X][2 * q + 1]);
-                auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[X][2 * q] - (float)h2[0], pw[X][2 * q + 1] - (float)h2[1]);
-                union { decltype(h2) h; uint32_t u; } hb, lb;
-                hb.h = h2;
-                lb.h = l2;
-                hi.w[q] = hb.u;
-                lo.w[q] = lb.u;
-              }
-              const uint32_t L = (uint32_t)(16 * g + 4 * (X >> 1) + col);
-              const uint32_t base = ((X & 1) ? wsx(L) + 4096u * par : pbx(L) + MF_XBUF * par);
-              const uint32_t base8 = ((X & 1) ? wsx(L + 8u) + 4096u * par : pbx(L + 8u) + MF_XBUF * par);
-              *(mf_lds_u128*)(uintptr_t)base = hi.u;
-              *(mf_lds_u128*)(uintptr_t)base8 = lo.u;
-            }
+          for (int X = 0; X < 4; ++X) {
+            auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[X][0], pw[X][1]);
+            auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[X][0] - (float)h2[0], pw[X][1] - (float)h2[1]);
+            union { decltype(h2) h; uint32_t u; } hb, lb;
+            hb.h = h2;
+            lb.h = l2;
+            const uint32_t L = (uint32_t)(16 * g + 4 * (X >> 1) + c4);
+            const uint32_t base = ((X & 1) ? wsx(L) + 4096u * par : pbx(L) + MF_XBUF * par) + 4u * (uint32_t)kb;
+            const uint32_t base8 = ((X & 1) ? wsx(L + 8u) + 4096u * par : pbx(L + 8u) + MF_XBUF * par) + 4u * (uint32_t)kb;
+            *(mf_lds_u32*)(uintptr_t)base = hb.u;
+            *(mf_lds_u32*)(uintptr_t)base8 = lb.u;
           }
           *(mf_lds_u32*)(uintptr_t)(rsx((uint32_t)lane) + MF_XBUF * par) = __float_as_uint(resc);
           mf_publish(fl_addr, T + (uint32_t)c + 1u);
@@ -1599,7 +1591,7 @@ __device__ __forceinline__ void hm_role_main(const akv_hyb_mfma_args& a, const i
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);
         T += (uint32_t)nchunks;
         float lsum = l_run;
-        lsum = mf_rows_sum(lsum);
+        lsum = mf_banks_sum(mf_rows_sum(lsum));
         if (col < 4 && g == 0) {
           const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * 4 + col);
           a.part_ml[slot * 2] = m_run * 0.6931471805599453f;
