@@ -441,7 +441,52 @@ struct mf_start {
   int g0, g1;              // the workgroup's range of the global block axis
   int s, sb0, sb1, ctx;    // first segment: sequence (-1: search the prefix), its first and one-past-last global block, its tokens
   int pbwin;
+  uint32_t lutw[6];        // the words of the workspace's table block this thread turns into table entries (mf_fill_tables)
 };
+
+// The byte-pair tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) holds the entry's words (requested at
+// the kernel's entry, before anything else) and writes 8 of its 32 copies with 16-byte stores.  The words of the
+// workspace block are pairs indexed by two nibbles (first code << 4 | second code).
+template <int BITS>
+__device__ __forceinline__ void mf_load_table_words(const uint32_t* __restrict__ lut, uint32_t (&w)[6]) {
+  const int e = threadIdx.x >> 2;
+  if constexpr (BITS == 2) {
+    // entry = one code byte.  K: four coordinates (codes from the top bits down) as (hi pair, lo pair) twice.
+    // V: the same coordinate of four tokens (codes from the bottom bits up).
+    const int k01 = ((e >> 6) << 4) | ((e >> 4) & 3), k23 = (((e >> 2) & 3) << 4) | (e & 3);
+    const int v01 = ((e & 3) << 4) | ((e >> 2) & 3), v23 = (((e >> 4) & 3) << 4) | (e >> 6);
+    w[0] = lut[MF_W_KHI + k01]; w[1] = lut[MF_W_KLO + k01]; w[2] = lut[MF_W_KHI + k23]; w[3] = lut[MF_W_KLO + k23];
+    w[4] = lut[MF_W_VHI + v01]; w[5] = lut[MF_W_VHI + v23];
+  } else {
+    // 4-bit: entry = one code byte (two codes).  3-bit: entry = a 6-bit field, K (first code << 3 | second
+    // code) of one token, V (code of the odd token << 3 | code of the even token) of one coordinate; 64 entries.
+    int ke = e, ve = e;
+    if constexpr (BITS == 3) {
+      ke = (((e >> 3) & 7) << 4) | (e & 7);
+      ve = ((e & 7) << 4) | ((e >> 3) & 7);
+    }
+    w[0] = lut[MF_W_KHI + ke]; w[1] = lut[MF_W_KLO + ke]; w[2] = lut[MF_W_VHI + ve];
+    w[3] = 0u; w[4] = 0u; w[5] = 0u;
+  }
+}
+template <int BITS>
+__device__ __forceinline__ void mf_fill_tables(const uint32_t (&w)[6]) {
+  const int e = threadIdx.x >> 2, qt = threadIdx.x & 3;
+  mf_lds_u128* ka = (mf_lds_u128*)(uintptr_t)(uint32_t)(e * 256 + qt * 64);
+  mf_lds_u128* va = (mf_lds_u128*)(uintptr_t)(uint32_t)(MF_TABB + e * 256 + qt * (BITS == 2 ? 64 : 32));
+  if constexpr (BITS == 2) {
+    // K: 16 copies of 16 bytes (this thread: copies 4qt .. 4qt+3); V: 32 copies of 8 bytes (copies 8qt .. 8qt+7)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ka[i] = (mf_u32x4){w[0], w[1], w[2], w[3]};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) va[i] = (mf_u32x4){w[4], w[5], w[4], w[5]};
+  } else if (BITS == 4 || e < 64) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ka[i] = (mf_u32x4){w[0], w[1], w[0], w[1]};    // K copies 8qt .. 8qt+7 (8 bytes each)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) va[i] = (mf_u32x4){w[2], w[2], w[2], w[2]};    // V copies 8qt .. 8qt+7 (4 bytes each)
+  }
+}
 
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
 // separate instantiations entered through one uniform branch, so that neither keeps the other's
@@ -489,6 +534,17 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   int pbwin = st.pbwin, win_c0 = 0;
   bool fresh = st.s >= 0;
   const int gqa = a.QH / a.KVH;
+  // The tables are written by all wavefronts of the workgroup once, AFTER each has requested what its first chunks
+  // need: the fill (LDS stores from registers and the barrier that publishes them) then runs beside those round
+  // trips to memory instead of in front of them.
+  bool filled = false;
+  auto fill_once = [&]() {
+    if (!filled) {
+      mf_fill_tables<BITS>(st.lutw);
+      mf_barrier();          // (orders LDS traffic only: the rows just requested keep flying)
+      filled = true;
+    }
+  };
 
   int gcur = g0;
   while (gcur < g1) {
@@ -521,6 +577,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
       // for ALL loads, prefetches included, wherever the loop first touches their registers.)
       if (nchunks <= 0) continue;
       if (!active) {
+        fill_once();
         if constexpr (SYNC)
           for (int i = 0; i <= nchunks; ++i) mf_barrier();     // the workgroup's barriers are counted by all
         continue;
@@ -824,6 +881,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_sched_barrier(0);     // queue order = chunk order, as in the loop
         load_chunk(rb, 1);
         __builtin_amdgcn_sched_barrier(0);
+        fill_once();
         *(mf_lds_u32*)(uintptr_t)nw_addr = __float_as_uint(norm_out(ra.nrm));     // norms of chunk 0, ahead of the first barrier
         // pairs of chunks with the same loads on every path (an early exit from the middle of the
         // body would make the compiler wait for the newest prefetch at the top of every iteration)
@@ -972,6 +1030,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
         mf_vraw ra;
         load_chunk(ra, 0);
+        fill_once();
         if constexpr (SYNC) mf_barrier();
         for (int c = 0; c < nchunks; ++c) {
           if (c - win_c0 >= MF_WIN) load_window(c);
@@ -1009,6 +1068,7 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
   // segment: both requested here, ahead of the table fill, so that the two dependent trips to memory that every
   // wavefront would otherwise start with after the fill run beside it
   mf_start st;
+  mf_load_table_words<BITS>(x.lut, st.lutw);      // (first: these loads depend on nothing)
   {
     const int32_t* rec = x.wgdesc + (size_t)blockIdx.x * AKV_WGREC;
     st.g0 = rec[AKV_WGREC_G0];
@@ -1024,43 +1084,6 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
       st.pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, st.s * a.bt_stride + bi), a.num_blocks);
     }
   }
-  // ---- tables (layout at MF_LDS_BYTES): thread (entry e, quarter qt) reads the entry's three words once
-  // and writes 8 of its 32 copies with 16-byte stores
-  // The words of the workspace block are pairs indexed by two nibbles (first code << 4 | second code).
-  {
-    const int e = threadIdx.x >> 2, qt = threadIdx.x & 3;
-    uint4* ka = (uint4*)(lds_raw + e * 256 + qt * 64);
-    uint4* va = (uint4*)(lds_raw + MF_TABB + e * 256 + qt * (BITS == 2 ? 64 : 32));
-    if constexpr (BITS == 2) {
-      // entry = one code byte.  K: four coordinates (codes from the top bits down) as (hi pair, lo pair) twice,
-      // 16 copies of 16 bytes.  V: the same coordinate of four tokens (codes from the bottom bits up), 32
-      // copies of 8 bytes.
-      const int k01 = ((e >> 6) << 4) | ((e >> 4) & 3), k23 = (((e >> 2) & 3) << 4) | (e & 3);
-      const uint4 kq = make_uint4(x.lut[MF_W_KHI + k01], x.lut[MF_W_KLO + k01], x.lut[MF_W_KHI + k23], x.lut[MF_W_KLO + k23]);
-      const int v01 = ((e & 3) << 4) | ((e >> 2) & 3), v23 = (((e >> 4) & 3) << 4) | (e >> 6);
-      const uint32_t va01 = x.lut[MF_W_VHI + v01], va23 = x.lut[MF_W_VHI + v23];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ka[i] = kq;                            // K copies 4qt .. 4qt+3
-#pragma unroll
-      for (int i = 0; i < 4; ++i) va[i] = make_uint4(va01, va23, va01, va23);   // V copies 8qt .. 8qt+7
-    } else {
-      // 4-bit: entry = one code byte (two codes).  3-bit: entry = a 6-bit field, K (first code << 3 | second
-      // code) of one token, V (code of the odd token << 3 | code of the even token) of one coordinate; 64 entries.
-      int ke = e, ve = e;
-      if constexpr (BITS == 3) {
-        ke = (((e >> 3) & 7) << 4) | (e & 7);
-        ve = ((e & 7) << 4) | ((e >> 3) & 7);
-      }
-      const uint32_t khi = x.lut[MF_W_KHI + ke], klo = x.lut[MF_W_KLO + ke], vhi = x.lut[MF_W_VHI + ve];
-      if (BITS == 4 || e < 64) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ka[i] = make_uint4(khi, klo, khi, klo);    // K copies 8qt .. 8qt+7 (8 bytes each)
-#pragma unroll
-        for (int i = 0; i < 2; ++i) va[i] = make_uint4(vhi, vhi, vhi, vhi);    // V copies 8qt .. 8qt+7 (4 bytes each)
-      }
-    }
-  }
-  __syncthreads();
   if ((wave >> 3) == 0) mf_role_main<0, BITS, PACK4>(a, x, wave & 7, st);
   else mf_role_main<1, BITS, PACK4>(a, x, wave & 7, st);
 }
