@@ -371,10 +371,19 @@ __device__ __forceinline__ float mf_to_bank(float old, float src) {
   static_assert(K >= 1 && K <= 3, "bank 0 holds its own values");
   return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), 0x110 + 4 * K /*row_shr:4K*/, 0xf, 1 << K, false));
 }
-// mf_dpp_bank<CTRL, K>: lanes of bank K receive `src` through the row operation CTRL, the others keep `old`
+// mf_dpp_bank<CTRL, K>: lanes of bank K receive `src` through the row operation CTRL, the others keep `old`;
+// mf_dpp_banks<CTRL, MASK>: the same for a set of banks
 template <int CTRL, int K>
 __device__ __forceinline__ float mf_dpp_bank(float old, float src) {
   return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), CTRL, 0xf, 1 << K, false));
+}
+template <int CTRL, int MASK>
+__device__ __forceinline__ float mf_dpp_banks(float old, float src) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), CTRL, 0xf, MASK, false));
+}
+template <int CTRL, int MASK>
+__device__ __forceinline__ uint32_t mf_dpp_banks_u(uint32_t old, uint32_t src) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, MASK, false);
 }
 // mf_pair_from_bank<Q>: lanes 0..3 of a row receive `hi` of lanes 4Q + c, lanes 8..11 receive `lo` of lanes 4Q + c,
 // every other lane zero (quad_perm 0,1,2,3 is the shift by nothing)
@@ -491,7 +500,7 @@ __device__ __forceinline__ void mf_fill_tables(const uint32_t (&w)[6]) {
 // One role of the pipeline (ROLE 0 = score wavefront, 1 = value wavefront).  The two roles are
 // separate instantiations entered through one uniform branch, so that neither keeps the other's
 // loop-invariant registers alive.
-template <int ROLE, int BITS, bool PACK4>
+template <int ROLE, int BITS, int PACK>
 __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_mfma_extra& x, const int hs, const mf_start& st) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15, g = lane >> 4;
@@ -642,9 +651,10 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         const uint32_t ktile1 = bs32 ? 16u * (uint32_t)a.kps_pos : 0u;   // second tile inside the same block
         const uint32_t nw_addr = XB0 + (32u * (uint32_t)nhead + 10u + (nrm_is_v ? 1u : 0u)) * XS + (uint32_t)ntok * 4u;
         const uint32_t nr_addr = XB0 + (32u * hs + 10u) * XS + (uint32_t)g * 16u;
-        // (packed form: the lane's bank kb = token pair; its two norms are eight of those sixteen bytes)
-        const int kb = (lane >> 2) & 3;
-        const uint32_t nr2_addr = nr_addr + 64u * (uint32_t)(kb >> 1) + 8u * (uint32_t)(kb & 1);
+        // (packed form, four lanes per head: the lane's bank kb = token pair, its two norms are eight of those sixteen
+        // bytes; two lanes per head: kb = tile, all sixteen bytes of that tile)
+        const int kb = PACK == 4 ? (lane >> 2) & 3 : (lane >> 3) & 1;
+        const uint32_t nr2_addr = PACK == 4 ? nr_addr + 64u * (uint32_t)(kb >> 1) + 8u * (uint32_t)(kb & 1) : nr_addr + 64u * (uint32_t)kb;
         // what a lane hands over: a key norm as it is, a value norm as log2 |v| clamped below at -60 (a zero
         // vector then weighs 2^-60 of its codes: nothing at any output precision; NaN and negative norms,
         // which only rows outside a context can hold, come out as -60 as well)
@@ -671,7 +681,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         };
         // (`rn` holds the next chunk: its norms go out at the end of this step, behind the barrier that ends it)
         auto produce = [&](mf_kraw& r, const mf_kraw& rn, int c, const uint32_t par) {
-          float sv[8];
+          float sv[4];
           {
             // 8 steps of two MFMAs; the table reads of step n+2 are issued before the MFMAs of step n.
             //   4-bit: step = (tile j, dword st), 4 reads (one per code byte: hi and lo of two coordinates)
@@ -732,7 +742,18 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             __builtin_amdgcn_sched_barrier(0);   // not earlier: the loads reuse the registers just read
             load_chunk(r, c + 2);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (PACK4) {
+            if constexpr (PACK == 2) {
+              // Five to eight query heads per kv head: columns 0..7 carry the sums of the float16 roundings of the
+              // queries, 8..15 those of their remainders.  The packed copy has two lanes per head: lane c keeps tile 0
+              // (values 0..3), lane 8 + c takes tile 1 (values 4..7); each gets the other term of its tile from the
+              // other lane by one row shift of eight that writes half of the row.
+#pragma unroll
+              for (int jj = 0; jj < 4; ++jj) {
+                const float hi = mf_dpp_banks<0x118 /*row_shr:8*/, 0xc>(acc[0][jj], acc[1][jj]);
+                const float lo = mf_dpp_banks<0x108 /*row_shl:8*/, 0x3>(acc[1][jj], acc[0][jj]);
+                sv[jj] = hi + lo;
+              }
+            } else if constexpr (PACK == 4) {
               // At most four query heads per kv head: only columns 0..3 (the float16 roundings of the queries) and
               // 8..11 (their remainders) of a row of sixteen lanes carry sums, eight per lane.  Everything from
               // here to the weights runs on a PACKED copy instead: lane 4k + c of a row takes the token pair k
@@ -752,16 +773,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
                 lo = mf_dpp_bank<0x114 /*row_shr:4*/, 3>(lo, acc[1][2 + jj]);
                 sv[jj] = hi + lo;
               }
-            } else {
-            // columns c and c + 8 carry the hi and lo part of the same query head; only lanes of
-            // columns [0,8) keep a meaningful softmax state (the others see the lo part alone)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              union { mf_u32x4 u; float f[4]; } kn;
-              kn.u = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + 64u * j);
-#pragma unroll
-              for (int i = 0; i < 4; ++i) sv[4 * j + i] = (acc[j][i] + mf_from_hi_cols(acc[j][i])) * kn.f[i];
-            }
             }
           }
           // The value norms arrive as log2 |v| (clamped below at -60, see the hand-over of the norms) and the
@@ -770,8 +781,26 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
           // value product with the same relative precision for tiny and for huge value vectors.  The
           // denominator sums the plain p = exp2(score - max) in the same frame (at most 2^60 each); the frame
           // cancels between numerator and denominator and travels as `m` of the partial result.
-          float tv[8];
-          if constexpr (PACK4) {
+          float tv[4];
+          if constexpr (PACK == 2) {
+            // the lane's tile: four key norms and four log2 of value norms, sixteen bytes each
+            union { mf_u32x4 u; float f[4]; } kn, vn;
+            kn.u = *(mf_lds_u128*)(uintptr_t)(nr2_addr + XPAR * par);
+            vn.u = *(mf_lds_u128*)(uintptr_t)(nr2_addr + XPAR * par + XS);
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+              sv[jj] *= kn.f[jj];
+              tv[jj] = sv[jj] + vn.f[jj];
+            }
+            if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
+              // (a row past the context may hold anything, NaN norms included: both sums are overwritten)
+              const int tok0 = blk_lo * bs + 32 * c + 16 * kb + 4 * g;
+              const bool tile_ok = kb == 0 || bs32 || 2 * c + 1 < nblk;
+#pragma unroll
+              for (int jj = 0; jj < 4; ++jj)
+                if (!(tile_ok && tok0 + jj < t_end)) { sv[jj] = -INFINITY; tv[jj] = -INFINITY; }
+            }
+          } else {
             // the lane's token pair: key norms and log2 of the value norms, eight bytes each
             union { mf_u32x2 u; float f[2]; } kn, vn;
             kn.u = *(mf_lds_cu64*)(uintptr_t)(nr2_addr + XPAR * par);
@@ -789,29 +818,48 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
               for (int jj = 0; jj < 2; ++jj)
                 if (!(tile_ok && tok0 + jj < t_end)) { sv[jj] = -INFINITY; tv[jj] = -INFINITY; }
             }
-          } else {
-          union { mf_u32x4 u[2]; float f[8]; } vn;
-          vn.u[0] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS);
-          vn.u[1] = *(mf_lds_u128*)(uintptr_t)((nr_addr + XPAR * par) + XS + 64u);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) tv[i] = sv[i] + vn.f[i];
-          if (c == nchunks - 1) {     // only the last chunk of a segment can hold masked tokens
-            // (a row past the context may hold anything, NaN norms included: both sums are overwritten)
-            const int tok0 = blk_lo * bs + 32 * c;
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const int tok = tok0 + 16 * j + 4 * g + i;
-                const bool ok = (tok < t_end) && (j == 0 || bs32 || 2 * c + 1 < nblk);
-                if (!ok) { sv[4 * j + i] = -INFINITY; tv[4 * j + i] = -INFINITY; }
-              }
-          }
           }
           // running softmax in the log2 domain (scale * log2 e is folded into the query operand)
           union { mf_u32x4 u; uint32_t w[4]; } cv;
           float resc_out;
-          if constexpr (PACK4) {
+          if constexpr (PACK == 2) {
+            // both lanes of a head agree on its running maximum; each keeps the sum of its own tile
+            float mx = fmaxf(fmaxf(tv[0], tv[1]), fmaxf(tv[2], tv[3]));
+            mx = fmaxf(mx, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(mx), 0x128 /*row_ror:8*/, 0xf, 0xf, false)));
+            mx = mf_rows_max(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
+            m_run = m_new;
+            float psum = 0.f, pw[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+              psum += __builtin_amdgcn_exp2f(sv[jj] - m_new);            // 0 for masked tokens
+              pw[jj] = __builtin_amdgcn_exp2f(tv[jj] - m_new);           // p |v| <= 1; 0 for masked tokens
+            }
+            l_run = l_run * resc + psum;
+            uint32_t hb[2], lb[2];      // the tile's two token pairs as float16 hi + lo
+#pragma unroll
+            for (int pp = 0; pp < 2; ++pp) {
+              auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * pp], pw[2 * pp + 1]);
+              auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * pp] - (float)h2[0], pw[2 * pp + 1] - (float)h2[1]);
+              union { decltype(h2) h; uint32_t u; } hu, lu;
+              hu.h = h2;
+              lu.h = l2;
+              hb[pp] = hu.u;
+              lb[pp] = lu.u;
+            }
+            // operand dword qq = token pair q(qq) = pair q % 2 of tile q / 2: columns 0..7 take its hi form, columns
+            // 8..15 its lo form, each from the lane of the pair's tile (its own, or the one eight lanes away)
+            // (2-bit: the value side's operand takes the tokens as 4g, 4g+1 of both tiles, then 4g+2, 4g+3 of both)
+            auto tile0 = [&](int pp) { return mf_dpp_banks_u<0x118 /*row_shr:8*/, 0xc>(hb[pp], lb[pp]); };
+            auto tile1 = [&](int pp) { return mf_dpp_banks_u<0x108 /*row_shl:8*/, 0x3>(lb[pp], hb[pp]); };
+            if constexpr (BITS == 2) {
+              cv.w[0] = tile0(0); cv.w[1] = tile1(0); cv.w[2] = tile0(1); cv.w[3] = tile1(1);
+            } else {
+              cv.w[0] = tile0(0); cv.w[1] = tile0(1); cv.w[2] = tile1(0); cv.w[3] = tile1(1);
+            }
+            resc_out = resc;
+          } else {
             // every lane of a row knows the running maximum of its head c; the sum is kept per lane (its own
             // pair's share) and added up over the banks when the segment ends
             float mx = fmaxf(tv[0], tv[1]);
@@ -836,37 +884,6 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
             cv.w[2] = mf_pair_from_bank<BITS == 2 ? 1 : 2>(hb.u, lb.u);
             cv.w[3] = mf_pair_from_bank<3>(hb.u, lb.u);
             resc_out = resc;
-          } else {
-          float mx = fmaxf(fmaxf(fmaxf(tv[0], tv[1]), fmaxf(tv[2], tv[3])), fmaxf(fmaxf(tv[4], tv[5]), fmaxf(tv[6], tv[7])));
-          mx = mf_rows_max(mx);
-          const float m_new = fmaxf(m_run, mx);
-          const float resc = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first chunk
-          m_run = m_new;
-          float psum = 0.f;
-          float pw[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            psum += __builtin_amdgcn_exp2f(sv[i] - m_new);            // 0 for masked tokens
-            pw[i] = __builtin_amdgcn_exp2f(tv[i] - m_new);            // p |v| <= 1; 0 for masked tokens
-          }
-          // weights as float16 hi + lo, two at a time: hi = pw truncated to float16, lo = pw - hi (exact
-          // in float32, then truncated); columns [0,8) keep hi, columns [8,16) take the lo pair of the
-          // column eight to their left (one row shift per packed pair)
-          // (2-bit: the value side's operand takes the tokens as 4g, 4g+1 of both tiles, then 4g+2, 4g+3 of both)
-#pragma unroll
-          for (int qq = 0; qq < 4; ++qq) {
-            const int q = BITS == 2 ? ((qq & 1) << 1 | (qq >> 1)) : qq;      // the pair of tokens operand dword qq holds
-            auto h2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q], pw[2 * q + 1]);
-            auto l2 = __builtin_amdgcn_cvt_pkrtz(pw[2 * q] - (float)h2[0], pw[2 * q + 1] - (float)h2[1]);
-            union { decltype(h2) h; uint32_t u; } hb, lb;
-            hb.h = h2;
-            lb.h = l2;
-            const uint32_t lo_left = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)lb.u, 0x118 /*row_shr:8*/, 0xf, 0xf, true);
-            cv.w[qq] = col < 8 ? hb.u : lo_left;
-          }
-          l_run = l_run * resc + psum;
-          const float resc_left = mf_from_lo_cols(resc);
-          resc_out = col < 8 ? resc : resc_left;
           }
           // the buffer was last read for chunk c - 2, two barriers ago
           *(mf_lds_u128*)(uintptr_t)(pb_addr + XPAR * par) = cv.u;
@@ -901,7 +918,9 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
         __builtin_amdgcn_s_waitcnt(MF_WAIT_VM0);   // the lookahead past the last chunk is never consumed
         float lsum = l_run;
         lsum = mf_rows_sum(lsum);
-        if constexpr (PACK4) lsum = mf_banks_sum(lsum);      // every lane of a row summed its own token pair
+        // every lane of a row summed its own share
+        if constexpr (PACK == 4) lsum = mf_banks_sum(lsum);
+        else lsum += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(lsum), 0x128 /*row_ror:8*/, 0xf, 0xf, false));
         if (active && col < gqa && g == 0) {
           const size_t slot = (size_t)(blockIdx.x + s) * a.QH + (h * gqa + col);
           a.part_ml[slot * 2] = m_run * 0.6931471805599453f;   // back to the natural-log domain
@@ -1060,7 +1079,7 @@ __device__ __forceinline__ void mf_role_main(const akv_attn_args& a, const akv_m
   }
 }
 
-template <int BITS, bool PACK4>
+template <int BITS, int PACK>
 __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args a, akv_mfma_extra x) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wavefront-uniform on purpose
@@ -1084,8 +1103,8 @@ __global__ __launch_bounds__(MF_THREADS) void akv_attn_mfma_kernel(akv_attn_args
       st.pbwin = (int)akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, st.s * a.bt_stride + bi), a.num_blocks);
     }
   }
-  if ((wave >> 3) == 0) mf_role_main<0, BITS, PACK4>(a, x, wave & 7, st);
-  else mf_role_main<1, BITS, PACK4>(a, x, wave & 7, st);
+  if ((wave >> 3) == 0) mf_role_main<0, BITS, PACK>(a, x, wave & 7, st);
+  else mf_role_main<1, BITS, PACK>(a, x, wave & 7, st);
 }
 
 // ----------------------------------------------------------------------------------
@@ -1164,19 +1183,20 @@ int akv_attn_mfma_run(const void* query, int q_dtype, int64_t qs_seq, int64_t qs
   if (q_dtype == AKV_F16) MF_PRO(AKV_F16); else if (q_dtype == AKV_BF16) MF_PRO(AKV_BF16); else MF_PRO(AKV_F32);
 #undef MF_PRO
   AKV_LAUNCH_CHECK("akv_attn_mfma_prologue_kernel");
-  // at most four query heads per kv head (or group): the score wavefronts work on packed scores
+  // the score wavefronts work on packed scores: four lanes per query head with at most four heads per kv head
+  // (or group), two lanes per head with five to eight
   const bool pack4 = a.QH / a.KVH <= 4;
   static bool configured = false;
   if (!configured) {
 #define MF_CFG(B, P, L) AKV_HIP(hipFuncSetAttribute((const void*)akv_attn_mfma_kernel<B, P>, hipFuncAttributeMaxDynamicSharedMemorySize, L))
-    MF_CFG(4, false, MF_LDS_BYTES); MF_CFG(4, true, MF_LDS_BYTES);
-    MF_CFG(3, false, MF_LDS_BYTES); MF_CFG(3, true, MF_LDS_BYTES);
-    MF_CFG(2, false, MF_LDS_BYTES_2BIT); MF_CFG(2, true, MF_LDS_BYTES_2BIT);
+    MF_CFG(4, 2, MF_LDS_BYTES); MF_CFG(4, 4, MF_LDS_BYTES);
+    MF_CFG(3, 2, MF_LDS_BYTES); MF_CFG(3, 4, MF_LDS_BYTES);
+    MF_CFG(2, 2, MF_LDS_BYTES_2BIT); MF_CFG(2, 4, MF_LDS_BYTES_2BIT);
 #undef MF_CFG
     configured = true;
   }
-#define MF_RUN(B, L) do { if (pack4) AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, true>), grid, MF_THREADS, L, stream, a, x); \
-                         else AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, false>), grid, MF_THREADS, L, stream, a, x); } while (0)
+#define MF_RUN(B, L) do { if (pack4) AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, 4>), grid, MF_THREADS, L, stream, a, x); \
+                         else AKV_LAUNCH_TIMED((akv_attn_mfma_kernel<B, 2>), grid, MF_THREADS, L, stream, a, x); } while (0)
   if (bits == 4) MF_RUN(4, MF_LDS_BYTES);
   else if (bits == 3) MF_RUN(3, MF_LDS_BYTES);
   else MF_RUN(2, MF_LDS_BYTES_2BIT);
