@@ -20,9 +20,13 @@
 //            coordinate pair repeated to face the hi and the lo half; columns [0,8) = fp16 rounding
 //            of q', columns [8,16) = fp16 of the remainder (q' to ~22 bits at no extra MFMA).
 //            Result: lane (col, g) holds tokens 4g..4g+3 of the tile for column col.
-//   softmax  running max / sum per column in the log2 domain; the weights p * |v| of a lane are
-//            exactly the k-slice of the B operand of the next product (tokens 4g..4g+3 of both
-//            tiles), again split hi / lo over columns [0,8) / [8,16).
+//   softmax  running max / sum per query head in the log2 domain, on a PACKED copy of the scores: of the
+//            sixteen columns only gqa (roundings) + gqa (remainders) carry sums, so the lanes of a row
+//            share the eight tokens of a head -- four lanes a head (a token pair each) with at most four
+//            query heads, two lanes (a tile each) with five to eight -- and exponentials and float16
+//            splits are issued a quarter / half as often.  The weights p * |v| go back, by row shifts, to
+//            where they are exactly the k-slice of the B operand of the next product (tokens 4g..4g+3 of
+//            both tiles), again split hi / lo over columns [0,8) / [8,16).
 //   values   O^T[coord, col] += sum_token Vhat[token, coord] * P[token, col]
 //            A = Vhat^T: lane (m, g) loads dword m (coordinates 8m..8m+7) of its 8 tokens and
 //            builds, for each of the 8 coordinates, the 8-token k-slice; M-tile j row m is
