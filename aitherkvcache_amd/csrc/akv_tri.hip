@@ -540,8 +540,12 @@ static size_t tri_roles_lds_bytes(int kvh, int gqa_pass, bool q_half) {
 }
 
 typedef __attribute__((address_space(3))) const tri_half2 tri_lds_chalf2;
+typedef uint32_t tri_u32x4 __attribute__((ext_vector_type(4)));
+typedef float tri_f32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const tri_u32x4 tri_lds_cu32x4;
+typedef __attribute__((address_space(3))) const tri_f32x4 tri_lds_cf32x4;
 
-template <int GQ, bool PAGED, bool QH16>
+template <int GQ, bool PAGED, bool QH16, bool KP>
 __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int KVH = a.KVH;
@@ -551,14 +555,11 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // [4 arrays][KVH] x TRH_HEAD_PITCH
   unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
   float* alpha_lds = (float*)(tiles + (size_t)KVH * TRR_WAVE_BYTES);             // [2][KVH][TRR_ALPHA_FLOATS]
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool value_role = wv >= KVH;                            // wavefront-uniform
   const int h = value_role ? wv - KVH : wv;
   unsigned char* vt = tiles + (size_t)h * TRR_WAVE_BYTES;
   unsigned char* wt0 = vt + TRH_VT_BYTES;                        // weight buffer i at wt0 + i * 4 * TRH_WT_PITCH
-  if (value_role) {   // every use leaves the tile zero again; weight rows of absent query heads stay zero
-    for (int i = lane; i < TRR_WAVE_BYTES / 4; i += 64) ((uint32_t*)vt)[i] = 0u;
-  }
   const int col_n = lane & 15, grp = lane >> 4;
   const int col_q = col_n & 3, col_e = (col_n >> 2) & 1;
   // a weight dword is (hi | lo << 16) of one token: the lane takes its half into its parity slot
@@ -567,7 +568,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   const int gqa = a.QH / KVH;
   const int b = blockIdx.y, split = blockIdx.x;
   const float inv_sqrt_d = 1.0f / sqrtf(128.f);
-  if (tid < 64) theta[tid] = a.theta[tid];
+  const float theta_mine = tid < 64 ? a.theta[tid] : 0.f;
 
   // tokens of this batch element; ranges start on multiples of 64 (PAGED: of the block size too)
   const int64_t S = PAGED ? max((int64_t)0, min(akv_load_index(a.context_lens, a.cl_itype, b), a.S)) : a.S;
@@ -575,8 +576,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   const int64_t s0 = min(S, (int64_t)split * per);
   const int64_t s1 = min(S, s0 + per);
   const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)S;
-  const bool kp_wide = a.kpos && a.kp_itype == AKV_I64;
-  const unsigned char* kp_base = a.kpos ? (const unsigned char*)a.kpos : (const unsigned char*)a.theta;
+  const bool kp_wide = KP && a.kp_itype == AKV_I64;          // KP: key positions are given (otherwise 0..S-1)
 
   // the thread's row of a chunk: token r / KVH, head r % KVH; the first KVH wavefronts fetch the key arrays,
   // the others the value arrays
@@ -585,57 +585,89 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   const size_t arr = (size_t)KVH * TRH_HEAD_PITCH;
   unsigned char* st_wr = stage + (value_role ? 2 * arr : 0) + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
   const unsigned char* st_rd = stage + (value_role ? 2 * arr : 0) + (size_t)h * TRH_HEAD_PITCH + lane * 16;
-  const int64_t last_row = ((int64_t)b * a.S + max(s1, (int64_t)1)) * KVH - 1;
-  const uint8_t* src_idx = value_role ? a.v_idx : a.k_idx;
-  const uint8_t* src_cf = value_role ? a.v_cf : a.k_cf;
-  const unsigned short* src_sc = (const unsigned short*)(value_role ? a.v_sc : a.k_sc);
+  // Not PAGED: the rows of batch element b start at a wavefront-uniform address and a row is named by a
+  // 32-bit number (the host sends longer sequences to the other kernel).
+  const int64_t row_b = PAGED ? 0 : (int64_t)b * a.S * KVH;
+  const uint32_t last_rel = (uint32_t)max(s1, (int64_t)1) * KVH - 1;
+  const uint8_t* src_idx = (value_role ? a.v_idx : a.k_idx) + row_b * 12;
+  const uint8_t* src_cf = (value_role ? a.v_cf : a.k_cf) + row_b * 12;
+  const unsigned char* src_sc = (const unsigned char*)(value_role ? a.v_sc : a.k_sc) + row_b * 2;
+  const unsigned char* kp_b = KP ? (const unsigned char*)a.kpos + (int64_t)b * a.S * (kp_wide ? 8 : 4) : nullptr;
+  const int s1m = (int)s1 - 1;
 
   struct tri_rows { uint32_t x[2][3]; unsigned short sc; uint32_t kp_lo, kp_hi; };
   auto fetch = [&](tri_rows& rr, int64_t c0) {
-    int64_t row;
+    const uint32_t* p0;
+    const uint32_t* p1;
     if (PAGED) {
-      const int64_t tcl = max((int64_t)0, min(c0 + my_t, s1 - 1));           // tokens past the range: its last token
-      const int64_t blk = tcl / a.block_size;
+      const int tcl = max(0, min((int)c0 + my_t, s1m));                      // tokens past the range: its last token
+      const int blk = tcl / a.block_size;
       int64_t phys = akv_load_index(a.block_tables, a.bt_itype, (int64_t)b * a.bt_stride + blk);
       phys = max((int64_t)0, min(phys, a.num_blocks - 1));                   // (an empty sequence reads a padding entry)
-      row = ((phys * a.block_size) + (tcl - blk * a.block_size)) * KVH + my_h;
+      const int64_t row = ((phys * a.block_size) + (tcl - blk * a.block_size)) * KVH + my_h;
+      p0 = (const uint32_t*)(src_idx + row * 12);
+      p1 = (const uint32_t*)(src_cf + row * 12);
+      rr.sc = *(const unsigned short*)(src_sc + row * 2);
     } else {
-      row = min(((int64_t)b * a.S + c0) * KVH + r, last_row);                // rows past the range: its last row
+      const uint32_t rel = min((uint32_t)c0 * KVH + r, last_rel);            // rows past the range: its last row
+      p0 = (const uint32_t*)(src_idx + (size_t)(rel * 12u));
+      p1 = (const uint32_t*)(src_cf + (size_t)(rel * 12u));
+      rr.sc = *(const unsigned short*)(src_sc + (size_t)(rel * 2u));
     }
-    const uint32_t* p0 = (const uint32_t*)(src_idx + row * 12);
-    const uint32_t* p1 = (const uint32_t*)(src_cf + row * 12);
 #pragma unroll
     for (int w = 0; w < 3; ++w) { rr.x[0][w] = p0[w]; rr.x[1][w] = p1[w]; }
-    rr.sc = src_sc[row];
     // the score wavefront's own token positions (lane = token), as two dwords
-    const int64_t tc = max((int64_t)0, min(c0 + lane, s1 - 1));
-    const int64_t pe = (a.kpos && !value_role) ? ((int64_t)b * a.S + tc) * (kp_wide ? 8 : 4) : 0;
-    rr.kp_lo = *(const uint32_t*)(kp_base + pe);
-    rr.kp_hi = *(const uint32_t*)(kp_base + pe + (kp_wide ? 4 : 0));
+    rr.kp_lo = 0; rr.kp_hi = 0;
+    if constexpr (KP) {
+      const uint32_t pe = value_role ? 0u : (uint32_t)max(0, min((int)c0 + lane, s1m)) * (kp_wide ? 8u : 4u);
+      rr.kp_lo = *(const uint32_t*)(kp_b + (size_t)pe);
+      rr.kp_hi = *(const uint32_t*)(kp_b + (size_t)pe + (kp_wide ? 4 : 0));
+    }
   };
 
-  for (int qg = 0; qg < gqa; qg += GQ) {
-    __syncthreads();
-    for (int i = tid; i < KVH * GQ * 128; i += blockDim.x) {
+  {
+    // One workgroup serves GQ query heads of every kv head (grid z: which ones).  (A loop over the groups
+    // inside the kernel would keep every value that only one role uses alive through the other role's
+    // loop as well -- the loop's back edge joins the two -- and the kernel then needs more than its 128
+    // registers; a reload from scratch memory is counted with the global loads, so waiting for it
+    // waits for every row in flight.)
+    const int qg = blockIdx.z * GQ;
+    // The first chunk and the queries are requested before anything waits: the workgroup has KVH x 128
+    // threads and KVH x GQ x 128 query elements, GQ per thread (element j of thread tid is number
+    // tid + j x KVH x 128).
+    tri_rows nxt;
+    fetch(nxt, s0);
+    float qv[GQ];
+    unsigned short qraw[GQ];
+#pragma unroll
+    for (int j = 0; j < GQ; ++j) {
+      const int i = tid + j * KVH * 128;
       const int hh = i / (GQ * 128), rem = i - hh * (GQ * 128);
       const int q = rem >> 7, d = rem & 127;
       const int64_t off = ((int64_t)b * a.QH + (hh * gqa + qg + q)) * 128 + d;
+      qv[j] = 0.f; qraw[j] = 0;
+      if (QH16) qraw[j] = ((const unsigned short*)a.query)[off];
+      else if (a.q_dtype == AKV_BF16) qv[j] = akv_elem<AKV_BF16>::load(a.query, off);
+      else qv[j] = akv_elem<AKV_F32>::load(a.query, off);
+    }
+    {   // every use leaves a tile zero again; weight rows of absent query heads stay zero
+      for (int i = tid; i < KVH * (TRR_WAVE_BYTES / 16); i += KVH * 128) ((uint4*)tiles)[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (tid < 64) theta[tid] = theta_mine;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < GQ; ++j) {
+      const int i = tid + j * KVH * 128;
+      const int hh = i / (GQ * 128), rem = i - hh * (GQ * 128);
+      const int q = rem >> 7, d = rem & 127;
       unsigned char* row = (unsigned char*)q_lds + ((size_t)hh * 64 + (d >> 1)) * QROW;
-      if (QH16) {
-        *(unsigned short*)(row + (q * 2 + (d & 1)) * 2) = ((const unsigned short*)a.query)[off];
-      } else {
-        float v;
-        if (a.q_dtype == AKV_F16) v = akv_elem<AKV_F16>::load(a.query, off);
-        else if (a.q_dtype == AKV_BF16) v = akv_elem<AKV_BF16>::load(a.query, off);
-        else v = akv_elem<AKV_F32>::load(a.query, off);
-        *(float*)(row + (q * 2 + (d & 1)) * 4) = v;
-      }
+      if (QH16) *(unsigned short*)(row + (q * 2 + (d & 1)) * 2) = qraw[j];
+      else *(float*)(row + (q * 2 + (d & 1)) * 4) = qv[j];
     }
     const uint32_t q_base = 64 * sizeof(float) + (uint32_t)h * 64 * QROW;
     // One step of the staging pipeline, the same in both roles (two workgroup barriers): the chunk fetched
     // during the previous step goes to the staging area, the next one is requested, the wavefront's own
     // two entries per token come back.
-    tri_rows nxt;
     uint32_t kp_lo = 0, kp_hi = 0;
     auto stage_step = [&](int64_t c0, uint4& e0, uint4& e1, uint32_t& other_sc) {
       *(uint4*)(st_wr) = make_uint4(nxt.x[0][0], nxt.x[0][1], nxt.x[0][2], nxt.sc);
@@ -649,7 +681,6 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
       other_sc = *(const uint32_t*)(st_rd + (value_role ? 0 : 2 * arr) + 12);
       __syncthreads();
     };
-    fetch(nxt, s0);
 
     if (!value_role) {
       float m[GQ], l[GQ];
@@ -665,7 +696,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
         const uint32_t ki[3] = {e0.x, e0.y, e0.z}, kc[3] = {e1.x, e1.y, e1.z};
         const float ksc = __half2float(__ushort_as_half((unsigned short)e0.w));
         const float vsc = __half2float(__ushort_as_half((unsigned short)vsc_raw));
-        const float kp = !a.kpos ? (float)(valid ? t : s1 - 1)
+        const float kp = !KP ? (float)(valid ? (int)t : s1m)
                          : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
         const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
         const float kscale = ksc * (inv_sqrt_d / 15.f);
@@ -702,18 +733,33 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
           const float ka = k0 * cs - k1 * sn;
           const float kb = k1 * cs + k0 * sn;
           const uint32_t qrow = idx4 * (QROW / 4) + q_base;      // LDS address of the pair's row of this head
+          if constexpr (GQ == 4 && QH16) {
+            const tri_u32x4 qv = *(tri_lds_cu32x4*)(uintptr_t)qrow;
 #pragma unroll
-          for (int q = 0; q < GQ; ++q) {
-            if (QH16) {
-              const tri_half2 qq = *(tri_lds_chalf2*)(uintptr_t)(qrow + 4 * q);
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t qw = qv[q];
+              const tri_half2 qq = __builtin_bit_cast(tri_half2, qw);
               sc[q] = fmaf((float)qq.y, kb, fmaf((float)qq.x, ka, sc[q]));
-            } else {
-              const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
-              sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+            }
+          } else if constexpr (GQ == 4) {
+            const tri_f32x4 qa = *(tri_lds_cf32x4*)(uintptr_t)qrow;
+            const tri_f32x4 qb = *(tri_lds_cf32x4*)(uintptr_t)(qrow + 16);
+            sc[0] = fmaf(qa[1], kb, fmaf(qa[0], ka, sc[0]));
+            sc[1] = fmaf(qa[3], kb, fmaf(qa[2], ka, sc[1]));
+            sc[2] = fmaf(qb[1], kb, fmaf(qb[0], ka, sc[2]));
+            sc[3] = fmaf(qb[3], kb, fmaf(qb[2], ka, sc[3]));
+          } else {
+#pragma unroll
+            for (int q = 0; q < GQ; ++q) {
+              if (QH16) {
+                const tri_half2 qq = *(tri_lds_chalf2*)(uintptr_t)(qrow + 4 * q);
+                sc[q] = fmaf((float)qq.y, kb, fmaf((float)qq.x, ka, sc[q]));
+              } else {
+                const tri_f32x2 qq = *(tri_lds_cfloat2*)(uintptr_t)(qrow + 8 * q);
+                sc[q] = fmaf(qq.y, kb, fmaf(qq.x, ka, sc[q]));
+              }
             }
           }
-          // (with 128 registers per lane the query rows of all twelve pairs cannot be requested at once)
-          if ((f & 3) == 3) __builtin_amdgcn_sched_barrier(0);
         }
         float p[GQ], alpha[GQ];
         bool rescale = false;
@@ -724,22 +770,37 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
           sv[q] = valid ? sc[q] * kscale : -INFINITY;
           mx[q] = sv[q] + bias;
         }
-        if (GQ == 4) {
-          tri_row16_max4(mx[0], mx[1 % GQ], mx[2 % GQ], mx[3 % GQ]);
+        // The maxima are searched only when some token of the chunk exceeds one of them (the running
+        // maxima are the same in every lane, so the test is one comparison per query head and a vote);
+        // otherwise every factor is one and the sums just grow.
+        bool grow = false;
 #pragma unroll
-          for (int q = 0; q < GQ; ++q) mx[q] = tri_rows_max(mx[q]);
+        for (int q = 0; q < GQ; ++q) grow |= mx[q] > m[q];
+        if (__builtin_amdgcn_ballot_w64(grow) != 0ull) {
+          if (GQ == 4) {
+            tri_row16_max4(mx[0], mx[1 % GQ], mx[2 % GQ], mx[3 % GQ]);
+#pragma unroll
+            for (int q = 0; q < GQ; ++q) mx[q] = tri_rows_max(mx[q]);
+          } else {
+#pragma unroll
+            for (int q = 0; q < GQ; ++q) mx[q] = tri_wave_max(mx[q]);
+          }
+#pragma unroll
+          for (int q = 0; q < GQ; ++q) {
+            const float mn = fmaxf(m[q], mx[q]);
+            alpha[q] = __expf(m[q] - mn);
+            l[q] *= alpha[q];
+            m[q] = mn;
+          }
+          rescale = true;
         } else {
 #pragma unroll
-          for (int q = 0; q < GQ; ++q) mx[q] = tri_wave_max(mx[q]);
+          for (int q = 0; q < GQ; ++q) alpha[q] = 1.f;
         }
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float mn = fmaxf(m[q], mx[q]);
-          alpha[q] = __expf(m[q] - mn);
-          rescale |= (mn != m[q]);
-          p[q] = valid ? __expf(sv[q] - mn) : 0.f;
-          l[q] = l[q] * alpha[q] + p[q];
-          m[q] = mn;
+          p[q] = valid ? __expf(sv[q] - m[q]) : 0.f;
+          l[q] += p[q];
         }
         unsigned char* wt = wt0 + buf * 4 * TRH_WT_PITCH;
 #pragma unroll
@@ -846,17 +907,18 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
       }
       __syncthreads();             // the weights of the last chunk
       if (have_prev) consume(buf ^ 1);
-#pragma unroll
-      for (int q = 0; q < GQ; ++q) {
-        const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + q)) * a.nsplit + split;
+      {
+        // columns 0..7 hold the high parts of (query head, parity), columns 8..15 the low parts
+        const size_t slot = ((size_t)b * a.QH + (h * gqa + qg + (GQ == 4 ? col_q : 0))) * a.nsplit + split;
+        float* dst = a.part_acc + slot * 128 + 8 * grp + col_e;
+        const bool mine = col_n < 8 && col_q < GQ;
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float hi = oacc[mt][i];
             const float lo = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(hi), 0x108 /*row_shl:8*/, 0xf, 0xf, true));
-            if (col_n < 8 && col_q == q)
-              a.part_acc[slot * 128 + 2 * (16 * mt + 4 * grp + i) + col_e] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
+            if (mine) dst[32 * mt + 2 * i] = (hi + lo) * (1.f / (15.f * TRI_WSCALE));
           }
       }
     }
@@ -918,24 +980,24 @@ __global__ void tri_zero_kernel(float* out, size_t n) {
 
 // launch of the all-heads kernel for (gq, qh, lds, hgrid, num_kv_heads, stream, a) of the caller; more than 64 KB
 // of dynamic LDS has to be allowed once per kernel
-template <int GQ, bool PAGED, bool QH16>
+template <int GQ, bool PAGED, bool QH16, bool KP>
 static int tri_heads_launch(dim3 hgrid, int kvh, size_t lds, hipStream_t stream, const tri_args& a) {
   static size_t configured = 0;
   if (configured < lds) {
-    AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<GQ, PAGED, QH16>,
+    AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<GQ, PAGED, QH16, KP>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     configured = lds;
   }
-  AKV_LAUNCH_TIMED((tri_decode_heads_kernel<GQ, PAGED, QH16>), hgrid, kvh * 128, lds, stream, a);
+  AKV_LAUNCH_TIMED((tri_decode_heads_kernel<GQ, PAGED, QH16, KP>), hgrid, kvh * 128, lds, stream, a);
   return AKV_OK;
 }
-#define TRI_HEADS_LAUNCH(PAGED)                                                                                      \
+#define TRI_HEADS_LAUNCH(PAGED, KP)                                                                                  \
   do {                                                                                                               \
     int rc_;                                                                                                         \
-    if (gq == 4) rc_ = qh ? tri_heads_launch<4, PAGED, true>(hgrid, num_kv_heads, lds, stream, a)                    \
-                          : tri_heads_launch<4, PAGED, false>(hgrid, num_kv_heads, lds, stream, a);                  \
-    else rc_ = qh ? tri_heads_launch<1, PAGED, true>(hgrid, num_kv_heads, lds, stream, a)                            \
-                  : tri_heads_launch<1, PAGED, false>(hgrid, num_kv_heads, lds, stream, a);                          \
+    if (gq == 4) rc_ = qh ? tri_heads_launch<4, PAGED, true, KP>(hgrid, num_kv_heads, lds, stream, a)                \
+                          : tri_heads_launch<4, PAGED, false, KP>(hgrid, num_kv_heads, lds, stream, a);              \
+    else rc_ = qh ? tri_heads_launch<1, PAGED, true, KP>(hgrid, num_kv_heads, lds, stream, a)                        \
+                  : tri_heads_launch<1, PAGED, false, KP>(hgrid, num_kv_heads, lds, stream, a);                      \
     if (rc_ != AKV_OK) return rc_;                                                                                   \
   } while (0)
 
@@ -1008,7 +1070,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   const bool f12 = !wide && num_freqs == 12 &&
                    ((((uintptr_t)k_indices | (uintptr_t)k_coeffs | (uintptr_t)v_indices | (uintptr_t)v_coeffs) & 3) == 0);
   const bool dense = d == 128;
-  if (dense && f12 && num_kv_heads <= 8) {
+  if (dense && f12 && num_kv_heads <= 8 && (uint64_t)seq_len * num_kv_heads * 12 < (1ull << 32)) {
     // one workgroup per (token range, batch element), a wavefront per kv head
     const int gq = gqa % 4 == 0 ? 4 : 1;
     const bool qh = q_dtype == AKV_F16;
@@ -1016,15 +1078,16 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
     if (lds <= 160 * 1024) {
       int cus = akv_cached_cu_count();
       if (cus <= 0) cus = 256;
-      int64_t n = (cus + batch - 1) / batch;
+      const int passes = gqa / gq;
+      int64_t n = (cus + batch * passes - 1) / (batch * passes);
       const int64_t by_len = (seq_len + 63) / 64;
       if (n > by_len) n = by_len;
       if (n > TRI_MAX_SPLITS) n = TRI_MAX_SPLITS;
       if (n < 1) n = 1;
       a.nsplit = (int)n;
       a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
-      dim3 hgrid(a.nsplit, batch);
-      TRI_HEADS_LAUNCH(false);
+      dim3 hgrid(a.nsplit, batch, passes);
+      if (key_positions) TRI_HEADS_LAUNCH(false, true); else TRI_HEADS_LAUNCH(false, false);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
       AKV_LAUNCH_CHECK("tri_reduce_kernel");
@@ -1088,10 +1151,11 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const int gq = gqa % 4 == 0 ? 4 : 1;
   const bool qh = q_dtype == AKV_F16;
   const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
-  if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024)
+  if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024 ||
+      max_blocks_per_seq * block_size >= ((int64_t)1 << 31))
     return akv_fail(AKV_ERR_UNSUPPORTED,
-                    "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads and 4-byte "
-                    "aligned arrays");
+                    "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads, 4-byte "
+                    "aligned arrays and fewer than 2^31 tokens per sequence");
   if (batch == 0) return AKV_OK;
   AKV_REQUIRE(out != nullptr, "akv_tri_decode_paged: null pointer");
   if (max_blocks_per_seq == 0) {   // block tables without columns: every sequence is empty
@@ -1117,7 +1181,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   a.context_lens = context_lens; a.cl_itype = cl_itype; a.block_size = block_size; a.num_blocks = num_blocks;
   int cus = akv_cached_cu_count();
   if (cus <= 0) cus = 256;
-  int64_t n = (cus + batch - 1) / batch;
+  const int passes = gqa / gq;
+  int64_t n = (cus + batch * passes - 1) / (batch * passes);
   const int64_t by_len = (a.S + 63) / 64;
   if (n > by_len) n = by_len;
   if (n > TRI_MAX_SPLITS) n = TRI_MAX_SPLITS;
@@ -1126,8 +1191,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
-  dim3 hgrid(a.nsplit, batch);
-  TRI_HEADS_LAUNCH(true);
+  dim3 hgrid(a.nsplit, batch, passes);
+  TRI_HEADS_LAUNCH(true, false);
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");
