@@ -571,10 +571,12 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   const float theta_mine = tid < 64 ? a.theta[tid] : 0.f;
 
   // tokens of this batch element; ranges start on multiples of 64 (PAGED: of the block size too)
-  const int64_t S = PAGED ? max((int64_t)0, min(akv_load_index(a.context_lens, a.cl_itype, b), a.S)) : a.S;
-  const int64_t per = PAGED ? (((S + a.nsplit - 1) / a.nsplit + 63) & ~(int64_t)63) : (a.S + a.nsplit - 1) / a.nsplit;
-  const int64_t s0 = min(S, (int64_t)split * per);
-  const int64_t s1 = min(S, s0 + per);
+  // (token numbers fit 32 bits: the host sends longer sequences elsewhere)
+  const int S = PAGED ? (int)max((int64_t)0, min(akv_load_index(a.context_lens, a.cl_itype, b), a.S)) : (int)a.S;
+  const int per_raw = (int)(((uint32_t)S + (uint32_t)a.nsplit - 1u) / (uint32_t)a.nsplit);
+  const int per = PAGED ? ((per_raw + 63) & ~63) : per_raw;
+  const int s0 = min(S, split * per);
+  const int s1 = min(S, s0 + per);
   const float qp = a.qpos ? (float)akv_load_index(a.qpos, a.qp_itype, b) : (float)S;
   const bool kp_wide = KP && a.kp_itype == AKV_I64;          // KP: key positions are given (otherwise 0..S-1)
 
@@ -588,19 +590,19 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   // Not PAGED: the rows of batch element b start at a wavefront-uniform address and a row is named by a
   // 32-bit number (the host sends longer sequences to the other kernel).
   const int64_t row_b = PAGED ? 0 : (int64_t)b * a.S * KVH;
-  const uint32_t last_rel = (uint32_t)max(s1, (int64_t)1) * KVH - 1;
+  const uint32_t last_rel = (uint32_t)max(s1, 1) * KVH - 1;
   const uint8_t* src_idx = (value_role ? a.v_idx : a.k_idx) + row_b * 12;
   const uint8_t* src_cf = (value_role ? a.v_cf : a.k_cf) + row_b * 12;
   const unsigned char* src_sc = (const unsigned char*)(value_role ? a.v_sc : a.k_sc) + row_b * 2;
   const unsigned char* kp_b = KP ? (const unsigned char*)a.kpos + (int64_t)b * a.S * (kp_wide ? 8 : 4) : nullptr;
-  const int s1m = (int)s1 - 1;
+  const int s1m = s1 - 1;
 
   struct tri_rows { uint32_t x[2][3]; unsigned short sc; uint32_t kp_lo, kp_hi; };
-  auto fetch = [&](tri_rows& rr, int64_t c0) {
+  auto fetch = [&](tri_rows& rr, int c0) {
     const uint32_t* p0;
     const uint32_t* p1;
     if (PAGED) {
-      const int tcl = max(0, min((int)c0 + my_t, s1m));                      // tokens past the range: its last token
+      const int tcl = max(0, min(c0 + my_t, s1m));                      // tokens past the range: its last token
       const int blk = tcl / a.block_size;
       int64_t phys = akv_load_index(a.block_tables, a.bt_itype, (int64_t)b * a.bt_stride + blk);
       phys = max((int64_t)0, min(phys, a.num_blocks - 1));                   // (an empty sequence reads a padding entry)
@@ -619,7 +621,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
     // the score wavefront's own token positions (lane = token), as two dwords
     rr.kp_lo = 0; rr.kp_hi = 0;
     if constexpr (KP) {
-      const uint32_t pe = value_role ? 0u : (uint32_t)max(0, min((int)c0 + lane, s1m)) * (kp_wide ? 8u : 4u);
+      const uint32_t pe = value_role ? 0u : (uint32_t)max(0, min(c0 + lane, s1m)) * (kp_wide ? 8u : 4u);
       rr.kp_lo = *(const uint32_t*)(kp_b + (size_t)pe);
       rr.kp_hi = *(const uint32_t*)(kp_b + (size_t)pe + (kp_wide ? 4 : 0));
     }
@@ -669,7 +671,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
     // during the previous step goes to the staging area, the next one is requested, the wavefront's own
     // two entries per token come back.
     uint32_t kp_lo = 0, kp_hi = 0;
-    auto stage_step = [&](int64_t c0, uint4& e0, uint4& e1, uint32_t& other_sc) {
+    auto stage_step = [&](int c0, uint4& e0, uint4& e1, uint32_t& other_sc) {
       *(uint4*)(st_wr) = make_uint4(nxt.x[0][0], nxt.x[0][1], nxt.x[0][2], nxt.sc);
       *(uint4*)(st_wr + arr) = make_uint4(nxt.x[1][0], nxt.x[1][1], nxt.x[1][2], nxt.sc);
       kp_lo = nxt.kp_lo; kp_hi = nxt.kp_hi;
@@ -687,16 +689,16 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
 #pragma unroll
       for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
       int buf = 0;
-      for (int64_t c0 = s0; c0 < s1; c0 += 64) {
+      for (int c0 = s0; c0 < s1; c0 += 64) {
         uint4 e0, e1;
         uint32_t vsc_raw;
         stage_step(c0, e0, e1, vsc_raw);
-        const int64_t t = c0 + lane;
+        const int t = c0 + lane;
         const bool valid = t < s1;
         const uint32_t ki[3] = {e0.x, e0.y, e0.z}, kc[3] = {e1.x, e1.y, e1.z};
         const float ksc = __half2float(__ushort_as_half((unsigned short)e0.w));
         const float vsc = __half2float(__ushort_as_half((unsigned short)vsc_raw));
-        const float kp = !KP ? (float)(valid ? (int)t : s1m)
+        const float kp = !KP ? (float)(valid ? t : s1m)
                          : kp_wide ? (float)(int64_t)(((uint64_t)kp_hi << 32) | kp_lo) : (float)(int32_t)kp_lo;
         const float delta = a.post_rope ? 0.f : __fsub_rn(kp, qp);
         const float kscale = ksc * (inv_sqrt_d / 15.f);
@@ -762,8 +764,9 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
           }
         }
         float p[GQ], alpha[GQ];
-        bool rescale = false;
-        const float bias = __logf(fmaxf(vsc, 5.9604645e-8f));
+        // (the bias only places the maxima: the hardware logarithm is good enough, and a float16 scale is
+        // never a float32 denormal)
+        const float bias = __builtin_amdgcn_logf(fmaxf(vsc, 5.9604645e-8f)) * 0.6931471805599453f;
         float sv[GQ], mx[GQ];
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
@@ -773,6 +776,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
         // The maxima are searched only when some token of the chunk exceeds one of them (the running
         // maxima are the same in every lane, so the test is one comparison per query head and a vote);
         // otherwise every factor is one and the sums just grow.
+        float* al = alpha_lds + ((size_t)buf * KVH + h) * TRR_ALPHA_FLOATS;
         bool grow = false;
 #pragma unroll
         for (int q = 0; q < GQ; ++q) grow |= mx[q] > m[q];
@@ -792,32 +796,33 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
             l[q] *= alpha[q];
             m[q] = mn;
           }
-          rescale = true;
-        } else {
+          if (lane < 5) {        // m is the same in every lane, and so are the factors; entry 4: "some factor is not one"
+            float av = 1.f;
 #pragma unroll
-          for (int q = 0; q < GQ; ++q) alpha[q] = 1.f;
+            for (int q = 0; q < GQ; ++q) av = lane == q ? alpha[q] : av;
+            if (lane < GQ || lane == 4) al[lane] = av;
+          }
+        } else if (lane == 4) {
+          al[4] = 0.f;
         }
+        // (a token past the range has the score minus infinity and the weight exp(-inf) = 0: the maxima
+        // are finite once a chunk has been seen, and every chunk has a token inside the range)
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          p[q] = valid ? __expf(sv[q] - m[q]) : 0.f;
+          p[q] = __expf(sv[q] - m[q]);
           l[q] += p[q];
         }
+        // weight x value scale x 2^14 as float16 hi + lo: hi is the weight cut to float16's eleven bits, lo the
+        // exact rest; one conversion packs the two
         unsigned char* wt = wt0 + buf * 4 * TRH_WT_PITCH;
+        const float wsc = vsc * TRI_WSCALE;
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
-          const float w = p[q] * vsc * TRI_WSCALE;
-          auto h2 = __builtin_amdgcn_cvt_pkrtz(w, 0.f);
-          auto l2 = __builtin_amdgcn_cvt_pkrtz(w - (float)h2[0], 0.f);
-          union { decltype(h2) hv; uint32_t u; } hb, lb;
-          hb.hv = h2; lb.hv = l2;
-          *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = (hb.u & 0xffffu) | (lb.u << 16);
-        }
-        if (lane < 5) {          // m is the same in every lane, and so are the factors
-          float* al = alpha_lds + ((size_t)buf * KVH + h) * TRR_ALPHA_FLOATS;
-          float av = rescale ? 1.f : 0.f;
-#pragma unroll
-          for (int q = 0; q < GQ; ++q) av = lane == q ? alpha[q] : av;
-          if (lane < GQ || lane == 4) al[lane] = av;
+          const float w = p[q] * wsc;
+          const float w_hi = __uint_as_float(__float_as_uint(w) & 0xffffe000u);
+          union { decltype(__builtin_amdgcn_cvt_pkrtz(0.f, 0.f)) hv; uint32_t u; } pk;
+          pk.hv = __builtin_amdgcn_cvt_pkrtz(w_hi, w - w_hi);
+          *(uint32_t*)(wt + q * TRH_WT_PITCH + 4 * lane) = pk.u;
         }
         buf ^= 1;
       }
@@ -879,7 +884,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
         }
       };
       int buf = 0;
-      for (int64_t c0 = s0; c0 < s1; c0 += 64) {
+      for (int c0 = s0; c0 < s1; c0 += 64) {
         uint4 e0, e1;
         uint32_t unused;
         stage_step(c0, e0, e1, unused);
@@ -1152,10 +1157,10 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const bool qh = q_dtype == AKV_F16;
   const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
   if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024 ||
-      max_blocks_per_seq * block_size >= ((int64_t)1 << 31))
+      max_blocks_per_seq * block_size >= ((int64_t)1 << 30))
     return akv_fail(AKV_ERR_UNSUPPORTED,
                     "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads, 4-byte "
-                    "aligned arrays and fewer than 2^31 tokens per sequence");
+                    "aligned arrays and fewer than 2^30 tokens per sequence");
   if (batch == 0) return AKV_OK;
   AKV_REQUIRE(out != nullptr, "akv_tri_decode_paged: null pointer");
   if (max_blocks_per_seq == 0) {   // block tables without columns: every sequence is empty
