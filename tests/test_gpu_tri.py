@@ -279,6 +279,46 @@ def test_short_sequences_zero_and_large_values(dev, S, qdtype):
     assert np.max(np.abs(out - ref)) <= TOL * scale
 
 
+@pytest.mark.parametrize("qdtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("kp_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("QH,KVH", [(32, 8), (16, 2), (6, 2)])
+def test_key_positions_of_both_widths_and_query_types(dev, qdtype, kp_dtype, QH, KVH):
+    """Explicit key positions (32- and 64-bit) with every query type on the all-heads kernel, over several
+    ranges of a sequence; groups of four, eight (two groups on the grid) and three (one by one) query heads."""
+    cfg = TriAttentionConfig(num_kv_heads=KVH, num_query_heads=QH)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(QH * 100 + KVH)
+    B, S, D = 2, 1500, 128
+    keys = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    k_enc, v_enc = tri.encode_kv(t(keys, dev), t(vals, dev))
+    q = torch.from_numpy(rng.standard_normal((B, QH, D)).astype(np.float32)).to(dev).to(qdtype)
+    kpos = np.sort(rng.integers(0, 30000, size=(B, S)), axis=-1)
+    qpos = np.array([31000, 40000])
+    out = tri.decode_step(q, k_enc, v_enc, t(qpos, dev), torch.from_numpy(kpos).to(dev).to(kp_dtype)).cpu().numpy()
+    ref = O.tri_decode_step(q.float().cpu().numpy(), tuple(x.cpu().numpy() for x in k_enc),
+                            tuple(x.cpu().numpy() for x in v_enc), tri._theta.cpu().numpy(), qpos, kpos)
+    assert np.max(np.abs(out - ref)) <= TOL * max(1.0, float(np.abs(ref).max()))
+
+
+def test_scores_that_grow_along_the_sequence(dev):
+    """Post-RoPE scoring of keys that are multiples of one vector, growing with the position: every chunk of 64
+    tokens raises the running maxima (the sums are rescaled every time), and the last tokens carry the output."""
+    cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32, pre_rope=False)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(11)
+    B, S, KVH, QH, D = 2, 2000, 8, 32, 128
+    base = rng.standard_normal((1, 1, KVH, D))
+    keys = (base * np.linspace(0.05, 3.0, S)[None, :, None, None]).astype(np.float16)
+    vals = rng.standard_normal((B, S, KVH, D)).astype(np.float16)
+    k_enc, v_enc = tri.encode_kv(t(np.broadcast_to(keys, (B, S, KVH, D)).copy(), dev), t(vals, dev))
+    q = np.repeat(base[0, 0], QH // KVH, axis=0)[None].repeat(B, 0).astype(np.float32)      # aligned with the keys
+    out = tri.decode_step(t(q, dev), k_enc, v_enc).cpu().numpy()
+    ref = O.tri_decode_step(q, tuple(x.cpu().numpy() for x in k_enc), tuple(x.cpu().numpy() for x in v_enc),
+                            tri._theta.cpu().numpy(), pre_rope=False)
+    assert np.max(np.abs(out - ref)) <= TOL * max(1.0, float(np.abs(ref).max()))
+
+
 def test_empty_batch_and_empty_sequence(dev):
     cfg = TriAttentionConfig(num_kv_heads=8, num_query_heads=32)
     tri = TriAttention(cfg, device=str(dev))
