@@ -1257,26 +1257,39 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: the vector index and the search stay scalar
   const int P = d >> 1;
   const bool have = lane < P;
-  for (int64_t v = (int64_t)blockIdx.x * 4 + wave; v < n; v += (int64_t)gridDim.x * 4) {
-    float x0 = 0.f, x1 = 0.f;
-    if (have) {
-      x0 = akv_elem<XDT>::load(x, v * xs + 2 * lane);
-      x1 = akv_elem<XDT>::load(x, v * xs + 2 * lane + 1);
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  // the lane's pair of a vector is requested one vector ahead
+  auto fetch = [&](int64_t vv, float& p0, float& p1) {
+    p0 = 0.f; p1 = 0.f;
+    if (have && vv < n) {
+      p0 = akv_elem<XDT>::load(x, vv * xs + 2 * lane);
+      p1 = akv_elem<XDT>::load(x, vv * xs + 2 * lane + 1);
     }
+  };
+  float nx0, nx1;
+  fetch((int64_t)blockIdx.x * 4 + wave, nx0, nx1);
+  for (int64_t v = (int64_t)blockIdx.x * 4 + wave; v < n; v += stride) {
+    const float x0 = nx0, x1 = nx1;
+    fetch(v + stride, nx0, nx1);
     const float e = akv_add_rn(akv_mul_rn(x0, x0), akv_mul_rn(x1, x1));
     // non-negative floats and NaNs order like their bit patterns; lanes beyond the last pair sort last
     const uint32_t key = have ? (__float_as_uint(e) & 0x7fffffffu) + 1u : 0u;
     // The F-th largest key by a bitwise search (largest T with at least F keys >= T: one compare and a
     // population count per bit), then everything above it plus, of the keys equal to it, the lowest
     // lanes -- the order torch.topk's result has once it is sorted by index with ties to the lower index.
-    // (Once exactly F keys reach the threshold the remaining bits cannot change the set: the search stops there,
-    // after about half of its steps on keys without ties.)
+    // (Once exactly F keys reach the threshold the remaining bits cannot change the set: the search stops there
+    // -- looked at after every four bits --, after about half of its steps on keys without ties.  Written out
+    // bit by bit, a step is one vector compare against a scalar and four scalar instructions.)
     uint32_t T = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = T | (1u << bit);
-      const int cnt = __popcll(__ballot(key >= cand));
-      if (cnt >= F) T = cand;
-      if (cnt == F) break;
+#pragma unroll
+    for (int grp = 7; grp >= 0; --grp) {
+#pragma unroll
+      for (int b = 3; b >= 0; --b) {
+        const uint32_t cand = T | (1u << (4 * grp + b));
+        const int cnt = __builtin_popcountll(__builtin_amdgcn_ballot_w64(key >= cand));
+        T = cnt >= F ? cand : T;
+      }
+      if (__builtin_popcountll(__builtin_amdgcn_ballot_w64(key >= T)) == F) break;
     }
     const bool above = key > T, equal = key == T;
     const int need = F - __popcll(__ballot(above));
@@ -1287,13 +1300,20 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
     const int pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
     float amax = keep ? fmaxf(fabsf(x0), fabsf(x1)) : 0.f;
     if (keep && (x0 != x0 || x1 != x1)) amax = __uint_as_float(0x7fc00000u);   // torch.amax propagates NaN
-    // wave maximum that keeps a NaN
-    float m = amax;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float o = __shfl_xor(m, off, 64);
-      m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
+    // wave maximum that keeps a NaN: the values are non-negative or that one NaN pattern, which order like
+    // their bit patterns with the NaN on top (lane rotations inside rows of sixteen, then the row swaps)
+    uint32_t mb = __float_as_uint(amax);
+    mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x128 /*row_ror:8*/, 0xf, 0xf, false));
+    mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x124 /*row_ror:4*/, 0xf, 0xf, false));
+    mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x122 /*row_ror:2*/, 0xf, 0xf, false));
+    mb = max(mb, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mb, 0x121 /*row_ror:1*/, 0xf, 0xf, false));
+    {
+      auto r32 = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+      mb = max(r32[0], r32[1]);
+      auto r16 = __builtin_amdgcn_permlane16_swap(mb, mb, false, false);
+      mb = max(r16[0], r16[1]);
     }
+    const float m = __uint_as_float(mb);
     const float scale = (m != m) ? m : fmaxf(m, 1e-8f);
     if (keep && cbits == 16) {
       indices[v * F + pos] = (uint8_t)lane;
