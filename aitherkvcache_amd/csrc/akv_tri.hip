@@ -939,7 +939,7 @@ __global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict
   const size_t pair = blockIdx.x;  // b * QH + qh
   // the first partial sums of the thread's coordinate are requested before the weights exist: the
   // two round trips to memory overlap (D <= 128 coordinates take one pass of the 128 threads)
-  constexpr int PRE = 16;
+  constexpr int PRE = 32;
   float pre[PRE];
   {
     const int i0 = min((int)threadIdx.x, D - 1);
@@ -947,17 +947,18 @@ __global__ __launch_bounds__(128) void tri_reduce_kernel(const float* __restrict
     for (int s = 0; s < PRE; ++s) pre[s] = part_acc[(pair * nsplit + min(s, nsplit - 1)) * D + i0];
   }
   if (threadIdx.x < 64) {
-    float m = -INFINITY;
-    for (int s = threadIdx.x; s < nsplit; s += 64) m = fmaxf(m, part_ml[(pair * nsplit + s) * 2]);
-    m = akv_wave_max(m);
-    float l = 0.f;
-    for (int s = threadIdx.x; s < nsplit; s += 64) {
-      const float ms = part_ml[(pair * nsplit + s) * 2];
-      const float ws = ms > -INFINITY ? __expf(ms - m) : 0.f;
-      w[s] = ws;
-      l += ws * part_ml[(pair * nsplit + s) * 2 + 1];
-    }
-    l = akv_wave_sum(l);
+    // (maximum, sum) of ranges lane and lane + 64, one 8-byte load each, requested together
+    static_assert(TRI_MAX_SPLITS <= 128, "two ranges per lane");
+    const int sa = threadIdx.x, sb = threadIdx.x + 64;
+    float2 mla = make_float2(-INFINITY, 0.f), mlb = make_float2(-INFINITY, 0.f);
+    if (sa < nsplit) mla = *(const float2*)(part_ml + (pair * nsplit + sa) * 2);
+    if (sb < nsplit) mlb = *(const float2*)(part_ml + (pair * nsplit + sb) * 2);
+    const float m = akv_wave_max(fmaxf(mla.x, mlb.x));
+    const float wa = mla.x > -INFINITY ? __expf(mla.x - m) : 0.f;
+    const float wb = mlb.x > -INFINITY ? __expf(mlb.x - m) : 0.f;
+    if (sa < nsplit) w[sa] = wa;
+    if (sb < nsplit) w[sb] = wb;
+    const float l = akv_wave_sum(wa * mla.y + wb * mlb.y);
     if (threadIdx.x == 0) red[0] = l > 0.f ? 1.f / l : 0.f;
   }
   __syncthreads();
