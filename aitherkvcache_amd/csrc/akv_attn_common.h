@@ -136,12 +136,7 @@ __device__ __forceinline__ void akv_block_prefix_scan(const void* context_lens, 
   // exclusive scan over the 256 threads: inclusive scan inside each wavefront by lane shifts, then
   // the four wavefront totals through LDS
   const int lane = tid & 63, wave = tid >> 6;
-  int inc = sum;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int up = __shfl_up(inc, d, 64);
-    if (lane >= d) inc += up;
-  }
+  const int inc = akv_wave_inclusive_scan(sum);
   if (lane == 63) scratch[wave] = inc;
   __syncthreads();
   int base = 0;
@@ -210,22 +205,15 @@ __device__ __forceinline__ void akv_attn_partition(int32_t* prefix, int S, int G
       ctx = (int)akv_seq_tokens(context_lens, cl_itype, lane, block_size, max_blocks_per_seq);
       n = (ctx + block_size - 1) / block_size;
     }
-    int inc = n;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int up = __shfl_up(inc, d, 64);
-      if (lane >= d) inc += up;
-    }
-    const int total = __shfl(inc, 63, 64);
+    const int inc = akv_wave_inclusive_scan(n);
+    const int total = __builtin_amdgcn_readlane(inc, 63);
     const int b0 = inc - n;
     if (lane < S) prefix[lane] = b0;
     if (lane == 0) prefix[S] = total;
     p_pref[lane] = b0;
     p_ctx[lane] = ctx;
     const int c = (n + cb - 1) / cb;                             // chunks of the lane's sequence
-    int sumc = c;
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) sumc += __shfl_xor(sumc, m, 64);
+    const int sumc = akv_wave_sum(c);
     const int nz = __popcll(__ballot(c > 0));
     const int aligned = (nz >= 1 && nz * 8 <= G) ? 1 : 0;
     if (aligned) {
@@ -233,18 +221,11 @@ __device__ __forceinline__ void akv_attn_partition(int32_t* prefix, int S, int G
       if (lo < 1) lo = 1;
       while (lo < hi) {
         const int mid = (lo + hi) >> 1;
-        int tot = (c + mid - 1) / mid;
-#pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
+        const int tot = akv_wave_sum((c + mid - 1) / mid);
         if (tot <= G) hi = mid; else lo = mid + 1;
       }
       const int k = (c + lo - 1) / lo;
-      int kinc = k;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(kinc, d, 64);
-        if (lane >= d) kinc += up;
-      }
+      const int kinc = akv_wave_inclusive_scan(k);
       p_wfirst[lane] = kinc - k;
       if (lane == 63) p_wfirst[64] = kinc;
       if (lane < S) {

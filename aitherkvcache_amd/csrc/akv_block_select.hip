@@ -113,12 +113,7 @@ __device__ __forceinline__ uint32_t bs_column_key(const float* __restrict__ sc, 
 // exclusive scan of one int per thread over the 1024 threads of the workgroup; also returns the total
 __device__ __forceinline__ int bs_block_scan(int v, int* lds /*[17]*/, int& total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int inc = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int up = __shfl_up(inc, d, 64);
-    if (lane >= d) inc += up;
-  }
+  const int inc = akv_wave_inclusive_scan(v);
   __syncthreads();
   if (lane == 63) lds[wave] = inc;
   __syncthreads();

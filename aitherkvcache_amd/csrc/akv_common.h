@@ -179,17 +179,78 @@ __device__ __forceinline__ float akv_sub_rn(float a, float b) {
 }
 
 // ----------------------------------------------------------------------------------
-// device: wavefront (64-lane) reductions; every lane receives the result
+// device: the value of lane (lane ^ M), by data-parallel primitives and the row swaps: no trip through the LDS
+// crossbar (a shuffle is one, some hundred cycles under load).  M is a power of two below 64.
+// ----------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ uint32_t akv_dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+template <int M>
+__device__ __forceinline__ uint32_t akv_lane_xor_u32(uint32_t v) {
+  static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "a single bit of the lane number");
+  if constexpr (M == 1) return akv_dpp_u32<0xB1>(v);                      // quad_perm [1,0,3,2]
+  else if constexpr (M == 2) return akv_dpp_u32<0x4E>(v);                 // quad_perm [2,3,0,1]
+  else if constexpr (M == 4) return akv_dpp_u32<0x141>(akv_dpp_u32<0x1B>(v));   // quad_perm [3,2,1,0] (^3), then row_half_mirror (^7)
+  else if constexpr (M == 8) return akv_dpp_u32<0x128>(v);                // row_ror:8
+  else {
+    // fed the same value twice, the swaps leave (rows 0,1,0,1 | 2,3,2,3) and (rows 0,0,2,2 | 1,1,3,3)
+    const bool upper = (threadIdx.x & M) != 0;
+    if constexpr (M == 16) {
+      auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+      return upper ? r[0] : r[1];
+    } else {
+      auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+      return upper ? r[0] : r[1];
+    }
+  }
+}
+template <int M> __device__ __forceinline__ float akv_lane_xor(float v) {
+  return __uint_as_float(akv_lane_xor_u32<M>(__float_as_uint(v)));
+}
+template <int M> __device__ __forceinline__ int akv_lane_xor(int v) { return (int)akv_lane_xor_u32<M>((uint32_t)v); }
+
+// ----------------------------------------------------------------------------------
+// device: wavefront (64-lane) reductions; every lane receives the result.  (The butterfly of a shuffle loop
+// -- partner lane ^ 32 first, lane ^ 1 last -- so the sums round as they always did.)
 // ----------------------------------------------------------------------------------
 __device__ __forceinline__ float akv_wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, AKV_WAVE);
+  v += akv_lane_xor<32>(v);
+  v += akv_lane_xor<16>(v);
+  v += akv_lane_xor<8>(v);
+  v += akv_lane_xor<4>(v);
+  v += akv_lane_xor<2>(v);
+  v += akv_lane_xor<1>(v);
   return v;
 }
 __device__ __forceinline__ float akv_wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, AKV_WAVE));
+  v = fmaxf(v, akv_lane_xor<32>(v));
+  v = fmaxf(v, akv_lane_xor<16>(v));
+  v = fmaxf(v, akv_lane_xor<8>(v));
+  v = fmaxf(v, akv_lane_xor<4>(v));
+  v = fmaxf(v, akv_lane_xor<2>(v));
+  v = fmaxf(v, akv_lane_xor<1>(v));
   return v;
+}
+__device__ __forceinline__ int akv_wave_sum(int v) {
+  v += akv_lane_xor<32>(v);
+  v += akv_lane_xor<16>(v);
+  v += akv_lane_xor<8>(v);
+  v += akv_lane_xor<4>(v);
+  v += akv_lane_xor<2>(v);
+  v += akv_lane_xor<1>(v);
+  return v;
+}
+// inclusive prefix sum over the 64 lanes: shifts inside the rows of sixteen (lanes without a source add zero),
+// then the totals of the rows below
+__device__ __forceinline__ int akv_wave_inclusive_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111 /*row_shr:1*/, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112 /*row_shr:2*/, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114 /*row_shr:4*/, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118 /*row_shr:8*/, 0xf, 0xf, true);
+  const int t0 = __builtin_amdgcn_readlane(v, 15), t1 = __builtin_amdgcn_readlane(v, 31), t2 = __builtin_amdgcn_readlane(v, 47);
+  const int row = (threadIdx.x & 63) >> 4;
+  return v + (row >= 1 ? t0 : 0) + (row >= 2 ? t1 : 0) + (row >= 3 ? t2 : 0);
 }
 
 // ----------------------------------------------------------------------------------

@@ -418,12 +418,12 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       const bool g1 = (g & 1) != 0;
       float mine;
       if constexpr (MT == 1) {
-        const float a01 = ss[0] + __shfl_xor(ss[0], 16, 64);
-        mine = a01 + __shfl_xor(a01, 32, 64);                 // all four lanes of a row hold its sum
+        const float a01 = ss[0] + akv_lane_xor<16>(ss[0]);     // (row swaps, not shuffles: the step waits for this chain)
+        mine = a01 + akv_lane_xor<32>(a01);                   // all four lanes of a row hold its sum
       } else {
         static_assert(MT <= 2, "two M-tiles at most");
-        const float a01 = (g1 ? ss[MT - 1] : ss[0]) + __shfl_xor(g1 ? ss[0] : ss[MT - 1], 16, 64);
-        mine = a01 + __shfl_xor(a01, 32, 64);                 // lanes g and g + 2 both hold M-tile g & 1
+        const float a01 = (g1 ? ss[MT - 1] : ss[0]) + akv_lane_xor<16>(g1 ? ss[0] : ss[MT - 1]);
+        mine = a01 + akv_lane_xor<32>(a01);                   // lanes g and g + 2 both hold M-tile g & 1
       }
       const float nrm = sqrtf(mine);
       const uint32_t my_unscale = (MT > 1 && g1) ? unscale[MT - 1] : unscale[0];

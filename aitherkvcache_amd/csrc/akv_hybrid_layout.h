@@ -21,12 +21,18 @@
 #define HYB_BND1 275
 
 // 64-point Walsh-Hadamard transform across the lanes of a wavefront
+template <int H>
+__device__ __forceinline__ float hyb_fwht_step(float v, int lane) {
+  const float o = akv_lane_xor<H>(v);
+  return (lane & H) ? akv_sub_rn(o, v) : akv_add_rn(v, o);
+}
 __device__ __forceinline__ float hyb_fwht64(float v, int lane) {
-#pragma unroll
-  for (int h = 1; h < 64; h <<= 1) {
-    const float o = __shfl_xor(v, h, AKV_WAVE);
-    v = (lane & h) ? akv_sub_rn(o, v) : akv_add_rn(v, o);
-  }
+  v = hyb_fwht_step<1>(v, lane);
+  v = hyb_fwht_step<2>(v, lane);
+  v = hyb_fwht_step<4>(v, lane);
+  v = hyb_fwht_step<8>(v, lane);
+  v = hyb_fwht_step<16>(v, lane);
+  v = hyb_fwht_step<32>(v, lane);
   return v;
 }
 
