@@ -329,9 +329,9 @@ int akv_tri_scores(const void* query, int q_dtype,
  *   0..ctx-1; query_pos [B] or NULL (= ctx); out [B][QH][d] float32, zeros where ctx == 0.
  *   Coefficients are int4 (the only width the reference's cache stores, cache.py:66-85); pre_rope as for
  *   akv_tri_decode_step.
- * Workspace as for akv_tri_decode_step.  Built for d = 128, num_freqs = 12, at most 8 kv heads
- * and 4-byte aligned arrays; anything else returns AKV_ERR_UNSUPPORTED (gather, then
- * akv_tri_decode_step).
+ * Workspace as for akv_tri_decode_step.  Built for d = 128, num_freqs = 12, at most 8 kv heads,
+ * 4-byte aligned arrays and max_blocks_per_seq * block_size < 2^30; anything else returns
+ * AKV_ERR_UNSUPPORTED (gather, then akv_tri_decode_step).
  * ------------------------------------------------------------------------------- */
 int akv_tri_decode_paged(const void* query, int q_dtype,
                          const uint8_t* k_indices, const uint8_t* k_coeffs, const void* k_scales,
