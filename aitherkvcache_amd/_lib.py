@@ -77,6 +77,16 @@ SIGNATURES = {
                                    _p, _i, _i64, _i64,
                                    _i, _i, _i, _i, _i64, _i64, _f,
                                    _p, _sz, _p]),
+    "akv_hybrid25_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
+    "akv_hybrid25_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
+                                       _p, _i64, _i64, _i64, _i, _i64, _p]),
+    "akv_hybrid25_decode": (_i, [_p, _i64, _i64, _p, _p, _i64, _p]),
+    "akv_hybrid25_paged_attn": (_i, [_p, _i, _i64, _i64,
+                                     _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,
+                                     _p, _i, _i64, _p, _i, _p,
+                                     _p, _i, _i64, _i64,
+                                     _i, _i, _i, _i, _i64, _i64, _f,
+                                     _p, _sz, _p]),
     "akv_block_rep_update": (_i, [_p, _i, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "akv_block_rep_finalize": (_i, [_p, _i, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "akv_block_scores": (_i, [_p, _p, _p, _p, _p, _i, _i64, _p, _i, _i, _i, _i, _i, _i64, _i, _i64, _p, _p]),

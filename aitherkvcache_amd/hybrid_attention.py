@@ -1,11 +1,11 @@
-"""Encode-on-write and paged decode attention for the tq35 hybrid cache.
+"""Encode-on-write and paged decode attention for the hybrid (tq35 / tq25) cache.
 
 The reference has no fused path for hybrid data: its tq::hybrid_decode_step
 (aither_kvcache/vllm/hooks.py:240-345) encodes the new token, decompresses every block the
 batch addresses with HybridTurboQuant.decode and runs dense SDPA.  Here the same attention
-(softmax(q K^T * scale) V over the decoded rows) is computed directly on the packed 64-byte
-rows by one kernel sequence, and the new token is written by one scatter kernel.
-Cache tensors are uint8 [num_blocks, block_size, num_kv_heads, >= 64] (norms are inside the
+(softmax(q K^T * scale) V over the decoded rows) is computed directly on the packed rows (64 bytes
+for tq35, 44 for tq25) by one kernel sequence, and the new token is written by one scatter kernel.
+Cache tensors are uint8 [num_blocks, block_size, num_kv_heads, >= packed_dim] (norms are inside the
 rows); strided views with 4-byte aligned rows are accepted.
 """
 from typing import Optional
@@ -17,7 +17,7 @@ from . import _lib
 
 def hybrid_encode_and_store(htq, x: torch.Tensor, slot_mapping: torch.Tensor, cache: torch.Tensor,
                             block_size: int = 16, max_blocks: int = 0) -> None:
-    """Write x [num_tokens, num_kv_heads, 128] into cache[blk, pos, head, :64] for
+    """Write x [num_tokens, num_kv_heads, 128] into cache[blk, pos, head, :packed_dim] for
     slot = blk * block_size + pos; negative slots and blocks >= max_blocks are skipped."""
     if max_blocks == 0:
         max_blocks = cache.shape[0]
@@ -36,7 +36,7 @@ def hybrid_encode_and_store(htq, x: torch.Tensor, slot_mapping: torch.Tensor, ca
     if x.stride(-1) != 1:
         x = x.contiguous()
     slots = slot_mapping if slot_mapping.is_contiguous() else slot_mapping.contiguous()
-    _lib.check(_lib.lib().akv_hybrid_encode_paged(
+    _lib.check(getattr(_lib.lib(), htq._abi + "_encode_paged")(
         x.data_ptr(), _lib.dtype_code(x), num_tokens, num_kv_heads, x.stride(0), x.stride(1),
         slots.data_ptr(), _lib.itype_code(slots), table.data_ptr(),
         cache.data_ptr(), cache.stride(0), cache.stride(1), cache.stride(2),
@@ -80,8 +80,8 @@ class HybridPagedAttention:
         if num_seqs == 0:
             return out
         for name, t in (("k_cache", k_cache), ("v_cache", v_cache)):
-            if t.dtype != torch.uint8 or t.stride(-1) != 1 or t.shape[-1] < 64:
-                raise ValueError(f"{name} must be uint8 with contiguous rows of >= 64 bytes")
+            if t.dtype != torch.uint8 or t.stride(-1) != 1 or t.shape[-1] < self._htq.packed_dim:
+                raise ValueError(f"{name} must be uint8 with contiguous rows of >= {self._htq.packed_dim} bytes")
         bt = block_tables if block_tables.stride(-1) == 1 else block_tables.contiguous()
         cl = context_lens if context_lens.is_contiguous() else context_lens.contiguous()
         L = _lib.lib()
@@ -89,7 +89,7 @@ class HybridPagedAttention:
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != dev:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=dev)
         ws = self._workspace
-        _lib.check(L.akv_hybrid_paged_attn(
+        _lib.check(getattr(L, self._htq._abi + "_paged_attn")(
             q.data_ptr(), _lib.dtype_code(q), q.stride(0), q.stride(1),
             k_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
             v_cache.data_ptr(), v_cache.stride(0), v_cache.stride(1), v_cache.stride(2),

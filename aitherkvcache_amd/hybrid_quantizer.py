@@ -1,17 +1,19 @@
-"""Hybrid bit-width quantizer (tq35) on MI355X, with the interface of the reference's
+"""Hybrid bit-width quantizer (tq35, tq25) on MI355X, with the interface of the reference's
 aither_kvcache/hybrid_quantizer.py (HybridTurboQuant.encode/decode/calibrate_uniform, layouts).
 
-A 128-d vector is split into dims [0,64) and [64,128).  Each half is L2-normalised, rotated
+tq35: a 128-d vector is split into dims [0,64) and [64,128).  Each half is L2-normalised, rotated
 by a sign-flipped 64-point Walsh-Hadamard transform, scalar-quantised (3-bit / 2-bit
 Lloyd-Max codebook of the sphere-coordinate Beta law), and the residual is sketched with one
 sign bit per coordinate after a second sign-flipped Hadamard transform (QJL).  The two norms
 of a half travel as fp16 inside the 64-byte row (hybrid_quantizer.py:92-123,706-779).
+tq25: dims [0,32) at 2 bits and [32,128) at 1 bit, 44-byte rows; the 96 coordinates of the second
+group are transformed as a 64-point and a 32-point block and divided by sqrt(96), as the reference's
+fwht_general does (hybrid_quantizer.py:154-193) -- not a unitary transform, and kept that way.
 
 encode / decode are HIP kernels (one wavefront per vector, butterflies across lanes); the
 codebooks and sign vectors are built on the host at construction, as in the reference.
-Only `tq35` has kernels.  `calibrate_uniform()` is the configuration they are written for;
-`calibrate(sample)` runs the same kernels on coordinates permuted into group order.  `tq25` is
-recognised (layout arithmetic works) but raises NotImplementedError when used.
+`calibrate_uniform()` is the configuration the kernels are written for; `calibrate(sample)` runs the
+same kernels on coordinates permuted into group order.  head_dim is 128.
 """
 from __future__ import annotations
 
@@ -74,6 +76,14 @@ def _make_hybrid_layout(head_dim: int, mode: str) -> HybridLayout:
 # iteration leaves there is summation noise (0.0 for the 3-bit book, -2**-58 for the 2-bit
 # book), and it decides which code an all-zero group receives -- so the literal values are
 # kept.  Decoded values do not depend on it (such a group has norm 0).
+# (tq25: the one-bit book's only boundary is such noise, -2**-57)
+_TQ25_BOOKS = {
+    (32, 2): (np.array([-0.26338478922843933, -0.07983556389808655, 0.07983556389808655,
+                        0.26338478922843933], dtype=np.float32),
+              np.array([-0.17161017656326294, 0.0, 0.17161017656326294], dtype=np.float32)),
+    (96, 1): (np.array([-0.08164610713720322, 0.08164610713720322], dtype=np.float32),
+              np.array([-6.938893903907228e-18], dtype=np.float32)),
+}
 _TQ35_D64 = {
     3: (np.array([-0.264565646648407, -0.16685186326503754, -0.09433808922767639,
                   -0.03065413422882557, 0.03065413422882557, 0.09433808922767639,
@@ -164,6 +174,8 @@ def dimension_aware_codebook(dim: int, bits: int) -> Tuple[torch.Tensor, torch.T
     """(centroids [2^bits], inner boundaries [2^bits - 1]) float32 CPU tensors."""
     if dim == 64 and bits in _TQ35_D64:
         c, b = _TQ35_D64[bits]
+    elif (dim, bits) in _TQ25_BOOKS:
+        c, b = _TQ25_BOOKS[(dim, bits)]
     else:
         c, b = _lloyd_on_grid(dim, bits)
     return torch.from_numpy(c.copy()), torch.from_numpy(b.copy())
@@ -171,7 +183,7 @@ def dimension_aware_codebook(dim: int, bits: int) -> Tuple[torch.Tensor, torch.T
 
 class HybridTurboQuant:
     """htq = HybridTurboQuant(head_dim=128, mode="tq35"); htq.calibrate_uniform()
-    packed = htq.encode(kv)        # uint8 [..., 64]
+    packed = htq.encode(kv)        # uint8 [..., 64] (tq25: [..., 44])
     kv_hat = htq.decode(packed)    # float32 [..., 128]
     """
 
@@ -221,6 +233,14 @@ class HybridTurboQuant:
             tab[256:264], tab[264:268] = c0, c1
             tab[268:275], tab[275:278] = bnd0, bnd1
             self._table = tab.to(device)
+        elif mode == "tq25" and head_dim == 128:
+            tab = torch.zeros(_lib.HYB_TABLE_FLOATS, dtype=torch.float32)
+            tab[0:32], tab[32:128], tab[128:160], tab[160:256] = signs
+            tab[256:260], tab[260:262] = c0, c1
+            tab[262:265], tab[265:266] = bnd0, bnd1
+            self._table = tab.to(device)
+        # entry points of the mode (include/aitherkv.h)
+        self._abi = "akv_hybrid25" if mode == "tq25" else "akv_hybrid"
 
     # -- calibration ----------------------------------------------------------------------
     def calibrate_uniform(self, num_kv_heads: int = 1) -> None:
@@ -295,8 +315,7 @@ class HybridTurboQuant:
                                "before encode/decode.")
         if self._table is None:
             raise NotImplementedError(
-                f"HIP kernels exist for mode 'tq35' at head_dim 128 only (got {self.mode!r}, "
-                f"head_dim {self.head_dim})")
+                f"HIP kernels exist for head_dim 128 only (got mode {self.mode!r}, head_dim {self.head_dim})")
 
     @property
     def kernel_table(self) -> torch.Tensor:
@@ -305,7 +324,7 @@ class HybridTurboQuant:
 
     # -- encode / decode --------------------------------------------------------------------
     def encode(self, x: torch.Tensor) -> torch.Tensor:
-        """[..., 128] float -> uint8 [..., 64]."""
+        """[..., 128] float -> uint8 [..., packed_dim] (64 for tq35, 44 for tq25)."""
         self._ensure_ready()
         assert x.shape[-1] == self.head_dim, f"Expected last dim {self.head_dim}, got {x.shape[-1]}"
         dev = _lib.require_gpu(x, self._table)
@@ -317,13 +336,13 @@ class HybridTurboQuant:
             xf = xf.contiguous()
         n = xf.shape[0]
         out = torch.empty(n, self.layout.packed_dim, dtype=torch.uint8, device=dev)
-        _lib.check(_lib.lib().akv_hybrid_encode(
+        _lib.check(getattr(_lib.lib(), self._abi + "_encode")(
             xf.data_ptr(), _lib.dtype_code(xf), n, xf.stride(0) if n else self.head_dim,
             self._table.data_ptr(), out.data_ptr(), self.layout.packed_dim, _lib.stream_ptr(dev)))
         return out.reshape(batch + [self.layout.packed_dim])
 
     def decode(self, packed: torch.Tensor) -> torch.Tensor:
-        """uint8 [..., 64] -> float32 [..., 128]."""
+        """uint8 [..., packed_dim] -> float32 [..., 128]."""
         self._ensure_ready()
         assert packed.shape[-1] == self.layout.packed_dim, \
             f"Expected last dim {self.layout.packed_dim}, got {packed.shape[-1]}"
@@ -334,7 +353,7 @@ class HybridTurboQuant:
             pf = pf.contiguous()
         n = pf.shape[0]
         out = torch.empty(n, self.head_dim, dtype=torch.float32, device=dev)
-        _lib.check(_lib.lib().akv_hybrid_decode(
+        _lib.check(getattr(_lib.lib(), self._abi + "_decode")(
             pf.data_ptr(), pf.stride(0) if n else self.layout.packed_dim, n, self._table.data_ptr(),
             out.data_ptr(), self.head_dim, _lib.stream_ptr(dev)))
         return self.from_group_order(out).reshape(batch + [self.head_dim])

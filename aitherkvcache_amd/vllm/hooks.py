@@ -77,7 +77,7 @@ def decode_step(query, key, value, kv_cache, output, k_norms, v_norms, slot_mapp
 def hybrid_decode_step(query, key, value, kv_cache, output, slot_mapping, block_table, seq_lens,
                        layer_idx: int, num_heads: int, num_kv_heads: int, head_size: int,
                        scale: float, num_actual: int) -> torch.Tensor:
-    """Body of tq::hybrid_decode_step; kv_cache uint8 [blocks, 2, block_size, kv_heads, 64]."""
+    """Body of tq::hybrid_decode_step; kv_cache uint8 [blocks, 2, block_size, kv_heads, packed_dim] (64 bytes for tq35, 44 for tq25)."""
     htq = _tq_quantizers[head_size]
     key_cache, value_cache = kv_cache[:, 0], kv_cache[:, 1]
     block_size = key_cache.shape[1]

@@ -281,6 +281,42 @@ int akv_hybrid_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------
+ * HybridTurboQuant, mode tq25 with calibrate_uniform() groups (dims 0..31 at 2-bit MSE, dims 32..127
+ * at 1-bit MSE, each with a 1-bit QJL residual sketch and fp16 norms inside the 44-byte row; the 96
+ * coordinates of group 1 are transformed as a 64-point and a 32-point block and divided by sqrt(96)) --
+ * aither_kvcache/hybrid_quantizer.py:59-65 (mode), :154-193 (transform of 96 points), :616-779 (encode),
+ * :785-933 (decode).  Same arguments as the tq35 entry points above; `hyb_table` is a device
+ * float32[AKV_HYB_TABLE_FLOATS] laid out as
+ *   [0,128)   Hadamard signs in coordinate order (group 0's 32, then group 1's 96)
+ *   [128,256) QJL signs likewise
+ *   [256,260) group-0 centroids (4)     [260,262) group-1 centroids (2)
+ *   [262,265) group-0 boundaries (3)    [265]     group-1 boundary
+ * Rows: [0,8) group-0 codes, [8,12) group-0 sign bits, [12,16) group-0 norm and residual norm (fp16 LE),
+ * [16,28) group-1 codes, [28,40) group-1 sign bits, [40,44) group-1 norms.  head_dim is 128.
+ * akv_hybrid25_paged_attn is the attention of tq::hybrid_decode_step (aither_kvcache/vllm/hooks.py:240-345)
+ * on such rows; its workspace has the size akv_hybrid_paged_attn_workspace_bytes gives.
+ * ------------------------------------------------------------------------------- */
+#define AKV_HYB25_PACKED_BYTES 44
+int akv_hybrid25_encode(const void* x, int x_dtype, int64_t n, int64_t x_stride,
+                        const float* hyb_table, uint8_t* out, int64_t out_stride_bytes, void* stream);
+int akv_hybrid25_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads,
+                              int64_t xs_token, int64_t xs_head,
+                              const void* slot_mapping, int slot_itype, const float* hyb_table,
+                              uint8_t* out, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                              int block_size, int64_t max_blocks, void* stream);
+int akv_hybrid25_decode(const uint8_t* packed, int64_t packed_stride_bytes, int64_t n,
+                        const float* hyb_table, float* out, int64_t out_stride, void* stream);
+int akv_hybrid25_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,
+                            const uint8_t* k_cache, int64_t kps_blk, int64_t kps_pos, int64_t kps_head,
+                            const uint8_t* v_cache, int64_t vps_blk, int64_t vps_pos, int64_t vps_head,
+                            const void* block_tables, int bt_itype, int64_t bt_stride,
+                            const void* context_lens, int cl_itype, const float* hyb_table,
+                            void* out, int out_dtype, int64_t os_seq, int64_t os_head,
+                            int num_seqs, int num_q_heads, int num_kv_heads,
+                            int block_size, int64_t num_blocks, int64_t max_blocks_per_seq, float scale,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------
  * TriAttention.decode_step -- aither_kvcache/triattention/attention.py:186-280 with
  * TrigSeriesScorer.score (scorer.py:115-208):
  *   k/v_indices [B][S][KVH][F] uint8; k/v_coeffs by coeff_bits (scorer.py:84-113):

@@ -1,4 +1,4 @@
-"""CPU oracle for the TurboQuant / tq35 / TriAttention hot path  --  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the TurboQuant / tq35 and tq25 / TriAttention hot path  --  TEST INFRASTRUCTURE ONLY.
 
 This module is a plain numpy restatement of the reference's algorithm for the
 path (encode-on-write -> paged decode attention -> TriAttention decode_step).
@@ -18,18 +18,20 @@ reference tree).  How each one is pinned:
       batch_decompress_active_blocks (its decode by the golden vectors; its block
       selection and scatter by a per-block loop in tests/test_oracle_pins.py),
       fwht, structured_hadamard, dimension_aware_codebook,
-      hybrid_encode, hybrid_decode, rope_frequencies, spectral_encode,
+      hybrid_encode, hybrid_decode (mode tq25, with fwht_general over 96 points, by
+      tests/golden/golden_tq25.npz, also written by the reference itself, and by the block
+      structure of the 96-point matrix), rope_frequencies, spectral_encode,
       tri_scores, tri_decode_step (coefficient widths 8 / 16 and post-RoPE scoring by
       tests/golden/golden_tri_widths.npz, also written by the reference itself),
       spectral_fetch_sequence / tri_decode_step_paged (indexing only, on top of the pinned
       tri_decode_step: checked against a token-by-token loop in tests/test_oracle_pins.py)
   derived here (the reference has no such function; it always decompresses
-  tq35 data before attending): hybrid_paged_attention is *defined* as
+  tq35 / tq25 data before attending): hybrid_paged_attention is *defined* as
   hybrid_decode -> dense f32 softmax attention, i.e. the reference's
   tq::hybrid_decode_step (vllm/hooks.py:294-345) without its bf16 down-cast.
 
 Inputs that only torch's CPU generator / LAPACK can produce (the rotation matrix
-and the tq35 sign vectors) are arguments here; the tests take them from the
+and the tq35 / tq25 sign vectors) are arguments here; the tests take them from the
 golden file.
 """
 from __future__ import annotations
@@ -472,7 +474,7 @@ def block_select(scores, block_tables, context_lens, block_size, max_selected, n
 
 
 # --------------------------------------------------------------------------------------
-# hybrid_quantizer.py (tq35, calibrate_uniform)
+# hybrid_quantizer.py (tq35 and tq25, calibrate_uniform)
 # --------------------------------------------------------------------------------------
 def fwht(x):
     """fwht_pow2, hybrid_quantizer.py:130-151: unnormalised Walsh-Hadamard butterflies over the
@@ -490,13 +492,30 @@ def fwht(x):
     return x
 
 
+def fwht_general(x):
+    """fwht_general, hybrid_quantizer.py:154-193: a length that is no power of two is cut into
+    descending powers of two (96 = 64 + 32) and every piece is transformed on its own."""
+    x = np.asarray(x, dtype=f32)
+    n = x.shape[-1]
+    if n > 0 and (n & (n - 1)) == 0:
+        return fwht(x)
+    out, at = np.array(x, dtype=f32, copy=True), 0
+    while n > 0:
+        p = 1 << (n.bit_length() - 1)
+        out[..., at:at + p] = fwht(x[..., at:at + p])
+        at, n = at + p, n - p
+    return out
+
+
 def structured_hadamard(x, signs, inverse=False):
-    """structured_hadamard, hybrid_quantizer.py:200-234 with normalized=True."""
+    """structured_hadamard, hybrid_quantizer.py:200-234 with normalized=True (the division by
+    sqrt(dim) is a float32 division by the float32 value of the square root, as torch's CPU
+    kernel divides a float32 tensor by a Python number)."""
     dim = x.shape[-1]
     if inverse:
-        y = fwht(x) * signs
+        y = fwht_general(x) * signs
     else:
-        y = fwht(x * signs)
+        y = fwht_general(x * signs)
     return (y / f32(math.sqrt(dim))).astype(f32)
 
 
@@ -555,26 +574,30 @@ def unpack_multibit(packed, dim, bits):
 
 
 class HybridParams:
-    """The constants HybridTurboQuant(head_dim=128, mode='tq35') holds after
-    calibrate_uniform(): hybrid_quantizer.py:52-58,92-123,486-547,590-603.
+    """The constants HybridTurboQuant(head_dim=128, mode) holds after calibrate_uniform():
+    hybrid_quantizer.py:52-65,92-123,486-547,590-603.  tq35: dims 0..63 at 3 bits and 64..127 at
+    2 bits (64-byte rows); tq25: dims 0..31 at 2 bits and 32..127 at 1 bit (44-byte rows).
     The sign vectors come from torch's CPU generator (seed 42) and are arguments."""
 
-    def __init__(self, g0_had, g1_had, g0_qjl, g1_qjl, head_dim=128, codebooks=None):
+    def __init__(self, g0_had, g1_had, g0_qjl, g1_qjl, head_dim=128, codebooks=None, mode="tq35"):
         assert head_dim == 128
         self.head_dim = head_dim
-        self.g_dim = (64, 64)
-        self.mse_bits = (3, 2)
+        self.mode = mode
+        self.g_dim = {"tq35": (64, 64), "tq25": (32, 96)}[mode]
+        self.mse_bits = {"tq35": (3, 2), "tq25": (2, 1)}[mode]
         self.had = (np.asarray(g0_had, f32), np.asarray(g1_had, f32))
         self.qjl = (np.asarray(g0_qjl, f32), np.asarray(g1_qjl, f32))
+        assert self.had[0].shape == (self.g_dim[0],) and self.had[1].shape == (self.g_dim[1],)
         if codebooks is None:
-            codebooks = (dimension_aware_codebook(64, 3), dimension_aware_codebook(64, 2))
+            codebooks = tuple(dimension_aware_codebook(self.g_dim[g], self.mse_bits[g]) for g in (0, 1))
         self.centroids = (codebooks[0][0], codebooks[1][0])
         self.boundaries = (codebooks[0][1], codebooks[1][1])
-        self.qjl_scale = (math.sqrt(math.pi / 2.0) / 64, math.sqrt(math.pi / 2.0) / 64)
+        self.qjl_scale = tuple(math.sqrt(math.pi / 2.0) / self.g_dim[g] for g in (0, 1))
         # byte layout: [mse | qjl bits | norm fp16 | residual norm fp16] per group
-        self.mse_bytes = (24, 16)
-        self.group_bytes = (24 + 8 + 4, 16 + 8 + 4)
-        self.packed_dim = 64
+        self.mse_bytes = tuple(-(-self.g_dim[g] * self.mse_bits[g] // 8) for g in (0, 1))
+        self.sign_bytes = tuple(-(-self.g_dim[g] // 8) for g in (0, 1))
+        self.group_bytes = tuple(self.mse_bytes[g] + self.sign_bytes[g] + 4 for g in (0, 1))
+        self.packed_dim = sum(self.group_bytes)
 
 
 def _hybrid_encode_group(xg, hp: HybridParams, g):
@@ -596,20 +619,27 @@ def _hybrid_encode_group(xg, hp: HybridParams, g):
 
 
 def hybrid_encode(x, hp: HybridParams):
-    """HybridTurboQuant.encode with calibrate_uniform groups (dims 0..63 / 64..127),
+    """HybridTurboQuant.encode with calibrate_uniform groups (the first g0 dims / the rest),
     hybrid_quantizer.py:616-704."""
     x = np.asarray(x)
     flat = x.reshape(-1, 128).astype(f32)
-    out = np.concatenate([_hybrid_encode_group(flat[:, :64], hp, 0),
-                          _hybrid_encode_group(flat[:, 64:], hp, 1)], axis=-1)
-    return out.reshape(x.shape[:-1] + (64,))
+    d0 = hp.g_dim[0]
+    out = np.concatenate([_hybrid_encode_group(flat[:, :d0], hp, 0),
+                          _hybrid_encode_group(flat[:, d0:], hp, 1)], axis=-1)
+    return out.reshape(x.shape[:-1] + (hp.packed_dim,))
 
 
-def _hadamard_matrix64():
-    h = np.array([[1.0]])
-    while h.shape[0] < 64:
-        h = np.block([[h, h], [h, -h]])
-    return h
+def _hadamard_matrix(n):
+    """Float64 matrix of fwht_general over n points (block diagonal for 96 = 64 + 32), unnormalised."""
+    out, at = np.zeros((n, n)), 0
+    while n - at > 0:
+        p = 1 << ((n - at).bit_length() - 1)
+        h = np.array([[1.0]])
+        while h.shape[0] < p:
+            h = np.block([[h, h], [h, -h]])
+        out[at:at + p, at:at + p] = h
+        at += p
+    return out
 
 
 def hybrid_encode_margins(x, packed, hp: HybridParams):
@@ -630,13 +660,15 @@ def hybrid_encode_margins(x, packed, hp: HybridParams):
                             of the float64 value, in fp16 steps (bit patterns)
     Same operations as _hybrid_encode_group (hybrid_quantizer.py:706-779) carried in float64."""
     x = np.asarray(x).reshape(-1, 128).astype(f32).astype(np.float64)
-    packed = np.asarray(packed, dtype=np.uint8).reshape(-1, 64)
-    H = _hadamard_matrix64() / 8.0
+    packed = np.asarray(packed, dtype=np.uint8).reshape(-1, hp.packed_dim)
     out = {"code_ulps": [], "sign_ulps": [], "norm_steps": [], "rnorm_steps": []}
-    for g, (lo, off) in enumerate(((0, 0), (64, 36))):
-        xg = x[:, lo:lo + 64]
+    for g, (lo, off) in enumerate(((0, 0), (hp.g_dim[0], hp.group_bytes[0]))):
+        G = hp.g_dim[g]
+        # (the reference divides by the float32 value of sqrt(dim))
+        H = _hadamard_matrix(G) / float(f32(math.sqrt(G)))
+        xg = x[:, lo:lo + G]
         pg = packed[:, off:off + hp.group_bytes[g]]
-        mb = hp.mse_bytes[g]
+        mb, sb = hp.mse_bytes[g], hp.sign_bytes[g]
         n64 = np.sqrt(np.sum(xg * xg, axis=-1))
         # the reference divides by the float32 norm + 1e-10 (float32 arithmetic)
         unit = xg / (n64.astype(f32) + f32(1e-10)).astype(np.float64)[:, None]
@@ -644,7 +676,7 @@ def hybrid_encode_margins(x, packed, hp: HybridParams):
         rot = (unit * had) @ H
         b = hp.boundaries[g].astype(np.float64)
         idx64 = np.clip(np.searchsorted(b, rot, side="left"), 0, (1 << hp.mse_bits[g]) - 1)
-        idx = unpack_multibit(pg[:, :mb], 64, hp.mse_bits[g]).astype(np.int64)
+        idx = unpack_multibit(pg[:, :mb], G, hp.mse_bits[g]).astype(np.int64)
         # boundaries between the stored code and the float64 code: the farthest one decides
         far = np.where(idx > idx64, b[np.clip(idx - 1, 0, len(b) - 1)], b[np.clip(idx, 0, len(b) - 1)])
         # the rounding error of a butterfly sum is absolute, of the size of the terms summed: a result
@@ -656,10 +688,10 @@ def hybrid_encode_margins(x, packed, hp: HybridParams):
         res = unit - mse_hat
         rn64 = np.sqrt(np.sum(res * res, axis=-1))
         proj = (res * hp.qjl[g].astype(np.float64)) @ H
-        sgn = unpack_multibit(pg[:, mb:mb + 8], 64, 1).astype(bool)
+        sgn = unpack_multibit(pg[:, mb:mb + sb], G, 1).astype(bool)
         row_ulp = np.spacing(np.maximum(np.max(np.abs(proj), axis=-1), 1e-30).astype(f32)).astype(np.float64)
         out["sign_ulps"].append(np.where(sgn != (proj >= 0), np.abs(proj) / row_ulp[:, None], 0.0))
-        for key, val, at in (("norm_steps", n64, mb + 8), ("rnorm_steps", rn64, mb + 10)):
+        for key, val, at in (("norm_steps", n64, mb + sb), ("rnorm_steps", rn64, mb + sb + 2)):
             stored = np.ascontiguousarray(pg[:, at:at + 2]).view(np.uint16).reshape(-1).astype(np.int64)
             want = val.astype(np.float16).view(np.uint16).astype(np.int64)
             out[key].append(stored - want)
@@ -668,22 +700,23 @@ def hybrid_encode_margins(x, packed, hp: HybridParams):
 
 def _hybrid_decode_group(pg, hp: HybridParams, g):
     """_decode_single_group, hybrid_quantizer.py:876-933."""
-    mb = hp.mse_bytes[g]
-    idx = unpack_multibit(pg[:, :mb], 64, hp.mse_bits[g]).astype(np.int64)
+    mb, sb, G = hp.mse_bytes[g], hp.sign_bytes[g], hp.g_dim[g]
+    idx = unpack_multibit(pg[:, :mb], G, hp.mse_bits[g]).astype(np.int64)
     mse_hat = structured_hadamard(hp.centroids[g][idx], hp.had[g], inverse=True)
-    sgn = 2.0 * unpack_multibit(pg[:, mb:mb + 8], 64, 1).astype(f32) - 1.0
+    sgn = 2.0 * unpack_multibit(pg[:, mb:mb + sb], G, 1).astype(f32) - 1.0
     qjl_hat = structured_hadamard((sgn * f32(hp.qjl_scale[g])).astype(f32), hp.qjl[g], inverse=True)
-    n = np.ascontiguousarray(pg[:, mb + 8:mb + 10]).view(np.float16).reshape(-1).astype(f32)
-    rn = np.ascontiguousarray(pg[:, mb + 10:mb + 12]).view(np.float16).reshape(-1).astype(f32)
+    n = np.ascontiguousarray(pg[:, mb + sb:mb + sb + 2]).view(np.float16).reshape(-1).astype(f32)
+    rn = np.ascontiguousarray(pg[:, mb + sb + 2:mb + sb + 4]).view(np.float16).reshape(-1).astype(f32)
     return ((mse_hat + qjl_hat * rn[:, None]) * n[:, None]).astype(f32)
 
 
 def hybrid_decode(packed, hp: HybridParams):
     """HybridTurboQuant.decode, hybrid_quantizer.py:785-874; returns float32."""
     packed = np.asarray(packed, dtype=np.uint8)
-    flat = packed.reshape(-1, 64)
-    out = np.concatenate([_hybrid_decode_group(flat[:, :36], hp, 0),
-                          _hybrid_decode_group(flat[:, 36:], hp, 1)], axis=-1)
+    flat = packed.reshape(-1, hp.packed_dim)
+    b0 = hp.group_bytes[0]
+    out = np.concatenate([_hybrid_decode_group(flat[:, :b0], hp, 0),
+                          _hybrid_decode_group(flat[:, b0:], hp, 1)], axis=-1)
     return out.reshape(packed.shape[:-1] + (128,))
 
 
@@ -704,7 +737,7 @@ def hybrid_paged_attention(query, k_cache, v_cache, block_tables, context_lens, 
                            scale, block_size=16, dtype=f32):
     """tq::hybrid_decode_step's attention (vllm/hooks.py:294-345) in float32: decompress every
     addressed token with hybrid_decode, mask by context length, dense softmax attention.
-    Caches are [blocks, block_size, KVH, 64] uint8.  Returns float32 [S, QH, D]."""
+    Caches are [blocks, block_size, KVH, hp.packed_dim] uint8.  Returns float32 [S, QH, D]."""
     query = np.asarray(query)
     S, QH, D = query.shape
     out = np.zeros((S, QH, D), dtype=dtype)

@@ -32,3 +32,10 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="session")
+def tq25():
+    """HybridTurboQuant in mode tq25 (sign vectors, codebooks, encode / decode), produced by the reference
+    itself (tests/golden/make_golden_tq25.py)."""
+    return np.load(os.path.join(ROOT, "tests", "golden", "golden_tq25.npz"))

@@ -176,10 +176,36 @@ def test_hybrid_layout_and_errors():
     with pytest.raises(RuntimeError, match="HIP devices only"):
         h.encode(torch.zeros(1, 128))
     assert h.compression_ratio() == 4.0 and "calibrated" in repr(h)
+    with pytest.raises(NotImplementedError, match="head_dim 128 only"):
+        h64 = HybridTurboQuant(head_dim=64, device="cpu")
+        h64.calibrate_uniform()
+        h64.encode(torch.zeros(1, 64))
+
+
+def test_tq25_constants_match_the_reference(tq25):
+    """Mode tq25 on the host: the sign vectors of seed 42, the two codebooks (literal tables: the one-bit
+    book's boundary is float64 summation noise in the reference) and the kernel table's layout."""
     t = HybridTurboQuant(mode="tq25", device="cpu")
-    t.calibrate_uniform()
-    with pytest.raises(NotImplementedError):
+    assert (t._g0_dim, t._g1_dim, t._g0_mse_bits, t._g1_mse_bits, t.packed_dim) == (32, 96, 2, 1, 44)
+    for nm, got in (("g0_had", t._g0_had_signs), ("g1_had", t._g1_had_signs), ("g0_qjl", t._g0_qjl_signs),
+                    ("g1_qjl", t._g1_qjl_signs), ("g0_centroids", t._g0_centroids), ("g0_boundaries", t._g0_boundaries),
+                    ("g1_centroids", t._g1_centroids), ("g1_boundaries", t._g1_boundaries)):
+        assert np.array_equal(got.numpy(), tq25[nm]), nm
+    tab = t._table.numpy()
+    assert tab.shape == (_lib.HYB_TABLE_FLOATS,)
+    assert np.array_equal(tab[0:32], tq25["g0_had"]) and np.array_equal(tab[32:128], tq25["g1_had"])
+    assert np.array_equal(tab[128:160], tq25["g0_qjl"]) and np.array_equal(tab[160:256], tq25["g1_qjl"])
+    assert np.array_equal(tab[256:260], tq25["g0_centroids"]) and np.array_equal(tab[260:262], tq25["g1_centroids"])
+    assert np.array_equal(tab[262:265], tq25["g0_boundaries"]) and np.array_equal(tab[265:266], tq25["g1_boundaries"])
+    assert t._abi == "akv_hybrid25" and HybridTurboQuant(device="cpu")._abi == "akv_hybrid"
+    t.calibrate_uniform(num_kv_heads=2)
+    assert t._group0_indices.shape == (2, 32) and int(t._group1_indices[1, 0]) == 32
+    with pytest.raises(RuntimeError, match="HIP devices only"):
         t.encode(torch.zeros(1, 128))
+    # the grid iteration itself gives the same centroids as the literal tables
+    from aitherkvcache_amd.hybrid_quantizer import _lloyd_on_grid
+    for (d, b), nm in (((32, 2), "g0"), ((96, 1), "g1")):
+        assert np.array_equal(_lloyd_on_grid(d, b)[0], tq25[nm + "_centroids"])
 
 
 def test_tri_config_and_theta(golden):

@@ -360,3 +360,69 @@ def test_boundary_distance_counts_ulps_of_the_largest_term_under_cancellation():
     floored = O.boundary_ulp_distance(y, b, floor=np.array([0.018, 0.018]))
     assert abs(floored[0] - 3.99e-9 / np.spacing(np.float32(0.018))) < 1e-6 and floored[0] < 3
     assert floored[1] == plain[1]
+
+
+# ---- hybrid, mode tq25 -------------------------------------------------------------------------
+def tq25_params(tq25):
+    books = ((tq25["g0_centroids"], tq25["g0_boundaries"]), (tq25["g1_centroids"], tq25["g1_boundaries"]))
+    return O.HybridParams(tq25["g0_had"], tq25["g1_had"], tq25["g0_qjl"], tq25["g1_qjl"], codebooks=books, mode="tq25")
+
+
+def test_tq25_oracle_reproduces_the_reference_rows(tq25):
+    """Rows and decoded vectors of the reference itself (groups of 32 and 96 coordinates, 44-byte rows): the
+    oracle's encode and decode give them bit for bit, for one head and for two."""
+    hp = tq25_params(tq25)
+    assert hp.packed_dim == int(tq25["packed_dim"]) == 44 and hp.group_bytes == (16, 28)
+    assert np.array_equal(O.hybrid_encode(tq25["x"], hp), tq25["packed"])
+    assert np.array_equal(O.hybrid_decode(tq25["packed"], hp), tq25["decoded"])
+    assert np.array_equal(O.hybrid_encode(tq25["x_heads2"], hp), tq25["packed_heads2"])
+    assert np.array_equal(O.hybrid_decode(tq25["packed_heads2"], hp), tq25["decoded_heads2"])
+    # the grid iteration: centroids bit for bit; the middle boundary of a symmetric book is float64 summation
+    # noise in the reference (0.0 and -2^-57 here) and in the oracle's restatement alike
+    for nm, (d, b) in (("g0", (32, 2)), ("g1", (96, 1))):
+        c, bd = O.dimension_aware_codebook(d, b)
+        assert np.array_equal(c, tq25[nm + "_centroids"])
+        mid = len(bd) // 2
+        assert np.array_equal(np.delete(bd, mid), np.delete(tq25[nm + "_boundaries"], mid))
+        assert abs(float(bd[mid])) < 1e-16 and abs(float(tq25[nm + "_boundaries"][mid])) < 1e-16
+    m = O.hybrid_encode_margins(tq25["x"], tq25["packed"], hp)
+    assert all(float(np.abs(v[g]).max()) == 0 for v in m.values() for g in (0, 1))
+
+
+def test_transform_of_96_points_is_two_blocks():
+    """fwht_general on 96 points = a 64-point and a 32-point Hadamard matrix side by side; the structured
+    transform divides both by sqrt(96), so forward-then-inverse scales the blocks by 64/96 and 32/96 (the
+    reference's transform is not unitary at this length)."""
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((6, 96)).astype(np.float32)
+    H = O._hadamard_matrix(96)
+    assert np.array_equal(H[:64, 64:], np.zeros((64, 32))) and np.array_equal(H, H.T)
+    assert np.array_equal(H[:64, :64] @ H[:64, :64], 64 * np.eye(64)) and np.array_equal(H[64:, 64:] @ H[64:, 64:], 32 * np.eye(32))
+    assert np.allclose(O.fwht_general(x), x @ H, atol=1e-4)
+    assert np.array_equal(O.fwht_general(x[:, :64]), O.fwht(x[:, :64]))
+    s = np.sign(rng.standard_normal(96)).astype(np.float32)
+    back = O.structured_hadamard(O.structured_hadamard(x, s), s, inverse=True)
+    assert np.allclose(back[:, :64], x[:, :64] * (64 / 96), atol=1e-5)
+    assert np.allclose(back[:, 64:], x[:, 64:] * (32 / 96), atol=1e-5)
+
+
+def test_tq25_margins_catch_defects(tq25):
+    hp = tq25_params(tq25)
+    rng = np.random.default_rng(10)
+    x = (rng.standard_normal((2000, 128)) * rng.lognormal(0, 0.5, (2000, 1))).astype(np.float32)
+    p = O.hybrid_encode(x, hp)
+    m = O.hybrid_encode_margins(x, p, hp)
+    for g in (0, 1):
+        assert m["code_ulps"][g].max() <= 4 and m["sign_ulps"][g].max() <= 4
+        assert np.abs(m["norm_steps"][g]).max() <= 1 and np.abs(m["rnorm_steps"][g]).max() <= 1
+    bad = p.copy()
+    bad[7, 3] ^= 0x40          # a group-0 code bit
+    bad[9, 9] ^= 0x01          # a group-0 sign bit
+    bad[11, 20] ^= 0x40        # a group-1 code bit
+    bad[12, 33] ^= 0x02        # a group-1 sign bit
+    bad[13, 41] ^= 0x04        # group-1 norm, fp16 high byte
+    m = O.hybrid_encode_margins(x, bad, hp)
+    assert m["code_ulps"][0][7].max() > 1e3 and m["sign_ulps"][0][9].max() > 1e3
+    assert m["code_ulps"][1][11].max() > 1e3 and m["sign_ulps"][1][12].max() > 1e3
+    assert abs(int(m["norm_steps"][1][13])) > 100
+    assert m["code_ulps"][0][8].max() == 0 and m["sign_ulps"][1][9].max() == 0
