@@ -6,7 +6,7 @@ from typing import NamedTuple, Optional
 class CacheFormat(NamedTuple):
     kind: str             # "uniform" or "hybrid"
     bits: Optional[int]   # uniform: 4 / 3 / 2
-    mode: Optional[str]   # hybrid: "tq35"
+    mode: Optional[str]   # hybrid: "tq35" or "tq25"
     packed_bytes_d128: int
     norms_in_row: bool
 
@@ -17,6 +17,7 @@ KV_CACHE_DTYPES = {
     "tq-t2nc": CacheFormat("uniform", 2, None, 32, False),
     "tq-t35nc": CacheFormat("hybrid", None, "tq35", 64, True),
     "tq35": CacheFormat("hybrid", None, "tq35", 64, True),
+    "tq25": CacheFormat("hybrid", None, "tq25", 44, True),
 }
 
 

@@ -59,7 +59,10 @@ def slots_of(tables, s, start, stop):
     return [int(tables[s][p // BS]) * BS + p % BS for p in range(start, stop)]
 
 
-def hybrid_params(golden):
+def hybrid_params(golden, tq25=None):
+    if tq25 is not None:
+        books = ((tq25["g0_centroids"], tq25["g0_boundaries"]), (tq25["g1_centroids"], tq25["g1_boundaries"]))
+        return O.HybridParams(tq25["g0_had"], tq25["g1_had"], tq25["g0_qjl"], tq25["g1_qjl"], codebooks=books, mode="tq25")
     books = tuple((golden[f"hyb_centroids_64_{k}"], golden[f"hyb_boundaries_64_{k}"]) for k in (3, 2))
     return O.HybridParams(golden["hyb_g0_had_signs"], golden["hyb_g1_had_signs"],
                           golden["hyb_g0_qjl_signs"], golden["hyb_g1_qjl_signs"], codebooks=books)
@@ -197,13 +200,14 @@ def test_primary_decode_without_separate_cache_update(golden, dev, impl_cls):
     assert int((impl_cls._primary_k_norms[0] > 0).sum()) == 4 * 2 * KVH
 
 
-def test_primary_hybrid_decode(golden, dev, impl_cls):
-    layers, htq = make_layers(impl_cls, golden, dev, "tq35")
+@pytest.mark.parametrize("mode,row", [("tq35", 64), ("tq25", 44)])
+def test_primary_hybrid_decode(golden, tq25, dev, impl_cls, mode, row):
+    layers, htq = make_layers(impl_cls, golden, dev, mode)
     impl = layers[1]
-    hp = hybrid_params(golden)
+    hp = hybrid_params(golden, tq25 if mode == "tq25" else None)
     rng = np.random.default_rng(78)
-    kv_cache = torch.zeros(*B.TurboQuantBackend.get_kv_cache_shape(NB, BS, KVH, 128, "tq35"), dtype=torch.uint8, device=dev)
-    assert kv_cache.shape[-1] == 64
+    kv_cache = torch.zeros(*B.TurboQuantBackend.get_kv_cache_shape(NB, BS, KVH, 128, mode), dtype=torch.uint8, device=dev)
+    assert kv_cache.shape[-1] == row
     tables = np.array([[4, 8, 0], [1, 6, 0]], dtype=np.int32)
     hist = 21
     seen = {}
@@ -230,7 +234,7 @@ def test_primary_hybrid_decode(golden, dev, impl_cls):
     ref = O.hybrid_paged_attention(qd, kv_cache[:, 0].cpu().numpy(), kv_cache[:, 1].cpu().numpy(), tables,
                                    np.array([hist + 1, hist + 1]), hp, impl.scale, dtype=np.float64)
     assert np.max(np.abs(outd.view(2, QH, 128).cpu().numpy().astype(np.float64) - ref)) <= 2e-3
-    assert impl_cls._primary_k_norms is None            # tq35 rows carry their norms
+    assert impl_cls._primary_k_norms is None            # hybrid rows carry their norms
 
 
 def test_shadow_copy_serves_decode(golden, dev, impl_cls, monkeypatch):

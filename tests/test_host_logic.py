@@ -236,6 +236,7 @@ def test_kv_cache_dtype_names_and_ops():
     assert resolve_kv_cache_dtype("tq35").mode == "tq35"
     assert tq_dim_for_head(128, resolve_kv_cache_dtype("tq-t4nc")) == 68
     assert tq_dim_for_head(128, resolve_kv_cache_dtype("tq-t35nc")) == 64
+    assert resolve_kv_cache_dtype("tq25").mode == "tq25" and tq_dim_for_head(128, resolve_kv_cache_dtype("tq25")) == 44
     with pytest.raises(ValueError):
         resolve_kv_cache_dtype("fp8")
     assert register_custom_ops() and register_custom_ops()
