@@ -56,6 +56,16 @@ def test_library_loads_and_reports_version():
         _lib.check(rc)
     with pytest.raises(ValueError):
         _lib.check(_lib.AKV_ERR_INVALID)
+    # the tq25 entry points check like their tq35 counterparts: sizes, null pointers, rows shorter than 44 bytes
+    assert L.akv_hybrid25_encode(None, 0, 0, 128, None, None, 44, None) == _lib.AKV_OK
+    assert L.akv_hybrid25_encode(None, 0, -1, 128, None, None, 44, None) == _lib.AKV_ERR_INVALID
+    assert L.akv_hybrid25_encode(None, 0, 3, 128, None, None, 44, None) == _lib.AKV_ERR_INVALID
+    assert b"akv_hybrid25_encode" in L.akv_last_error()
+    buf = (ctypes.c_char * 4096)()
+    ptr = ctypes.addressof(buf)
+    assert L.akv_hybrid25_encode(ptr, 0, 3, 128, ptr, ptr, 43, None) == _lib.AKV_ERR_INVALID
+    assert L.akv_hybrid25_decode(ptr, 40, 3, ptr, ptr, 128, None) == _lib.AKV_ERR_INVALID
+    assert L.akv_hybrid25_decode(None, 44, 0, None, None, 128, None) == _lib.AKV_OK
 
 
 # ---- TurboQuant surface -------------------------------------------------------------------
