@@ -53,6 +53,9 @@ struct tri_args {
   const void* block_tables; int bt_itype; int64_t bt_stride;
   const void* context_lens; int cl_itype;
   int block_size; int64_t num_blocks;
+  // token -> block without a division: a shift when the block size is a power of two (bs_shift), else
+  // floor(t / block_size) = (t x bs_magic) >> (32 + bs_mshift), exact for t < 2^30 and block sizes from 3
+  int bs_shift; uint32_t bs_magic; int bs_mshift;
   float* part_acc;  // [B][QH][nsplit][D]
   float* part_ml;   // [B][QH][nsplit][2]
 };
@@ -545,7 +548,7 @@ typedef float tri_f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) const tri_u32x4 tri_lds_cu32x4;
 typedef __attribute__((address_space(3))) const tri_f32x4 tri_lds_cf32x4;
 
-template <int GQ, bool PAGED, bool QH16, bool KP>
+template <int GQ, bool PAGED, bool QH16, bool KP, bool BSP2>
 __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int KVH = a.KVH;
@@ -598,18 +601,55 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   const int s1m = s1 - 1;
 
   struct tri_rows { uint32_t x[2][3]; unsigned short sc; uint32_t kp_lo, kp_hi; };
+  // PAGED: the block table entry of the thread's token of a chunk, as two dwords (both index widths by the
+  // same two loads: a load under a branch would make every later wait a wait for all loads)
+  const bool bt_wide = PAGED && a.bt_itype == AKV_I64;
+  const unsigned char* bt_b = PAGED ? (const unsigned char*)a.block_tables + (int64_t)b * a.bt_stride * (bt_wide ? 8 : 4) : nullptr;
+  const uint32_t blk_last = BSP2 ? (uint32_t)max(s1m, 0) >> a.bs_shift : 0u;
+  const uint32_t blk_rows = (uint32_t)a.block_size * (uint32_t)KVH;
+  const uint32_t row_in_blk = ((uint32_t)(s0 + my_t) & (uint32_t)(a.block_size - 1)) * (uint32_t)KVH + (uint32_t)my_h;
+  uint32_t bt_lo = 0, bt_hi = 0;
+  auto table_entry = [&](int c0) {
+    uint32_t blk;
+    if constexpr (BSP2) {
+      blk = min((uint32_t)(c0 + my_t) >> a.bs_shift, blk_last);         // tokens past the range: its last block
+    } else {
+      const uint32_t tcl = (uint32_t)max(0, min(c0 + my_t, s1m));
+      blk = __umulhi(tcl, a.bs_magic) >> a.bs_mshift;
+    }
+    const uint32_t be = blk * (bt_wide ? 8u : 4u);
+    bt_lo = *(const uint32_t*)(bt_b + (size_t)be);
+    bt_hi = *(const uint32_t*)(bt_b + (size_t)be + (bt_wide ? 4 : 0));
+  };
   auto fetch = [&](tri_rows& rr, int c0) {
     const uint32_t* p0;
     const uint32_t* p1;
     if (PAGED) {
-      const int tcl = max(0, min(c0 + my_t, s1m));                      // tokens past the range: its last token
-      const int blk = tcl / a.block_size;
-      int64_t phys = akv_load_index(a.block_tables, a.bt_itype, (int64_t)b * a.bt_stride + blk);
-      phys = max((int64_t)0, min(phys, a.num_blocks - 1));                   // (an empty sequence reads a padding entry)
-      const int64_t row = ((phys * a.block_size) + (tcl - blk * a.block_size)) * KVH + my_h;
-      p0 = (const uint32_t*)(src_idx + row * 12);
-      p1 = (const uint32_t*)(src_cf + row * 12);
-      rr.sc = *(const unsigned short*)(src_sc + row * 2);
+      // The table entry of the thread's token was requested one chunk earlier: everything between the two
+      // barriers of a step is waited for by all sixteen wavefronts, a dependent load there is paid per chunk.
+      const bool hi_zero = !bt_wide || bt_hi == 0u;
+      if constexpr (BSP2) {
+        // Blocks of 1 .. 64 tokens (a power of two): chunks start on multiples of the block size, so the
+        // token's place inside its block never changes and a row is (block x rows per block + a constant);
+        // 32-bit byte offsets from wavefront-uniform bases (the host sends larger caches to the other form).
+        // An entry outside the cache belongs to a token past the range: any row of the cache serves.
+        const uint32_t phys = hi_zero ? min(bt_lo, (uint32_t)a.num_blocks - 1u) : 0u;
+        const uint32_t row = __umul24(phys, blk_rows) + row_in_blk;
+        const uint32_t o12 = (row << 3) + (row << 2);
+        p0 = (const uint32_t*)(src_idx + (size_t)o12);
+        p1 = (const uint32_t*)(src_cf + (size_t)o12);
+        rr.sc = *(const unsigned short*)(src_sc + (size_t)(row << 1));
+      } else {
+        const uint32_t tcl = (uint32_t)max(0, min(c0 + my_t, s1m));     // tokens past the range: its last token
+        const uint32_t blk = __umulhi(tcl, a.bs_magic) >> a.bs_mshift;
+        const uint32_t off = tcl - blk * (uint32_t)a.block_size;
+        int64_t phys = bt_wide ? (int64_t)(((uint64_t)bt_hi << 32) | bt_lo) : (int64_t)(int32_t)bt_lo;
+        phys = max((int64_t)0, min(phys, a.num_blocks - 1));                 // (an empty sequence reads a padding entry)
+        const uint32_t row = ((uint32_t)phys * (uint32_t)a.block_size + off) * (uint32_t)KVH + (uint32_t)my_h;
+        p0 = (const uint32_t*)(src_idx + (size_t)row * 12);
+        p1 = (const uint32_t*)(src_cf + (size_t)row * 12);
+        rr.sc = *(const unsigned short*)(src_sc + (size_t)row * 2);
+      }
     } else {
       const uint32_t rel = min((uint32_t)c0 * KVH + r, last_rel);            // rows past the range: its last row
       p0 = (const uint32_t*)(src_idx + (size_t)(rel * 12u));
@@ -619,6 +659,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
 #pragma unroll
     for (int w = 0; w < 3; ++w) { rr.x[0][w] = p0[w]; rr.x[1][w] = p1[w]; }
     // the score wavefront's own token positions (lane = token), as two dwords
+    if constexpr (PAGED) table_entry(c0 + 64);
     rr.kp_lo = 0; rr.kp_hi = 0;
     if constexpr (KP) {
       const uint32_t pe = value_role ? 0u : (uint32_t)max(0, min(c0 + lane, s1m)) * (kp_wide ? 8u : 4u);
@@ -638,6 +679,7 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
     // threads and KVH x GQ x 128 query elements, GQ per thread (element j of thread tid is number
     // tid + j x KVH x 128).
     tri_rows nxt;
+    if constexpr (PAGED) table_entry(s0);
     fetch(nxt, s0);
     float qv[GQ];
     unsigned short qraw[GQ];
@@ -986,24 +1028,24 @@ __global__ void tri_zero_kernel(float* out, size_t n) {
 
 // launch of the all-heads kernel for (gq, qh, lds, hgrid, num_kv_heads, stream, a) of the caller; more than 64 KB
 // of dynamic LDS has to be allowed once per kernel
-template <int GQ, bool PAGED, bool QH16, bool KP>
+template <int GQ, bool PAGED, bool QH16, bool KP, bool BSP2>
 static int tri_heads_launch(dim3 hgrid, int kvh, size_t lds, hipStream_t stream, const tri_args& a) {
   static size_t configured = 0;
   if (configured < lds) {
-    AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<GQ, PAGED, QH16, KP>,
+    AKV_HIP(hipFuncSetAttribute((const void*)tri_decode_heads_kernel<GQ, PAGED, QH16, KP, BSP2>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     configured = lds;
   }
-  AKV_LAUNCH_TIMED((tri_decode_heads_kernel<GQ, PAGED, QH16, KP>), hgrid, kvh * 128, lds, stream, a);
+  AKV_LAUNCH_TIMED((tri_decode_heads_kernel<GQ, PAGED, QH16, KP, BSP2>), hgrid, kvh * 128, lds, stream, a);
   return AKV_OK;
 }
-#define TRI_HEADS_LAUNCH(PAGED, KP)                                                                                  \
+#define TRI_HEADS_LAUNCH(PAGED, KP, BSP2)                                                                            \
   do {                                                                                                               \
     int rc_;                                                                                                         \
-    if (gq == 4) rc_ = qh ? tri_heads_launch<4, PAGED, true, KP>(hgrid, num_kv_heads, lds, stream, a)                \
-                          : tri_heads_launch<4, PAGED, false, KP>(hgrid, num_kv_heads, lds, stream, a);              \
-    else rc_ = qh ? tri_heads_launch<1, PAGED, true, KP>(hgrid, num_kv_heads, lds, stream, a)                        \
-                  : tri_heads_launch<1, PAGED, false, KP>(hgrid, num_kv_heads, lds, stream, a);                      \
+    if (gq == 4) rc_ = qh ? tri_heads_launch<4, PAGED, true, KP, BSP2>(hgrid, num_kv_heads, lds, stream, a)          \
+                          : tri_heads_launch<4, PAGED, false, KP, BSP2>(hgrid, num_kv_heads, lds, stream, a);        \
+    else rc_ = qh ? tri_heads_launch<1, PAGED, true, KP, BSP2>(hgrid, num_kv_heads, lds, stream, a)                  \
+                  : tri_heads_launch<1, PAGED, false, KP, BSP2>(hgrid, num_kv_heads, lds, stream, a);                \
     if (rc_ != AKV_OK) return rc_;                                                                                   \
   } while (0)
 
@@ -1066,7 +1108,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.cbits = coeff_bits; a.post_rope = pre_rope ? 0 : 1;
   a.nsplit = tri_pick_splits(batch, num_kv_heads, seq_len);
   a.block_tables = nullptr; a.bt_itype = AKV_I32; a.bt_stride = 0; a.context_lens = nullptr; a.cl_itype = AKV_I32;
-  a.block_size = 0; a.num_blocks = 0;
+  a.block_size = 0; a.num_blocks = 0; a.bs_shift = 0; a.bs_magic = 0; a.bs_mshift = 0;
   float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
@@ -1093,7 +1135,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
       a.nsplit = (int)n;
       a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
       dim3 hgrid(a.nsplit, batch, passes);
-      if (key_positions) TRI_HEADS_LAUNCH(false, true); else TRI_HEADS_LAUNCH(false, false);
+      if (key_positions) TRI_HEADS_LAUNCH(false, true, true); else TRI_HEADS_LAUNCH(false, false, true);
       AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
       tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
       AKV_LAUNCH_CHECK("tri_reduce_kernel");
@@ -1158,10 +1200,16 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const bool qh = q_dtype == AKV_F16;
   const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
   if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024 ||
-      max_blocks_per_seq * block_size >= ((int64_t)1 << 30))
+      max_blocks_per_seq * block_size >= ((int64_t)1 << 30) || block_size >= (1 << 30) ||
+      (double)num_blocks * block_size * num_kv_heads >= 4294967296.0)
     return akv_fail(AKV_ERR_UNSUPPORTED,
                     "akv_tri_decode_paged: needs head_dim 128, 12 frequencies, at most 8 kv heads, 4-byte "
-                    "aligned arrays and fewer than 2^30 tokens per sequence");
+                    "aligned arrays, fewer than 2^30 tokens per sequence and fewer than 2^32 rows in the cache");
+  // blocks of 1 .. 64 tokens (a power of two) in a cache whose arrays stay below 4 GB: rows by 32-bit offsets
+  const bool bs_small = (block_size & (block_size - 1)) == 0 && block_size <= 64 && num_blocks < (1 << 24) &&
+                        (double)num_blocks * block_size * num_kv_heads * 12.0 < 4294967296.0;
+  if (!bs_small && block_size < 3)
+    return akv_fail(AKV_ERR_UNSUPPORTED, "akv_tri_decode_paged: blocks of %d tokens in a cache of 4 GB arrays or more", block_size);
   if (batch == 0) return AKV_OK;
   AKV_REQUIRE(out != nullptr, "akv_tri_decode_paged: null pointer");
   if (max_blocks_per_seq == 0) {   // block tables without columns: every sequence is empty
@@ -1185,6 +1233,15 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   a.cbits = 4; a.post_rope = pre_rope ? 0 : 1;
   a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
   a.context_lens = context_lens; a.cl_itype = cl_itype; a.block_size = block_size; a.num_blocks = num_blocks;
+  a.bs_shift = 0; a.bs_magic = 0; a.bs_mshift = 0;
+  if (bs_small) {
+    a.bs_shift = __builtin_ctz((unsigned)block_size);
+  } else {
+    // block_size >= 3 here: k = 30 + ceil(log2 block_size) >= 32 and magic = ceil(2^k / block_size) < 2^31
+    const int k = 30 + (32 - __builtin_clz((unsigned)block_size - 1));
+    a.bs_magic = (uint32_t)((((uint64_t)1 << k) + (uint64_t)block_size - 1) / (uint64_t)block_size);
+    a.bs_mshift = k - 32;
+  }
   int cus = akv_cached_cu_count();
   if (cus <= 0) cus = 256;
   const int passes = gqa / gq;
@@ -1198,7 +1255,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
   dim3 hgrid(a.nsplit, batch, passes);
-  TRI_HEADS_LAUNCH(true, false);
+  if (bs_small) TRI_HEADS_LAUNCH(true, false, true);
+  else TRI_HEADS_LAUNCH(true, false, false);
   AKV_LAUNCH_CHECK("tri_decode_heads_kernel");
   tri_reduce_kernel<<<batch * num_q_heads, 128, 0, stream>>>(a.part_acc, a.part_ml, a.nsplit, d, out);
   AKV_LAUNCH_CHECK("tri_reduce_kernel");

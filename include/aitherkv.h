@@ -366,8 +366,10 @@ int akv_tri_scores(const void* query, int q_dtype,
  *   Coefficients are int4 (the only width the reference's cache stores, cache.py:66-85); pre_rope as for
  *   akv_tri_decode_step.
  * Workspace as for akv_tri_decode_step.  Built for d = 128, num_freqs = 12, at most 8 kv heads,
- * 4-byte aligned arrays and max_blocks_per_seq * block_size < 2^30; anything else returns
- * AKV_ERR_UNSUPPORTED (gather, then akv_tri_decode_step).
+ * 4-byte aligned arrays, max_blocks_per_seq * block_size < 2^30 and num_blocks * block_size * KVH < 2^32
+ * (blocks of 1 or 2 tokens: arrays below 4 GB); anything else returns AKV_ERR_UNSUPPORTED (gather, then
+ * akv_tri_decode_step).  Blocks of 1 .. 64 tokens (a power of two) in arrays below 4 GB take the shortest
+ * path: rows by 32-bit offsets and no division per chunk.
  * ------------------------------------------------------------------------------- */
 int akv_tri_decode_paged(const void* query, int q_dtype,
                          const uint8_t* k_indices, const uint8_t* k_coeffs, const void* k_scales,

@@ -185,7 +185,9 @@ def test_spectral_encode_energies_a_rounding_apart(dev, bits):
 
 
 @pytest.mark.parametrize("KVH,QH,bt_dtype,BS", [(8, 32, torch.int32, 16), (2, 8, torch.int64, 16), (4, 4, torch.int32, 16),
-                                                 (8, 32, torch.int64, 32), (1, 4, torch.int32, 8), (16, 16, torch.int32, 16)])
+                                                 (8, 32, torch.int64, 32), (1, 4, torch.int32, 8), (16, 16, torch.int32, 16),
+                                                 (8, 32, torch.int32, 24), (2, 8, torch.int64, 3), (4, 16, torch.int32, 100),
+                                                 (8, 8, torch.int32, 1)])
 def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
     """decode_step_paged over a block pool with permuted block tables, ragged context lengths (one
     empty, one ending inside a block, one filling its table) against the oracle's fetch + decode and
@@ -196,8 +198,8 @@ def test_paged_decode_vs_oracle(dev, KVH, QH, bt_dtype, BS):
     rng = np.random.default_rng(100 + KVH)
     D = 128
     lens = [0, 1, 777, 2048, 1500]
-    B, max_bps = len(lens), 2048 // BS
-    NB = 6400 // BS
+    B, max_bps = len(lens), -(-2048 // BS)        # (block sizes that are no power of two among them)
+    NB = 6400 // BS + 8
     cache = SpectralKVCache(cfg, max_blocks=NB, device=str(dev))
     perm = rng.permutation(NB)
     tables = np.full((B, max_bps), -7, dtype=np.int64)        # padding entries are never dereferenced
