@@ -49,6 +49,7 @@ struct tri_args {
   int cbits;       // coefficient width: 4 (a byte per pair), 8 (two bytes per pair), 16 (two float16 per pair, scales unused)
   int post_rope;   // keys were stored after RoPE: plain sparse dot product, positions unused
   int nsplit;
+  int two_stages;      // all-heads kernel: the staging area exists twice and a step has one barrier instead of two
   // paged cache (arrays are [num_blocks][block_size][KVH][...]; S = max_blocks_per_seq * block_size)
   const void* block_tables; int bt_itype; int64_t bt_stride;
   const void* context_lens; int cl_itype;
@@ -527,7 +528,7 @@ typedef __attribute__((address_space(3))) const tri_f32x2 tri_lds_cfloat2;
 // tokens (lane = token), keeps the running softmax and leaves the weights (x value scale, float16 hi + lo)
 // and the factors by which earlier sums shrink in LDS; the VALUE wavefront (wavefront KVH + h) scatters the
 // chunk's value coefficients into its dense tile and, one chunk behind, multiplies them by those weights on
-// the matrix cores.  The two workgroup barriers that order the staging area also order the hand-over
+// the matrix cores.  The workgroup barriers that order the staging area also order the hand-over
 // (weights are double-buffered).  Four wavefronts share a SIMD instead of two: the chains of dependent
 // LDS reads, transcendentals and products of one role run in the shadow of the other's.
 #define TRR_WAVE_BYTES (TRH_VT_BYTES + 2 * 4 * TRH_WT_PITCH)
@@ -537,13 +538,25 @@ typedef __attribute__((address_space(3))) const tri_f32x2 tri_lds_cfloat2;
 // multiply-adds take them directly), others as float32 with 16 bytes of padding
 static constexpr int tri_qrow_bytes(int gqa_pass, bool q_half) { return q_half ? gqa_pass * 4 : gqa_pass * 8 + TRH_Q_PAD; }
 
-static size_t tri_roles_lds_bytes(int kvh, int gqa_pass, bool q_half) {
+// One staging area: per role (keys, values) the index rows with the scale (16 bytes per token) and the coefficient
+// rows (12 bytes per token), head after head.
+#define TRH_CF_PITCH (64 * 12 + 32)
+static constexpr size_t tri_stage_bytes(int kvh) { return 2 * (size_t)kvh * (TRH_HEAD_PITCH + TRH_CF_PITCH); }
+static size_t tri_roles_lds_bytes(int kvh, int gqa_pass, bool q_half, bool two_stages) {
   return 64 * sizeof(float) + (size_t)kvh * 64 * tri_qrow_bytes(gqa_pass, q_half) + 64 +
-         4 * (size_t)kvh * TRH_HEAD_PITCH + (size_t)kvh * TRR_WAVE_BYTES + 2 * (size_t)kvh * TRR_ALPHA_FLOATS * sizeof(float);
+         (two_stages ? 2 : 1) * tri_stage_bytes(kvh) + (size_t)kvh * TRR_WAVE_BYTES +
+         2 * (size_t)kvh * TRR_ALPHA_FLOATS * sizeof(float);
+}
+// With the staging area doubled a step needs one workgroup barrier (chunk k + 1 is written into the area that
+// chunk k - 1 was read from, and every wavefront has passed the barrier of chunk k since it read that one);
+// taken whenever the 160 KB of LDS hold it.
+static bool tri_two_stages(int kvh, int gqa_pass, bool q_half) {
+  return tri_roles_lds_bytes(kvh, gqa_pass, q_half, true) <= 160 * 1024;
 }
 
 typedef __attribute__((address_space(3))) const tri_half2 tri_lds_chalf2;
 typedef uint32_t tri_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t tri_u32x3 __attribute__((ext_vector_type(3), aligned(4)));
 typedef float tri_f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) const tri_u32x4 tri_lds_cu32x4;
 typedef __attribute__((address_space(3))) const tri_f32x4 tri_lds_cf32x4;
@@ -555,8 +568,9 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   float* theta = (float*)lds_raw;                               // [64]
   float* q_lds = theta + 64;                                    // [KVH][64 pairs][GQ][even, odd]
   constexpr int QROW = tri_qrow_bytes(GQ, QH16);                // bytes of one pair's row of the query table
-  unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // [4 arrays][KVH] x TRH_HEAD_PITCH
-  unsigned char* tiles = stage + 4 * (size_t)KVH * TRH_HEAD_PITCH;
+  unsigned char* stage = (unsigned char*)q_lds + (size_t)KVH * 64 * QROW + 64;   // one or two staging areas
+  const uint32_t stage_bytes = (uint32_t)tri_stage_bytes(KVH);
+  unsigned char* tiles = stage + (a.two_stages ? 2 : 1) * (size_t)stage_bytes;
   float* alpha_lds = (float*)(tiles + (size_t)KVH * TRR_WAVE_BYTES);             // [2][KVH][TRR_ALPHA_FLOATS]
   const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool value_role = wv >= KVH;                            // wavefront-uniform
@@ -587,9 +601,14 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
   // the others the value arrays
   const int r = tid - (value_role ? KVH * 64 : 0);
   const int my_t = r / KVH, my_h = r - my_t * KVH;
-  const size_t arr = (size_t)KVH * TRH_HEAD_PITCH;
-  unsigned char* st_wr = stage + (value_role ? 2 * arr : 0) + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
-  const unsigned char* st_rd = stage + (value_role ? 2 * arr : 0) + (size_t)h * TRH_HEAD_PITCH + lane * 16;
+  // (inside an area: [keys: index rows | coefficient rows][values: index rows | coefficient rows])
+  const size_t arr_i = (size_t)KVH * TRH_HEAD_PITCH, arr_c = (size_t)KVH * TRH_CF_PITCH, role_b = arr_i + arr_c;
+  unsigned char* st_wr = stage + (value_role ? role_b : 0) + (size_t)my_h * TRH_HEAD_PITCH + my_t * 16;
+  unsigned char* st_wr_c = stage + (value_role ? role_b : 0) + arr_i + (size_t)my_h * TRH_CF_PITCH + my_t * 12;
+  const unsigned char* st_rd = stage + (value_role ? role_b : 0) + (size_t)h * TRH_HEAD_PITCH + lane * 16;
+  const unsigned char* st_rd_c = stage + (value_role ? role_b : 0) + arr_i + (size_t)h * TRH_CF_PITCH + lane * 12;
+  // (score wavefront: the value scale of its token is the fourth dword of the value side's index entry)
+  const unsigned char* st_rd_o = stage + (value_role ? 0 : role_b) + (size_t)h * TRH_HEAD_PITCH + lane * 16 + 12;
   // Not PAGED: the rows of batch element b start at a wavefront-uniform address and a row is named by a
   // 32-bit number (the host sends longer sequences to the other kernel).
   const int64_t row_b = PAGED ? 0 : (int64_t)b * a.S * KVH;
@@ -713,17 +732,18 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
     // during the previous step goes to the staging area, the next one is requested, the wavefront's own
     // two entries per token come back.
     uint32_t kp_lo = 0, kp_hi = 0;
-    auto stage_step = [&](int c0, uint4& e0, uint4& e1, uint32_t& other_sc) {
-      *(uint4*)(st_wr) = make_uint4(nxt.x[0][0], nxt.x[0][1], nxt.x[0][2], nxt.sc);
-      *(uint4*)(st_wr + arr) = make_uint4(nxt.x[1][0], nxt.x[1][1], nxt.x[1][2], nxt.sc);
+    uint32_t area = 0;                 // byte offset of the staging area of this step
+    auto stage_step = [&](int c0, uint4& e0, tri_u32x3& e1, uint32_t& other_sc) {
+      *(uint4*)(st_wr + area) = make_uint4(nxt.x[0][0], nxt.x[0][1], nxt.x[0][2], nxt.sc);
+      *(tri_u32x3*)(st_wr_c + area) = (tri_u32x3){nxt.x[1][0], nxt.x[1][1], nxt.x[1][2]};
       kp_lo = nxt.kp_lo; kp_hi = nxt.kp_hi;
       __syncthreads();
       fetch(nxt, c0 + 64);
-      e0 = *(const uint4*)(st_rd);
-      e1 = *(const uint4*)(st_rd + arr);
-      // (score wavefront: the value scale of its token, fourth dword of the value index entry)
-      other_sc = *(const uint32_t*)(st_rd + (value_role ? 0 : 2 * arr) + 12);
-      __syncthreads();
+      e0 = *(const uint4*)(st_rd + area);
+      e1 = *(const tri_u32x3*)(st_rd_c + area);
+      other_sc = *(const uint32_t*)(st_rd_o + area);
+      if (a.two_stages) area ^= stage_bytes;            // (wavefront-uniform)
+      else __syncthreads();
     };
 
     if (!value_role) {
@@ -732,7 +752,8 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
       for (int q = 0; q < GQ; ++q) { m[q] = -INFINITY; l[q] = 0.f; }
       int buf = 0;
       for (int c0 = s0; c0 < s1; c0 += 64) {
-        uint4 e0, e1;
+        uint4 e0;
+        tri_u32x3 e1;
         uint32_t vsc_raw;
         stage_step(c0, e0, e1, vsc_raw);
         const int t = c0 + lane;
@@ -927,7 +948,8 @@ __global__ __launch_bounds__(1024) void tri_decode_heads_kernel(tri_args a) {
       };
       int buf = 0;
       for (int c0 = s0; c0 < s1; c0 += 64) {
-        uint4 e0, e1;
+        uint4 e0;
+        tri_u32x3 e1;
         uint32_t unused;
         stage_step(c0, e0, e1, unused);
         if (have_prev) consume(buf ^ 1);
@@ -1108,7 +1130,7 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
   a.cbits = coeff_bits; a.post_rope = pre_rope ? 0 : 1;
   a.nsplit = tri_pick_splits(batch, num_kv_heads, seq_len);
   a.block_tables = nullptr; a.bt_itype = AKV_I32; a.bt_stride = 0; a.context_lens = nullptr; a.cl_itype = AKV_I32;
-  a.block_size = 0; a.num_blocks = 0; a.bs_shift = 0; a.bs_magic = 0; a.bs_mshift = 0;
+  a.block_size = 0; a.num_blocks = 0; a.bs_shift = 0; a.bs_magic = 0; a.bs_mshift = 0; a.two_stages = 0;
   float* wsf = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.part_acc = wsf;
   a.part_ml = wsf + (size_t)batch * num_q_heads * a.nsplit * d;
@@ -1122,8 +1144,10 @@ extern "C" int akv_tri_decode_step(const void* query, int q_dtype, const uint8_t
     // one workgroup per (token range, batch element), a wavefront per kv head
     const int gq = gqa % 4 == 0 ? 4 : 1;
     const bool qh = q_dtype == AKV_F16;
-    const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
+    const bool two = tri_two_stages(num_kv_heads, gq, qh);
+    const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh, two);
     if (lds <= 160 * 1024) {
+      a.two_stages = two ? 1 : 0;
       int cus = akv_cached_cu_count();
       if (cus <= 0) cus = 256;
       const int passes = gqa / gq;
@@ -1198,7 +1222,8 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   const int gqa = num_q_heads / num_kv_heads;
   const int gq = gqa % 4 == 0 ? 4 : 1;
   const bool qh = q_dtype == AKV_F16;
-  const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh);
+  const bool two = tri_two_stages(num_kv_heads, gq, qh);
+  const size_t lds = tri_roles_lds_bytes(num_kv_heads, gq, qh, two);
   if (d != 128 || num_freqs != 12 || num_kv_heads > 8 || !aligned || lds > 160 * 1024 ||
       max_blocks_per_seq * block_size >= ((int64_t)1 << 30) || block_size >= (1 << 30) ||
       (double)num_blocks * block_size * num_kv_heads >= 4294967296.0)
@@ -1233,6 +1258,7 @@ extern "C" int akv_tri_decode_paged(const void* query, int q_dtype, const uint8_
   a.cbits = 4; a.post_rope = pre_rope ? 0 : 1;
   a.block_tables = block_tables; a.bt_itype = bt_itype; a.bt_stride = bt_stride;
   a.context_lens = context_lens; a.cl_itype = cl_itype; a.block_size = block_size; a.num_blocks = num_blocks;
+  a.two_stages = two ? 1 : 0;
   a.bs_shift = 0; a.bs_magic = 0; a.bs_mshift = 0;
   if (bs_small) {
     a.bs_shift = __builtin_ctz((unsigned)block_size);
