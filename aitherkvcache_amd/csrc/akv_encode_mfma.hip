@@ -133,10 +133,20 @@ __device__ __forceinline__ uint32_t em_cell(float y) {
 }
 
 // MT: M-tiles (16 vectors each) per wavefront step -- MT, or 1 for float32 input
-template <int BITS, bool PAGED, int XDT, bool DIRECT, int MT>
+// SPLIT (calls of a few thousand vectors, e.g. one serving step): a workgroup is eight wavefronts that share ONE
+// step of 16 vectors, wavefront w computes N-tile w with its eighth of the B operand straight from memory in
+// registers -- no 64 KB fill, no cell table, one barrier; the codes meet in LDS and 256 threads pack and store
+// them.  Same products, same reciprocal, same comparison against the boundaries: the same codes.
+#define EM_SPLIT_WAVES 8
+#define EM_SPLIT_CODES 0           // [16 vectors][128 coordinates] code bytes
+#define EM_SPLIT_WAVE_OFF 2048
+#define EM_SPLIT_LDS_BYTES (EM_SPLIT_WAVE_OFF + EM_SPLIT_WAVES * EM_WAVE_BYTES)
+template <int BITS, bool PAGED, int XDT, bool DIRECT, int MT, bool SPLIT = false>
 __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_args a, const uint4* __restrict__ bop) {
   extern __shared__ __align__(16) unsigned char lds[];
   static_assert(MT <= MT && (XDT != AKV_F32 || MT == 1), "the LDS regions are sized for MT tiles");
+  static_assert(!SPLIT || (MT == 1 && XDT != AKV_F32 && !DIRECT), "the split form: one M-tile of 16-bit rows");
+  constexpr uint32_t WAVE_OFF = SPLIT ? EM_SPLIT_WAVE_OFF : EM_WAVE_OFF;
   constexpr int ROWS = 16 * MT;                       // vectors per wavefront step
   constexpr int XB = XDT == AKV_F32 ? 4 : 2;          // bytes per input element
   constexpr int NA = XDT == AKV_F32 ? 2 : 1;          // float16 terms of the input operand
@@ -180,7 +190,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   };
   const float* bnd = (const float*)(lds + EM_BND_OFF);
 
-  unsigned char* wl = lds + EM_WAVE_OFF + wave * EM_WAVE_BYTES;
+  unsigned char* wl = lds + WAVE_OFF + wave * EM_WAVE_BYTES;
   int64_t* src_off = (int64_t*)wl;                    // address of the vector, or 0
   int64_t* dst_p = (int64_t*)(wl + ROWS * 8);      // address of the packed row, or 0
   int64_t* dst_n = (int64_t*)(wl + ROWS * 16);     // address of the norm
@@ -188,7 +198,19 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 
   const int64_t n_total = (PAGED && a.x2) ? 2 * a.n : a.n;      // a second tensor rides along (K and V of a step)
   const int64_t steps = (n_total + ROWS - 1) / ROWS;
-  const int64_t stride = (int64_t)gridDim.x * EM_WAVES;
+  const int64_t stride = SPLIT ? (int64_t)gridDim.x : (int64_t)gridDim.x * EM_WAVES;
+  // SPLIT: the wavefront's N-tile of the B operand, both terms, four k-steps
+  em_half8 Bh[4], Bl[4];
+  if constexpr (SPLIT) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      union { uint4 u; em_half8 h; } ch, cl;
+      ch.u = bop[(wave * 4 + ks) * 64 + lane];
+      cl.u = bop[2048 + (wave * 4 + ks) * 64 + lane];
+      Bh[ks] = ch.h;
+      Bl[ks] = cl.h;
+    }
+  }
 
   // A operands of one step straight from memory (zeros past the end): lane l resolves the source
   // row of vector base + l, the lanes of an M-tile pick the rows up through LDS
@@ -440,9 +462,57 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
         if constexpr (DIRECT) {
           if ((uint32_t)base + lane < (uint32_t)a.n) a.norms[(uint32_t)base + lane] = nrm;
         } else {
-          if (dst_p[lane] != 0) *(float*)(uintptr_t)dst_n[lane] = nrm;
+          if (dst_p[lane] != 0 && (!SPLIT || wave == 0)) *(float*)(uintptr_t)dst_n[lane] = nrm;
         }
       }
+    }
+    if constexpr (SPLIT) {
+      // ---- the wavefront's tile: products, reciprocal, comparison with every boundary, code bytes to LDS
+      union { em_u32x4 u; em_float4 f; } rc;
+      rc.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(WAVE_OFF + wave * EM_WAVE_BYTES + ROWS * 24 + (4 * g) * 4);
+      em_float4 acc = (em_float4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[0][ks], Bh[ks], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[0][ks], Bl[ks], acc, 0, 0, 0);
+      }
+      uint8_t* codes = lds + EM_SPLIT_CODES;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float y = acc[i] * rc.f[i];
+        uint32_t code = 0;
+#pragma unroll
+        for (int k = 0; k < NB; ++k) code += (a.table[k] < y) ? 1u : 0u;
+        if (!(rc.f[i] == rc.f[i])) code = (uint32_t)NB;            // NaN vector: last level everywhere
+        codes[(4 * g + i) * 128 + 8 * col + wave] = (uint8_t)code;
+      }
+      __syncthreads();
+      if (threadIdx.x < 256) {
+        const int row = threadIdx.x >> 4, grp = threadIdx.x & 15;
+        const int64_t dp = dst_p[row];
+        if (dp != 0) {
+          const uint2 c8 = *(const uint2*)(codes + row * 128 + 8 * grp);
+          auto code_of = [&](int t) { return ((t < 4 ? c8.x : c8.y) >> (8 * (t & 3))) & 0xffu; };
+          uint32_t v = 0;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int t = BITS == 4 ? 6 - (k & ~1) + (k & 1) : BITS == 3 ? k : ((k + 4) & 7);
+            v = (v << BITS) + code_of(t);
+          }
+          uint8_t* prow = (uint8_t*)(uintptr_t)dp;
+          if (BITS == 4) {
+            *(uint32_t*)(prow + 4 * grp) = v;
+          } else if (BITS == 3) {
+            prow[3 * grp] = (uint8_t)(v >> 16);
+            prow[3 * grp + 1] = (uint8_t)(v >> 8);
+            prow[3 * grp + 2] = (uint8_t)v;
+          } else {
+            *(uint16_t*)(prow + 2 * grp) = (uint16_t)v;
+          }
+        }
+      }
+      __syncthreads();      // the code bytes are rewritten by the next step
+      return;
     }
     // ---- rotate, search, pack
     uint32_t packed[MT][4];
@@ -454,7 +524,7 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       union { em_u32x4 u; em_float4 f; } cv;
-      cv.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(EM_WAVE_OFF + wave * EM_WAVE_BYTES + ROWS * 24 + (16 * mt + 4 * g) * 4);
+      cv.u = *(em_lds_u128*)(uintptr_t)(uint32_t)(WAVE_OFF + wave * EM_WAVE_BYTES + ROWS * 24 + (16 * mt + 4 * g) * 4);
       rv[mt] = cv.f;
     }
     // N-tiles are software-pipelined: the matrix-core work of tile nt + 1 is issued together with
@@ -586,9 +656,16 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   };
 
   // the rows of a step are requested at the end of the step before it (the first: before the set-up)
-  const int64_t first = (int64_t)wave * gridDim.x + blockIdx.x;
+  const int64_t first = SPLIT ? (int64_t)blockIdx.x : (int64_t)wave * gridDim.x + blockIdx.x;
   uint4 R[MT][NP];
   fetch(R, first);
+  if constexpr (SPLIT) {
+    for (int64_t step = first; step < steps; step += stride) {      // (the same steps in every wavefront)
+      encode_step(std::true_type{}, step, R);
+      fetch(R, step + stride);
+    }
+    return;
+  }
   setup();
   const bool linear_search = ((const uint32_t*)(lds + EM_PAR_OFF))[0] != 0;   // uniform
   if (__builtin_expect(!linear_search, 1)) {
@@ -601,6 +678,18 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
       encode_step(std::true_type{}, step, R);
       fetch(R, step + stride);
     }
+  }
+}
+
+// the split form exists for paged calls of 16-bit rows; returns false where it does not
+template <int BB, bool PG, int DT, bool DR>
+static bool em_launch_split(int grid, hipStream_t stream, const akv_gen_args& a, const uint4* bop) {
+  if constexpr (PG && DT != AKV_F32 && !DR) {
+    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, true, DT, false, 1, true>), grid, EM_SPLIT_WAVES * 64, EM_SPLIT_LDS_BYTES,
+                     stream, a, bop);
+    return true;
+  } else {
+    return false;
   }
 }
 
@@ -628,6 +717,8 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   // vectors per wavefront step: twice the workgroups, half the chain of products and searches that its one busy
   // wavefront per workgroup walks through alone.
   const bool narrow = paged && x_dtype != AKV_F32 && (n_total + EM_ROWS - 1) / EM_ROWS < cus;
+  // ... and one that leaves a workgroup at most two steps of 16 vectors shares each step among eight wavefronts
+  const bool split = narrow && (n_total + 15) / 16 <= 2 * (int64_t)cus && !getenv("AKV_ENCODE_NO_SPLIT");
   const int rows_per_step = (x_dtype == AKV_F32 || narrow) ? 16 : EM_ROWS;
   const int64_t steps = (n_total + rows_per_step - 1) / rows_per_step;
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
@@ -645,6 +736,7 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   } while (0)
 #define EM_LAUNCH(BB, PG, DT, DR)                                                                     \
   do {                                                                                               \
+    if (split && em_launch_split<BB, PG, DT, DR>(grid, stream, a, bop)) break;                       \
     if (DT == AKV_F32 || (PG && narrow)) EM_LAUNCH_MT(BB, PG, DT, DR, 1);                             \
     else EM_LAUNCH_MT(BB, PG, DT, DR, (DT == AKV_F32 ? 1 : EM_MT));                                   \
   } while (0)

@@ -191,6 +191,8 @@ def bench_encode(torch, akv, L, dev, steps, warmup, cpu, cpu_seconds, sweep=True
     step_ms = timed(torch, lambda: akv.fused_encode_and_store(c, 0, k, v, slots), steps, warmup)
     res["step_256tok_us"] = step_ms * 1e3
     res["step_256tok_bytes"] = 2 * T * H * 324 + T * 8
+    # the kernel of that step by itself (events on its dispatch): what a caller without Python's call cost pays
+    res["step_256tok_kernel_us"] = kernel_ms(torch, L, lambda: akv.fused_encode_and_store(c, 0, k, v, slots), 64) * 1e3
     # (b) bandwidth regime
     n = 1 << 20
     # two inputs alternated (2 x 268 MB): one alone would partly sit in the 256 MB last-level cache

@@ -264,6 +264,43 @@ def test_paged_update_strided_cache(golden, dev, bits, itype):
     assert torch.all(norms[:2] == 0)
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_small_paged_calls_share_a_step_among_wavefronts(golden, dev, bits, dtype, monkeypatch):
+    """A paged call of a few thousand vectors runs the form in which eight wavefronts share a step of 16 vectors
+    (an N-tile each); a larger call, and the same call with that form switched off, run a wavefront per step.
+    Codes, norms and untouched rows are the same byte for byte -- also with a NaN vector, an infinite one, a zero one,
+    skipped slots and a token count that is no multiple of 16."""
+    tq = make_tq(golden, dev, bits)
+    P = tq._packed_dim
+    NB, BS, H = 40, 16, 8
+    rng = np.random.default_rng(500 + bits)
+    for T in (1, 37, 256, 600):                       # 8 .. 4,800 vectors: one step, ragged, a serving step, two steps per workgroup
+        x = kv_like(rng, (T, H, 128)).astype(np.float32)
+        if T > 30:
+            x[3, 1, 5] = np.nan
+            x[4, 2, 7] = np.inf
+            x[5, 0] = 0
+        xd = torch.from_numpy(x).to(dev).to(dtype)
+        slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+        slots[::9] = -1
+        sd = torch.from_numpy(slots).to(dev)
+        outs = []
+        for off in ("", "1"):
+            if off:
+                monkeypatch.setenv("AKV_ENCODE_NO_SPLIT", "1")
+            else:
+                monkeypatch.delenv("AKV_ENCODE_NO_SPLIT", raising=False)
+            kp = torch.full((NB, BS, H, P + 4), 0xAB, dtype=torch.uint8, device=dev)
+            kn = torch.full((NB, BS, H), -5.0, device=dev)
+            akv.fused_kv_update(xd, sd, kp[..., :P], kn, tq.rotation, tq.boundaries_inner, bits, BS)
+            outs.append((kp.cpu().numpy(), kn.cpu().numpy()))
+        monkeypatch.delenv("AKV_ENCODE_NO_SPLIT", raising=False)
+        assert np.array_equal(outs[0][0], outs[1][0]), (bits, dtype, T)
+        assert np.array_equal(outs[0][1], outs[1][1], equal_nan=True), (bits, dtype, T)
+        assert int(np.sum(outs[0][1] != -5.0)) == int(np.sum(slots >= 0)) * H
+
+
 def test_fused_encode_and_store(golden, dev):
     class Cache:
         pass
