@@ -681,11 +681,11 @@ __global__ __launch_bounds__(EM_THREADS) void akv_encode_mfma_kernel(akv_gen_arg
   }
 }
 
-// the split form exists for paged calls of 16-bit rows; returns false where it does not
+// the split form exists for 16-bit rows addressed row by row; returns false where it does not
 template <int BB, bool PG, int DT, bool DR>
 static bool em_launch_split(int grid, hipStream_t stream, const akv_gen_args& a, const uint4* bop) {
-  if constexpr (PG && DT != AKV_F32 && !DR) {
-    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, true, DT, false, 1, true>), grid, EM_SPLIT_WAVES * 64, EM_SPLIT_LDS_BYTES,
+  if constexpr (DT != AKV_F32 && !DR) {
+    AKV_LAUNCH_TIMED((akv_encode_mfma_kernel<BB, PG, DT, false, 1, true>), grid, EM_SPLIT_WAVES * 64, EM_SPLIT_LDS_BYTES,
                      stream, a, bop);
     return true;
   } else {
@@ -717,9 +717,10 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   // vectors per wavefront step: twice the workgroups, half the chain of products and searches that its one busy
   // wavefront per workgroup walks through alone.
   const bool narrow = paged && x_dtype != AKV_F32 && (n_total + EM_ROWS - 1) / EM_ROWS < cus;
-  // ... and one that leaves a workgroup at most two steps of 16 vectors shares each step among eight wavefronts
-  const bool split = narrow && (n_total + 15) / 16 <= 2 * (int64_t)cus && !getenv("AKV_ENCODE_NO_SPLIT");
-  const int rows_per_step = (x_dtype == AKV_F32 || narrow) ? 16 : EM_ROWS;
+  // ... and one (paged or flat) that leaves a workgroup at most two steps of 16 vectors shares each step among
+  // eight wavefronts
+  const bool split = x_dtype != AKV_F32 && (n_total + 15) / 16 <= 2 * (int64_t)cus && !getenv("AKV_ENCODE_NO_SPLIT");
+  const int rows_per_step = (x_dtype == AKV_F32 || narrow || split) ? 16 : EM_ROWS;
   const int64_t steps = (n_total + rows_per_step - 1) / rows_per_step;
   // steps are dealt round-robin over workgroups first, so a small call (one serving step) spreads
   // over as many CUs as it has steps instead of filling the wavefronts of a few
@@ -746,7 +747,7 @@ int akv_encode_mfma_try(const akv_gen_args& a, bool paged, int x_dtype, int d, i
   const bool direct = !paged && a.n < ((int64_t)1 << 31) / (xbytes * a.xs0 > a.ps0 ? xbytes * a.xs0 : a.ps0);
   if (paged) {
     if (bits == 4) EM_LAUNCH_DT(4, true, false); else if (bits == 3) EM_LAUNCH_DT(3, true, false); else EM_LAUNCH_DT(2, true, false);
-  } else if (direct) {
+  } else if (direct && !split) {
     if (bits == 4) EM_LAUNCH_DT(4, false, true); else if (bits == 3) EM_LAUNCH_DT(3, false, true); else EM_LAUNCH_DT(2, false, true);
   } else {
     if (bits == 4) EM_LAUNCH_DT(4, false, false); else if (bits == 3) EM_LAUNCH_DT(3, false, false); else EM_LAUNCH_DT(2, false, false);

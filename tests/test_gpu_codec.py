@@ -299,6 +299,19 @@ def test_small_paged_calls_share_a_step_among_wavefronts(golden, dev, bits, dtyp
         assert np.array_equal(outs[0][0], outs[1][0]), (bits, dtype, T)
         assert np.array_equal(outs[0][1], outs[1][1], equal_nan=True), (bits, dtype, T)
         assert int(np.sum(outs[0][1] != -5.0)) == int(np.sum(slots >= 0)) * H
+        # the same vectors through the flat entry point (TurboQuant.encode), with and without the shared steps
+        flat = []
+        for off in ("", "1"):
+            if off:
+                monkeypatch.setenv("AKV_ENCODE_NO_SPLIT", "1")
+            else:
+                monkeypatch.delenv("AKV_ENCODE_NO_SPLIT", raising=False)
+            p_, n_ = tq.encode(xd.reshape(-1, 128))
+            flat.append((p_.cpu().numpy(), n_.cpu().numpy()))
+        monkeypatch.delenv("AKV_ENCODE_NO_SPLIT", raising=False)
+        assert np.array_equal(flat[0][0], flat[1][0]) and np.array_equal(flat[0][1], flat[1][1], equal_nan=True)
+        ok = slots >= 0
+        assert np.array_equal(outs[0][0][slots[ok] // BS, slots[ok] % BS][..., :P], flat[0][0].reshape(T, H, P)[ok])
 
 
 def test_fused_encode_and_store(golden, dev):
