@@ -17,6 +17,7 @@
 #include "akv_hybrid_layout.h"
 
 static bool hyb_lane_disabled();
+static bool hyb_lane_forced();
 static const float kHybKappa = (float)(1.2533141373155001 / 64.0);  // sqrt(pi/2) / 64
 
 __device__ __forceinline__ float hyb_half_bits_to_float(uint32_t b) {
@@ -589,6 +590,11 @@ static int hyb_grid(int64_t n) {
   return (int)(g < 1 ? 1 : (g > cap ? cap : g));
 }
 
+static bool hyb_lane_forced() {
+  const char* e = getenv("AKV_HYBRID_LANE_ENCODE");        // (read per call: tests switch it)
+  return e && e[0] == '1';
+}
+
 static bool hyb_lane_disabled() {
   static int v = -1;
   if (v < 0) {
@@ -602,8 +608,12 @@ template <bool PAGED>
 static int hyb_launch_encode(int dt, const hyb_enc_args& a, hipStream_t stream) {
   // 16-byte aligned input rows and packed rows: one lane per vector
   const int64_t xal = dt == AKV_F32 ? 3 : 7;      // elements per 16 bytes, minus one
+  // ... and enough of them: a lane walks its vector's six transforms alone (20 us however few vectors there are),
+  // a wavefront per vector takes 7 us for a serving step of 2,048 vectors and 0.8 ns more per vector; they meet
+  // near 16 K vectors
   const bool lane_form = (((uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.ps0 | (uintptr_t)(PAGED ? a.ps1 | a.ps2 : 0)) & 15) == 0 &&
-                         ((a.xs0 | (PAGED ? a.xs1 : 0)) & xal) == 0 && !hyb_lane_disabled();
+                         ((a.xs0 | (PAGED ? a.xs1 : 0)) & xal) == 0 && !hyb_lane_disabled() &&
+                         (a.n >= 16384 || hyb_lane_forced());
   if (lane_form) {
     const int lgrid = (int)((a.n + 255) / 256);
     switch (dt) {
@@ -662,8 +672,9 @@ extern "C" int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_by
   if (n == 0) return AKV_OK;
   AKV_REQUIRE(packed && hyb_table && out, "akv_hybrid_decode: null pointer");
   AKV_REQUIRE(packed_stride_bytes >= 64 && out_stride >= 128, "akv_hybrid_decode: stride smaller than row");
+  // (a lane per vector from 64 K vectors on; below that a wavefront per vector ends two to three microseconds earlier)
   if (!hyb_lane_disabled() && (((uintptr_t)packed | (uintptr_t)packed_stride_bytes | (uintptr_t)out) & 15) == 0 &&
-      (out_stride & 3) == 0) {
+      (out_stride & 3) == 0 && (n >= 65536 || hyb_lane_forced())) {
     hyb_decode_lane_kernel<<<(int)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(packed, packed_stride_bytes, n,
                                                                                   hyb_table, kHybKappa, out, out_stride);
     AKV_LAUNCH_CHECK("hyb_decode_lane_kernel");

@@ -321,10 +321,12 @@ def test_hybrid_decode_step_replays_from_a_graph(golden, dev):
             _ = (torch.randn(1 << 16, device=dev) * 2).sum().item()
 
 
-def test_both_codec_forms_agree(golden, dev):
-    """Rows that are 16-byte aligned take the lane-per-vector kernels, any others the
-    wavefront-per-vector kernels: same bytes from both on the same vectors (paged store into rows of
-    pitch 68, flat encode of an input whose rows start at odd element offsets), same decoded floats."""
+def test_both_codec_forms_agree(golden, dev, monkeypatch):
+    """Large calls on rows that are 16-byte aligned take the lane-per-vector kernels, small calls and any other
+    rows the wavefront-per-vector kernels (here the lane form is switched on for the small call as well): same bytes
+    from both on the same vectors (paged store into rows of pitch 68, flat encode of an input whose rows start at
+    odd element offsets), same decoded floats."""
+    monkeypatch.setenv("AKV_HYBRID_LANE_ENCODE", "1")
     h = akv.HybridTurboQuant(device=str(dev))
     h.calibrate_uniform(num_kv_heads=4)
     rng = np.random.default_rng(71)
@@ -344,6 +346,16 @@ def test_both_codec_forms_agree(golden, dev):
     d_a = h.decode(aligned.reshape(-1, 64))
     d_p = h.decode(pitched.reshape(-1, 68)[:, :64])
     assert torch.equal(d_a, d_p)
+    # the choice by size: the same small call without the switch (a wavefront per vector), and a call large enough
+    # for the lane form by itself against its own pitched twin
+    monkeypatch.delenv("AKV_HYBRID_LANE_ENCODE")
+    small = torch.zeros_like(aligned)
+    akv.hybrid_encode_and_store(h, x, slots, small, BS)
+    assert torch.equal(small, aligned)
+    big = t(kv_like(rng, (20000, 128)), dev)
+    wide = torch.zeros(20000, 131, dtype=big.dtype, device=dev)
+    wide[:, 3:] = big
+    assert torch.equal(h.encode(big), h.encode(wide[:, 3:]))
 
 
 def test_one_object_across_batch_sizes(golden, dev):
