@@ -92,6 +92,7 @@ SIGNATURES = {
     "akv_block_scores": (_i, [_p, _p, _p, _p, _p, _i, _i64, _p, _i, _i, _i, _i, _i, _i64, _i, _i64, _p, _p]),
     "akv_block_select": (_i, [_p, _p, _i, _i64, _p, _i, _i, _i64, _i, _i, _i, _i, _p, _p, _p]),
     "akv_tri_encode": (_i, [_p, _i, _i64, _i, _i64, _i, _i, _p, _p, _p, _p]),
+    "akv_tri_encode_paged": (_i, [_p, _i, _i64, _i, _i, _i64, _i64, _i, _p, _i, _i64, _p, _p, _p, _p]),
     "akv_tri_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "akv_tri_scores": (_i, [_p, _i, _p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i64, _i, _i, _i, _i, _i, _i, _p]),
     "akv_tri_decode_step": (_i, [_p, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i,

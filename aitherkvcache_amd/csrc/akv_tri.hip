@@ -1334,10 +1334,15 @@ extern "C" int akv_tri_scores(const void* query, int q_dtype, const uint8_t* k_i
 // number of kept lanes below them.  Arithmetic follows the reference operation by operation
 // (separately rounded squares and sum, true division by the scale, round half to even).
 // ----------------------------------------------------------------------------------
-template <int XDT>
+// PAGED (encode-on-write): vector v is (token v / kvh, head v % kvh) of a [tokens][kv heads] tensor with
+// element strides xs / xs_head, and its row goes to row slot x kvh + head of the block pool, slot =
+// block x block_size + position from slot_mapping; tokens whose slot is negative or not below num_slots are skipped.
+struct tri_enc_paged { int64_t xs_head; int kvh; const void* slots; int slot_itype; int64_t num_slots; };
+template <int XDT, bool PAGED = false>
 __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict__ x, int64_t n, int d, int64_t xs,
                                                          int F, int cbits, uint8_t* __restrict__ indices,
-                                                         uint8_t* __restrict__ coeffs, __half* __restrict__ scales) {
+                                                         uint8_t* __restrict__ coeffs, __half* __restrict__ scales,
+                                                         tri_enc_paged pg = {}) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in every lane: the vector index and the search stay scalar
   const int P = d >> 1;
@@ -1347,15 +1352,27 @@ __global__ __launch_bounds__(256) void tri_encode_kernel(const void* __restrict_
   auto fetch = [&](int64_t vv, float& p0, float& p1) {
     p0 = 0.f; p1 = 0.f;
     if (have && vv < n) {
-      p0 = akv_elem<XDT>::load(x, vv * xs + 2 * lane);
-      p1 = akv_elem<XDT>::load(x, vv * xs + 2 * lane + 1);
+      int64_t off = vv * xs;
+      if constexpr (PAGED) {
+        const int64_t tok = vv / pg.kvh;
+        off = tok * xs + (vv - tok * pg.kvh) * pg.xs_head;
+      }
+      p0 = akv_elem<XDT>::load(x, off + 2 * lane);
+      p1 = akv_elem<XDT>::load(x, off + 2 * lane + 1);
     }
   };
   float nx0, nx1;
   fetch((int64_t)blockIdx.x * 4 + wave, nx0, nx1);
-  for (int64_t v = (int64_t)blockIdx.x * 4 + wave; v < n; v += stride) {
+  for (int64_t vsrc = (int64_t)blockIdx.x * 4 + wave; vsrc < n; vsrc += stride) {
     const float x0 = nx0, x1 = nx1;
-    fetch(v + stride, nx0, nx1);
+    fetch(vsrc + stride, nx0, nx1);
+    int64_t v = vsrc;               // row of the outputs
+    if constexpr (PAGED) {
+      const int64_t tok = vsrc / pg.kvh;
+      const int64_t slot = akv_load_index(pg.slots, pg.slot_itype, tok);
+      if (slot < 0 || slot >= pg.num_slots) continue;          // (wavefront-uniform)
+      v = slot * pg.kvh + (vsrc - tok * pg.kvh);
+    }
     const float e = akv_add_rn(akv_mul_rn(x0, x0), akv_mul_rn(x1, x1));
     // non-negative floats and NaNs order like their bit patterns; lanes beyond the last pair sort last
     const uint32_t key = have ? (__float_as_uint(e) & 0x7fffffffu) + 1u : 0u;
@@ -1444,6 +1461,37 @@ extern "C" int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int6
     case AKV_F16: tri_encode_kernel<AKV_F16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
     case AKV_BF16: tri_encode_kernel<AKV_BF16><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
     default: tri_encode_kernel<AKV_F32><<<grid, 256, 0, stream>>>(x, n, d, x_stride, num_freqs, coeff_bits, indices, (uint8_t*)coeffs, (__half*)scales); break;
+  }
+  AKV_LAUNCH_CHECK("tri_encode_kernel");
+  return AKV_OK;
+}
+
+// SpectralKVEncoder.encode of a step's K or V vectors written straight into the block pool of a paged spectral
+// cache (SpectralKVCache.store_token, aither_kvcache/triattention/cache.py:106-140, for every token of the step at
+// once): int4 coefficients, the only width that cache stores.
+extern "C" int akv_tri_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads, int d,
+                                    int64_t xs_token, int64_t xs_head, int num_freqs, const void* slot_mapping,
+                                    int slot_itype, int64_t num_slots, uint8_t* indices, uint8_t* coeffs,
+                                    void* scales, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  AKV_REQUIRE(num_tokens >= 0 && num_kv_heads > 0 && num_slots >= 0, "akv_tri_encode_paged: bad sizes");
+  AKV_REQUIRE(akv_valid_dtype(x_dtype) && akv_valid_itype(slot_itype), "akv_tri_encode_paged: bad dtype");
+  AKV_REQUIRE(d > 0 && d % 2 == 0, "akv_tri_encode_paged: head_dim=%d must be even", d);
+  AKV_REQUIRE(num_freqs > 0 && num_freqs <= d / 2, "akv_tri_encode_paged: num_freqs=%d out of range", num_freqs);
+  if (d > 128) return akv_fail(AKV_ERR_UNSUPPORTED, "akv_tri_encode_paged: head_dim=%d above 128 (one lane per pair)", d);
+  if (num_tokens == 0 || num_slots == 0) return AKV_OK;
+  AKV_REQUIRE(x && slot_mapping && indices && coeffs && scales, "akv_tri_encode_paged: null pointer");
+  AKV_REQUIRE(xs_head >= d && xs_token >= d, "akv_tri_encode_paged: stride smaller than row");
+  const int64_t n = num_tokens * num_kv_heads;
+  const int64_t want = (n + 3) / 4;
+  const int cap = akv_cached_cu_count() * 32;
+  const int grid = (int)(want < cap ? want : cap);
+  tri_enc_paged pg;
+  pg.xs_head = xs_head; pg.kvh = num_kv_heads; pg.slots = slot_mapping; pg.slot_itype = slot_itype; pg.num_slots = num_slots;
+  switch (x_dtype) {
+    case AKV_F16: tri_encode_kernel<AKV_F16, true><<<grid, 256, 0, stream>>>(x, n, d, xs_token, num_freqs, 4, indices, coeffs, (__half*)scales, pg); break;
+    case AKV_BF16: tri_encode_kernel<AKV_BF16, true><<<grid, 256, 0, stream>>>(x, n, d, xs_token, num_freqs, 4, indices, coeffs, (__half*)scales, pg); break;
+    default: tri_encode_kernel<AKV_F32, true><<<grid, 256, 0, stream>>>(x, n, d, xs_token, num_freqs, 4, indices, coeffs, (__half*)scales, pg); break;
   }
   AKV_LAUNCH_CHECK("tri_encode_kernel");
   return AKV_OK;

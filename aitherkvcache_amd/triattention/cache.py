@@ -12,6 +12,7 @@ from typing import Optional, Tuple
 
 import torch
 
+from .. import _lib
 from .config import TriAttentionConfig
 from .encoder import SpectralEncoding
 
@@ -55,6 +56,43 @@ class SpectralKVCache:
         for dst, src in zip(self._arrays(), tuple(k_enc) + tuple(v_enc)):
             dst[block_idx, slot_idx] = src
         self._block_fill[block_idx] = max(self._block_fill[block_idx], slot_idx + 1)
+
+    def encode_and_store(self, keys: torch.Tensor, values: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+        """Encode-on-write of a step: keys / values [num_tokens, kv_heads, head_dim] (keys before RoPE) are encoded
+        (SpectralKVEncoder.encode, reference encoder.py:73-149) and written into the block pool at
+        slot = block * block_size + position per token, one launch per tensor -- what the reference does with
+        encode followed by store_token per token (cache.py:106-140).  Negative slots and slots past the cache are
+        skipped.  No counterpart in the reference."""
+        T, KVH, D = keys.shape
+        if KVH != self.num_kv_heads or D != self.config.head_dim or values.shape != keys.shape:
+            raise ValueError(f"keys / values {tuple(keys.shape)} / {tuple(values.shape)} do not fit kv_heads="
+                             f"{self.num_kv_heads}, head_dim={self.config.head_dim}")
+        if slot_mapping.numel() != T:
+            raise ValueError("slot_mapping must hold one slot per token")
+        if T == 0:
+            return
+        dev = _lib.require_gpu(keys, values, self.k_indices)
+        sm = slot_mapping if slot_mapping.dtype in (torch.int32, torch.int64) else slot_mapping.long()
+        host_slots = None if sm.is_cuda else sm.tolist()
+        sm = sm.to(dev).contiguous()
+        L = _lib.lib()
+        for x, (idx, cf, sc) in ((keys, (self.k_indices, self.k_packed, self.k_scales)),
+                                 (values, (self.v_indices, self.v_packed, self.v_scales))):
+            if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+                x = x.float()
+            if x.stride(-1) != 1:
+                x = x.contiguous()
+            _lib.check(L.akv_tri_encode_paged(
+                x.data_ptr(), _lib.dtype_code(x), T, KVH, D, x.stride(0), x.stride(1), self.num_freqs,
+                sm.data_ptr(), _lib.itype_code(sm), self.max_blocks * self.block_size,
+                idx.data_ptr(), cf.data_ptr(), sc.data_ptr(), _lib.stream_ptr(dev)))
+        # (the fill counters serve memory_stats alone: they follow slots given as host data, and are not read back
+        # from the device for slots that live there)
+        if host_slots is not None:
+            for s_ in host_slots:
+                if 0 <= s_ < self.max_blocks * self.block_size:
+                    b, p_ = divmod(s_, self.block_size)
+                    self._block_fill[b] = max(self._block_fill[b], p_ + 1)
 
     def store_block(self, block_idx: int, k_enc: SpectralEncoding, v_enc: SpectralEncoding,
                     num_tokens: Optional[int] = None) -> None:

@@ -400,6 +400,18 @@ int akv_tri_decode_paged(const void* query, int q_dtype,
 int akv_tri_encode(const void* x, int x_dtype, int64_t n, int d, int64_t x_stride, int num_freqs,
                    int coeff_bits, uint8_t* indices, void* coeffs, void* scales, void* stream);
 
+/* Encode-on-write for the paged spectral cache: SpectralKVEncoder.encode (encoder.py:73-149, int4 coefficients)
+ * of x [num_tokens][num_kv_heads][d] (element strides xs_token, xs_head) written straight into the block pool --
+ * what the reference does token by token with SpectralKVCache.store_token (aither_kvcache/triattention/cache.py:
+ * 106-140) after encoding.  slot_mapping [num_tokens]: slot = block * block_size + position; a token whose slot is
+ * negative or not below num_slots (= num_blocks * block_size) is skipped.  indices, coeffs
+ * [num_slots][num_kv_heads][num_freqs] uint8 and scales [num_slots][num_kv_heads] fp16, contiguous (the cache's
+ * k_* or v_* tensors). */
+int akv_tri_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int num_kv_heads, int d,
+                         int64_t xs_token, int64_t xs_head, int num_freqs,
+                         const void* slot_mapping, int slot_itype, int64_t num_slots,
+                         uint8_t* indices, uint8_t* coeffs, void* scales, void* stream);
+
 /* ---------------------------------------------------------------------------------
  * Block selection for sparse decode attention -- aither_kvcache/block_selector.py.
  * The attention entry points take the filtered table and context lengths as they are.

@@ -589,3 +589,53 @@ def test_benchmark_method_reports_times_and_quality(dev):
     assert rep["seq_len"] == 300 and rep["batch_size"] == 2 and rep["compression_ratio"] > 5
     assert -1.0 <= rep["cosine_similarity"] <= 1.0 and rep["mse"] >= 0
 
+
+@pytest.mark.parametrize("KVH,BS,dtype,it", [(8, 16, torch.float16, torch.int64), (2, 8, torch.bfloat16, torch.int32),
+                                             (4, 24, torch.float32, torch.int64)])
+def test_encode_on_write_into_the_paged_cache(dev, KVH, BS, dtype, it):
+    """SpectralKVCache.encode_and_store: a step's keys and values encoded and written into the block pool by one
+    launch per tensor -- the rows are those of encode (byte for byte, and the oracle's), they land at their slots,
+    skipped tokens (negative slots, slots past the cache) and every other row stay untouched; strided inputs; a
+    decode step over the written cache agrees with the oracle."""
+    from aitherkvcache_amd.triattention import SpectralKVCache
+    cfg = TriAttentionConfig(num_kv_heads=KVH, num_query_heads=4 * KVH, block_size=BS)
+    tri = TriAttention(cfg, device=str(dev))
+    rng = np.random.default_rng(300 + KVH)
+    NB, T, D = 12, 70, 128
+    cache = SpectralKVCache(cfg, max_blocks=NB, device=str(dev))
+    for a in cache._arrays():
+        a.fill_(7)
+    pair_std = (np.arange(D // 2) + 1.0) ** -0.75
+    keys = (rng.standard_normal((T, KVH, D // 2, 2)) * pair_std[:, None]).reshape(T, KVH, D).astype(np.float32)
+    vals = rng.standard_normal((T, KVH, D)).astype(np.float32)
+    kd, vd = t(keys, dev).to(dtype), t(vals, dev).to(dtype)
+    wide = torch.zeros(T, KVH, D + 8, dtype=dtype, device=dev)       # values through a strided view
+    wide[..., :D] = vd
+    slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+    slots[::11] = -1
+    slots[5] = NB * BS + 3
+    cache.encode_and_store(kd, wide[..., :D], t(slots, dev).to(it))
+    k_enc, v_enc = tri.encode_kv(kd[None], vd[None])
+    ok = (slots >= 0) & (slots < NB * BS)
+    arrays = [a.cpu().numpy() for a in cache._arrays()]
+    for got, want in zip(arrays, [x[0].cpu().numpy() for x in tuple(k_enc) + tuple(v_enc)]):
+        flat = got.reshape((NB * BS,) + got.shape[2:])
+        assert np.array_equal(flat[slots[ok]], want[ok])
+        untouched = np.ones(NB * BS, bool)
+        untouched[slots[ok]] = False
+        assert np.all(flat[untouched] == 7)
+    ref = O.spectral_encode(kd.float().cpu().numpy(), 12, 4)
+    assert np.array_equal(arrays[0].reshape(NB * BS, KVH, 12)[slots[ok]], ref[0][ok])
+    assert np.array_equal(arrays[1].reshape(NB * BS, KVH, 12)[slots[ok]], ref[1][ok])
+    # the written tokens as one sequence, read back through a block table
+    seq = np.flatnonzero(ok)[:BS * 3]
+    cache2 = SpectralKVCache(cfg, max_blocks=NB, device=str(dev))
+    table = rng.permutation(NB)[:4]
+    sl = np.array([table[j // BS] * BS + j % BS for j in range(len(seq))], dtype=np.int64)
+    cache2.encode_and_store(kd[seq], vd[seq], torch.from_numpy(sl))               # (slots as host data)
+    q = rng.standard_normal((1, 4 * KVH, D)).astype(np.float32)
+    out = tri.decode_step_paged(t(q, dev), cache2, t(table[None], dev), torch.tensor([len(seq)], device=dev)).cpu().numpy()
+    refo = O.tri_decode_step_paged(q, [a.cpu().numpy() for a in cache2._arrays()], table[None], [len(seq)], BS,
+                                   tri._theta.cpu().numpy())
+    assert np.max(np.abs(out - refo)) <= TOL
+    assert cache2.memory_stats()["used_blocks"] == -(-len(seq) // BS)
