@@ -9,11 +9,11 @@ from .quantizer import TurboQuant, TurboQuantConfig
 from .hybrid_quantizer import HybridTurboQuant, HybridLayout, GroupLayout
 from .fused_kv_update import fused_tq4_kv_update, fused_kv_update, fused_kv_update_pair, fused_encode_and_store
 from .fused_attention import TQPagedAttention
-from .hybrid_attention import HybridPagedAttention, hybrid_encode_and_store
+from .hybrid_attention import HybridPagedAttention, hybrid_encode_and_store, hybrid_encode_and_store_pair
 
 __all__ = [
     "TurboQuant", "TurboQuantConfig", "HybridTurboQuant", "HybridLayout", "GroupLayout",
     "fused_tq4_kv_update", "fused_kv_update", "fused_kv_update_pair", "fused_encode_and_store", "TQPagedAttention",
-    "HybridPagedAttention", "hybrid_encode_and_store",
+    "HybridPagedAttention", "hybrid_encode_and_store", "hybrid_encode_and_store_pair",
 ]
 __version__ = "0.1.0"

@@ -69,6 +69,8 @@ SIGNATURES = {
     "akv_hybrid_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
                                      _p, _i64, _i64, _i64, _i, _i64, _p]),
+    "akv_hybrid_encode_paged_kv": (_i, [_p, _p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
+                                        _p, _p, _i64, _i64, _i64, _i, _i64, _p]),
     "akv_hybrid_decode": (_i, [_p, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid_paged_attn_workspace_bytes": (_sz, [_i, _i]),
     "akv_hybrid_paged_attn": (_i, [_p, _i, _i64, _i64,
@@ -80,6 +82,8 @@ SIGNATURES = {
     "akv_hybrid25_encode": (_i, [_p, _i, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid25_encode_paged": (_i, [_p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
                                        _p, _i64, _i64, _i64, _i, _i64, _p]),
+    "akv_hybrid25_encode_paged_kv": (_i, [_p, _p, _i, _i64, _i, _i64, _i64, _p, _i, _p,
+                                          _p, _p, _i64, _i64, _i64, _i, _i64, _p]),
     "akv_hybrid25_decode": (_i, [_p, _i64, _i64, _p, _p, _i64, _p]),
     "akv_hybrid25_paged_attn": (_i, [_p, _i, _i64, _i64,
                                      _p, _i64, _i64, _i64, _p, _i64, _i64, _i64,

@@ -29,6 +29,7 @@ __device__ __forceinline__ float hyb_half_bits_to_float(uint32_t b) {
 // ----------------------------------------------------------------------------------
 struct hyb_enc_args {
   const void* x; int64_t n; int64_t xs0, xs1; int heads;
+  const void* x2; uint8_t* out2;     // paged, wavefront per vector: a second tensor (V beside K) with the same strides, or null
   const void* slots; int slot_itype; int block_size; int64_t max_blocks;
   const float* table;
   uint8_t* out; int64_t ps0, ps1, ps2;
@@ -78,10 +79,14 @@ __global__ __launch_bounds__(256) void hyb_encode_kernel(hyb_enc_args a) {
   for (int i = threadIdx.x; i < AKV_HYB_TABLE_FLOATS; i += 256) tab[i] = a.table[i];
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int64_t n = (int64_t)blockIdx.x * 4 + wave; n < a.n; n += (int64_t)gridDim.x * 4) {
+  const int64_t n_total = (PAGED && a.x2) ? 2 * a.n : a.n;
+  for (int64_t nn = (int64_t)blockIdx.x * 4 + wave; nn < n_total; nn += (int64_t)gridDim.x * 4) {
+    const bool second = PAGED && nn >= a.n;                     // (wavefront-uniform)
+    const int64_t n = second ? nn - a.n : nn;
+    const void* xb = second ? a.x2 : a.x;
     const int64_t off = PAGED ? (n / a.heads) * a.xs0 + (n % a.heads) * a.xs1 : n * a.xs0;
-    const float x0 = akv_elem<XDT>::load(a.x, off + lane);
-    const float x1 = akv_elem<XDT>::load(a.x, off + 64 + lane);
+    const float x0 = akv_elem<XDT>::load(xb, off + lane);
+    const float x1 = akv_elem<XDT>::load(xb, off + 64 + lane);
     hyb_encode_group<3>(x0, lane, tab + HYB_HAD0, tab + HYB_QJL0, tab + HYB_CEN0, tab + HYB_BND0,
                         codes[wave], signs[wave], rows[wave], 0);
     hyb_encode_group<2>(x1, lane, tab + HYB_HAD1, tab + HYB_QJL1, tab + HYB_CEN1, tab + HYB_BND1,
@@ -93,7 +98,7 @@ __global__ __launch_bounds__(256) void hyb_encode_kernel(hyb_enc_args a) {
       if (slot < 0) continue;
       const int64_t blk = slot / a.block_size, pos = slot % a.block_size;
       if (blk >= a.max_blocks) continue;
-      dst = a.out + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+      dst = (second ? a.out2 : a.out) + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
     } else {
       dst = a.out + n * a.ps0;
     }
@@ -613,7 +618,7 @@ static int hyb_launch_encode(int dt, const hyb_enc_args& a, hipStream_t stream) 
   // near 16 K vectors
   const bool lane_form = (((uintptr_t)a.x | (uintptr_t)a.out | (uintptr_t)a.ps0 | (uintptr_t)(PAGED ? a.ps1 | a.ps2 : 0)) & 15) == 0 &&
                          ((a.xs0 | (PAGED ? a.xs1 : 0)) & xal) == 0 && !hyb_lane_disabled() &&
-                         (a.n >= 16384 || hyb_lane_forced());
+                         (a.n >= 16384 || hyb_lane_forced()) && a.x2 == nullptr;
   if (lane_form) {
     const int lgrid = (int)((a.n + 255) / 256);
     switch (dt) {
@@ -624,7 +629,7 @@ static int hyb_launch_encode(int dt, const hyb_enc_args& a, hipStream_t stream) 
     AKV_LAUNCH_CHECK("hyb_encode_lane_kernel");
     return AKV_OK;
   }
-  const int grid = hyb_grid(a.n);
+  const int grid = hyb_grid((PAGED && a.x2) ? 2 * a.n : a.n);
   switch (dt) {
     case AKV_F16: hyb_encode_kernel<AKV_F16, PAGED><<<grid, 256, 0, stream>>>(a); break;
     case AKV_BF16: hyb_encode_kernel<AKV_BF16, PAGED><<<grid, 256, 0, stream>>>(a); break;
@@ -662,6 +667,34 @@ extern "C" int akv_hybrid_encode_paged(const void* x, int x_dtype, int64_t num_t
   a.x = x; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
   a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
   a.table = hyb_table; a.out = out; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
+  return hyb_launch_encode<true>(x_dtype, a, (hipStream_t)stream);
+}
+
+// K and V of a step in one launch while the call is small (a wavefront per vector); two launches of the form
+// for large calls otherwise.  Both tensors and both caches have the strides given.
+extern "C" int akv_hybrid_encode_paged_kv(const void* x_k, const void* x_v, int x_dtype, int64_t num_tokens,
+                                          int num_kv_heads, int64_t xs_token, int64_t xs_head,
+                                          const void* slot_mapping, int slot_itype,
+                                          const float* hyb_table, uint8_t* out_k, uint8_t* out_v, int64_t ps_blk,
+                                          int64_t ps_pos, int64_t ps_head, int block_size,
+                                          int64_t max_blocks, void* stream) {
+  AKV_REQUIRE(num_tokens >= 0 && num_kv_heads > 0, "akv_hybrid_encode_paged_kv: bad sizes");
+  if (num_tokens == 0 || max_blocks == 0) return AKV_OK;
+  AKV_REQUIRE(x_k && x_v && out_k && out_v, "akv_hybrid_encode_paged_kv: null pointer");
+  if (num_tokens * num_kv_heads >= 16384) {
+    const int rc = akv_hybrid_encode_paged(x_k, x_dtype, num_tokens, num_kv_heads, xs_token, xs_head, slot_mapping,
+                                           slot_itype, hyb_table, out_k, ps_blk, ps_pos, ps_head, block_size, max_blocks, stream);
+    if (rc) return rc;
+    return akv_hybrid_encode_paged(x_v, x_dtype, num_tokens, num_kv_heads, xs_token, xs_head, slot_mapping,
+                                   slot_itype, hyb_table, out_v, ps_blk, ps_pos, ps_head, block_size, max_blocks, stream);
+  }
+  AKV_REQUIRE(akv_valid_dtype(x_dtype) && akv_valid_itype(slot_itype), "akv_hybrid_encode_paged_kv: bad dtype");
+  AKV_REQUIRE(block_size > 0 && max_blocks >= 0, "akv_hybrid_encode_paged_kv: bad block_size/max_blocks");
+  AKV_REQUIRE(slot_mapping && hyb_table, "akv_hybrid_encode_paged_kv: null pointer");
+  hyb_enc_args a = {};
+  a.x = x_k; a.x2 = x_v; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
+  a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
+  a.table = hyb_table; a.out = out_k; a.out2 = out_v; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
   return hyb_launch_encode<true>(x_dtype, a, (hipStream_t)stream);
 }
 

@@ -76,6 +76,7 @@ struct h25_roles {
 // ----------------------------------------------------------------------------------
 struct h25_enc_args {
   const void* x; int64_t n; int64_t xs0, xs1; int heads;
+  const void* x2; uint8_t* out2;     // paged: a second tensor (V beside K) with the same strides, or null
   const void* slots; int slot_itype; int block_size; int64_t max_blocks;
   const float* table;
   uint8_t* out; int64_t ps0, ps1, ps2;
@@ -92,10 +93,14 @@ __global__ __launch_bounds__(256) void h25_encode_kernel(h25_enc_args a) {
   const float had_a = tab[H25_HAD + r.ca], had_b = tab[H25_HAD + r.cb];
   const float qjl_a = tab[H25_QJL + r.ca], qjl_b = tab[H25_QJL + r.cb];
   const float root_b = r.b0 ? kH25Root0 : kH25Root1;
-  for (int64_t n = (int64_t)blockIdx.x * 4 + wave; n < a.n; n += (int64_t)gridDim.x * 4) {
+  const int64_t n_total = (PAGED && a.x2) ? 2 * a.n : a.n;
+  for (int64_t nn = (int64_t)blockIdx.x * 4 + wave; nn < n_total; nn += (int64_t)gridDim.x * 4) {
+    const bool second = PAGED && nn >= a.n;                     // (wavefront-uniform)
+    const int64_t n = second ? nn - a.n : nn;
+    const void* xsrc = second ? a.x2 : a.x;
     const int64_t off = PAGED ? (n / a.heads) * a.xs0 + (n % a.heads) * a.xs1 : n * a.xs0;
-    const float xa = akv_elem<XDT>::load(a.x, off + r.ca);
-    const float xb = akv_elem<XDT>::load(a.x, off + r.cb);
+    const float xa = akv_elem<XDT>::load(xsrc, off + r.ca);
+    const float xb = akv_elem<XDT>::load(xsrc, off + r.cb);
     // norms: group 0 = the lower half's second values, group 1 = all first values + the upper half's second values
     const float sb = h25_half_sum(akv_mul_rn(xb, xb));
     const float n0 = sqrtf(h25_lane_value(sb, 0));
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(256) void h25_encode_kernel(h25_enc_args a) {
       if (slot < 0) continue;
       const int64_t blk = slot / a.block_size, pos = slot % a.block_size;
       if (blk >= a.max_blocks) continue;
-      dst = a.out + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
+      dst = (second ? a.out2 : a.out) + blk * a.ps0 + pos * a.ps1 + head * a.ps2;
     } else {
       dst = a.out + n * a.ps0;
     }
@@ -467,7 +472,7 @@ static int h25_grid(int64_t n) {
 
 template <bool PAGED>
 static int h25_launch_encode(int dt, const h25_enc_args& a, hipStream_t stream) {
-  const int grid = h25_grid(a.n);
+  const int grid = h25_grid((PAGED && a.x2) ? 2 * a.n : a.n);
   switch (dt) {
     case AKV_F16: h25_encode_kernel<AKV_F16, PAGED><<<grid, 256, 0, stream>>>(a); break;
     case AKV_BF16: h25_encode_kernel<AKV_BF16, PAGED><<<grid, 256, 0, stream>>>(a); break;
@@ -505,6 +510,24 @@ extern "C" int akv_hybrid25_encode_paged(const void* x, int x_dtype, int64_t num
   a.x = x; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
   a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
   a.table = hyb_table; a.out = out; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
+  return h25_launch_encode<true>(x_dtype, a, (hipStream_t)stream);
+}
+
+extern "C" int akv_hybrid25_encode_paged_kv(const void* x_k, const void* x_v, int x_dtype, int64_t num_tokens,
+                                            int num_kv_heads, int64_t xs_token, int64_t xs_head,
+                                            const void* slot_mapping, int slot_itype,
+                                            const float* hyb_table, uint8_t* out_k, uint8_t* out_v, int64_t ps_blk,
+                                            int64_t ps_pos, int64_t ps_head, int block_size,
+                                            int64_t max_blocks, void* stream) {
+  AKV_REQUIRE(num_tokens >= 0 && num_kv_heads > 0, "akv_hybrid25_encode_paged_kv: bad sizes");
+  AKV_REQUIRE(akv_valid_dtype(x_dtype) && akv_valid_itype(slot_itype), "akv_hybrid25_encode_paged_kv: bad dtype");
+  AKV_REQUIRE(block_size > 0 && max_blocks >= 0, "akv_hybrid25_encode_paged_kv: bad block_size/max_blocks");
+  if (num_tokens == 0 || max_blocks == 0) return AKV_OK;
+  AKV_REQUIRE(x_k && x_v && slot_mapping && hyb_table && out_k && out_v, "akv_hybrid25_encode_paged_kv: null pointer");
+  h25_enc_args a = {};
+  a.x = x_k; a.x2 = x_v; a.n = num_tokens * num_kv_heads; a.xs0 = xs_token; a.xs1 = xs_head; a.heads = num_kv_heads;
+  a.slots = slot_mapping; a.slot_itype = slot_itype; a.block_size = block_size; a.max_blocks = max_blocks;
+  a.table = hyb_table; a.out = out_k; a.out2 = out_v; a.ps0 = ps_blk; a.ps1 = ps_pos; a.ps2 = ps_head;
   return h25_launch_encode<true>(x_dtype, a, (hipStream_t)stream);
 }
 

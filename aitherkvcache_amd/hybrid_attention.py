@@ -43,6 +43,36 @@ def hybrid_encode_and_store(htq, x: torch.Tensor, slot_mapping: torch.Tensor, ca
         block_size, max_blocks, _lib.stream_ptr(dev)))
 
 
+def hybrid_encode_and_store_pair(htq, key: torch.Tensor, value: torch.Tensor, slot_mapping: torch.Tensor,
+                                 k_cache: torch.Tensor, v_cache: torch.Tensor, block_size: int = 16,
+                                 max_blocks: int = 0) -> None:
+    """K and V of a step (the two encodes of tq::hybrid_decode_step, reference vllm/hooks.py:271-284) in one call:
+    one launch while the step is small.  Tensors or caches that differ in dtype, shape or strides go through
+    hybrid_encode_and_store one after the other."""
+    same = (key.shape == value.shape and key.dtype == value.dtype and key.stride() == value.stride()
+            and key.dim() == 3 and key.stride(-1) == 1 and key.dtype in (torch.float16, torch.bfloat16, torch.float32)
+            and k_cache.shape == v_cache.shape and k_cache.stride() == v_cache.stride()
+            and k_cache.dtype == torch.uint8 and v_cache.dtype == torch.uint8 and k_cache.stride(-1) == 1
+            and k_cache.shape[-1] >= htq.packed_dim and htq.group_order is None
+            and slot_mapping.is_contiguous() and key.shape[-1] == htq.head_dim)
+    if not same:
+        hybrid_encode_and_store(htq, key, slot_mapping, k_cache, block_size, max_blocks)
+        hybrid_encode_and_store(htq, value, slot_mapping, v_cache, block_size, max_blocks)
+        return
+    num_tokens, num_kv_heads, _ = key.shape
+    if num_tokens == 0:
+        return
+    if max_blocks == 0:
+        max_blocks = k_cache.shape[0]
+    table = htq.kernel_table
+    dev = _lib.require_gpu(key, value, slot_mapping, k_cache, v_cache, table)
+    _lib.check(getattr(_lib.lib(), htq._abi + "_encode_paged_kv")(
+        key.data_ptr(), value.data_ptr(), _lib.dtype_code(key), num_tokens, num_kv_heads, key.stride(0), key.stride(1),
+        slot_mapping.data_ptr(), _lib.itype_code(slot_mapping), table.data_ptr(),
+        k_cache.data_ptr(), v_cache.data_ptr(), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+        block_size, max_blocks, _lib.stream_ptr(dev)))
+
+
 class HybridPagedAttention:
     """attn = HybridPagedAttention(htq, num_query_heads=32)
     out = attn.forward(query, k_cache, v_cache, block_tables, context_lens, scale=...)"""

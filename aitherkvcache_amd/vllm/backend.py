@@ -188,7 +188,7 @@ def _make_impl_class():
 
     from ..fused_attention import TQPagedAttention
     from ..fused_kv_update import fused_encode_and_store, fused_kv_update_pair
-    from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store
+    from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store_pair
     from . import hooks
     from .cache import TQGPUCache
     from .decompress import batch_decompress_active_blocks
@@ -299,8 +299,7 @@ def _make_impl_class():
             k_rows, v_rows = primary_views(kv_cache, self.head_size, fmt)
             block_size = kv_cache.shape[2]
             if fmt.kind == "hybrid":
-                hybrid_encode_and_store(tq, key, slot_mapping, k_rows, block_size=block_size)
-                hybrid_encode_and_store(tq, value, slot_mapping, v_rows, block_size=block_size)
+                hybrid_encode_and_store_pair(tq, key, value, slot_mapping, k_rows, v_rows, block_size=block_size)
                 return
             self._ensure_norms(kv_cache)
             li = self._tq_layer_idx

@@ -18,7 +18,7 @@ import torch
 
 from ..fused_attention import TQPagedAttention
 from ..fused_kv_update import fused_kv_update_pair
-from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store
+from ..hybrid_attention import HybridPagedAttention, hybrid_encode_and_store_pair
 from ..hybrid_quantizer import HybridTurboQuant
 from ..quantizer import TurboQuant
 
@@ -82,8 +82,7 @@ def hybrid_decode_step(query, key, value, kv_cache, output, slot_mapping, block_
     key_cache, value_cache = kv_cache[:, 0], kv_cache[:, 1]
     block_size = key_cache.shape[1]
     n = key.shape[0]
-    hybrid_encode_and_store(htq, key, slot_mapping[:n], key_cache, block_size=block_size)
-    hybrid_encode_and_store(htq, value, slot_mapping[:n], value_cache, block_size=block_size)
+    hybrid_encode_and_store_pair(htq, key, value, slot_mapping[:n], key_cache, value_cache, block_size=block_size)
     attn = _tq_fused_attn.get((layer_idx, head_size))
     if attn is None:
         attn = HybridPagedAttention(htq, num_heads)

@@ -262,6 +262,13 @@ int akv_hybrid_encode_paged(const void* x, int x_dtype, int64_t num_tokens, int 
                             const void* slot_mapping, int slot_itype, const float* hyb_table,
                             uint8_t* out, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
                             int block_size, int64_t max_blocks, void* stream);
+/* K and V of a step in one call (both tensors with the strides given, both caches with the strides given): the two
+ * encodes of tq::hybrid_decode_step, aither_kvcache/vllm/hooks.py:271-284; one launch while the call is small. */
+int akv_hybrid_encode_paged_kv(const void* x_k, const void* x_v, int x_dtype, int64_t num_tokens, int num_kv_heads,
+                               int64_t xs_token, int64_t xs_head,
+                               const void* slot_mapping, int slot_itype, const float* hyb_table,
+                               uint8_t* out_k, uint8_t* out_v, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                               int block_size, int64_t max_blocks, void* stream);
 int akv_hybrid_decode(const uint8_t* packed, int64_t packed_stride_bytes, int64_t n,
                       const float* hyb_table, float* out, int64_t out_stride, void* stream);
 /* Decode attention over a tq35 paged cache.  The reference has no fused kernel for this: its
@@ -304,6 +311,11 @@ int akv_hybrid25_encode_paged(const void* x, int x_dtype, int64_t num_tokens, in
                               const void* slot_mapping, int slot_itype, const float* hyb_table,
                               uint8_t* out, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
                               int block_size, int64_t max_blocks, void* stream);
+int akv_hybrid25_encode_paged_kv(const void* x_k, const void* x_v, int x_dtype, int64_t num_tokens, int num_kv_heads,
+                                 int64_t xs_token, int64_t xs_head,
+                                 const void* slot_mapping, int slot_itype, const float* hyb_table,
+                                 uint8_t* out_k, uint8_t* out_v, int64_t ps_blk, int64_t ps_pos, int64_t ps_head,
+                                 int block_size, int64_t max_blocks, void* stream);
 int akv_hybrid25_decode(const uint8_t* packed, int64_t packed_stride_bytes, int64_t n,
                         const float* hyb_table, float* out, int64_t out_stride, void* stream);
 int akv_hybrid25_paged_attn(const void* query, int q_dtype, int64_t qs_seq, int64_t qs_head,

@@ -220,3 +220,33 @@ def test_ranked_calibration_is_the_codec_on_permuted_coordinates(tq25, dev):
     ub = u.decode(p).cpu().numpy()
     for k in range(KVH):
         assert np.array_equal(back[:, k, order[k]], ub[:, k])
+
+
+@pytest.mark.parametrize("mode,row", [("tq35", 64), ("tq25", 44)])
+def test_key_and_value_of_a_step_in_one_call(golden, tq25, dev, mode, row):
+    """hybrid_encode_and_store_pair: K and V of a step by one call -- the same bytes as two single calls, for a
+    small step (one launch), a large one (the form for large calls, twice), skipped slots, pitched caches, and
+    tensors whose strides differ (two single calls underneath)."""
+    h = akv.HybridTurboQuant(mode=mode, device=str(dev))
+    h.calibrate_uniform(num_kv_heads=4)
+    rng = np.random.default_rng(61)
+    KVH, BS = 4, 16
+    for T, NB in ((1, 4), (37, 8), (300, 24), (5000, 320)):
+        k, v = t(kv_like(rng, (T, KVH, 128)), dev), t(kv_like(rng, (T, KVH, 128)), dev)
+        slots = rng.permutation(NB * BS)[:T].astype(np.int64)
+        slots[::13] = -1
+        sd = t(slots, dev)
+        kv = torch.full((NB, 2, BS, KVH, row + 4), 0xAB, dtype=torch.uint8, device=dev)      # the serving layout
+        akv.hybrid_encode_and_store_pair(h, k, v, sd, kv[:, 0, :, :, :row], kv[:, 1, :, :, :row], BS)
+        ref = torch.full_like(kv, 0xAB)
+        akv.hybrid_encode_and_store(h, k, sd, ref[:, 0, :, :, :row], BS)
+        akv.hybrid_encode_and_store(h, v, sd, ref[:, 1, :, :, :row], BS)
+        assert torch.equal(kv, ref), (mode, T)
+    wide = torch.zeros(37, KVH, 136, dtype=k.dtype, device=dev)
+    k37, v37 = k[:37].contiguous(), v[:37]
+    wide[..., :128] = v37
+    a = torch.zeros(8, BS, KVH, row, dtype=torch.uint8, device=dev)
+    b = torch.zeros_like(a)
+    sl = torch.arange(37, device=dev)
+    akv.hybrid_encode_and_store_pair(h, k37, wide[..., :128], sl, a, b, BS)
+    assert torch.equal(a.reshape(-1, KVH, row)[:37], h.encode(k37)) and torch.equal(b.reshape(-1, KVH, row)[:37], h.encode(v37))
