@@ -15,6 +15,7 @@
 #include "akv_common.h"
 
 #define BS_THREADS 1024
+#define BS_COLS 4            // table columns per wavefront of the scoring kernel
 
 __global__ __launch_bounds__(64) void bs_update_kernel(const void* __restrict__ bidx, int itype, const uint8_t* __restrict__ kp,
                                                        int64_t ps_tok, int64_t ps_head, const float* __restrict__ kn,
@@ -77,20 +78,36 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const float* __restrict_
   const int64_t ctx = akv_load_index(cl, cl_itype, s);
   const int64_t nb = (ctx + block_size - 1) / block_size;
   const int n = KVH * HD;
-  for (int j = 0; j < 16; ++j) {
-    const int64_t col = (int64_t)blockIdx.x * 64 + wave * 16 + j;
-    if (col >= B) break;
-    float r = -INFINITY;
-    if (col < nb) {
-      int64_t blk = akv_load_index(bt, bt_itype, s * bt_stride + col);
-      blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
-      const float* re = rep_e + (size_t)blk * n;
-      const float* ro = rep_o + (size_t)blk * n;
-      float acc = 0.f;
-      for (int i = lane; i < n; i += 64) acc = fmaf(qm[i], re[i], fmaf(qm[n + i], ro[i], acc));
-      r = akv_wave_sum(acc);
-    }
-    if (lane == 0) scores[(size_t)s * B + col] = r;
+  // A wavefront takes BS_COLS columns at once: their table entries, then their representatives, are requested
+  // together (one column after the other is a chain of two trips to memory per column -- 22 us for 128 columns of
+  // 16 sequences); every column's sum is formed in the order it always was.
+  const int64_t col0 = (int64_t)blockIdx.x * (4 * BS_COLS) + wave * BS_COLS;
+  const float* re[BS_COLS];
+  const float* ro[BS_COLS];
+  bool live[BS_COLS];
+#pragma unroll
+  for (int j = 0; j < BS_COLS; ++j) {
+    const int64_t col = col0 + j;
+    live[j] = col < B && col < nb;
+    int64_t blk = live[j] ? akv_load_index(bt, bt_itype, s * bt_stride + col) : 0;
+    blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
+    re[j] = rep_e + (size_t)blk * n;
+    ro[j] = rep_o + (size_t)blk * n;
+  }
+  float acc[BS_COLS];
+#pragma unroll
+  for (int j = 0; j < BS_COLS; ++j) acc[j] = 0.f;
+  for (int i = lane; i < n; i += 64) {
+    const float qe = qm[i], qo = qm[n + i];
+#pragma unroll
+    for (int j = 0; j < BS_COLS; ++j)
+      if (live[j]) acc[j] = fmaf(qe, re[j][i], fmaf(qo, ro[j][i], acc[j]));
+  }
+#pragma unroll
+  for (int j = 0; j < BS_COLS; ++j) {
+    const int64_t col = col0 + j;
+    const float r = live[j] ? akv_wave_sum(acc[j]) : -INFINITY;
+    if (lane == 0 && col < B) scores[(size_t)s * B + col] = r;
   }
 }
 
@@ -155,14 +172,29 @@ __global__ __launch_bounds__(BS_THREADS) void bs_select_kernel(const float* __re
       if ((key & known) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int above = 0, bucket = 255;
-      for (; bucket > 0; --bucket) {
-        if (above + hist[bucket] >= krem) break;
-        above += hist[bucket];
+    {
+      // the highest bucket at which the count of keys in it and above reaches krem (bucket 0 if none does): thread
+      // b < 256 knows how many keys lie above its bucket from a scan over the buckets, and exactly one thread finds
+      // above < krem <= above + its own count.  (One thread walking down from bucket 255 read up to 255 counters
+      // one after the other, four times: 25-50 us per call.)
+      const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      const int mine = threadIdx.x < 256 ? hist[threadIdx.x] : 0;
+      const int inc = akv_wave_inclusive_scan(mine);
+      if (threadIdx.x < 256 && lane == 63) scan_lds[wave] = inc;
+      __syncthreads();
+      if (threadIdx.x < 256) {
+        int below_waves = 0, total = 0;
+        for (int w = 0; w < 4; ++w) {
+          const int t = scan_lds[w];
+          if (w < wave) below_waves += t;
+          total += t;
+        }
+        const int above = total - (below_waves + inc);       // keys in buckets above this one
+        if (above < krem && (threadIdx.x == 0 || above + mine >= krem)) {
+          sh_prefix = prefix | ((uint32_t)threadIdx.x << shift);
+          sh_krem = krem - above;
+        }
       }
-      sh_prefix = prefix | ((uint32_t)bucket << shift);
-      sh_krem = krem - above;
     }
     __syncthreads();
     prefix = sh_prefix;
@@ -248,7 +280,7 @@ extern "C" int akv_block_scores(const float* q_even, const float* q_odd, const f
   AKV_REQUIRE(q_even && q_odd && rep_even && rep_odd && block_tables && context_lens && scores, "akv_block_scores: null pointer");
   const size_t lds = (size_t)2 * num_kv_heads * half_d * sizeof(float);
   if (lds > 48 * 1024) return akv_fail(AKV_ERR_UNSUPPORTED, "akv_block_scores: kv_heads x half_d = %d too large", num_kv_heads * half_d);
-  const dim3 grid((unsigned)((max_blocks_per_seq + 63) / 64), (unsigned)num_seqs);
+  const dim3 grid((unsigned)((max_blocks_per_seq + 4 * BS_COLS - 1) / (4 * BS_COLS)), (unsigned)num_seqs);
   bs_scores_kernel<<<grid, 256, lds, (hipStream_t)stream>>>(q_even, q_odd, rep_even, rep_odd, block_tables, bt_itype, bt_stride,
                                                            context_lens, cl_itype, num_q_heads, num_kv_heads, half_d,
                                                            max_blocks_per_seq, block_size, num_blocks, scores);
