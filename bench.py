@@ -342,6 +342,24 @@ def cpu_attention_baseline(w, tq, bits, seconds):
     return tokens, compute, [s for s, _ in used]
 
 
+def cpu_attention_loop_form(w, tq, bits, tokens=2048):
+    """The reference's literal CPU attention (a Python loop per token, TQPagedAttentionRef.forward) on a slice:
+    the longest sequence's first `tokens` tokens, one kv head and its four query heads.  Seconds per (token, kv head)."""
+    from oracle import tq_oracle as O
+    R = tq.rotation.cpu().numpy()
+    c = tq.centroids.cpu().numpy()
+    s = int(np.argmax(w["ctx_np"]))
+    n = int(min(tokens, w["ctx_np"][s]))
+    nb = -(-n // 16)
+    blocks = w["tables"][s, :nb].long()
+    kp, kn = w["kp"][blocks][:, :, :1].cpu().numpy(), w["kn"][blocks][:, :, :1].cpu().numpy()
+    vp, vn = w["vp"][blocks][:, :, :1].cpu().numpy(), w["vn"][blocks][:, :, :1].cpu().numpy()
+    q = w["q"][s:s + 1, :4].cpu().numpy()
+    t0 = time.perf_counter()
+    O.paged_attention_loop(q, kp, kn, vp, vn, np.arange(nb)[None], np.array([n]), R, c, bits)
+    return (time.perf_counter() - t0) / n, n
+
+
 def cpu_hybrid_baseline(w, tq, seconds):
     """The oracle's tq35 attention (decompress every addressed row, dense softmax attention) on whole
     sequences of the batch, in batch order, until the time budget is used."""
@@ -465,6 +483,11 @@ def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_second
         cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
                    "sample": f"numpy float32 oracle (gather, unpack, codebook, einsum, softmax, einsum, inverse "
                              f"rotation) on whole sequences {seqs} of the batch = {toks} context tokens"}
+        per_tok_s, n_loop = cpu_attention_loop_form(ws[0], tq, bits)
+        cpu_obj["loop_form"] = {"value": per_tok / 8 / per_tok_s / 1e9, "unit": "GB/s", "cores": 1,
+                                "us_per_token_and_kv_head": per_tok_s * 1e6,
+                                "sample": f"the reference's per-token Python loop (TQPagedAttentionRef.forward as the oracle "
+                                          f"restates it) on {n_loop} tokens of the longest sequence, one kv head, four query heads"}
     del ws, calls, attn
     torch.cuda.empty_cache()
     return res, roof, cpu_obj
