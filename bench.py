@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TurboQuant hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode4|decode4_b256|decode3|decode2|tq35|tri|encode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode4|decode4_b256|decode3|decode2|tq35|tq25|tri|encode]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The default workload is the headline one: paged decode attention over a tq-t4nc cache
@@ -23,7 +23,7 @@ having been written by the encode-on-write kernel.  One JSON line is printed:
              360 MB, the size of the headline step's cache: context for the fraction of the nominal peak
 
 Algorithmic bytes per context token = 8 heads x (64 B codes + 4 B norm) x (K and V) = 1088 B
-(104 / 72 / 128 B x 8 for 3-bit / 2-bit / tq35), plus queries, outputs and block tables.
+(104 / 72 / 128 / 88 B x 8 for 3-bit / 2-bit / tq35 / tq25), plus queries, outputs and block tables.
 """
 import argparse
 import ctypes
@@ -59,7 +59,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="decode4",
-                    choices=["decode4", "decode4_b256", "decode3", "decode2", "tq35", "tri", "encode"])
+                    choices=["decode4", "decode4_b256", "decode3", "decode2", "tq35", "tq25", "tri", "encode"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true",
                     help="skip the 3-bit / 2-bit / tq35 / TriAttention workloads that the default run reports beside the headline one")
@@ -283,8 +283,8 @@ def decode_workload(torch, akv, dev, tq, bits_or_mode, seed, num_seqs, ctx):
     KVH, QH, BS = 8, 32, 16
     nblk = -(-ctx // BS)
     NB = int(nblk.sum())
-    hybrid = bits_or_mode == "tq35"
-    P = 64 if hybrid else tq._packed_dim
+    hybrid = bits_or_mode in ("tq35", "tq25")
+    P = tq.layout.packed_dim if hybrid else tq._packed_dim
     kp = torch.zeros(NB, BS, KVH, P, dtype=torch.uint8, device=dev)
     vp = torch.zeros_like(kp)
     kn = vn = None
@@ -361,12 +361,16 @@ def cpu_attention_loop_form(w, tq, bits, tokens=2048):
 
 
 def cpu_hybrid_baseline(w, tq, seconds):
-    """The oracle's tq35 attention (decompress every addressed row, dense softmax attention) on whole
+    """The oracle's tq35 / tq25 attention (decompress every addressed row, dense softmax attention) on whole
     sequences of the batch, in batch order, until the time budget is used."""
     from oracle import tq_oracle as O
     tab = tq.kernel_table.cpu().numpy()
-    hp = O.HybridParams(tab[0:64], tab[64:128], tab[128:192], tab[192:256],
-                        codebooks=((tab[256:264], tab[268:275]), (tab[264:268], tab[275:278])))
+    if tq.mode == "tq25":
+        hp = O.HybridParams(tab[0:32], tab[32:128], tab[128:160], tab[160:256],
+                            codebooks=((tab[256:260], tab[262:265]), (tab[260:262], tab[265:266])), mode="tq25")
+    else:
+        hp = O.HybridParams(tab[0:64], tab[64:128], tab[128:192], tab[192:256],
+                            codebooks=((tab[256:264], tab[268:275]), (tab[264:268], tab[275:278])))
     q = w["q"].float().cpu().numpy()
     tokens, compute, used = 0, 0.0, []
     t0 = time.perf_counter()
@@ -434,11 +438,11 @@ def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_second
         bits, per_tok, tq = 4, 1088, tq4
     else:
         ctx = np.full(64, 8192, dtype=np.int64)
-        bits = {"decode3": 3, "decode2": 2, "tq35": "tq35"}[workload]
-        per_tok = {"decode3": 8 * 104, "decode2": 8 * 72, "tq35": 8 * 128}[workload]
+        bits = {"decode3": 3, "decode2": 2, "tq35": "tq35", "tq25": "tq25"}[workload]
+        per_tok = {"decode3": 8 * 104, "decode2": 8 * 72, "tq35": 8 * 128, "tq25": 8 * 88}[workload]
         name = f"config 3: paged decode attention, {workload}, 32Q/8KV d=128, batch 64 x 8192, block 16, seed 3"
-        if bits == "tq35":
-            tq = akv.HybridTurboQuant(device=str(dev))
+        if bits in ("tq35", "tq25"):
+            tq = akv.HybridTurboQuant(mode=bits, device=str(dev))
             tq.calibrate_uniform(8)
         else:
             tq = akv.TurboQuant(head_dim=128, bits=bits, device=str(dev))
@@ -446,7 +450,7 @@ def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_second
     # two copies of the cache, alternated, so that no step finds its data in the 256 MB
     # last-level cache left by the previous one
     ws = [decode_workload(torch, akv, dev, tq, bits, seed + 100 * i, len(ctx), ctx) for i in range(2)]
-    if bits == "tq35":
+    if bits in ("tq35", "tq25"):
         attn = akv.HybridPagedAttention(tq, 32)
         calls = [lambda w=w: attn.forward(w["q"], w["kp"], w["vp"], w["tables"], w["ctx"], scale=1 / math.sqrt(128))
                  for w in ws]
@@ -465,7 +469,8 @@ def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_second
     ms = timed(torch, step, steps, warmup)
     kms = kernel_ms(torch, L, step, max(20, steps))
     res = dict(metric="tq-t4nc paged-decode attn GB/s" if workload == "decode4" else f"{workload} paged-decode attn GB/s",
-               value=algo_bytes / ms / 1e6, ms_per_step=ms, dtype=DECODE_DTYPE,
+               value=algo_bytes / ms / 1e6, ms_per_step=ms,
+               dtype="f32 (vector kernels, no matrix cores)" if bits == "tq25" else DECODE_DTYPE,
                config={"workload": name, "context_tokens": tokens, "algorithmic_bytes_per_step": algo_bytes,
                        "cache_copies_alternated": 2, "preconditioning_s": PRECONDITION_S})
     achieved = tokens * per_tok / kms / 1e6
@@ -473,7 +478,7 @@ def run_decode(torch, akv, L, dev, workload, tq4, steps, warmup, cpu, cpu_second
             **traffic_fields(workload), "kernel": "main decode-attention kernel", "kernel_ms": kms,
             "algorithmic_bytes_per_launch": tokens * per_tok}
     cpu_obj = None
-    if cpu and bits == "tq35":
+    if cpu and bits in ("tq35", "tq25"):
         toks, secs, what = cpu_hybrid_baseline(ws[0], tq, cpu_seconds)
         cpu_obj = {"value": toks * per_tok / secs / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
                    "sample": f"numpy float32 oracle (hybrid_decode of every addressed row, dense softmax "
@@ -589,7 +594,7 @@ def main():
            "scaling": "weak", "vs_baseline": None, "data": "synthetic", "unit": "GB/s"}
     cpu_obj = None
 
-    if args.workload in ("decode4", "decode4_b256", "decode3", "decode2", "tq35"):
+    if args.workload in ("decode4", "decode4_b256", "decode3", "decode2", "tq35", "tq25"):
         res, roof, cpu_obj = run_decode(torch, akv, L, dev, args.workload, tq4, args.steps, args.warmup, cpu,
                                         args.cpu_seconds, cores)
         out.update(res)
