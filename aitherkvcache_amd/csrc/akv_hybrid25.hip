@@ -262,28 +262,55 @@ __global__ __launch_bounds__(256) void h25_attn_prologue_kernel(
 }
 
 #define H25_WAVES 8
-#define H25_VROW 11      // dwords of a row (an odd pitch: the lanes' rows start in different banks)
+#define H25_VDW 11       // dwords of a row
+#define H25_LUT_POS 144  // two-bit fields of a row's code and sign bytes (9 dwords x 16)
 
+typedef uint32_t h25_u4 __attribute__((ext_vector_type(4)));
+typedef float h25_f4 __attribute__((ext_vector_type(4)));
+template <int GQ>
+struct alignas(GQ * 4) h25_qv { float v[GQ]; };
+
+// LDS of one wavefront, in floats:
+//   lut [144][4][GQ]   partial dot products of the GQ query heads with the coordinates a two-bit field of a key
+//                      row covers, for each of its four values (a 2-bit code: one coordinate of group 0; two
+//                      1-bit codes or two sign bits: two coordinates)
+//   p   [GQ][4][64]    weights of the chunk's tokens: p vn0 | p vn0 vr0 kappa0 | p vn1 | p vn1 vr1 kappa1
+//   v   [11][64]       the chunk's value rows, dword-major (token = lane)
 template <int GQ>
 struct h25_attn_cfg {
-  static constexpr size_t wave_floats = 64 * GQ * 4 + 64 * H25_VROW;
-  static size_t lds_bytes(int QH) { return ((size_t)QH * 256 + H25_WAVES * wave_floats + 8) * 4; }
+  static constexpr size_t lut_floats = (size_t)H25_LUT_POS * 4 * GQ;
+  static constexpr size_t wave_floats = lut_floats + 64 * GQ * 4 + 64 * H25_VDW;
+  static size_t lds_bytes(int) { return (H25_WAVES * wave_floats + 8) * 4; }
 };
 
 template <int GQ>
 __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
   typedef h25_attn_cfg<GQ> cfg;
+  typedef h25_qv<GQ> qv;
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  float* q_lds = (float*)lds_raw;                          // [QH][256]
-  float* wave_base = q_lds + (size_t)a.QH * 256;
+  float* wave_base = (float*)lds_raw;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float* p_lds = wave_base + wave * cfg::wave_floats;      // [64][GQ][4]
-  uint32_t* v_lds = (uint32_t*)(p_lds + 64 * GQ * 4);      // [64][11]
-  float* cen = wave_base + H25_WAVES * cfg::wave_floats;   // 4 + 2 centroids
-  if (threadIdx.x < 6) cen[threadIdx.x] = a.table[H25_CEN0 + threadIdx.x];
-  const float* cen0 = cen;
-  const float* cen1 = cen + 4;
+  qv* lut = (qv*)(wave_base + wave * cfg::wave_floats);
+  float* p_lds = wave_base + wave * cfg::wave_floats + cfg::lut_floats;
+  uint32_t* v_lds = (uint32_t*)(p_lds + 64 * GQ * 4);
+  float cen0[4], cen1[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) cen0[i] = a.table[H25_CEN0 + i];
+  cen1[0] = a.table[H25_CEN1]; cen1[1] = a.table[H25_CEN1 + 1];
   const h25_roles r(lane);
+
+  // value phase, lane = coordinate pair: where the lane's bits sit in a row (dword, shift) and what they mean
+  const int sh_a = 8 * ((lane >> 3) & 3) + 7 - (lane & 7);
+  const int dw_a = 4 + (lane >> 5);                 // group-1 code dword; its sign dword is 3 further
+  const int jb = 32 + lane;                         // lanes 32..63: position of the second coordinate in group 1
+  const int dw_bm = r.b0 ? (lane >> 4) : 6;
+  const int sh_bm = r.b0 ? 8 * ((lane >> 2) & 3) + 6 - 2 * (lane & 3) : 8 * ((jb >> 3) & 3) + 7 - (jb & 7);
+  const uint32_t mask_b = r.b0 ? 3u : 1u;
+  const int dw_bs = r.b0 ? 2 : 9;
+  const int sh_bs = r.b0 ? 8 * (lane >> 3) + 7 - (lane & 7) : sh_bm;
+  const float tb0 = r.b0 ? cen0[0] : cen1[0], tb1 = r.b0 ? cen0[1] : cen1[1];
+  const float tb2 = r.b0 ? cen0[2] : cen1[0], tb3 = r.b0 ? cen0[3] : cen1[1];
+  const int kb_m = r.b0 ? 0 : 2, kb_s = r.b0 ? 1 : 3;
 
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
@@ -304,13 +331,35 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
     const int t1 = (int)min((int64_t)blk_hi * bs, ctx);
     g = sb0 + blk_hi;
 
-    __syncthreads();
-    for (int i = threadIdx.x; i < a.QH * 256; i += blockDim.x)
-      q_lds[i] = a.qt[(size_t)s * a.QH * 256 + i];
-    __syncthreads();
-
     for (int h = wave; h < a.KVH; h += H25_WAVES) {
       for (int qg = 0; qg < gqa; qg += GQ) {
+        // ---- table of the group's query heads (the wavefront's previous look-ups are done: LDS is in order)
+        {
+          const float* Q = a.qt + ((size_t)s * a.QH + (h * gqa + qg)) * 256;
+          for (int e = lane; e < H25_LUT_POS * 4; e += 64) {
+            const int pos = e >> 2, v = e & 3;
+            const int di = pos >> 4, b = (pos >> 2) & 3, k = pos & 3;
+            qv o;
+            if (di < 2) {
+#pragma unroll
+              for (int q = 0; q < GQ; ++q) o.v[q] = Q[q * 256 + pos] * cen0[v];
+            } else {
+              const bool sign = di == 2 || di >= 6;
+              const int base = di == 2 ? 128 : (di < 6 ? 32 : 160);
+              const int ob = di == 2 ? b : 4 * ((di - 3) % 3) + b;
+              const int j0 = base + 8 * ob + 2 * k;
+              const float f_hi = sign ? ((v & 2) ? 1.f : -1.f) : cen1[v >> 1];
+              const float f_lo = sign ? ((v & 1) ? 1.f : -1.f) : cen1[v & 1];
+#pragma unroll
+              for (int q = 0; q < GQ; ++q) o.v[q] = fmaf(Q[q * 256 + j0], f_hi, Q[q * 256 + j0 + 1] * f_lo);
+            }
+            lut[e] = o;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
         float m[GQ], l[GQ], acc[GQ][4];
 #pragma unroll
         for (int q = 0; q < GQ; ++q) {
@@ -318,7 +367,6 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[q][i] = 0.f;
         }
-        const float* qh = q_lds + (size_t)(h * gqa + qg) * 256;
 
         for (int c0 = t0; c0 < t1; c0 += 64) {
           const int t = c0 + lane;
@@ -326,46 +374,40 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
           const int tc = valid ? t : t1 - 1;
           const int64_t phys = akv_clamp_block(akv_load_index(a.block_tables, a.bt_itype, s * a.bt_stride + tc / bs), a.num_blocks);
           const int pos = tc % bs;
-          // ---- scores: lane = token, its key row in registers
-          uint32_t row[H25_VROW];
+          // ---- scores: lane = token, its key row in registers, one look-up per two-bit field
+          uint32_t row[H25_VDW], vrow[H25_VDW];
           {
             const uint32_t* kr = (const uint32_t*)(a.kc + phys * a.kps_blk + pos * a.kps_pos + h * a.kps_head);
+            const uint32_t* vr = (const uint32_t*)(a.vc + phys * a.vps_blk + pos * a.vps_pos + h * a.vps_head);
 #pragma unroll
-            for (int i = 0; i < H25_VROW; ++i) row[i] = kr[i];
+            for (int i = 0; i < H25_VDW; ++i) row[i] = kr[i];
+#pragma unroll
+            for (int i = 0; i < H25_VDW; ++i) vrow[i] = vr[i];
           }
-          auto kb = [&](int o) { return (row[o >> 2] >> (8 * (o & 3))) & 0xffu; };
           float d0[GQ], e0[GQ], d1[GQ], e1[GQ];
 #pragma unroll
           for (int q = 0; q < GQ; ++q) { d0[q] = e0[q] = d1[q] = e1[q] = 0.f; }
 #pragma unroll
-          for (int j = 0; j < 32; ++j) {
-            const float cv = cen0[akv_stream_code<2>(j, kb)];
-            const float sv = ((kb(8 + (j >> 3)) >> (7 - (j & 7))) & 1u) ? 1.f : -1.f;
+          for (int di = 0; di < 9; ++di) {
+            const uint32_t w = row[di < 3 ? di : di + 1];
 #pragma unroll
-            for (int q = 0; q < GQ; ++q) {
-              d0[q] = fmaf(qh[q * 256 + j], cv, d0[q]);
-              e0[q] = fmaf(qh[q * 256 + 128 + j], sv, e0[q]);
-            }
-          }
+            for (int c = 0; c < 16; ++c) {
+              const uint32_t v = (w >> (8 * (c >> 2) + 6 - 2 * (c & 3))) & 3u;
+              const qv e = lut[(16 * di + c) * 4 + v];
 #pragma unroll
-          for (int j = 0; j < 96; ++j) {
-            const float cv = cen1[(kb(16 + (j >> 3)) >> (7 - (j & 7))) & 1u];
-            const float sv = ((kb(28 + (j >> 3)) >> (7 - (j & 7))) & 1u) ? 1.f : -1.f;
-#pragma unroll
-            for (int q = 0; q < GQ; ++q) {
-              d1[q] = fmaf(qh[q * 256 + 32 + j], cv, d1[q]);
-              e1[q] = fmaf(qh[q * 256 + 160 + j], sv, e1[q]);
+              for (int q = 0; q < GQ; ++q) {
+                if (di < 2) d0[q] += e.v[q];
+                else if (di == 2) e0[q] += e.v[q];
+                else if (di < 6) d1[q] += e.v[q];
+                else e1[q] += e.v[q];
+              }
             }
           }
           const float kn0 = h25_half_bits_to_float(row[3]), kr0 = h25_half_bits_to_float(row[3] >> 16);
           const float kn1 = h25_half_bits_to_float(row[10]), kr1 = h25_half_bits_to_float(row[10] >> 16);
-          // ---- value row: norms from registers, codes through LDS
-          uint32_t vrow[H25_VROW];
-          {
-            const uint32_t* vr = (const uint32_t*)(a.vc + phys * a.vps_blk + pos * a.vps_pos + h * a.vps_head);
+          // ---- value rows go to LDS dword-major; their norms stay here
 #pragma unroll
-            for (int i = 0; i < H25_VROW; ++i) { vrow[i] = vr[i]; v_lds[lane * H25_VROW + i] = vrow[i]; }
-          }
+          for (int i = 0; i < H25_VDW; ++i) v_lds[i * 64 + lane] = vrow[i];
           const float vn0 = h25_half_bits_to_float(vrow[3]), vr0 = h25_half_bits_to_float(vrow[3] >> 16);
           const float vn1 = h25_half_bits_to_float(vrow[10]), vr1 = h25_half_bits_to_float(vrow[10] >> 16);
 #pragma unroll
@@ -380,26 +422,46 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[q][i] *= alpha;
             m[q] = mn;
-            float4 pw;
-            pw.x = p * vn0; pw.y = p * vn0 * vr0 * kH25Kappa0; pw.z = p * vn1; pw.w = p * vn1 * vr1 * kH25Kappa1;
-            *(float4*)(p_lds + (lane * GQ + q) * 4) = pw;
+            float* pw = p_lds + q * 256 + lane;
+            pw[0] = valid ? p * vn0 : 0.f;
+            pw[64] = valid ? p * vn0 * vr0 * kH25Kappa0 : 0.f;
+            pw[128] = valid ? p * vn1 : 0.f;
+            pw[192] = valid ? p * vn1 * vr1 * kH25Kappa1 : 0.f;
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          // ---- value sums: lane = coordinate pair, one token after the other
+          // ---- value sums: lane = coordinate pair, four tokens per read (the weights of tokens past the end are zero)
           const int nt = min(64, t1 - c0);
-          for (int tt = 0; tt < nt; ++tt) {
-            const uint8_t* vb = (const uint8_t*)(v_lds + tt * H25_VROW);
-            float cen_a, sg_a, cen_b, sg_b;
-            h25_row_values(r, [&](int o) { return (uint32_t)vb[o]; }, cen0, cen1, cen_a, sg_a, cen_b, sg_b);
+          for (int t4 = 0; t4 < nt; t4 += 4) {
+            const h25_u4 wam = *(const h25_u4*)(v_lds + dw_a * 64 + t4);
+            const h25_u4 was = *(const h25_u4*)(v_lds + (dw_a + 3) * 64 + t4);
+            const h25_u4 wbm = *(const h25_u4*)(v_lds + dw_bm * 64 + t4);
+            const h25_u4 wbs = *(const h25_u4*)(v_lds + dw_bs * 64 + t4);
+            float cen_a[4], nsg_a[4], cen_b[4], nsg_b[4];     // nsg = -sign: bit set -> -1
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t xam = wam[i], xas = was[i], xbm = wbm[i], xbs = wbs[i];
+              cen_a[i] = ((xam >> sh_a) & 1u) ? cen1[1] : cen1[0];
+              nsg_a[i] = __uint_as_float((((xas >> sh_a) & 1u) << 31) | 0x3f800000u);
+              const uint32_t cb = (xbm >> sh_bm) & mask_b;
+              const float lo = (cb & 1u) ? tb1 : tb0, hi = (cb & 1u) ? tb3 : tb2;
+              cen_b[i] = (cb & 2u) ? hi : lo;
+              nsg_b[i] = __uint_as_float((((xbs >> sh_bs) & 1u) << 31) | 0x3f800000u);
+            }
 #pragma unroll
             for (int q = 0; q < GQ; ++q) {
-              const float4 pw = *(const float4*)(p_lds + (tt * GQ + q) * 4);
-              acc[q][0] = fmaf(pw.z, cen_a, acc[q][0]);
-              acc[q][1] = fmaf(pw.w, sg_a, acc[q][1]);
-              acc[q][2] = fmaf(r.b0 ? pw.x : pw.z, cen_b, acc[q][2]);
-              acc[q][3] = fmaf(r.b0 ? pw.y : pw.w, sg_b, acc[q][3]);
+              const float* pq = p_lds + q * 256 + t4;
+              const h25_f4 pz = *(const h25_f4*)(pq + 128), pw = *(const h25_f4*)(pq + 192);
+              const h25_f4 pbm = *(const h25_f4*)(pq + kb_m * 64), pbs = *(const h25_f4*)(pq + kb_s * 64);
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const float z = pz[i], w = pw[i], bm = pbm[i], bsw = pbs[i];
+                acc[q][0] = fmaf(z, cen_a[i], acc[q][0]);
+                acc[q][1] = fmaf(-w, nsg_a[i], acc[q][1]);
+                acc[q][2] = fmaf(bm, cen_b[i], acc[q][2]);
+                acc[q][3] = fmaf(-bsw, nsg_b[i], acc[q][3]);
+              }
             }
           }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
