@@ -305,12 +305,13 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
   const int jb = 32 + lane;                         // lanes 32..63: position of the second coordinate in group 1
   const int dw_bm = r.b0 ? (lane >> 4) : 6;
   const int sh_bm = r.b0 ? 8 * ((lane >> 2) & 3) + 6 - 2 * (lane & 3) : 8 * ((jb >> 3) & 3) + 7 - (jb & 7);
-  const uint32_t mask_b = r.b0 ? 3u : 1u;
   const int dw_bs = r.b0 ? 2 : 9;
   const int sh_bs = r.b0 ? 8 * (lane >> 3) + 7 - (lane & 7) : sh_bm;
   const float tb0 = r.b0 ? cen0[0] : cen1[0], tb1 = r.b0 ? cen0[1] : cen1[1];
   const float tb2 = r.b0 ? cen0[2] : cen1[0], tb3 = r.b0 ? cen0[3] : cen1[1];
   const int kb_m = r.b0 ? 0 : 2, kb_s = r.b0 ? 1 : 3;
+  const uint32_t c1lo = __float_as_uint(cen1[0]), c1hi = __float_as_uint(cen1[1]);
+  const uint32_t ub0 = __float_as_uint(tb0), ub1 = __float_as_uint(tb1), ub2 = __float_as_uint(tb2), ub3 = __float_as_uint(tb3);
 
   const int G = gridDim.x;
   const int total = a.prefix[a.S];
@@ -442,12 +443,16 @@ __global__ __launch_bounds__(512) void h25_attn_kernel(h25_attn_args a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const uint32_t xam = wam[i], xas = was[i], xbm = wbm[i], xbs = wbs[i];
-              cen_a[i] = ((xam >> sh_a) & 1u) ? cen1[1] : cen1[0];
-              nsg_a[i] = __uint_as_float((((xas >> sh_a) & 1u) << 31) | 0x3f800000u);
-              const uint32_t cb = (xbm >> sh_bm) & mask_b;
-              const float lo = (cb & 1u) ? tb1 : tb0, hi = (cb & 1u) ? tb3 : tb2;
-              cen_b[i] = (cb & 2u) ? hi : lo;
-              nsg_b[i] = __uint_as_float((((xbs >> sh_bs) & 1u) << 31) | 0x3f800000u);
+              // a bit as a mask of 32 (one signed bit-field extract), values picked by bitwise select
+              const uint32_t ma = (uint32_t)__builtin_amdgcn_sbfe((int)xam, sh_a, 1);
+              cen_a[i] = __uint_as_float((c1hi & ma) | (c1lo & ~ma));
+              nsg_a[i] = __uint_as_float(((uint32_t)__builtin_amdgcn_sbfe((int)xas, sh_a, 1) & 0x80000000u) | 0x3f800000u);
+              // lanes of group 1 have tb2 = tb0 and tb3 = tb1: whatever sits in the bit above their code changes nothing
+              const uint32_t m0 = (uint32_t)__builtin_amdgcn_sbfe((int)xbm, sh_bm, 1);
+              const uint32_t m1 = (uint32_t)__builtin_amdgcn_sbfe((int)xbm, sh_bm + 1, 1);
+              const uint32_t lo = (ub1 & m0) | (ub0 & ~m0), hi = (ub3 & m0) | (ub2 & ~m0);
+              cen_b[i] = __uint_as_float((hi & m1) | (lo & ~m1));
+              nsg_b[i] = __uint_as_float(((uint32_t)__builtin_amdgcn_sbfe((int)xbs, sh_bs, 1) & 0x80000000u) | 0x3f800000u);
             }
 #pragma unroll
             for (int q = 0; q < GQ; ++q) {
